@@ -1,0 +1,190 @@
+"""The cache of a model: a slot for each live sequence; per group of layers
+with the same needs, paged keys and values with a block table; beside them,
+fixed-size state per slot.
+
+Layout of a key/value group (``entries`` = schedule entries that keep a cache
+in this group):
+    k  [entries, pages, kv_heads, 64, head_dim]   a token's key is a row
+    v  [entries, pages, kv_heads, head_dim, 64]   a page's keys are contiguous per channel
+    block_table [slots, max_pages_per_slot] int32, on the device
+The reference's cache is [layer][kv_head][capacity][head_dim] per session
+(/root/reference/crates/nnis-rt/src/kv_cache.rs:1-5,98-110); pages replace the
+fixed capacity so that the memory follows the tokens actually held.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Any, Dict, List, Optional, Sequence, Tuple
+
+import torch
+
+from ..errors import CacheFull, InvalidInput
+from ..parts.base import KVRequest, StateRequest
+from .allocator import PAGE_TOKENS, FreeList, PageTable, pages_for
+
+
+@dataclass
+class KVView:
+    """What an attention-like mixer sees of the cache for one schedule entry."""
+
+    k_pages: torch.Tensor  # [pages, kv_heads, 64, head_dim]
+    v_pages: torch.Tensor  # [pages, kv_heads, head_dim, 64]
+    block_table: torch.Tensor  # [slots, max_pages_per_slot]
+    window: Optional[int]
+    read_only: bool  # this run reads another entry's cache and writes nothing
+
+
+@dataclass
+class StateView:
+    """Fixed-size state: one row per slot, zero when a sequence starts."""
+
+    state: torch.Tensor  # [slots, *shape]
+    read_only: bool
+
+
+class KVGroup:
+    def __init__(self, request: KVRequest, entries: List[int], pages: int, slots: int, max_positions: int,
+                 dtype: torch.dtype, device):
+        self.request = request
+        self.entries = entries  # schedule indices, in order
+        # a windowed group has storage and pages of its own; it keeps every
+        # page of a sequence (the kernels mask by the window), so that a whole
+        # prompt can be written before its scores are taken
+        per_slot = min(pages, pages_for(max_positions))
+        self.table = PageTable(pages, slots, per_slot)
+        self.k = torch.empty((len(entries), pages, request.kv_heads, PAGE_TOKENS, request.head_dim), dtype=dtype, device=device)
+        self.v = torch.empty((len(entries), pages, request.kv_heads, request.head_dim, PAGE_TOKENS), dtype=dtype, device=device)
+        pinned = torch.device(device).type == "cuda"
+        self.block_table_host = torch.zeros((slots, per_slot), dtype=torch.int32, pin_memory=pinned)
+        self.block_table = torch.zeros((slots, per_slot), dtype=torch.int32, device=device)
+        self._dirty = set()
+
+    def bytes_per_token(self) -> int:
+        return 2 * len(self.entries) * self.request.kv_heads * self.request.head_dim * self.k.element_size()
+
+    def grow(self, slot: int, new_length: int) -> None:
+        changed = self.table.grow(slot, new_length)
+        if changed:
+            row = self.table.rows[slot]
+            for index in changed:
+                self.block_table_host[slot, index] = row[index]
+            self._dirty.add(slot)
+
+    def flush(self) -> None:
+        """Copies the block-table rows that changed to the device."""
+        for slot in sorted(self._dirty):
+            self.block_table[slot].copy_(self.block_table_host[slot], non_blocking=True)
+        self._dirty.clear()
+
+
+class SequenceCache:
+    """Slots, pages and state for one model on one device.
+
+    ``max_tokens`` is the most tokens live sequences hold at any time, each
+    sequence's count rounded up to a whole page."""
+
+    def __init__(self, requests: Sequence[Tuple[int, Any]], shared: Dict[int, int], max_tokens: int, max_positions: int,
+                 dtype: torch.dtype, device, max_slots: Optional[int] = None):
+        """``requests``: (schedule index, KVRequest | StateRequest | None) for
+        entries that keep a cache; ``shared``: schedule index -> index of the
+        entry whose cache it reads."""
+        if max_tokens <= 0:
+            raise InvalidInput(f"max_tokens must be positive; got {max_tokens}")
+        self.device = torch.device(device)
+        self.dtype = dtype
+        self.max_positions = max_positions
+        self.pages = pages_for(max_tokens)
+        self.max_slots = min(self.pages, max_slots) if max_slots else self.pages
+        self.slots = FreeList(self.max_slots, "cache slot")
+        self.lengths: Dict[int, int] = {}
+
+        self.kv_groups: List[KVGroup] = []
+        self.state_regions: Dict[str, torch.Tensor] = {}
+        self._views: Dict[int, Any] = {}
+        grouped: Dict[KVRequest, List[int]] = {}
+        for index, request in requests:
+            if isinstance(request, KVRequest):
+                grouped.setdefault(request, []).append(index)
+            elif isinstance(request, StateRequest):
+                region = self.add_state_region(f"entry{index}", request.shape, getattr(torch, request.dtype))
+                self._views[index] = StateView(region, read_only=False)
+            elif request is not None:
+                raise InvalidInput(f"schedule entry {index}: unknown cache request {request!r}")
+        for request, entries in grouped.items():
+            group = KVGroup(request, entries, self.pages, self.max_slots, max_positions, dtype, self.device)
+            self.kv_groups.append(group)
+            for position, index in enumerate(entries):
+                self._views[index] = KVView(group.k[position], group.v[position], group.block_table, request.window, False)
+        for index, owner in shared.items():
+            view = self._views.get(owner)
+            if isinstance(view, KVView):
+                self._views[index] = KVView(view.k_pages, view.v_pages, view.block_table, view.window, True)
+            elif isinstance(view, StateView):
+                self._views[index] = StateView(view.state, True)
+
+    # ---- state regions ----------------------------------------------------
+    def add_state_region(self, name: str, shape: Sequence[int], dtype: torch.dtype) -> torch.Tensor:
+        if name in self.state_regions:
+            raise InvalidInput(f"state region {name!r} exists already")
+        region = torch.zeros((self.max_slots, *shape), dtype=dtype, device=self.device)
+        self.state_regions[name] = region
+        return region
+
+    def view(self, schedule_index: int):
+        return self._views.get(schedule_index)
+
+    # ---- slots ---------------------------------------------------------------
+    def acquire(self) -> int:
+        slot = self.slots.take()
+        self.lengths[slot] = 0
+        for region in self.state_regions.values():
+            region[slot].zero_()
+        return slot
+
+    def release(self, slot: int) -> None:
+        self.slots.give_back(slot)
+        del self.lengths[slot]
+        for group in self.kv_groups:
+            group.table.release(slot)
+
+    def length(self, slot: int) -> int:
+        try:
+            return self.lengths[slot]
+        except KeyError:
+            raise InvalidInput(f"cache slot {slot} is not held") from None
+
+    def check_room(self, growth: Dict[int, int]) -> None:
+        """Raises before anything changes if the slots cannot grow by the given
+        token counts (all or nothing, as the reference's append:
+        /root/reference/crates/nnis-rt/src/kv_cache.rs:223-228)."""
+        for group in self.kv_groups:
+            need = 0
+            for slot, extra in growth.items():
+                new_length = self.length(slot) + extra
+                if new_length > self.max_positions:
+                    raise CacheFull(
+                        f"slot {slot} would hold {new_length} tokens; the model's positions end at {self.max_positions}"
+                    )
+                need += group.table.pages_needed(slot, new_length)
+            if need > group.table.pool.free:
+                raise CacheFull(
+                    f"the cache has {group.table.pool.free} free pages of {PAGE_TOKENS} tokens; this step needs {need}"
+                )
+
+    def grow(self, growth: Dict[int, int]) -> None:
+        """Reserves pages for the new tokens and advances the lengths."""
+        self.check_room(growth)
+        for slot, extra in growth.items():
+            new_length = self.lengths[slot] + extra
+            for group in self.kv_groups:
+                group.grow(slot, new_length)
+            self.lengths[slot] = new_length
+        for group in self.kv_groups:
+            group.flush()
+
+    def bytes_per_token(self) -> int:
+        return sum(group.bytes_per_token() for group in self.kv_groups)
+
+    def live_tokens(self) -> int:
+        return sum(self.lengths.values())

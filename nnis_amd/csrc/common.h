@@ -1,0 +1,98 @@
+// Shared helpers of the gfx950 kernels: element types, loads that widen to
+// 32-bit, wave and block reductions, and the error channel of the C entry
+// points.  Every entry point returns 0 on success; on refusal it returns a
+// non-zero code and leaves a message for nnis_last_error().
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+
+typedef __bf16 bf16_t;
+
+// element type codes shared with the Python side
+enum : int { NNIS_F32 = 0, NNIS_BF16 = 1 };
+
+constexpr int kWave = 64;        // lanes of a gfx950 wavefront
+constexpr int kPageTokens = 64;  // tokens a cache page holds
+
+extern thread_local char g_nnis_error[512];
+
+static inline int nnis_fail(const char* fmt, ...) {
+  va_list args;
+  va_start(args, fmt);
+  vsnprintf(g_nnis_error, sizeof(g_nnis_error), fmt, args);
+  va_end(args);
+  return 1;
+}
+
+#define NNIS_REQUIRE(cond, ...)                  \
+  do {                                           \
+    if (!(cond)) return nnis_fail(__VA_ARGS__);  \
+  } while (0)
+
+#define NNIS_LAUNCH_CHECK(name)                                                        \
+  do {                                                                                 \
+    hipError_t launch_error = hipGetLastError();                                       \
+    if (launch_error != hipSuccess)                                                    \
+      return nnis_fail("%s: launch failed: %s", name, hipGetErrorString(launch_error)); \
+  } while (0)
+
+static inline bool nnis_dtype_ok(int dtype) { return dtype == NNIS_F32 || dtype == NNIS_BF16; }
+static inline int nnis_dtype_size(int dtype) { return dtype == NNIS_F32 ? 4 : 2; }
+
+// ---- typed access -----------------------------------------------------------
+
+__device__ __forceinline__ float to_f32(float v) { return v; }
+__device__ __forceinline__ float to_f32(bf16_t v) { return (float)v; }
+
+template <typename T>
+__device__ __forceinline__ T from_f32(float v);
+template <>
+__device__ __forceinline__ float from_f32<float>(float v) { return v; }
+template <>
+__device__ __forceinline__ bf16_t from_f32<bf16_t>(float v) { return (bf16_t)v; }  // round to nearest even
+
+// element `index` of an array whose element type is only known at run time;
+// the branch is uniform over a launch
+__device__ __forceinline__ float load_as_f32(const void* base, int dtype, size_t index) {
+  return dtype == NNIS_F32 ? ((const float*)base)[index] : (float)((const bf16_t*)base)[index];
+}
+
+__device__ __forceinline__ void store_from_f32(void* base, int dtype, size_t index, float value) {
+  if (dtype == NNIS_F32) {
+    ((float*)base)[index] = value;
+  } else {
+    ((bf16_t*)base)[index] = (bf16_t)value;
+  }
+}
+
+// ---- reductions ---------------------------------------------------------------
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int offset = kWave / 2; offset > 0; offset >>= 1) v += __shfl_xor(v, offset, kWave);
+  return v;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int offset = kWave / 2; offset > 0; offset >>= 1) v = fmaxf(v, __shfl_xor(v, offset, kWave));
+  return v;
+}
+
+// sum over a block of up to 1024 threads; `scratch` holds at least 16 floats;
+// every thread gets the result
+__device__ __forceinline__ float block_sum(float v, float* scratch) {
+  const int lane = threadIdx.x % kWave;
+  const int wave = threadIdx.x / kWave;
+  const int waves = (blockDim.x + kWave - 1) / kWave;
+  v = wave_sum(v);
+  __syncthreads();  // scratch may still be read from a previous call
+  if (lane == 0) scratch[wave] = v;
+  __syncthreads();
+  float total = 0.0f;
+  for (int w = 0; w < waves; ++w) total += scratch[w];
+  return total;
+}

@@ -1,0 +1,307 @@
+// Row-wise kernels of the decoder: embedding gather, RMSNorm (optionally fused
+// with the residual sum and a row gather), rotate-half RoPE fused with the
+// write of keys and values into cache pages, SiLU-multiply and argmax.
+// Storage types are chosen at run time (32-bit float or bfloat16); every sum,
+// statistic and rotation is computed in 32-bit.
+#include "common.h"
+
+thread_local char g_nnis_error[512] = {0};
+
+extern "C" const char* nnis_last_error() { return g_nnis_error; }
+
+// -----------------------------------------------------------------------------
+// embedding: out[t, :] = table[ids[t], :]   (a row copy, no scaling;
+// /root/reference/crates/nnis-kernels/src/gather.rs:17-33)
+// -----------------------------------------------------------------------------
+__global__ void embed_kernel(const int* __restrict__ ids, const void* __restrict__ table, int table_dtype,
+                             float* __restrict__ out, int width, int vocab) {
+  const int token = blockIdx.x;
+  const int id = ids[token];
+  float* dst = out + (size_t)token * width;
+  if (id < 0 || id >= vocab) {  // padding rows carry -1; never read outside the table
+    for (int c = threadIdx.x; c < width; c += blockDim.x) dst[c] = 0.0f;
+    return;
+  }
+  const size_t base = (size_t)id * width;
+  for (int c = threadIdx.x; c < width; c += blockDim.x) dst[c] = load_as_f32(table, table_dtype, base + c);
+}
+
+extern "C" int nnis_embed(const int* ids, const void* table, int table_dtype, float* out, int tokens, int width,
+                          int vocab, void* stream) {
+  NNIS_REQUIRE(nnis_dtype_ok(table_dtype), "embed: unknown table dtype %d", table_dtype);
+  NNIS_REQUIRE(tokens >= 0 && width > 0 && vocab > 0, "embed: bad sizes tokens=%d width=%d vocab=%d", tokens, width, vocab);
+  if (tokens == 0) return 0;
+  hipLaunchKernelGGL(embed_kernel, dim3(tokens), dim3(256), 0, (hipStream_t)stream, ids, table, table_dtype, out,
+                     width, vocab);
+  NNIS_LAUNCH_CHECK("embed");
+  return 0;
+}
+
+// -----------------------------------------------------------------------------
+// RMSNorm: y[c] = (x[c] * (1/sqrt(mean(x^2) + eps))) * w[c]
+// (/root/reference/crates/nnis-model/src/kernels.rs:15-48: eps inside the
+// root, mean over the row, x*scale*weight in that order).
+//   delta != null : the row normalised is x + delta (sum in 32-bit); without
+//                   `rows` the sum is written back to x, which must be 32-bit.
+//   rows  != null : output row r reads input row rows[r]; nothing is written back.
+// -----------------------------------------------------------------------------
+__global__ void rmsnorm_kernel(void* __restrict__ x, int x_dtype, const void* __restrict__ delta, int delta_dtype,
+                               const void* __restrict__ weight, int weight_dtype, void* __restrict__ out,
+                               int out_dtype, const int* __restrict__ rows, int width, float inv_width, float eps) {
+  __shared__ float scratch[16];
+  const int out_row = blockIdx.x;
+  const int in_row = rows ? rows[out_row] : out_row;
+  const size_t in_base = (size_t)in_row * width;
+  const size_t out_base = (size_t)out_row * width;
+  const bool write_back = delta != nullptr && rows == nullptr;
+
+  float sumsq = 0.0f;
+  for (int c = threadIdx.x; c < width; c += blockDim.x) {
+    float v = load_as_f32(x, x_dtype, in_base + c);
+    if (delta) {
+      v += load_as_f32(delta, delta_dtype, in_base + c);
+      if (write_back) ((float*)x)[in_base + c] = v;
+    }
+    sumsq = fmaf(v, v, sumsq);
+  }
+  const float total = block_sum(sumsq, scratch);
+  const float scale = 1.0f / sqrtf(total * inv_width + eps);
+  for (int c = threadIdx.x; c < width; c += blockDim.x) {
+    float v = load_as_f32(x, x_dtype, in_base + c);  // holds the sum already when written back
+    if (delta && !write_back) v += load_as_f32(delta, delta_dtype, in_base + c);
+    store_from_f32(out, out_dtype, out_base + c, (v * scale) * load_as_f32(weight, weight_dtype, c));
+  }
+}
+
+extern "C" int nnis_rmsnorm(void* x, int x_dtype, const void* delta, int delta_dtype, const void* weight,
+                            int weight_dtype, void* out, int out_dtype, const int* rows, int out_rows, int width,
+                            float eps, void* stream) {
+  NNIS_REQUIRE(nnis_dtype_ok(x_dtype) && nnis_dtype_ok(weight_dtype) && nnis_dtype_ok(out_dtype),
+               "rmsnorm: unknown dtype (x %d, weight %d, out %d)", x_dtype, weight_dtype, out_dtype);
+  NNIS_REQUIRE(delta == nullptr || nnis_dtype_ok(delta_dtype), "rmsnorm: unknown delta dtype %d", delta_dtype);
+  NNIS_REQUIRE(!(delta != nullptr && rows == nullptr && x_dtype != NNIS_F32),
+               "rmsnorm: the residual sum is kept in 32-bit; x must be float32 when delta is added in place");
+  NNIS_REQUIRE(out_rows >= 0 && width > 0, "rmsnorm: bad sizes rows=%d width=%d", out_rows, width);
+  NNIS_REQUIRE(eps > 0.0f, "rmsnorm: eps must be positive, got %g", (double)eps);
+  if (out_rows == 0) return 0;
+  const int threads = width >= 1024 ? 256 : (width >= 256 ? 128 : 64);
+  hipLaunchKernelGGL(rmsnorm_kernel, dim3(out_rows), dim3(threads), 0, (hipStream_t)stream, x, x_dtype, delta,
+                     delta_dtype, weight, weight_dtype, out, out_dtype, rows, width, 1.0f / (float)width, eps);
+  NNIS_LAUNCH_CHECK("rmsnorm");
+  return 0;
+}
+
+// -----------------------------------------------------------------------------
+// rotate-half RoPE on queries and keys, fused with the cache write.
+//   qkv   [tokens, (heads + 2*kv_heads) * head_dim] : q heads, then k heads, then v heads
+//   q_out [tokens, heads * head_dim]
+//   K page layout  [page][kv_head][token in page][head_dim]
+//   V page layout  [page][kv_head][head_dim][token in page]   (keys contiguous)
+// pair j < rot_dim/2 of a head:  out[j] = x[j]*c - x[j+half]*s,
+//                                out[j+half] = x[j+half]*c + x[j]*s
+// with (c, s) = table[pos][j]  (/root/reference/crates/nnis-model/src/runtime_kernels.rs:38-66);
+// elements at and beyond rot_dim pass through.  V is not rotated
+// (/root/reference/crates/nnis-model/src/runtime.rs:997-1016).
+// A token whose slot is negative is padding: nothing is written for it.
+// -----------------------------------------------------------------------------
+struct RopeWriteArgs {
+  const void* qkv;
+  int qkv_dtype;
+  void* q_out;
+  int q_dtype;
+  const float* cos_table;  // [positions][rot_dim/2] or null (no rotation)
+  const float* sin_table;
+  int table_positions;
+  int rot_dim;
+  const int* tok_slot;
+  const int* tok_pos;
+  void* k_pages;  // null: this run keeps no cache of its own
+  void* v_pages;
+  int cache_dtype;
+  const int* block_table;  // [slots][max_pages]
+  int max_pages;
+  int heads, kv_heads, head_dim;
+};
+
+__global__ void rope_kv_write_kernel(RopeWriteArgs a) {
+  const int token = blockIdx.x;
+  const int slot = a.tok_slot[token];
+  if (slot < 0) return;
+  const int pos = a.tok_pos[token];
+  const int hd = a.head_dim;
+  const int half = a.rot_dim / 2;
+  const int row_width = (a.heads + 2 * a.kv_heads) * hd;
+  const size_t in_base = (size_t)token * row_width;
+  const bool rotate = a.cos_table != nullptr && pos < a.table_positions;
+  const float* cos_row = rotate ? a.cos_table + (size_t)pos * half : nullptr;
+  const float* sin_row = rotate ? a.sin_table + (size_t)pos * half : nullptr;
+
+  int page = -1;
+  if (a.k_pages) page = a.block_table[(size_t)slot * a.max_pages + pos / kPageTokens];
+  const int in_page = pos % kPageTokens;
+
+  // queries and keys: one work item per (head, element below head_dim/2 or pass-through element)
+  const int rot_heads = a.heads + a.kv_heads;
+  const int items_per_head = hd - half;  // `half` rotated pairs + (hd - rot_dim) pass-through elements
+  for (int item = threadIdx.x; item < rot_heads * items_per_head; item += blockDim.x) {
+    const int head = item / items_per_head;
+    const int e = item % items_per_head;
+    const size_t src = in_base + (size_t)head * hd;
+    float lo, hi = 0.0f;
+    int lo_index, hi_index = -1;
+    if (e < half) {
+      const float x0 = load_as_f32(a.qkv, a.qkv_dtype, src + e);
+      const float x1 = load_as_f32(a.qkv, a.qkv_dtype, src + e + half);
+      float c = 1.0f, s = 0.0f;
+      if (rotate) {
+        c = cos_row[e];
+        s = sin_row[e];
+      }
+      lo = x0 * c - x1 * s;
+      hi = x1 * c + x0 * s;
+      lo_index = e;
+      hi_index = e + half;
+    } else {
+      lo_index = e + half;  // element index in [rot_dim, head_dim)
+      lo = load_as_f32(a.qkv, a.qkv_dtype, src + lo_index);
+    }
+    if (head < a.heads) {
+      const size_t dst = ((size_t)token * a.heads + head) * hd;
+      store_from_f32(a.q_out, a.q_dtype, dst + lo_index, lo);
+      if (hi_index >= 0) store_from_f32(a.q_out, a.q_dtype, dst + hi_index, hi);
+    } else if (page >= 0) {
+      const int kv_head = head - a.heads;
+      const size_t dst = (((size_t)page * a.kv_heads + kv_head) * kPageTokens + in_page) * hd;
+      store_from_f32(a.k_pages, a.cache_dtype, dst + lo_index, lo);
+      if (hi_index >= 0) store_from_f32(a.k_pages, a.cache_dtype, dst + hi_index, hi);
+    }
+  }
+  // values: copied, transposed into the page
+  if (page >= 0) {
+    const size_t v_src = in_base + (size_t)(a.heads + a.kv_heads) * hd;
+    for (int item = threadIdx.x; item < a.kv_heads * hd; item += blockDim.x) {
+      const int kv_head = item / hd;
+      const int d = item % hd;
+      const float v = load_as_f32(a.qkv, a.qkv_dtype, v_src + item);
+      const size_t dst = (((size_t)page * a.kv_heads + kv_head) * hd + d) * kPageTokens + in_page;
+      store_from_f32(a.v_pages, a.cache_dtype, dst, v);
+    }
+  }
+}
+
+extern "C" int nnis_rope_kv_write(const void* qkv, int qkv_dtype, void* q_out, int q_dtype, const float* cos_table,
+                                  const float* sin_table, int table_positions, int rot_dim, const int* tok_slot,
+                                  const int* tok_pos, void* k_pages, void* v_pages, int cache_dtype,
+                                  const int* block_table, int max_pages, int tokens, int heads, int kv_heads,
+                                  int head_dim, void* stream) {
+  NNIS_REQUIRE(nnis_dtype_ok(qkv_dtype) && nnis_dtype_ok(q_dtype), "rope_kv_write: unknown dtype");
+  NNIS_REQUIRE(k_pages == nullptr || nnis_dtype_ok(cache_dtype), "rope_kv_write: unknown cache dtype %d", cache_dtype);
+  NNIS_REQUIRE((k_pages == nullptr) == (v_pages == nullptr), "rope_kv_write: key and value pages must come together");
+  NNIS_REQUIRE(k_pages == nullptr || (block_table != nullptr && max_pages > 0), "rope_kv_write: cache without a block table");
+  NNIS_REQUIRE(heads > 0 && kv_heads > 0 && head_dim > 0, "rope_kv_write: bad head sizes %d/%d/%d", heads, kv_heads, head_dim);
+  NNIS_REQUIRE(rot_dim >= 0 && rot_dim <= head_dim && rot_dim % 2 == 0,
+               "rope_kv_write: rot_dim %d must be even and at most head_dim %d", rot_dim, head_dim);
+  NNIS_REQUIRE((cos_table == nullptr) == (sin_table == nullptr), "rope_kv_write: cos and sin tables must come together");
+  if (tokens <= 0) return 0;
+  RopeWriteArgs a;
+  a.qkv = qkv; a.qkv_dtype = qkv_dtype; a.q_out = q_out; a.q_dtype = q_dtype;
+  a.cos_table = cos_table; a.sin_table = sin_table; a.table_positions = table_positions;
+  a.rot_dim = cos_table ? rot_dim : 0;
+  a.tok_slot = tok_slot; a.tok_pos = tok_pos; a.k_pages = k_pages; a.v_pages = v_pages;
+  a.cache_dtype = cache_dtype; a.block_table = block_table; a.max_pages = max_pages;
+  a.heads = heads; a.kv_heads = kv_heads; a.head_dim = head_dim;
+  const int work = (heads + 2 * kv_heads) * head_dim / 2;
+  const int threads = work >= 512 ? 256 : (work >= 128 ? 128 : 64);
+  hipLaunchKernelGGL(rope_kv_write_kernel, dim3(tokens), dim3(threads), 0, (hipStream_t)stream, a);
+  NNIS_LAUNCH_CHECK("rope_kv_write");
+  return 0;
+}
+
+// -----------------------------------------------------------------------------
+// SiLU-multiply on a fused [tokens, 2*inner] projection (gate columns first):
+// out = gate / (1 + exp(-gate)) * up
+// (/root/reference/crates/nnis-model/src/fused_swiglu.rs:14-28)
+// -----------------------------------------------------------------------------
+__global__ void silu_mul_kernel(const void* __restrict__ gate_up, int in_dtype, void* __restrict__ out, int out_dtype,
+                                int inner, size_t total) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+    const size_t row = i / inner;
+    const size_t col = i % inner;
+    const float g = load_as_f32(gate_up, in_dtype, row * 2 * inner + col);
+    const float u = load_as_f32(gate_up, in_dtype, row * 2 * inner + inner + col);
+    const float act = g / (1.0f + expf(-g));
+    store_from_f32(out, out_dtype, i, act * u);
+  }
+}
+
+extern "C" int nnis_silu_mul(const void* gate_up, int in_dtype, void* out, int out_dtype, int tokens, int inner,
+                             void* stream) {
+  NNIS_REQUIRE(nnis_dtype_ok(in_dtype) && nnis_dtype_ok(out_dtype), "silu_mul: unknown dtype");
+  NNIS_REQUIRE(tokens >= 0 && inner > 0, "silu_mul: bad sizes tokens=%d inner=%d", tokens, inner);
+  if (tokens == 0) return 0;
+  const size_t total = (size_t)tokens * inner;
+  size_t blocks = (total + 255) / 256;
+  if (blocks > 65536) blocks = 65536;
+  hipLaunchKernelGGL(silu_mul_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, gate_up, in_dtype,
+                     out, out_dtype, inner, total);
+  NNIS_LAUNCH_CHECK("silu_mul");
+  return 0;
+}
+
+// -----------------------------------------------------------------------------
+// argmax per row, lowest index on ties
+// (/root/reference/crates/nnis-kernels/src/top_k.rs:41-92: value descending,
+// then lower index).  NaN never wins.
+// -----------------------------------------------------------------------------
+__device__ __forceinline__ bool better(float v, int i, float best_v, int best_i) {
+  return v > best_v || (v == best_v && i < best_i);
+}
+
+__global__ void argmax_kernel(const float* __restrict__ logits, int* __restrict__ out, int vocab) {
+  __shared__ float s_val[16];
+  __shared__ int s_idx[16];
+  const float* row = logits + (size_t)blockIdx.x * vocab;
+  float best_v = -INFINITY;
+  int best_i = 0x7fffffff;
+  for (int c = threadIdx.x; c < vocab; c += blockDim.x) {
+    const float v = row[c];
+    if (better(v, c, best_v, best_i)) {
+      best_v = v;
+      best_i = c;
+    }
+  }
+#pragma unroll
+  for (int offset = kWave / 2; offset > 0; offset >>= 1) {
+    const float ov = __shfl_xor(best_v, offset, kWave);
+    const int oi = __shfl_xor(best_i, offset, kWave);
+    if (better(ov, oi, best_v, best_i)) {
+      best_v = ov;
+      best_i = oi;
+    }
+  }
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  if (lane == 0) {
+    s_val[wave] = best_v;
+    s_idx[wave] = best_i;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    const int waves = (blockDim.x + kWave - 1) / kWave;
+    for (int w = 1; w < waves; ++w) {
+      if (better(s_val[w], s_idx[w], best_v, best_i)) {
+        best_v = s_val[w];
+        best_i = s_idx[w];
+      }
+    }
+    out[blockIdx.x] = best_i == 0x7fffffff ? 0 : best_i;
+  }
+}
+
+extern "C" int nnis_argmax(const float* logits, int* out, int rows, int vocab, void* stream) {
+  NNIS_REQUIRE(rows >= 0 && vocab > 0, "argmax: bad sizes rows=%d vocab=%d", rows, vocab);
+  if (rows == 0) return 0;
+  const int threads = vocab >= 8192 ? 1024 : (vocab >= 1024 ? 256 : 64);
+  hipLaunchKernelGGL(argmax_kernel, dim3(rows), dim3(threads), 0, (hipStream_t)stream, logits, out, vocab);
+  NNIS_LAUNCH_CHECK("argmax");
+  return 0;
+}

@@ -1,0 +1,35 @@
+"""What one step brings: for each sequence its slot, its next tokens and the
+places whose logits are wanted.  ``StepContext`` is the same on the device:
+per packed token its slot and position, per sequence where it starts.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import List, Optional, Sequence
+
+import torch
+
+
+@dataclass
+class StepEntry:
+    slot: int
+    tokens: Sequence[int]
+    want: Optional[Sequence[int]] = None  # indices into tokens; None: the last one
+
+
+@dataclass
+class StepContext:
+    tokens: int  # packed tokens of the step (rows of every activation)
+    batch: int  # sequences of the step
+    tok_slot: torch.Tensor  # int32 [tokens]; negative marks a padding row
+    tok_pos: torch.Tensor  # int32 [tokens]: position of the token in its sequence
+    seq_slot: torch.Tensor  # int32 [batch]
+    seq_start: torch.Tensor  # int32 [batch + 1]: first packed row of each sequence
+    seq_pos0: torch.Tensor  # int32 [batch]: position of each sequence's first new token
+    decode: bool  # every sequence brings exactly one token
+    max_new: int  # most tokens any sequence brings
+    max_len: int  # longest sequence after this step
+    host_slots: List[int] = field(default_factory=list)
+    host_new: List[int] = field(default_factory=list)
+    host_pos0: List[int] = field(default_factory=list)

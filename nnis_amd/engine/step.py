@@ -1,0 +1,135 @@
+"""The step function: runs exactly the tokens it is given, as one batch, from
+the cache that earlier steps left, and returns the logits at the wanted
+places.  Sequences of a step may have any lengths; a prompt goes in one step,
+then one token at a time.  The reference's two entry points, ``prefill`` and
+``decode_one`` (/root/reference/crates/nnis-model/src/runtime.rs:756-790), are
+both this call; its validation rules (runtime.rs:1134-1163) are kept, and a
+refused step changes nothing.
+"""
+
+from __future__ import annotations
+
+from typing import List, Optional, Sequence
+
+import numpy as np
+import torch
+
+from ..cache import SequenceCache
+from ..errors import InvalidInput
+from .batch import StepContext, StepEntry
+
+
+class Engine:
+    def __init__(self, model, rt, max_tokens: int, max_slots: Optional[int] = None):
+        if not model.bound:
+            raise InvalidInput("the model has no weights bound; load it first")
+        self.model = model
+        self.rt = rt
+        self.vocab_size = model.spec.vocab_size
+        requests, shared = model.cache_requests()
+        self.cache = SequenceCache(requests, shared, max_tokens, model.spec.max_positions, rt.dtype, rt.device, max_slots)
+        self._staging = None
+        self._staging_dev = None
+
+    # ---- sequences -----------------------------------------------------------
+    def start_sequence(self) -> int:
+        return self.cache.acquire()
+
+    def end_sequence(self, slot: int) -> None:
+        self.cache.release(slot)
+
+    def length(self, slot: int) -> int:
+        return self.cache.length(slot)
+
+    # ---- one step ------------------------------------------------------------
+    def _validate(self, entries: Sequence[StepEntry]):
+        if not entries:
+            raise InvalidInput("a step needs at least one sequence")
+        seen = set()
+        growth = {}
+        for entry in entries:
+            if entry.slot in seen:
+                raise InvalidInput(f"slot {entry.slot} appears twice in one step")
+            seen.add(entry.slot)
+            self.cache.length(entry.slot)  # raises if the slot is not held
+            count = len(entry.tokens)
+            if count == 0:
+                raise InvalidInput(f"slot {entry.slot}: a step needs at least one token per sequence")
+            for token in entry.tokens:
+                if not 0 <= int(token) < self.vocab_size:
+                    # runtime.rs:1155-1163
+                    raise InvalidInput(f"token id {token} is out of range for vocabulary {self.vocab_size}")
+            if entry.want is not None:
+                for place in entry.want:
+                    if not 0 <= int(place) < count:
+                        raise InvalidInput(f"slot {entry.slot}: wanted place {place} is not among its {count} tokens")
+            growth[entry.slot] = count
+        self.cache.check_room(growth)
+        return growth
+
+    def _stage(self, arrays: List[np.ndarray]) -> List[torch.Tensor]:
+        """One pinned buffer, one copy to the device, views per array."""
+        total = sum(a.size for a in arrays)
+        if self._staging is None or self._staging.numel() < total:
+            size = max(1024, 1 << (total - 1).bit_length())
+            self._staging = torch.empty(size, dtype=torch.int32, pin_memory=True)
+            self._staging_dev = torch.empty(size, dtype=torch.int32, device=self.rt.device)
+        host = self._staging.numpy()
+        offset = 0
+        spans = []
+        for array in arrays:
+            host[offset:offset + array.size] = array
+            spans.append((offset, array.size))
+            offset += array.size
+        # the previous step's kernels may still read the device buffer: the
+        # copy is ordered after them on the same stream
+        self._staging_dev[:total].copy_(self._staging[:total], non_blocking=True)
+        return [self._staging_dev[o:o + n] for o, n in spans]
+
+    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        """Returns float32 logits [wanted places, vocab], in the order of the
+        entries and of each entry's ``want``."""
+        growth = self._validate(entries)
+        pos0 = [self.cache.length(e.slot) for e in entries]
+        counts = [len(e.tokens) for e in entries]
+        total = sum(counts)
+        ids = np.empty(total, dtype=np.int32)
+        tok_slot = np.empty(total, dtype=np.int32)
+        tok_pos = np.empty(total, dtype=np.int32)
+        seq_start = np.zeros(len(entries) + 1, dtype=np.int32)
+        want_rows: List[int] = []
+        row = 0
+        for index, entry in enumerate(entries):
+            n = counts[index]
+            ids[row:row + n] = np.asarray(entry.tokens, dtype=np.int32)
+            tok_slot[row:row + n] = entry.slot
+            tok_pos[row:row + n] = np.arange(pos0[index], pos0[index] + n, dtype=np.int32)
+            places = [n - 1] if entry.want is None else entry.want
+            want_rows.extend(row + int(p) for p in places)
+            row += n
+            seq_start[index + 1] = row
+        self.cache.grow(growth)
+
+        # the staging buffer is reused: wait until the previous step's copy has left it
+        torch.cuda.current_stream().synchronize() if self._staging is not None else None
+        dev = self._stage([
+            ids, tok_slot, tok_pos,
+            np.asarray([e.slot for e in entries], dtype=np.int32), seq_start,
+            np.asarray(pos0, dtype=np.int32), np.asarray(want_rows, dtype=np.int32),
+        ])
+        ctx = StepContext(
+            tokens=total,
+            batch=len(entries),
+            tok_slot=dev[1],
+            tok_pos=dev[2],
+            seq_slot=dev[3],
+            seq_start=dev[4],
+            seq_pos0=dev[5],
+            decode=all(n == 1 for n in counts),
+            max_new=max(counts),
+            max_len=max(p + n for p, n in zip(pos0, counts)),
+            host_slots=[e.slot for e in entries],
+            host_new=counts,
+            host_pos0=pos0,
+        )
+        return self.model.forward(dev[0], ctx, self.cache, dev[6], self.rt)

@@ -1,0 +1,253 @@
+"""Python face of the HIP kernels: checks operands against what a kernel and
+its grid assume, then launches it on the current stream.  Every function here
+runs hand-written device code; none has a host or library stand-in.
+"""
+
+from __future__ import annotations
+
+import ctypes
+from typing import Optional
+
+import torch
+
+from ..errors import KernelError
+from . import lib as _lib
+
+PAGE_TOKENS = 64
+
+_VOID = ctypes.c_void_p
+_INT = ctypes.c_int
+_FLT = ctypes.c_float
+_U64 = ctypes.c_uint64
+
+_CORE_SIGNATURES = {
+    "nnis_embed": [_VOID, _VOID, _INT, _VOID, _INT, _INT, _INT, _VOID],
+    "nnis_rmsnorm": [_VOID, _INT, _VOID, _INT, _VOID, _INT, _VOID, _INT, _VOID, _INT, _INT, _FLT, _VOID],
+    "nnis_rope_kv_write": [_VOID, _INT, _VOID, _INT, _VOID, _VOID, _INT, _INT, _VOID, _VOID, _VOID, _VOID, _INT,
+                           _VOID, _INT, _INT, _INT, _INT, _INT, _VOID],
+    "nnis_silu_mul": [_VOID, _INT, _VOID, _INT, _INT, _INT, _VOID],
+    "nnis_argmax": [_VOID, _VOID, _INT, _INT, _VOID],
+    "nnis_gemm_ordered": [_VOID, _INT, _VOID, _INT, _VOID, _INT, _INT, _INT, _INT, _VOID],
+}
+_ATTN_SIGNATURES = {
+    "nnis_attention_rows": [_VOID, _INT, _VOID, _INT, _VOID, _VOID, _INT, _VOID, _INT, _VOID, _VOID, _INT, _INT, _INT,
+                            _INT, _INT, _FLT, _VOID],
+}
+
+_DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1}
+
+
+def _code(t: torch.Tensor) -> int:
+    try:
+        return _DTYPE_CODE[t.dtype]
+    except KeyError:
+        raise KernelError(f"kernels take float32 or bfloat16 tensors, got {t.dtype}") from None
+
+
+def _bind(module: str, signatures):
+    lib = _lib.load_module(module)
+    if not getattr(lib, "_nnis_bound", False):
+        for name, argtypes in signatures.items():
+            fn = getattr(lib, name, None)
+            if fn is None:
+                continue  # a kernel that is not in this build; calling it raises below
+            fn.argtypes = argtypes
+            fn.restype = ctypes.c_int
+        lib._nnis_bound = True
+    return lib
+
+
+_core = None
+_attn = {}
+
+
+def core():
+    global _core
+    if _core is None:
+        _core = _bind("core", _CORE_SIGNATURES)
+    return _core
+
+
+def attention_module(head_dim: int):
+    if head_dim not in _attn:
+        if head_dim <= 0 or head_dim % 2 != 0 or head_dim > 256:
+            raise KernelError(f"attention kernels take an even head_dim up to 256, got {head_dim}")
+        _attn[head_dim] = _bind(f"attn_hd{head_dim}", _ATTN_SIGNATURES)
+    return _attn[head_dim]
+
+
+def _check(lib, status: int) -> None:
+    if status != 0:
+        raise KernelError(lib.nnis_last_error().decode(errors="replace"))
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _dev(t: torch.Tensor, what: str) -> None:
+    if not t.is_cuda:
+        raise KernelError(f"{what} must live on the GPU; this library has no host path")
+    if not t.is_contiguous():
+        raise KernelError(f"{what} must be contiguous")
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+# ---------------------------------------------------------------------------
+
+def embed(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[t, :] = table[ids[t], :] widened to 32-bit; ids outside the table give a zero row."""
+    _dev(ids, "ids"), _dev(table, "embedding table"), _dev(out, "out")
+    tokens, width = out.shape
+    if ids.dtype != torch.int32 or ids.numel() < tokens:
+        raise KernelError(f"embed: ids must be int32 with at least {tokens} entries")
+    if table.dim() != 2 or table.shape[1] != width or out.dtype != torch.float32:
+        raise KernelError(f"embed: table {tuple(table.shape)} / out {tuple(out.shape)} {out.dtype} do not fit")
+    lib = core()
+    _check(lib, lib.nnis_embed(ids.data_ptr(), table.data_ptr(), _code(table), out.data_ptr(), tokens, width,
+                               table.shape[0], _stream()))
+    return out
+
+
+def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor,
+            delta: Optional[torch.Tensor] = None, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out = rmsnorm(x [+ delta]) * weight.  Without ``rows`` and with ``delta``
+    the sum is written back into ``x`` (32-bit).  With ``rows`` (int32), output
+    row r reads input row rows[r]."""
+    _dev(x, "x"), _dev(weight, "norm weight"), _dev(out, "out")
+    width = x.shape[-1]
+    if weight.numel() != width or out.shape[-1] != width:
+        raise KernelError(f"rmsnorm: width {width} against weight {tuple(weight.shape)} and out {tuple(out.shape)}")
+    out_rows = out.numel() // width
+    if rows is None:
+        if x.numel() // width != out_rows:
+            raise KernelError(f"rmsnorm: {x.numel() // width} input rows against {out_rows} output rows")
+    else:
+        _dev(rows, "rows")
+        if rows.dtype != torch.int32 or rows.numel() < out_rows:
+            raise KernelError("rmsnorm: rows must be int32 with one entry per output row")
+    if delta is not None:
+        _dev(delta, "delta")
+        if delta.shape != x.shape:
+            raise KernelError(f"rmsnorm: delta {tuple(delta.shape)} against x {tuple(x.shape)}")
+    lib = core()
+    _check(lib, lib.nnis_rmsnorm(x.data_ptr(), _code(x), _ptr(delta), _code(delta) if delta is not None else 0,
+                                 weight.data_ptr(), _code(weight), out.data_ptr(), _code(out), _ptr(rows), out_rows,
+                                 width, float(eps), _stream()))
+    return out
+
+
+def rope_kv_write(qkv: torch.Tensor, q_out: torch.Tensor, cos: Optional[torch.Tensor], sin: Optional[torch.Tensor],
+                  rot_dim: int, tok_slot: torch.Tensor, tok_pos: torch.Tensor, k_pages: Optional[torch.Tensor],
+                  v_pages: Optional[torch.Tensor], block_table: Optional[torch.Tensor], heads: int, kv_heads: int,
+                  head_dim: int) -> torch.Tensor:
+    """Rotates queries and keys by their positions and writes keys and values
+    into the pages of each token's slot.  ``k_pages`` is
+    ``[pages, kv_heads, 64, head_dim]``, ``v_pages`` ``[pages, kv_heads,
+    head_dim, 64]``; both ``None`` for a run that keeps no cache of its own."""
+    _dev(qkv, "qkv"), _dev(q_out, "q_out"), _dev(tok_slot, "tok_slot"), _dev(tok_pos, "tok_pos")
+    tokens = qkv.shape[0]
+    if qkv.shape[1] != (heads + 2 * kv_heads) * head_dim or q_out.shape != (tokens, heads * head_dim):
+        raise KernelError(f"rope_kv_write: qkv {tuple(qkv.shape)} / q_out {tuple(q_out.shape)} do not fit "
+                          f"{heads}+2*{kv_heads} heads of {head_dim}")
+    if tok_slot.dtype != torch.int32 or tok_pos.dtype != torch.int32 or tok_slot.numel() < tokens or tok_pos.numel() < tokens:
+        raise KernelError("rope_kv_write: tok_slot / tok_pos must be int32 with one entry per token")
+    table_positions = 0
+    if cos is not None:
+        _dev(cos, "cos"), _dev(sin, "sin")
+        if cos.dtype != torch.float32 or sin.dtype != torch.float32 or cos.shape != sin.shape or cos.shape[1] != rot_dim // 2:
+            raise KernelError(f"rope_kv_write: tables {tuple(cos.shape)} do not fit rot_dim {rot_dim} in float32")
+        table_positions = cos.shape[0]
+    max_pages = 0
+    cache_code = 0
+    if k_pages is not None:
+        _dev(k_pages, "k_pages"), _dev(v_pages, "v_pages"), _dev(block_table, "block_table")
+        if tuple(k_pages.shape[1:]) != (kv_heads, PAGE_TOKENS, head_dim) or tuple(v_pages.shape[1:]) != (kv_heads, head_dim, PAGE_TOKENS):
+            raise KernelError(f"rope_kv_write: page shapes {tuple(k_pages.shape)} / {tuple(v_pages.shape)} do not fit")
+        if block_table.dtype != torch.int32 or block_table.dim() != 2:
+            raise KernelError("rope_kv_write: block_table must be int32 [slots, pages]")
+        max_pages = block_table.shape[1]
+        cache_code = _code(k_pages)
+    lib = core()
+    _check(lib, lib.nnis_rope_kv_write(qkv.data_ptr(), _code(qkv), q_out.data_ptr(), _code(q_out), _ptr(cos), _ptr(sin),
+                                       table_positions, rot_dim, tok_slot.data_ptr(), tok_pos.data_ptr(),
+                                       _ptr(k_pages), _ptr(v_pages), cache_code, _ptr(block_table), max_pages, tokens,
+                                       heads, kv_heads, head_dim, _stream()))
+    return q_out
+
+
+def silu_mul(gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    _dev(gate_up, "gate_up"), _dev(out, "out")
+    tokens, inner = out.shape
+    if gate_up.shape != (tokens, 2 * inner):
+        raise KernelError(f"silu_mul: gate_up {tuple(gate_up.shape)} against out {tuple(out.shape)}")
+    lib = core()
+    _check(lib, lib.nnis_silu_mul(gate_up.data_ptr(), _code(gate_up), out.data_ptr(), _code(out), tokens, inner, _stream()))
+    return out
+
+
+def argmax(logits: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    _dev(logits, "logits"), _dev(out, "out")
+    rows, vocab = logits.shape
+    if logits.dtype != torch.float32 or out.dtype != torch.int32 or out.numel() < rows:
+        raise KernelError("argmax: logits must be float32 [rows, vocab] and out int32 [rows]")
+    lib = core()
+    _check(lib, lib.nnis_argmax(logits.data_ptr(), out.data_ptr(), rows, vocab, _stream()))
+    return out
+
+
+def gemm_ordered(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[M, N] = x[M, K] @ w[N, K]^T, each element one ascending-k chain of
+    32-bit fused multiply-adds."""
+    _dev(x, "x"), _dev(w, "weight"), _dev(out, "out")
+    m, k = x.shape
+    n = w.shape[0]
+    if w.shape[1] != k or out.shape != (m, n):
+        raise KernelError(f"gemm: x {tuple(x.shape)} w {tuple(w.shape)} out {tuple(out.shape)} do not fit")
+    lib = core()
+    _check(lib, lib.nnis_gemm_ordered(x.data_ptr(), _code(x), w.data_ptr(), _code(w), out.data_ptr(), _code(out), m, n, k,
+                                      _stream()))
+    return out
+
+
+def attention_rows(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
+                   block_table: torch.Tensor, tok_slot: torch.Tensor, tok_pos: torch.Tensor, heads: int, kv_heads: int,
+                   head_dim: int, scale: float, window: int = 0) -> torch.Tensor:
+    """Causal attention of each token over the cached keys of its slot up to
+    its own position (32-bit arithmetic, any storage type)."""
+    _dev(q, "q"), _dev(out, "out"), _dev(k_pages, "k_pages"), _dev(v_pages, "v_pages"), _dev(block_table, "block_table")
+    tokens = q.shape[0]
+    if q.shape != (tokens, heads * head_dim) or out.shape != q.shape:
+        raise KernelError(f"attention: q {tuple(q.shape)} / out {tuple(out.shape)} do not fit {heads} heads of {head_dim}")
+    if tuple(k_pages.shape[1:]) != (kv_heads, PAGE_TOKENS, head_dim) or tuple(v_pages.shape[1:]) != (kv_heads, head_dim, PAGE_TOKENS):
+        raise KernelError(f"attention: page shapes {tuple(k_pages.shape)} / {tuple(v_pages.shape)} do not fit")
+    if k_pages.dtype != v_pages.dtype:
+        raise KernelError("attention: key and value pages differ in type")
+    if tok_slot.dtype != torch.int32 or tok_pos.dtype != torch.int32 or block_table.dtype != torch.int32:
+        raise KernelError("attention: tok_slot, tok_pos and block_table must be int32")
+    lib = attention_module(head_dim)
+    _check(lib, lib.nnis_attention_rows(q.data_ptr(), _code(q), out.data_ptr(), _code(out), k_pages.data_ptr(),
+                                        v_pages.data_ptr(), _code(k_pages), block_table.data_ptr(), block_table.shape[1],
+                                        tok_slot.data_ptr(), tok_pos.data_ptr(), tokens, heads, kv_heads, head_dim,
+                                        int(window), float(scale), _stream()))
+    return out
+
+
+# ---------------------------------------------------------------------------
+# dispatch by operand types
+# ---------------------------------------------------------------------------
+
+def linear(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out = x @ weight^T.  32-bit operands take the ordered 32-bit product;
+    bfloat16 operands take the matrix-core kernels."""
+    return gemm_ordered(x, weight, out)
+
+
+def attention(q: torch.Tensor, out: torch.Tensor, view, ctx, heads: int, kv_heads: int, head_dim: int, scale: float,
+              window: int = 0) -> torch.Tensor:
+    """Attention of the step's tokens over the cache ``view``."""
+    return attention_rows(q, out, view.k_pages, view.v_pages, view.block_table, ctx.tok_slot, ctx.tok_pos, heads,
+                          kv_heads, head_dim, scale, window)

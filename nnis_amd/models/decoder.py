@@ -1,0 +1,80 @@
+"""A decoder put together from a ``ModelSpec``: embedding, blocks run in the
+order of the schedule, final norm and head.  Nothing here names an
+architecture; which parts exist and how they are sized is the spec's business.
+"""
+
+from __future__ import annotations
+
+from typing import Any, Dict, List, Tuple
+
+import torch
+
+from ..parts import build_part
+from ..parts.base import TensorSpec
+from .spec import ModelSpec
+
+
+class DecoderModel:
+    def __init__(self, spec: ModelSpec):
+        spec.validate()
+        self.spec = spec
+        self.positions = {name: build_part("position", description) for name, description in spec.positions.items()}
+        self.embedding = build_part("embedding", spec.embedding)
+        self.layers = [build_part("block", description, positions=self.positions) for description in spec.layers]
+        self.final_norm = build_part("norm", spec.final_norm)
+        self.head = build_part("head", spec.head)
+        self.bound = False
+
+    # ---- weights -------------------------------------------------------------
+    def parts(self):
+        return [self.embedding, *self.positions.values(), *self.layers, self.final_norm, self.head]
+
+    def tensors(self) -> List[TensorSpec]:
+        out, seen = [], set()
+        for part in self.parts():
+            for tensor in part.tensors():
+                if tensor.name not in seen:
+                    seen.add(tensor.name)
+                    out.append(tensor)
+        return out
+
+    def bind(self, weights: Dict[str, torch.Tensor], rt) -> None:
+        for part in self.parts():
+            part.bind(weights, rt)
+        self.bound = True
+
+    def step_weight_bytes(self) -> int:
+        """Bytes of weights a decode step reads: every layer each time the
+        schedule runs it, the head, and no embedding table (a row per token)."""
+        total = sum(self.layers[entry.layer].weight_bytes() for entry in self.spec.schedule)
+        return total + self.final_norm.weight_bytes() + self.head.weight_bytes()
+
+    # ---- cache ---------------------------------------------------------------
+    def cache_requests(self) -> Tuple[List[Tuple[int, Any]], Dict[int, int]]:
+        requests, shared = [], {}
+        for index, entry in enumerate(self.spec.schedule):
+            if entry.reads_cache_of is None:
+                requests.append((index, self.layers[entry.layer].cache_request()))
+            else:
+                shared[index] = entry.reads_cache_of
+        return requests, shared
+
+    # ---- forward -------------------------------------------------------------
+    def forward(self, ids: torch.Tensor, ctx, cache, want_rows: torch.Tensor, rt) -> torch.Tensor:
+        """ids: int32 [tokens] on the device; want_rows: int32 indices of the
+        packed tokens whose logits are asked for.  Returns float32
+        [len(want_rows), vocab]."""
+        x = self.embedding.forward(ids, ctx.tokens, rt)
+        for position in self.positions.values():
+            x = position.embed(x, ctx, rt)
+        stream = (x, None)
+        for index, entry in enumerate(self.spec.schedule):
+            stream = self.layers[entry.layer].forward(stream, ctx, cache.view(index), rt)
+        x, pending = stream
+        if want_rows.shape[0] == 0:
+            return rt.empty(0, self.spec.vocab_size, dtype=torch.float32)
+        if pending is None:
+            normed = self.final_norm.forward(x, rt, rows=want_rows)
+        else:
+            normed = self.final_norm.add_forward(x, pending, rt, rows=want_rows)
+        return self.head.forward(normed, rt)

@@ -1,0 +1,74 @@
+"""Causal self-attention with grouped key/value heads over the cache
+(/root/reference/crates/nnis-model/src/runtime.rs:959-1038; formula
+/root/reference/crates/nnis-model/src/kernels.rs:66-125).  Queries, keys and
+values come from one fused projection; queries and keys are rotated by the
+position encoding handed in; keys and values go into the cache before the
+scores are taken, so the same code runs whole prompts and single tokens.
+"""
+
+from __future__ import annotations
+
+import math
+
+import torch
+
+from ..errors import InvalidInput
+from .base import KVRequest, Mixer, TensorSpec, register_part
+from .linear import Projection
+
+
+class CausalSelfAttention(Mixer):
+    def __init__(self, width, heads, kv_heads, head_dim, q, k, v, o, position=None, window=None, positions=None):
+        if heads % kv_heads != 0:
+            raise InvalidInput(f"{heads} query heads do not divide into {kv_heads} key/value heads")
+        self.width, self.heads, self.kv_heads, self.head_dim = int(width), int(heads), int(kv_heads), int(head_dim)
+        self.names = {"q": q, "k": k, "v": v, "o": o}
+        self.window = None if not window else int(window)
+        self.position = None
+        if position is not None:
+            if positions is None or position not in positions:
+                raise InvalidInput(f"attention names position encoding {position!r}, which the model does not define")
+            self.position = positions[position]
+        self.scale = 1.0 / math.sqrt(self.head_dim)  # runtime.rs:943
+        self.qkv = None
+        self.out = None
+
+    def tensors(self):
+        q_width, kv_width = self.heads * self.head_dim, self.kv_heads * self.head_dim
+        return [
+            TensorSpec(self.names["q"], (q_width, self.width)),
+            TensorSpec(self.names["k"], (kv_width, self.width)),
+            TensorSpec(self.names["v"], (kv_width, self.width)),
+            TensorSpec(self.names["o"], (self.width, q_width)),
+        ]
+
+    def bind(self, weights, rt):
+        # one projection for queries, keys and values: rows q heads, k heads, v heads
+        self.qkv = Projection(torch.cat([weights[self.names["q"]], weights[self.names["k"]], weights[self.names["v"]]], dim=0))
+        self.out = Projection(weights[self.names["o"]])
+
+    def weight_bytes(self):
+        return self.qkv.weight_bytes() + self.out.weight_bytes()
+
+    def cache_request(self):
+        return KVRequest(self.kv_heads, self.head_dim, self.window)
+
+    def forward(self, x, ctx, view, rt):
+        tokens = x.shape[0]
+        qkv = self.qkv(x, rt)
+        q = rt.empty(tokens, self.heads * self.head_dim)
+        tables = self.position.rotary() if self.position is not None else None
+        writes = not view.read_only
+        rt.ops.rope_kv_write(
+            qkv, q,
+            tables.cos if tables else None, tables.sin if tables else None, tables.rot_dim if tables else 0,
+            ctx.tok_slot, ctx.tok_pos,
+            view.k_pages if writes else None, view.v_pages if writes else None, view.block_table if writes else None,
+            self.heads, self.kv_heads, self.head_dim,
+        )
+        attn = rt.empty(tokens, self.heads * self.head_dim)
+        rt.ops.attention(q, attn, view, ctx, self.heads, self.kv_heads, self.head_dim, self.scale, self.window or 0)
+        return self.out(attn, rt)
+
+
+register_part("mixer", "causal_attention", CausalSelfAttention)

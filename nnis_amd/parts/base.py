@@ -1,0 +1,168 @@
+"""Interfaces of the parts a decoder is put together from, and their registry.
+
+A part is built from its own sizes and constants and from the checkpoint names
+of its tensors; it never sees a model configuration and does not know which
+model it is in.  A model description (``nnis_amd.models.spec``) names, layer
+by layer, which part kinds to use and with which parameters; ``build_part``
+turns one such entry into an object through the registry below.  A new mixer,
+feed-forward, norm or position encoding is added by registering a class under
+a new kind name; nothing else in the library keys on the kind.
+
+The interfaces:
+
+``Norm``
+    ``forward(x, rt, rows=None)`` -> normed rows in the activation type;
+    ``add_forward(residual, delta, rt, rows=None)`` -> the same after
+    ``residual += delta`` (the sum is taken and kept in 32-bit).
+``PositionEncoding``
+    ``rotary()`` -> ``RotaryTables`` or ``None`` (consumed by attention
+    mixers that rotate queries and keys); ``embed(x, ctx, rt)`` -> x, for
+    encodings added to the token embedding (default: unchanged).
+``Mixer``
+    ``cache_request()`` -> what the cache must hold for one use of this mixer
+    in the schedule (``KVRequest``, ``StateRequest`` or ``None``);
+    ``forward(x, ctx, view, rt)`` -> y, where ``x`` is ``[tokens, width]`` in
+    the activation type, ``ctx`` is the step's ``StepContext`` and ``view``
+    is the cache's view for this schedule entry.
+``FeedForward``
+    ``forward(x, ctx, rt)`` -> y, row-wise over the packed tokens.
+``Block``
+    ``forward(stream, ctx, view, rt)`` -> stream; the block owns the
+    arrangement of norm, mixer and feed-forward around the residual stream.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Any, Callable, Dict, List, Optional, Tuple
+
+from ..errors import InvalidInput
+
+
+@dataclass(frozen=True)
+class TensorSpec:
+    """A tensor a part reads from the checkpoint.
+
+    ``init`` tells the random-weights writer how to draw it: ``"matrix"`` is
+    N(0, 0.02) and ``"gain"`` is 1 + N(0, 0.01).  ``fallback`` names another
+    checkpoint tensor that stands in when this one is absent (a tied head)."""
+
+    name: str
+    shape: Tuple[int, ...]
+    init: str = "matrix"
+    fallback: Optional[str] = None
+
+
+@dataclass(frozen=True)
+class KVRequest:
+    """Keys and values of every token (``window is None``) or of the last
+    ``window`` tokens, for ``kv_heads`` heads of ``head_dim``."""
+
+    kv_heads: int
+    head_dim: int
+    window: Optional[int] = None
+
+
+@dataclass(frozen=True)
+class StateRequest:
+    """A block of fixed shape per sequence, zero when the sequence starts.
+    ``dtype`` is a torch dtype name; state is kept in it whatever the
+    activation type is."""
+
+    shape: Tuple[int, ...]
+    dtype: str = "float32"
+
+
+class Part:
+    """Common base: tensors in, bound device weights out."""
+
+    def tensors(self) -> List[TensorSpec]:
+        return []
+
+    def bind(self, weights: Dict[str, Any], rt: Any) -> None:
+        """Receives the loaded tensors (by checkpoint name, on the device, in
+        the stored type or widened for the 32-bit path) and keeps or repacks
+        what it needs."""
+
+    def weight_bytes(self) -> int:
+        """Bytes of weights one step has to read through this part."""
+        return 0
+
+
+class Norm(Part):
+    def forward(self, x, rt, rows=None):
+        raise NotImplementedError
+
+    def add_forward(self, residual, delta, rt, rows=None):
+        raise NotImplementedError
+
+
+@dataclass
+class RotaryTables:
+    cos: Any  # [positions, rot_dim/2] float32 on the device
+    sin: Any
+    rot_dim: int
+
+
+class PositionEncoding(Part):
+    def rotary(self) -> Optional[RotaryTables]:
+        return None
+
+    def embed(self, x, ctx, rt):
+        return x
+
+
+class Mixer(Part):
+    def cache_request(self):
+        return None
+
+    def forward(self, x, ctx, view, rt):
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, x, ctx, rt):
+        raise NotImplementedError
+
+
+class Block(Part):
+    def cache_request(self):
+        return None
+
+    def forward(self, stream, ctx, view, rt):
+        raise NotImplementedError
+
+
+# --------------------------------------------------------------------------
+# registry of part kinds
+# --------------------------------------------------------------------------
+
+_PART_KINDS: Dict[Tuple[str, str], Callable[..., Part]] = {}
+_ROLES = ("norm", "position", "mixer", "feed_forward", "block", "embedding", "head")
+
+
+def register_part(role: str, kind: str, factory: Callable[..., Part], replace: bool = False) -> None:
+    """Makes ``{"kind": kind, ...params}`` buildable for ``role``."""
+    if role not in _ROLES:
+        raise InvalidInput(f"unknown part role {role!r}; roles are {', '.join(_ROLES)}")
+    key = (role, kind)
+    if key in _PART_KINDS and not replace:
+        raise InvalidInput(f"part kind {kind!r} is already registered for role {role!r}")
+    _PART_KINDS[key] = factory
+
+
+def build_part(role: str, spec: Dict[str, Any], **extra) -> Part:
+    """``spec`` is ``{"kind": name, **parameters}``; ``extra`` carries objects
+    the description cannot hold as data (already-built sub-parts)."""
+    if "kind" not in spec:
+        raise InvalidInput(f"{role} description has no 'kind': {spec!r}")
+    key = (role, spec["kind"])
+    if key not in _PART_KINDS:
+        known = sorted(kind for (r, kind) in _PART_KINDS if r == role)
+        raise InvalidInput(f"unknown {role} kind {spec['kind']!r}; registered: {', '.join(known) or 'none'}")
+    params = {k: v for k, v in spec.items() if k != "kind"}
+    return _PART_KINDS[key](**params, **extra)
+
+
+def registered_kinds(role: str) -> List[str]:
+    return sorted(kind for (r, kind) in _PART_KINDS if r == role)

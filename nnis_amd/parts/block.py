@@ -1,0 +1,45 @@
+"""The pre-norm arrangement of a layer:
+x += mixer(norm1(x)); x += feed_forward(norm2(x))
+(/root/reference/crates/nnis-model/src/runtime.rs:945-1095).
+
+The residual stream is kept in 32-bit as a pair (x, pending): ``pending`` is a
+part's output not yet added.  The sum is taken by the next norm in the same
+kernel that normalises, so the stream is read and written once per part.
+"""
+
+from __future__ import annotations
+
+from .base import Block, build_part, register_part
+
+
+class PreNormBlock(Block):
+    def __init__(self, width, norm1, mixer, norm2, feed_forward, positions=None):
+        self.width = int(width)
+        self.norm1 = build_part("norm", norm1)
+        self.mixer = build_part("mixer", mixer, positions=positions)
+        self.norm2 = build_part("norm", norm2)
+        self.feed_forward = build_part("feed_forward", feed_forward)
+        self._parts = [self.norm1, self.mixer, self.norm2, self.feed_forward]
+
+    def tensors(self):
+        return [spec for part in self._parts for spec in part.tensors()]
+
+    def bind(self, weights, rt):
+        for part in self._parts:
+            part.bind(weights, rt)
+
+    def weight_bytes(self):
+        return sum(part.weight_bytes() for part in self._parts)
+
+    def cache_request(self):
+        return self.mixer.cache_request()
+
+    def forward(self, stream, ctx, view, rt):
+        x, pending = stream
+        normed = self.norm1.forward(x, rt) if pending is None else self.norm1.add_forward(x, pending, rt)
+        mixed = self.mixer.forward(normed, ctx, view, rt)
+        normed = self.norm2.add_forward(x, mixed, rt)
+        return x, self.feed_forward.forward(normed, ctx, rt)
+
+
+register_part("block", "pre_norm", PreNormBlock)
