@@ -16,7 +16,7 @@ __all__ = [
 
 def __getattr__(name):
     # heavy imports (torch) happen on first use
-    if name in ("load_model", "load_engine"):
+    if name in ("load_model", "load_engine", "generate"):
         from . import api
 
         return getattr(api, name)
@@ -25,8 +25,4 @@ def __getattr__(name):
         from .weights.random_init import write_random_model
 
         return write_random_model
-    if name == "generate":
-        from .engine.generate import generate
-
-        return generate
     raise AttributeError(name)

@@ -1,0 +1,237 @@
+// Seeded temperature / top-k / top-p sampling on the device, one block per row.
+//
+// Semantics are the reference's host sampler
+// (/root/reference/crates/nnis-model/src/sampling.rs:113-202): candidates in
+// order of logit descending, ties by lower id; top-k keeps the first k;
+// weights exp((l - l_max) / T) in 64-bit; top-p keeps the shortest prefix
+// whose weight reaches p * total (the crossing candidate stays); one
+// SplitMix64 draw u in [0,1) per token (sampling.rs:261-284); the result is
+// the first candidate whose cumulative weight exceeds u * total.
+//
+// No sort: a prefix of the sorted order is described by a cut (key, ties): all
+// tokens whose key is above `key`, and the first `ties` tokens (by id) whose key
+// equals it.  Each cut is found by a bitwise search over the 32-bit ordered
+// key with a block-wide sum per probe; sums are taken in a fixed order, so a
+// seed always gives the same token.  Sums differ from the reference's running
+// sum in the last bits only.
+#include "common.h"
+
+namespace {
+
+constexpr int kSampleThreads = 1024;
+
+__device__ __forceinline__ unsigned ordered_key(float v) {
+  if (v == 0.0f) v = 0.0f;  // -0 and +0 compare equal
+  const unsigned bits = __float_as_uint(v);
+  return (bits & 0x80000000u) ? ~bits : (bits | 0x80000000u);
+}
+
+template <typename T>
+__device__ __forceinline__ T block_total(T v, T* scratch) {
+#pragma unroll
+  for (int offset = kWave / 2; offset > 0; offset >>= 1) v += __shfl_xor(v, offset, kWave);
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  __syncthreads();
+  if (lane == 0) scratch[wave] = v;
+  __syncthreads();
+  T total = 0;
+  for (int w = 0; w < kSampleThreads / kWave; ++w) total += scratch[w];
+  return total;
+}
+
+__device__ __forceinline__ unsigned long long splitmix64_next(unsigned long long* state) {
+  *state += 0x9E3779B97F4A7C15ull;
+  unsigned long long z = *state;
+  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+  return z ^ (z >> 31);
+}
+
+struct RowView {
+  const float* logits;
+  const double* weights;
+  int vocab;
+};
+
+// weight of all tokens whose key is >= t
+__device__ double mass_at_least(const RowView& r, unsigned t, double* scratch) {
+  double sum = 0.0;
+  for (int c = threadIdx.x; c < r.vocab; c += kSampleThreads)
+    if (ordered_key(r.logits[c]) >= t) sum += r.weights[c];
+  return block_total(sum, scratch);
+}
+
+__device__ int count_at_least(const RowView& r, unsigned t, int* scratch) {
+  int count = 0;
+  for (int c = threadIdx.x; c < r.vocab; c += kSampleThreads)
+    if (ordered_key(r.logits[c]) >= t) ++count;
+  return block_total(count, scratch);
+}
+
+__global__ __launch_bounds__(kSampleThreads) void sample_kernel(
+    const float* __restrict__ logits, double* __restrict__ weights, int vocab, const int* __restrict__ row_slot,
+    unsigned long long* __restrict__ rng, const float* __restrict__ temperature, const int* __restrict__ top_k,
+    const float* __restrict__ top_p, int* __restrict__ out) {
+  __shared__ double scratch_d[kSampleThreads / kWave];
+  __shared__ int scratch_i[kSampleThreads / kWave];
+  __shared__ int found;
+  const int row = blockIdx.x;
+  const int slot = row_slot[row];
+  if (slot < 0) return;  // padding row (uniform over the block)
+  RowView r;
+  r.logits = logits + (size_t)row * vocab;
+  double* w = weights + (size_t)row * vocab;
+  r.weights = w;
+  r.vocab = vocab;
+
+  // maximum key, and a check that every logit is finite
+  unsigned key_max = 0;
+  int bad = 0;
+  for (int c = threadIdx.x; c < vocab; c += kSampleThreads) {
+    const float v = r.logits[c];
+    if (!isfinite(v)) bad = 1;
+    const unsigned key = ordered_key(v);
+    key_max = key > key_max ? key : key_max;
+  }
+  bad = block_total(bad, scratch_i);
+  if (bad) {
+    if (threadIdx.x == 0) out[row] = -1;  // the host raises: a non-finite logit is refused
+    return;
+  }
+#pragma unroll
+  for (int offset = kWave / 2; offset > 0; offset >>= 1) {
+    const unsigned other = __shfl_xor(key_max, offset, kWave);
+    key_max = other > key_max ? other : key_max;
+  }
+  __shared__ unsigned wave_keys[kSampleThreads / kWave];
+  if (threadIdx.x % kWave == 0) wave_keys[threadIdx.x / kWave] = key_max;
+  __syncthreads();
+  for (int i = 0; i < kSampleThreads / kWave; ++i) key_max = wave_keys[i] > key_max ? wave_keys[i] : key_max;
+  const unsigned max_bits = (key_max & 0x80000000u) ? (key_max & 0x7fffffffu) : ~key_max;
+  const double inv_t = 1.0 / (double)temperature[row];
+  const double max_scaled = (double)__uint_as_float(max_bits) * inv_t;
+  for (int c = threadIdx.x; c < vocab; c += kSampleThreads) w[c] = exp((double)r.logits[c] * inv_t - max_scaled);
+  __syncthreads();
+
+  // the kept prefix: everything with key > cut_key plus `cut_ties` tokens at cut_key
+  unsigned cut_key = 0;
+  int cut_ties = 0;          // meaningful only when limited
+  bool limited = false;
+  double total = mass_at_least(r, 0u, scratch_d);
+
+  const int k = top_k[row];
+  if (k > 0 && k < vocab) {
+    unsigned t = 0;
+    for (int bit = 31; bit >= 0; --bit) {
+      const unsigned probe = t | (1u << bit);
+      if (count_at_least(r, probe, scratch_i) >= k) t = probe;
+    }
+    const int above = count_at_least(r, t + 1u, scratch_i);
+    cut_key = t;
+    cut_ties = k - above;
+    limited = true;
+    const double weight_at = exp((double)__uint_as_float((t & 0x80000000u) ? (t & 0x7fffffffu) : ~t) * inv_t - max_scaled);
+    total = mass_at_least(r, t + 1u, scratch_d) + (double)cut_ties * weight_at;
+  }
+
+  const float p = top_p[row];
+  if (p > 0.0f && p <= 1.0f) {
+    const double threshold = (double)p * total;
+    unsigned t = 0;
+    for (int bit = 31; bit >= 0; --bit) {
+      const unsigned probe = t | (1u << bit);
+      const double mass = (limited && probe <= cut_key) ? total : mass_at_least(r, probe, scratch_d);
+      if (mass >= threshold) t = probe;
+    }
+    // t >= cut_key when limited, because the whole kept mass reaches the threshold
+    const double base = mass_at_least(r, t + 1u, scratch_d);
+    const double weight_at = exp((double)__uint_as_float((t & 0x80000000u) ? (t & 0x7fffffffu) : ~t) * inv_t - max_scaled);
+    int available = (limited && t == cut_key) ? cut_ties
+                                              : count_at_least(r, t, scratch_i) - count_at_least(r, t + 1u, scratch_i);
+    int need = 1;
+    double reached = base + weight_at;
+    while (need < available && reached < threshold) {
+      ++need;
+      reached += weight_at;
+    }
+    cut_key = t;
+    cut_ties = need;
+    limited = true;
+    total = base + (double)need * weight_at;
+  }
+
+  unsigned long long state = rng[slot];
+  const unsigned long long raw = splitmix64_next(&state);
+  const double unit = (double)(raw >> 11) * (1.0 / 9007199254740992.0);
+  const double draw = unit * total;
+
+  unsigned t = 0;
+  for (int bit = 31; bit >= 0; --bit) {
+    const unsigned probe = t | (1u << bit);
+    const double mass = (limited && probe <= cut_key) ? total : mass_at_least(r, probe, scratch_d);
+    if (mass > draw) t = probe;
+  }
+  const double base = mass_at_least(r, t + 1u, scratch_d);
+  const double weight_at = exp((double)__uint_as_float((t & 0x80000000u) ? (t & 0x7fffffffu) : ~t) * inv_t - max_scaled);
+  const int available = (limited && t == cut_key) ? cut_ties
+                                                  : count_at_least(r, t, scratch_i) - count_at_least(r, t + 1u, scratch_i);
+  int index = 0;
+  double reached = base + weight_at;
+  while (index + 1 < available && !(draw < reached)) {
+    ++index;
+    reached += weight_at;
+  }
+
+  // the index-th token (by id) whose key equals t: contiguous chunks per thread, then a scan
+  const int chunk = (vocab + kSampleThreads - 1) / kSampleThreads;
+  const int begin = threadIdx.x * chunk;
+  const int end = begin + chunk < vocab ? begin + chunk : vocab;
+  int mine = 0;
+  for (int c = begin; c < end; ++c)
+    if (ordered_key(r.logits[c]) == t) ++mine;
+  __shared__ int counts[kSampleThreads];
+  counts[threadIdx.x] = mine;
+  if (threadIdx.x == 0) found = -1;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int before = 0;
+    for (int i = 0; i < kSampleThreads; ++i) {
+      if (index < before + counts[i]) {
+        found = (i << 16) | (index - before);  // thread and its local index; chunk counts fit in 16 bits
+        break;
+      }
+      before += counts[i];
+    }
+  }
+  __syncthreads();
+  if (found >= 0 && threadIdx.x == (found >> 16)) {
+    int local = found & 0xffff;
+    for (int c = begin; c < end; ++c) {
+      if (ordered_key(r.logits[c]) == t) {
+        if (local == 0) {
+          out[row] = c;
+          break;
+        }
+        --local;
+      }
+    }
+  }
+  if (threadIdx.x == 0) {
+    rng[slot] = state;
+    if (found < 0) out[row] = -2;  // cannot happen for finite logits; reported rather than hidden
+  }
+}
+
+}  // namespace
+
+extern "C" int nnis_sample(const float* logits, double* weights, int rows, int vocab, const int* row_slot,
+                           unsigned long long* rng, const float* temperature, const int* top_k, const float* top_p,
+                           int* out, void* stream) {
+  NNIS_REQUIRE(rows >= 0 && vocab > 0, "sample: bad sizes rows=%d vocab=%d", rows, vocab);
+  NNIS_REQUIRE((long long)vocab <= 65535LL * kSampleThreads, "sample: vocabulary %d is too large for this kernel", vocab);
+  if (rows == 0) return 0;
+  hipLaunchKernelGGL(sample_kernel, dim3(rows), dim3(kSampleThreads), 0, (hipStream_t)stream, logits, weights, vocab,
+                     row_slot, rng, temperature, top_k, top_p, out);
+  NNIS_LAUNCH_CHECK("sample");
+  return 0;
+}

@@ -26,6 +26,7 @@ class Engine:
         self.model = model
         self.rt = rt
         self.vocab_size = model.spec.vocab_size
+        self.max_positions = model.spec.max_positions
         requests, shared = model.cache_requests()
         self.cache = SequenceCache(requests, shared, max_tokens, model.spec.max_positions, rt.dtype, rt.device, max_slots)
         self._staging = None
@@ -40,6 +41,13 @@ class Engine:
 
     def length(self, slot: int) -> int:
         return self.cache.length(slot)
+
+    def free_slots(self) -> int:
+        return self.cache.slots.free
+
+    def free_pages(self) -> int:
+        groups = self.cache.kv_groups
+        return min(g.table.pool.free for g in groups) if groups else 1 << 30
 
     # ---- one step ------------------------------------------------------------
     def _validate(self, entries: Sequence[StepEntry]):

@@ -28,6 +28,7 @@ _CORE_SIGNATURES = {
     "nnis_silu_mul": [_VOID, _INT, _VOID, _INT, _INT, _INT, _VOID],
     "nnis_argmax": [_VOID, _VOID, _INT, _INT, _VOID],
     "nnis_gemm_ordered": [_VOID, _INT, _VOID, _INT, _VOID, _INT, _INT, _INT, _INT, _VOID],
+    "nnis_sample": [_VOID, _VOID, _INT, _INT, _VOID, _VOID, _VOID, _VOID, _VOID, _VOID, _VOID],
 }
 _ATTN_SIGNATURES = {
     "nnis_attention_rows": [_VOID, _INT, _VOID, _INT, _VOID, _VOID, _INT, _VOID, _INT, _VOID, _VOID, _INT, _INT, _INT,
@@ -251,3 +252,27 @@ def attention(q: torch.Tensor, out: torch.Tensor, view, ctx, heads: int, kv_head
     """Attention of the step's tokens over the cache ``view``."""
     return attention_rows(q, out, view.k_pages, view.v_pages, view.block_table, ctx.tok_slot, ctx.tok_pos, heads,
                           kv_heads, head_dim, scale, window)
+
+
+def sample(logits: torch.Tensor, weights: torch.Tensor, row_slot: torch.Tensor, rng: torch.Tensor,
+           temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """Seeded sampling per row; rows whose slot is negative are skipped.  ``rng``
+    is int64 [slots] holding each sequence's SplitMix64 state; ``weights`` is
+    float64 scratch of at least [rows, vocab].  A row with a non-finite logit
+    gets -1."""
+    for t, what in ((logits, "logits"), (weights, "weights"), (row_slot, "row_slot"), (rng, "rng"),
+                    (temperature, "temperature"), (top_k, "top_k"), (top_p, "top_p"), (out, "out")):
+        _dev(t, what)
+    rows, vocab = logits.shape
+    if logits.dtype != torch.float32 or weights.dtype != torch.float64 or weights.numel() < rows * vocab:
+        raise KernelError("sample: logits must be float32 and weights float64 scratch of [rows, vocab]")
+    if rng.dtype != torch.int64 or row_slot.dtype != torch.int32 or top_k.dtype != torch.int32 or out.dtype != torch.int32:
+        raise KernelError("sample: rng must be int64; row_slot, top_k and out int32")
+    if temperature.dtype != torch.float32 or top_p.dtype != torch.float32:
+        raise KernelError("sample: temperature and top_p must be float32")
+    if min(row_slot.numel(), temperature.numel(), top_k.numel(), top_p.numel(), out.numel()) < rows:
+        raise KernelError("sample: per-row arrays are shorter than the rows")
+    lib = core()
+    _check(lib, lib.nnis_sample(logits.data_ptr(), weights.data_ptr(), rows, vocab, row_slot.data_ptr(), rng.data_ptr(),
+                                temperature.data_ptr(), top_k.data_ptr(), top_p.data_ptr(), out.data_ptr(), _stream()))
+    return out

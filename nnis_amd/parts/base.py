@@ -33,6 +33,7 @@ The interfaces:
 
 from __future__ import annotations
 
+import inspect
 from dataclasses import dataclass, field
 from typing import Any, Callable, Dict, List, Optional, Tuple
 
@@ -153,7 +154,7 @@ def register_part(role: str, kind: str, factory: Callable[..., Part], replace: b
 
 def build_part(role: str, spec: Dict[str, Any], **extra) -> Part:
     """``spec`` is ``{"kind": name, **parameters}``; ``extra`` carries objects
-    the description cannot hold as data (already-built sub-parts)."""
+    the description cannot hold as data (the model's position encodings)."""
     if "kind" not in spec:
         raise InvalidInput(f"{role} description has no 'kind': {spec!r}")
     key = (role, spec["kind"])
@@ -161,7 +162,13 @@ def build_part(role: str, spec: Dict[str, Any], **extra) -> Part:
         known = sorted(kind for (r, kind) in _PART_KINDS if r == role)
         raise InvalidInput(f"unknown {role} kind {spec['kind']!r}; registered: {', '.join(known) or 'none'}")
     params = {k: v for k, v in spec.items() if k != "kind"}
-    return _PART_KINDS[key](**params, **extra)
+    factory = _PART_KINDS[key]
+    # context objects go only to factories that name them (a mixer without a
+    # position encoding does not take ``positions``)
+    accepted = inspect.signature(factory).parameters
+    takes_any = any(p.kind is inspect.Parameter.VAR_KEYWORD for p in accepted.values())
+    context = {k: v for k, v in extra.items() if takes_any or k in accepted}
+    return factory(**params, **context)
 
 
 def registered_kinds(role: str) -> List[str]:

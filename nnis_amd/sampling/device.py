@@ -1,0 +1,69 @@
+"""Token selection on the device for a batch of logit rows: argmax for greedy
+rows, the sampling kernel for seeded rows.  Each sequence's generator state
+lives in the cache's per-slot state region, so a sequence's draws do not
+depend on what else is in the batch
+(/root/reference/crates/nnis-model/src/session_batch.rs:7-8)."""
+
+from __future__ import annotations
+
+from typing import List, Optional, Sequence
+
+import numpy as np
+import torch
+
+from ..errors import InvalidInput
+from .params import SamplingParams
+
+RNG_REGION = "sampler.rng"
+
+
+class DeviceSelector:
+    def __init__(self, engine):
+        self.engine = engine
+        self.rt = engine.rt
+        self.vocab_size = engine.vocab_size
+        cache = engine.cache
+        if RNG_REGION not in cache.state_regions:
+            cache.add_state_region(RNG_REGION, (), torch.int64)
+        self.rng = cache.state_regions[RNG_REGION]
+        self._weights = None
+
+    def start(self, slot: int, params: Optional[SamplingParams]) -> None:
+        """Called when a sequence starts: seeds its generator."""
+        if params is not None:
+            params.validate(self.vocab_size)
+            seed = params.seed if params.seed < (1 << 63) else params.seed - (1 << 64)
+            self.rng[slot] = seed
+
+    def select(self, logits: torch.Tensor, slots: Sequence[int], params: Sequence[Optional[SamplingParams]]) -> List[int]:
+        """One token per row of ``logits`` (float32 [rows, vocab] on the device)."""
+        rows = logits.shape[0]
+        ops = self.rt.ops
+        picked = torch.empty(rows, dtype=torch.int32, device=self.rt.device)
+        ops.argmax(logits, picked)
+        if any(p is not None for p in params):
+            row_slot = np.asarray([s if p is not None else -1 for s, p in zip(slots, params)], dtype=np.int32)
+            temperature = np.asarray([p.temperature if p is not None else 1.0 for p in params], dtype=np.float32)
+            top_k = np.asarray([(p.top_k or 0) if p is not None else 0 for p in params], dtype=np.int32)
+            top_p = np.asarray([(p.top_p or 0.0) if p is not None else 0.0 for p in params], dtype=np.float32)
+            if self._weights is None or self._weights.shape[0] < rows:
+                self._weights = torch.empty((max(rows, 8), self.vocab_size), dtype=torch.float64, device=self.rt.device)
+            sampled = torch.full((rows,), -3, dtype=torch.int32, device=self.rt.device)
+            ops.sample(
+                logits, self._weights,
+                torch.from_numpy(row_slot).to(self.rt.device), self.rng,
+                torch.from_numpy(temperature).to(self.rt.device), torch.from_numpy(top_k).to(self.rt.device),
+                torch.from_numpy(top_p).to(self.rt.device), sampled,
+            )
+            sampled_host = sampled.cpu().tolist()
+            picked_host = picked.cpu().tolist()
+            out = []
+            for row, p in enumerate(params):
+                if p is None:
+                    out.append(picked_host[row])
+                else:
+                    if sampled_host[row] < 0:
+                        raise InvalidInput(f"sampling refused row {row}: a logit is not finite")
+                    out.append(sampled_host[row])
+            return out
+        return picked.cpu().tolist()

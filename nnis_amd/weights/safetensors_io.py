@@ -105,12 +105,8 @@ class SafetensorsFile:
         return flat.view(shape)
 
     def close(self) -> None:
-        # tensors handed out may still view the mapping; closing is left to
-        # the garbage collector when any exist.
-        try:
-            self._map.close()
-        except (BufferError, ValueError):
-            pass
+        """Closes the file.  The mapping stays valid for as long as a tensor
+        handed out views it, and is released with the last of them."""
         self._file.close()
 
 

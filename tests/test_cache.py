@@ -1,0 +1,118 @@
+"""The cache's bookkeeping on the host: no slot or page is lost, held twice or
+freed twice; a refused growth changes nothing; slots given back are used again;
+state of fixed size starts at zero.  Behaviours kept from the reference's cache
+tests (/root/reference/crates/nnis-rt/src/kv_cache.rs:501-629: overflow leaves
+the length unchanged, reset reuses)."""
+
+import random
+
+import pytest
+import torch
+
+from nnis_amd.cache import FreeList, PageTable, SequenceCache, pages_for
+from nnis_amd.errors import CacheFull, InvalidInput
+from nnis_amd.parts.base import KVRequest, StateRequest
+
+
+def test_free_list_never_loses_or_doubles():
+    pool = FreeList(5, "slot")
+    taken = [pool.take() for _ in range(5)]
+    assert sorted(taken) == [0, 1, 2, 3, 4] and pool.free == 0
+    with pytest.raises(CacheFull):
+        pool.take()
+    pool.give_back(3)
+    with pytest.raises(InvalidInput, match="not held"):
+        pool.give_back(3)  # freed twice
+    with pytest.raises(InvalidInput):
+        pool.give_back(17)  # never given
+    assert pool.take() == 3  # used again
+    rng = random.Random(0)
+    held = set(pool.held)
+    for _ in range(2000):
+        if held and (rng.random() < 0.5 or pool.free == 0):
+            item = rng.choice(sorted(held))
+            pool.give_back(item)
+            held.remove(item)
+        else:
+            item = pool.take()
+            assert item not in held  # never held twice
+            held.add(item)
+        assert pool.free + len(held) == 5 and held == set(pool.held)
+    with pytest.raises(InvalidInput):
+        FreeList(0, "slot")
+
+
+def test_pages_follow_lengths():
+    assert [pages_for(n) for n in (0, 1, 64, 65, 128, 129)] == [0, 1, 1, 2, 2, 3]
+    table = PageTable(pages=4, slots=3, max_pages_per_slot=3)
+    assert table.grow(0, 1) == [0] and table.grow(0, 64) == [] and table.grow(0, 65) == [1]
+    assert table.grow(1, 100) == [0, 1]
+    with pytest.raises(CacheFull):
+        table.grow(2, 1)
+    assert table.rows[0] != table.rows[1] and not set(table.rows[0]) & set(table.rows[1])
+    table.release(0)
+    assert table.pool.free == 2 and 0 not in table.rows
+    table.grow(2, 128)
+    with pytest.raises(CacheFull, match="at most 3 pages"):
+        PageTable(pages=8, slots=1, max_pages_per_slot=3).grow(0, 64 * 4)
+
+
+def _cache(max_tokens=512, extra=()):
+    requests = [(0, KVRequest(2, 16)), (1, KVRequest(2, 16)), (2, KVRequest(1, 32, window=100)), *extra]
+    return SequenceCache(requests, {3: 1}, max_tokens=max_tokens, max_positions=300, dtype=torch.float32, device="cpu")
+
+
+def test_groups_have_storage_of_their_own():
+    cache = _cache(extra=[(4, StateRequest((3, 5)))])
+    assert len(cache.kv_groups) == 2  # all keys / a window of them
+    full, windowed = cache.kv_groups
+    assert full.k.shape == (2, 8, 2, 64, 16) and full.v.shape == (2, 8, 2, 16, 64)
+    assert windowed.k.shape == (1, 8, 1, 64, 32) and windowed.request.window == 100
+    assert cache.view(0).k_pages.data_ptr() != cache.view(1).k_pages.data_ptr()
+    shared = cache.view(3)  # reads entry 1's cache
+    assert shared.read_only and shared.k_pages.data_ptr() == cache.view(1).k_pages.data_ptr()
+    assert not cache.view(1).read_only
+    assert cache.view(4).state.shape == (8, 3, 5)
+    assert cache.bytes_per_token() == 2 * 2 * 2 * 16 * 4 + 2 * 1 * 1 * 32 * 4
+
+
+def test_slots_are_given_back_and_used_again():
+    cache = _cache(max_tokens=256)  # 4 pages, 4 slots
+    a, b = cache.acquire(), cache.acquire()
+    cache.grow({a: 70, b: 5})
+    assert cache.length(a) == 70 and cache.length(b) == 5 and cache.live_tokens() == 75
+    assert cache.kv_groups[0].table.pool.free == 1
+    # a refused growth changes nothing: neither lengths nor pages
+    with pytest.raises(CacheFull):
+        cache.grow({a: 60, b: 60})
+    assert cache.length(a) == 70 and cache.length(b) == 5 and cache.kv_groups[0].table.pool.free == 1
+    with pytest.raises(CacheFull, match="positions end at 300"):
+        cache.check_room({a: 231})
+    pages_of_a = list(cache.kv_groups[0].table.rows[a])
+    row = cache.kv_groups[0].block_table[a, :2].tolist()
+    assert row == pages_of_a  # the device table follows the host's
+    cache.release(a)
+    with pytest.raises(InvalidInput):
+        cache.release(a)
+    with pytest.raises(InvalidInput):
+        cache.length(a)
+    again = cache.acquire()
+    assert again == a and cache.length(again) == 0  # the slot is used again, empty
+    cache.grow({again: 128})
+    assert sorted(cache.kv_groups[0].table.rows[again]) == sorted(pages_of_a)  # and so are its pages
+    for slot in (again, b):
+        cache.release(slot)
+    assert all(g.table.pool.free == 4 for g in cache.kv_groups) and cache.slots.free == 4
+
+
+def test_state_starts_at_zero():
+    cache = _cache(extra=[(4, StateRequest((2,), "float32"))])
+    region = cache.add_state_region("extra", (), torch.int64)
+    slot = cache.acquire()
+    cache.view(4).state[slot] = 7.0
+    region[slot] = 99
+    cache.release(slot)
+    assert cache.acquire() == slot
+    assert cache.view(4).state[slot].abs().sum() == 0 and region[slot] == 0
+    with pytest.raises(InvalidInput):
+        cache.add_state_region("extra", (), torch.int64)

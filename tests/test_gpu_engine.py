@@ -1,0 +1,210 @@
+"""The engine in process: long decoding, the first tokens of a sequence, greedy
+generation through the entry points, sampling on the device against the host
+sampler, slot reuse, refused steps."""
+
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import plain_llama as P
+from configs import TINY_CONFIGS
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+TOL = {"float32": (2e-5, 2e-5), "bfloat16": (2e-2, 2e-2)}
+
+
+def _engine(model_dirs, name, dtype, max_tokens=1024):
+    from nnis_amd.api import load_engine
+
+    return load_engine(model_dirs[name], dtype=dtype, max_tokens=max_tokens)
+
+
+def _close(got, want, dtype, what):
+    atol, rtol = TOL[dtype]
+    error = (got - want).abs()
+    bound = atol + rtol * want.abs()
+    assert bool((error <= bound).all()), f"{what}: max error {error.max().item():.3g}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_long_decoding(model_dirs, name, dtype):
+    """A short prompt, then several pages of single-token steps: every
+    position's logits against the plain whole-sequence run."""
+    from nnis_amd.engine.batch import StepEntry
+
+    config, seed = TINY_CONFIGS[name]
+    total = config["max_position_embeddings"] - 3
+    ids = np.random.default_rng(seed).integers(0, config["vocab_size"], size=total).tolist()
+    want = P.PlainLlama(model_dirs[name]).logits(ids)
+    engine = _engine(model_dirs, name, dtype)
+    slot = engine.start_sequence()
+    rows = [engine.step([StepEntry(slot, ids[:3], [0, 1, 2])])]
+    for token in ids[3:]:
+        rows.append(engine.step([StepEntry(slot, [token], [0])]))
+    got = torch.cat(rows).cpu()
+    assert engine.length(slot) == total
+    _close(got, want, dtype, f"tiny {name} {dtype} long decoding")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_first_tokens(model_dirs, dtype):
+    """A sequence's very first tokens, fed one at a time from an empty slot,
+    next to a longer neighbour in the same batch."""
+    from nnis_amd.engine.batch import StepEntry
+
+    config, _ = TINY_CONFIGS["C"]
+    rng = np.random.default_rng(9)
+    short, long = rng.integers(0, config["vocab_size"], size=4).tolist(), rng.integers(0, config["vocab_size"], size=70).tolist()
+    plain = P.PlainLlama(model_dirs["C"])
+    engine = _engine(model_dirs, "C", dtype)
+    a, b = engine.start_sequence(), engine.start_sequence()
+    first = engine.step([StepEntry(a, short[:1], [0]), StepEntry(b, long[:67], [66])]).cpu()
+    _close(first[0], plain.logits(short[:1])[0], dtype, "first token")
+    _close(first[1], plain.logits(long[:67])[66], dtype, "neighbour")
+    for i in range(1, 4):
+        rows = engine.step([StepEntry(b, [long[66 + i]], [0]), StepEntry(a, [short[i]], None)]).cpu()
+        _close(rows[1], plain.logits(short[:i + 1])[i], dtype, f"token {i}")
+        _close(rows[0], plain.logits(long[:67 + i])[66 + i], dtype, f"neighbour {i}")
+
+
+def test_refused_steps_change_nothing(model_dirs):
+    from nnis_amd.engine.batch import StepEntry
+    from nnis_amd.errors import CacheFull, InvalidInput
+
+    engine = _engine(model_dirs, "A", "float32", max_tokens=128)
+    slot = engine.start_sequence()
+    engine.step([StepEntry(slot, [1, 2, 3], None)])
+    for bad in ([StepEntry(slot, [], None)], [StepEntry(slot, [512], None)], [StepEntry(slot, [1], [1])],
+                [StepEntry(slot, [1], None), StepEntry(slot, [2], None)], [StepEntry(7, [1], None)], []):
+        with pytest.raises(InvalidInput):
+            engine.step(bad)
+    with pytest.raises(CacheFull):
+        engine.step([StepEntry(slot, [1] * 126, None)])  # 129 tokens in a cache of 128
+    other = engine.start_sequence()
+    with pytest.raises(CacheFull):
+        engine.step([StepEntry(other, [1] * 10, None), StepEntry(slot, [1] * 70, None)])  # 1 + 2 pages of 2
+    assert engine.length(slot) == 3 and engine.length(other) == 0 and engine.free_pages() == 1
+    with pytest.raises(CacheFull, match="positions"):
+        big = _engine(model_dirs, "A", "float32", max_tokens=1024)
+        s = big.start_sequence()
+        big.step([StepEntry(s, [1] * 257, None)])  # the model has 256 positions
+
+
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_greedy_generation_through_the_entry_point(model_dirs, name):
+    import nnis_amd
+
+    config, seed = TINY_CONFIGS[name]
+    rng = np.random.default_rng(40 + seed)
+    prompts = [rng.integers(0, config["vocab_size"], size=n).tolist() for n in (5, 11, 17, 1, 66)]
+    plain = P.PlainLlama(model_dirs[name])
+    stops = config.get("eos_token_id", [])
+    stops = [stops] if isinstance(stops, int) else stops
+    want = [plain.greedy(p, 8, stops) for p in prompts]
+    # a cache of 6 pages and batches of at most 3: two batches, slots used again
+    got = nnis_amd.generate(model_dirs[name], prompts, max_new_tokens=8, dtype="float32", max_tokens=6 * 64, max_batch=3)
+    assert got == want
+    # bfloat16 may leave the 32-bit path at a near tie: every token it picks must be
+    # (nearly) the plain model's best continuation of what it has picked so far
+    got16 = nnis_amd.generate(model_dirs[name], prompts, max_new_tokens=8, dtype="bfloat16", max_tokens=6 * 64, max_batch=3)
+    for prompt, tokens in zip(prompts, got16):
+        assert 1 <= len(tokens) <= 8
+        logits = plain.logits(prompt + tokens)[len(prompt) - 1:-1]
+        for row, token in zip(logits, tokens):
+            assert row[token].item() >= row.max().item() - 3e-2
+
+
+def test_command_line(model_dirs):
+    plain = P.PlainLlama(model_dirs["B"])
+    prompt = [3, 141, 59, 26, 535]
+    run = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "nnis"), "generate", "--model", model_dirs["B"],
+                          "--prompt-ids", ",".join(map(str, prompt)), "--max-new-tokens", "6", "--dtype", "float32"],
+                         capture_output=True, text=True, timeout=300)
+    assert run.returncode == 0, run.stderr[-2000:]
+    assert [int(t) for t in run.stdout.strip().split(",")] == plain.greedy(prompt, 6)
+    run = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "nnis"), "generate-batch", "--model", model_dirs["B"],
+                          "--prompt-ids", "1,2,3", "--prompt-ids", "9", "--seed", "5", "--seed", "6", "--max-new-tokens", "4",
+                          "--temperature", "0.8", "--json"], capture_output=True, text=True, timeout=300)
+    assert run.returncode == 0, run.stderr[-2000:]
+    import json
+
+    payload = json.loads(run.stdout)
+    assert payload["session_count"] == 2 and [r["seed"] for r in payload["results"]] == [5, 6]
+    assert all(r["ok"] and len(r["text"].split(",")) == 4 for r in payload["results"])
+    run = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "nnis"), "generate", "--model", "/nonexistent",
+                          "--prompt-ids", "1"], capture_output=True, text=True, timeout=300)
+    assert run.returncode == 1 and run.stderr.startswith("nnis generate:")
+
+
+@pytest.mark.parametrize("options", [dict(), dict(temperature=0.8), dict(top_k=40), dict(top_p=0.7),
+                                     dict(temperature=1.3, top_k=200, top_p=0.95), dict(top_k=1)])
+def test_device_sampling_matches_the_host_sampler(options):
+    """Same logits, same seeds: the kernel picks what the reference's host
+    procedure picks, draw after draw (the generator state lives per slot)."""
+    from nnis_amd.kernels import ops
+    from nnis_amd.sampling import HostSampler, SamplingParams
+
+    vocab, rows, draws = 1000, 6, 40
+    rng = np.random.default_rng(3)
+    logits = (rng.standard_normal((rows, vocab)) * 2.5).astype(np.float32)
+    logits[0, 5] = logits[0, 900] = logits[0].max() + 0.5  # a tie at the top
+    logits[1, :] = 0.25  # all equal
+    logits[2, 17] = -0.0
+    logits[2, 18] = 0.0
+    dev = torch.from_numpy(logits).cuda()
+    slots = [4, 0, 7, 2, 5, -1]  # the last row is skipped
+    state = torch.zeros(8, dtype=torch.int64, device="cuda")
+    seeds = [11, 2**64 - 3, 13, 14, 15, 16]
+    hosts = []
+    for slot, seed in zip(slots, seeds):
+        if slot >= 0:
+            state[slot] = seed if seed < 2**63 else seed - 2**64
+        hosts.append(HostSampler(SamplingParams(seed=seed, **options), vocab))
+    temperature = torch.full((rows,), options.get("temperature", 1.0), dtype=torch.float32, device="cuda")
+    top_k = torch.full((rows,), options.get("top_k", 0), dtype=torch.int32, device="cuda")
+    top_p = torch.full((rows,), options.get("top_p", 0.0), dtype=torch.float32, device="cuda")
+    weights = torch.empty((rows, vocab), dtype=torch.float64, device="cuda")
+    row_slot = torch.tensor(slots, dtype=torch.int32, device="cuda")
+    for draw in range(draws):
+        out = torch.full((rows,), -7, dtype=torch.int32, device="cuda")
+        ops.sample(dev, weights, row_slot, state, temperature, top_k, top_p, out)
+        got = out.cpu().tolist()
+        assert got[5] == -7
+        for row in range(5):
+            assert got[row] == hosts[row].sample(logits[row]), (draw, row, options)
+    bad = dev.clone()
+    bad[3, 10] = float("nan")
+    out = torch.zeros(rows, dtype=torch.int32, device="cuda")
+    ops.sample(bad, weights, row_slot, state, temperature, top_k, top_p, out)
+    assert out[3].item() == -1 and out[0].item() >= 0
+
+
+def test_sampled_generation_is_seeded_and_per_sequence(model_dirs):
+    import nnis_amd
+    from nnis_amd.api import load_engine
+    from nnis_amd.sampling import HostSampler, SamplingParams
+
+    config, _ = TINY_CONFIGS["B"]
+    engine = load_engine(model_dirs["B"], dtype="float32", max_tokens=512)
+    prompts = [[1], [7, 8, 9, 10, 11, 12, 13], list(range(100, 123)), list(range(200, 240))]
+    seeds = [7, 8, 9, 10]
+    got = nnis_amd.generate(engine, prompts, max_new_tokens=12, sample=True, seed=seeds, temperature=0.8)
+    again = nnis_amd.generate(engine, prompts, max_new_tokens=12, sample=True, seed=seeds, temperature=0.8)
+    assert got == again and all(len(t) == 12 for t in got)
+    alone = nnis_amd.generate(engine, [prompts[2]], max_new_tokens=12, sample=True, seed=9, temperature=0.8)
+    assert alone[0] == got[2]  # what else is in the batch does not change a sequence
+    # the plain model and the host sampler, step by step
+    plain = P.PlainLlama(model_dirs["B"])
+    sampler = HostSampler(SamplingParams(seed=8, temperature=0.8), config["vocab_size"])
+    ids = list(prompts[1])
+    for token in got[1]:
+        assert sampler.sample(plain.logits(ids)[-1].numpy()) == token
+        ids.append(token)
+    assert engine.free_slots() == engine.cache.max_slots and engine.free_pages() == engine.cache.pages

@@ -1,0 +1,288 @@
+"""Each part alone against its plain function; the order of layers as data (a
+layer named twice, a layer that reads another layer's cache); and a toy mixer
+with state of its own, defined here, registered, built and stepped without a
+change to the library's files."""
+
+import math
+from dataclasses import dataclass
+
+import numpy as np
+import pytest
+import torch
+
+import plain_llama as P
+from gpu_helpers import assert_close, cache_for, context, runtime
+
+pytestmark = pytest.mark.gpu
+DTYPES = ["float32", "bfloat16"]
+
+
+def _w(shape, dtype, seed, gain=False):
+    g = torch.Generator().manual_seed(seed)
+    noise = torch.randn(shape, generator=g)
+    value = 1.0 + 0.1 * noise if gain else noise / math.sqrt(shape[-1])
+    return value.to(torch.bfloat16 if dtype == "bfloat16" else torch.float32)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_norm_part(dtype):
+    from nnis_amd.parts import build_part
+
+    rt = runtime(dtype)
+    width, eps = 70, 3e-4
+    norm = build_part("norm", {"kind": "rms", "width": width, "eps": eps, "weight": "n.w"})
+    assert [(t.name, t.shape, t.init) for t in norm.tensors()] == [("n.w", (70,), "gain")]
+    weight = _w((width,), dtype, 1, gain=True)
+    norm.bind({"n.w": weight.cuda()}, rt)
+    x = torch.randn(9, width) * 3
+    delta = torch.randn(9, width).to(rt.dtype)
+    assert_close(norm.forward(x.cuda(), rt), P.rms_norm(x, weight.float(), eps), dtype, "norm")
+    stream = x.cuda().clone()
+    got = norm.add_forward(stream, delta.cuda(), rt)
+    assert_close(got, P.rms_norm(x + delta.float(), weight.float(), eps), dtype, "add + norm")
+    assert torch.equal(stream.cpu(), x + delta.float())  # the residual sum is kept in 32-bit
+    rows = torch.tensor([8, 0, 3], dtype=torch.int32).cuda()
+    stream = x.cuda().clone()
+    got = norm.add_forward(stream, delta.cuda(), rt, rows=rows)
+    assert_close(got, P.rms_norm((x + delta.float())[[8, 0, 3]], weight.float(), eps), dtype, "gathered rows")
+    assert torch.equal(stream.cpu(), x)  # a gather writes nothing back
+
+
+def test_rotary_tables_equal_the_plain_ones():
+    from nnis_amd.parts import build_part
+
+    rt = runtime("float32")
+    for rot_dim, theta, positions in ((16, 10000.0, 256), (32, 100000.0, 512), (64, 130000.0, 8192)):
+        part = build_part("position", {"kind": "rotary_half", "rot_dim": rot_dim, "theta": theta, "max_positions": positions})
+        part.bind({}, rt)
+        tables = part.rotary()
+        cos, sin = P.rope_tables(positions, rot_dim, theta)
+        assert tables.rot_dim == rot_dim and tables.cos.dtype == torch.float32
+        assert np.abs(tables.cos.cpu().numpy() - cos).max() <= 6e-8 and np.abs(tables.sin.cpu().numpy() - sin).max() <= 6e-8
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("heads, kv_heads, head_dim, width", [(4, 2, 16, 64), (3, 1, 32, 80), (6, 6, 48, 100)])
+def test_attention_part(dtype, heads, kv_heads, head_dim, width):
+    """Two sequences of unequal length, whole and then continued by single
+    tokens, against the plain functions on each whole sequence."""
+    from nnis_amd.parts import build_part
+
+    rt = runtime(dtype)
+    rope = build_part("position", {"kind": "rotary_half", "rot_dim": head_dim, "theta": 5000.0, "max_positions": 300})
+    rope.bind({}, rt)
+    mixer = build_part("mixer", {"kind": "causal_attention", "width": width, "heads": heads, "kv_heads": kv_heads,
+                                 "head_dim": head_dim, "position": "r", "q": "q", "k": "k", "v": "v", "o": "o"},
+                       positions={"r": rope})
+    shapes = {t.name: t.shape for t in mixer.tensors()}
+    assert shapes == {"q": (heads * head_dim, width), "k": (kv_heads * head_dim, width),
+                      "v": (kv_heads * head_dim, width), "o": (width, heads * head_dim)}
+    weights = {n: _w(s, dtype, i) for i, (n, s) in enumerate(shapes.items())}
+    mixer.bind({n: w.cuda() for n, w in weights.items()}, rt)
+    cache = cache_for([mixer.cache_request()], rt)
+    lengths = (70, 9)
+    xs = [torch.randn(n + 3, width).to(rt.dtype) for n in lengths]
+    cos, sin = (torch.from_numpy(t) for t in P.rope_tables(300, head_dim, 5000.0))
+
+    def plain(x):
+        t = x.shape[0]
+        x = x.float()
+        q = P.linear(x, weights["q"].float()).view(t, heads, head_dim)
+        k = P.linear(x, weights["k"].float()).view(t, kv_heads, head_dim)
+        v = P.linear(x, weights["v"].float()).view(t, kv_heads, head_dim)
+        q, k = P.rope_rotate_half(q, cos[:t], sin[:t]), P.rope_rotate_half(k, cos[:t], sin[:t])
+        out = P.causal_attention(q, k, v, 1.0 / math.sqrt(head_dim)).reshape(t, heads * head_dim)
+        return P.linear(out, weights["o"].float())
+
+    want = [plain(x) for x in xs]
+    slots = [cache.acquire(), cache.acquire(), cache.acquire()][1:]  # not slot 0
+    ctx = context(cache, list(zip(slots, lengths)))
+    got = mixer.forward(torch.cat([x[:n] for x, n in zip(xs, lengths)]).cuda(), ctx, cache.view(0), rt)
+    assert_close(got[:70], want[0][:70], dtype, "prompt 0")
+    assert_close(got[70:], want[1][:9], dtype, "prompt 1")
+    for step in range(3):
+        ctx = context(cache, [(slots[1], 1), (slots[0], 1)])  # the other order
+        x = torch.stack([xs[1][9 + step], xs[0][70 + step]]).cuda()
+        got = mixer.forward(x, ctx, cache.view(0), rt)
+        assert_close(got[0], want[1][9 + step], dtype, f"decode {step} seq 1")
+        assert_close(got[1], want[0][70 + step], dtype, f"decode {step} seq 0")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_feed_forward_embedding_and_head_parts(dtype):
+    from nnis_amd.parts import build_part
+
+    rt = runtime(dtype)
+    width, inner, vocab = 72, 200, 333
+    ff = build_part("feed_forward", {"kind": "gated", "width": width, "inner": inner, "activation": "silu",
+                                     "gate": "g", "up": "u", "down": "d"})
+    weights = {"g": _w((inner, width), dtype, 1), "u": _w((inner, width), dtype, 2), "d": _w((width, inner), dtype, 3)}
+    ff.bind({n: w.cuda() for n, w in weights.items()}, rt)
+    x = torch.randn(11, width).to(rt.dtype)
+    want = P.swiglu(x.float(), weights["g"].float(), weights["u"].float(), weights["d"].float())
+    assert_close(ff.forward(x.cuda(), None, rt), want, dtype, "gated feed-forward")
+
+    table = _w((vocab, width), dtype, 4)
+    emb = build_part("embedding", {"kind": "table", "vocab_size": vocab, "width": width, "weight": "e"})
+    emb.bind({"e": table.cuda()}, rt)
+    ids = torch.tensor([0, 332, 17, 17], dtype=torch.int32)
+    got = emb.forward(ids.cuda(), 4, rt)
+    assert got.dtype == torch.float32 and torch.equal(got.cpu(), P.embedding(table.float(), ids.tolist()))
+    head = build_part("head", {"kind": "linear", "vocab_size": vocab, "width": width, "weight": "h", "tied_to": "e"})
+    assert head.tensors()[0].fallback == "e"
+    head.bind({"h": table.cuda()}, rt)
+    logits = head.forward(x.cuda(), rt)
+    assert logits.dtype == torch.float32
+    assert_close(logits, P.linear(x.float(), table.float()), dtype, "head")
+
+
+# ---------------------------------------------------------------------------
+# a toy architecture defined here: blocks whose mixer keeps a running sum per
+# sequence, next to attention blocks; one layer runs twice, one reads another's cache
+# ---------------------------------------------------------------------------
+
+def _register_toy():
+    from nnis_amd.config import register_architecture
+    from nnis_amd.models import ModelSpec, ScheduleEntry
+    from nnis_amd.parts import Mixer, StateRequest, TensorSpec, register_part
+    from nnis_amd.parts.linear import Projection
+
+    class RunningMean(Mixer):
+        """y_t = W * mean(x_0 .. x_t): the sum so far is the state."""
+
+        def __init__(self, width, weight):
+            self.width, self.weight_name, self.proj = width, weight, None
+
+        def tensors(self):
+            return [TensorSpec(self.weight_name, (self.width, self.width))]
+
+        def bind(self, weights, rt):
+            self.proj = Projection(weights[self.weight_name])
+
+        def cache_request(self):
+            return StateRequest((self.width,), "float32")
+
+        def forward(self, x, ctx, view, rt):
+            means = torch.empty(x.shape, dtype=torch.float32, device=x.device)
+            start = 0
+            for slot, count, pos0 in zip(ctx.host_slots, ctx.host_new, ctx.host_pos0):
+                sums = view.state[slot] + torch.cumsum(x[start:start + count].float(), dim=0)
+                if not view.read_only:
+                    view.state[slot] = sums[-1]
+                steps = torch.arange(pos0 + 1, pos0 + count + 1, device=x.device, dtype=torch.float32)
+                means[start:start + count] = sums / steps[:, None]
+                start += count
+            return self.proj(means.to(rt.dtype), rt)
+
+    @dataclass(frozen=True)
+    class ToyConfig:
+        width: int
+        vocab_size: int
+        layers: int
+        raw: dict
+
+        @classmethod
+        def from_dict(cls, raw):
+            return cls(raw["width"], raw["vocab_size"], raw["layers"], dict(raw))
+
+    def toy_spec(cfg):
+        w = cfg.width
+
+        def block(index, mixer):
+            p = f"blocks.{index}."
+            return {"kind": "pre_norm", "width": w,
+                    "norm1": {"kind": "rms", "width": w, "eps": 1e-5, "weight": p + "n1"}, "mixer": mixer,
+                    "norm2": {"kind": "rms", "width": w, "eps": 1e-5, "weight": p + "n2"},
+                    "feed_forward": {"kind": "gated", "width": w, "inner": 2 * w + 8, "gate": p + "g", "up": p + "u", "down": p + "d"}}
+
+        layers = []
+        for index in range(cfg.layers):
+            p = f"blocks.{index}."
+            if index % 2 == 0:
+                mixer = {"kind": "running_mean", "width": w, "weight": p + "mix"}
+            else:
+                mixer = {"kind": "causal_attention", "width": w, "heads": 2, "kv_heads": 1, "head_dim": 16,
+                         "position": "rope", "q": p + "q", "k": p + "k", "v": p + "v", "o": p + "o"}
+            layers.append(block(index, mixer))
+        # layer 0 runs twice (its second run keeps state of its own); the last
+        # entry runs layer 1 again on the cache that entry 1 filled
+        schedule = [ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(2), ScheduleEntry(0), ScheduleEntry(1, reads_cache_of=1)]
+        return ModelSpec(
+            architecture="ToyForCausalLM", width=w, vocab_size=cfg.vocab_size, max_positions=256, stored_dtype="bfloat16",
+            embedding={"kind": "table", "vocab_size": cfg.vocab_size, "width": w, "weight": "emb"},
+            positions={"rope": {"kind": "rotary_half", "rot_dim": 16, "theta": 1000.0, "max_positions": 256}},
+            layers=layers, schedule=schedule,
+            final_norm={"kind": "rms", "width": w, "eps": 1e-5, "weight": "norm"},
+            head={"kind": "linear", "vocab_size": cfg.vocab_size, "width": w, "weight": "head", "tied_to": None},
+            config_json=cfg.raw)
+
+    register_part("mixer", "running_mean", RunningMean, replace=True)
+    register_architecture("ToyForCausalLM", ToyConfig, toy_spec, replace=True)
+
+
+def _plain_toy(folder, ids):
+    """The toy model on one whole sequence with the plain functions."""
+    from safetensors import safe_open
+
+    with safe_open(folder + "/model.safetensors", framework="pt") as handle:
+        w = {n: handle.get_tensor(n).float() for n in handle.keys()}
+    t, width = len(ids), w["emb"].shape[1]
+    cos, sin = (torch.from_numpy(a) for a in P.rope_tables(256, 16, 1000.0))
+    x = P.embedding(w["emb"], ids)
+
+    def attention(p, h):
+        q = P.rope_rotate_half(P.linear(h, w[p + "q"]).view(t, 2, 16), cos[:t], sin[:t])
+        k = P.rope_rotate_half(P.linear(h, w[p + "k"]).view(t, 1, 16), cos[:t], sin[:t])
+        v = P.linear(h, w[p + "v"]).view(t, 1, 16)
+        return q, k, v
+
+    kept = {}
+    for entry, (layer, reads) in enumerate([(0, None), (1, None), (2, None), (0, None), (1, 1)]):
+        p = f"blocks.{layer}."
+        h = P.rms_norm(x, w[p + "n1"], 1e-5)
+        if layer % 2 == 0:
+            steps = torch.arange(1, t + 1, dtype=torch.float32)[:, None]
+            mixed = P.linear(torch.cumsum(h, 0) / steps, w[p + "mix"])
+        else:
+            q, k, v = attention(p, h)
+            if reads is None:
+                kept[entry] = (k, v)
+            else:
+                k, v = kept[reads]
+            mixed = P.linear(P.causal_attention(q, k, v, 0.25).reshape(t, 32), w[p + "o"])
+        x = x + mixed
+        x = x + P.swiglu(P.rms_norm(x, w[p + "n2"], 1e-5), w[p + "g"], w[p + "u"], w[p + "d"])
+    return P.linear(P.rms_norm(x, w["norm"], 1e-5), w["head"])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_toy_architecture_with_a_stateful_mixer(tmp_path, dtype):
+    import nnis_amd
+    from nnis_amd.api import load_engine
+    from nnis_amd.engine.batch import StepEntry
+
+    _register_toy()
+    folder = str(tmp_path / "toy")
+    raw = {"architectures": ["ToyForCausalLM"], "model_type": "toy", "width": 48, "vocab_size": 211, "layers": 3}
+    nnis_amd.write_random_model(folder, raw, seed=3)
+    engine = load_engine(folder, dtype=dtype, max_tokens=512)
+    # two attention entries keep keys and values (the third reads the second's); three keep a running sum
+    assert len(engine.cache.kv_groups) == 1 and len(engine.cache.kv_groups[0].entries) == 1
+    assert sorted(engine.cache.state_regions) == ["entry0", "entry2", "entry3"]
+    rng = np.random.default_rng(0)
+    a, b = rng.integers(0, 211, size=50).tolist(), rng.integers(0, 211, size=13).tolist()
+    want_a, want_b = _plain_toy(folder, a), _plain_toy(folder, b)
+    sa, sb = engine.start_sequence(), engine.start_sequence()
+    rows = engine.step([StepEntry(sa, a[:40], list(range(40))), StepEntry(sb, b[:3], [0, 1, 2])]).cpu()
+    assert_close(rows[:40], want_a[:40], dtype, "toy prompt a")
+    assert_close(rows[40:], want_b[:3], dtype, "toy prompt b")
+    for i in range(10):
+        rows = engine.step([StepEntry(sb, [b[3 + i]], [0]), StepEntry(sa, [a[40 + i]], [0])]).cpu()
+        assert_close(rows[0], want_b[3 + i], dtype, f"toy decode b {i}")
+        assert_close(rows[1], want_a[40 + i], dtype, f"toy decode a {i}")
+    # a slot used again starts from zero state
+    engine.end_sequence(sa)
+    again = engine.start_sequence()
+    assert again == sa
+    rows = engine.step([StepEntry(again, b, list(range(13)))]).cpu()
+    assert_close(rows, want_b, dtype, "toy reused slot")

@@ -1,0 +1,70 @@
+"""Trace replay through bin/trace_run, as a user runs it: the same requests
+whole, with the last 32 tokens one by one, and in batches of unequal lengths
+whose shorter requests end earlier, one batch after another so that slots and
+pages are used again -- in 32-bit and in bfloat16, against the plain
+implementation."""
+
+import numpy as np
+import pytest
+import torch
+
+import plain_llama as P
+import replay
+from configs import TINY_CONFIGS
+
+pytestmark = pytest.mark.gpu
+
+# lengths on purpose: 1 (a prompt that is only its first token), around a page's edge (63..65, 128..130), odd ones
+LENGTHS = [1, 7, 23, 40, 64, 65, 97, 130, 5, 63]
+
+
+def _requests(vocab, seed):
+    rng = np.random.default_rng(seed)
+    return {f"r{i}": rng.integers(0, vocab, size=n).tolist() for i, n in enumerate(LENGTHS)}
+
+
+def _compare(rows, plain_logits, atol, rtol, what):
+    worst = 0.0
+    for (name, position), row in rows.items():
+        want = plain_logits[name][position].numpy()
+        error = np.abs(row - want)
+        bound = atol + rtol * np.abs(want)
+        if np.any(error > bound):
+            index = int(np.argmax(error - bound))
+            raise AssertionError(f"{what}: request {name} position {position} logit {index}: "
+                                 f"got {row[index]:.6f}, plain {want[index]:.6f} (max error {error.max():.3g})")
+        worst = max(worst, float(error.max()))
+    return worst
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_schedules_agree_with_the_plain_model(model_dirs, tmp_path, name, dtype):
+    config, seed = TINY_CONFIGS[name]
+    vocab = config["vocab_size"]
+    requests = _requests(vocab, 100 + seed)
+    plain = P.PlainLlama(model_dirs[name], torch.float32)
+    plain_logits = {n: plain.logits(t) for n, t in requests.items()}
+    # 32-bit: rounding of sums only.  bfloat16: activations and cache keep 8 bits
+    # of mantissa; logits here are of order 1.
+    atol, rtol = (2e-5, 2e-5) if dtype == "float32" else (2e-2, 2e-2)
+
+    # every schedule in one process, one after another, with a cache too small
+    # to hold them side by side: 8 pages, the largest batch needs 7
+    steps = replay.whole(requests) + replay.tail_one_by_one(requests) + replay.unequal_batches(requests, batch=4, decode=32)
+    count_whole = len(replay.whole(requests))
+    count_tail = len(replay.tail_one_by_one(requests))
+    renamed = []
+    for number, step in enumerate(steps):  # one name space per schedule
+        tag = "w" if number < count_whole else ("t" if number < count_whole + count_tail else "b")
+        renamed.append({"entries": [dict(e, id=tag + e["id"]) for e in step["entries"]], "end": [tag + n for n in step.get("end", [])]})
+    rows = replay.run_trace(model_dirs[name], dtype, renamed, str(tmp_path), max_tokens=8 * 64, vocab=vocab)
+    assert len(rows) == 3 * sum(LENGTHS)
+    for tag, what in (("w", "whole"), ("t", "last 32 one by one"), ("b", "unequal batches")):
+        part = {(n[1:], p): row for (n, p), row in rows.items() if n[0] == tag}
+        assert len(part) == sum(LENGTHS)
+        _compare(part, plain_logits, atol, rtol, f"tiny {name} {dtype} {what}")
+    # the schedules agree with each other far more closely than with the plain model's rounding
+    between = max(float(np.abs(rows[("w" + n, p)] - rows[(tag + n, p)]).max())
+                  for tag in "tb" for n, t in requests.items() for p in range(len(t)))
+    assert between <= (1e-5 if dtype == "float32" else 2e-2), between

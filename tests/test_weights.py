@@ -1,0 +1,168 @@
+"""Weights by name: the writer and reader of the container, the random-weights
+mode, and the one error that lists everything wrong with a folder
+(/root/reference/crates/nnis-model/src/safetensors_loader.rs:1075-1157)."""
+
+import json
+import os
+import shutil
+import struct
+
+import pytest
+import torch
+
+import nnis_amd
+import nnis_amd.models  # noqa: F401
+from configs import TINY_A, TINY_B, TINY_C
+from nnis_amd.config import spec_from_config
+from nnis_amd.errors import WeightError
+from nnis_amd.models import DecoderModel
+from nnis_amd.weights import SafetensorsFile, load_weights, write_safetensors
+
+
+def _specs(config):
+    return DecoderModel(spec_from_config(config)[1]).tensors()
+
+
+def test_container_round_trip_against_the_package(tmp_path):
+    from safetensors import safe_open
+
+    tensors = [("a", torch.randn(3, 5)), ("b.c", torch.randn(7).to(torch.bfloat16)), ("i", torch.arange(6, dtype=torch.int32).view(2, 3))]
+    path = str(tmp_path / "x.safetensors")
+    write_safetensors(path, tensors, {"note": "t"})
+    with safe_open(path, framework="pt") as handle:  # the package reads what we wrote
+        for name, tensor in tensors:
+            assert torch.equal(handle.get_tensor(name), tensor)
+    ours = SafetensorsFile(path)
+    assert ours.entries["b.c"] == ("BF16", (7,)) and ours.metadata == {"note": "t"}
+    for name, tensor in tensors:
+        assert torch.equal(ours.tensor(name), tensor)
+
+
+def test_random_model_folder(model_dirs):
+    for name, config in (("A", TINY_A), ("B", TINY_B), ("C", TINY_C)):
+        folder = model_dirs[name]
+        assert sorted(os.listdir(folder)) == ["config.json", "model.safetensors"]
+        handle = SafetensorsFile(os.path.join(folder, "model.safetensors"))
+        names = set(handle.names())
+        assert ("lm_head.weight" in names) == (not config["tie_word_embeddings"])
+        stored = "BF16" if config["torch_dtype"] == "bfloat16" else "F32"
+        assert all(dtype == stored for dtype, _ in handle.entries.values())
+        gain = handle.tensor("model.norm.weight").float()
+        matrix = handle.tensor("model.layers.0.mlp.up_proj.weight").float()
+        assert abs(gain.mean().item() - 1.0) < 0.01 and 0.005 < gain.std().item() < 0.02
+        assert abs(matrix.mean().item()) < 0.002 and 0.017 < matrix.std().item() < 0.023
+
+
+def test_random_weights_follow_the_seed(tmp_path):
+    a, b, c = (str(tmp_path / n) for n in "abc")
+    nnis_amd.write_random_model(a, TINY_A, 5)
+    nnis_amd.write_random_model(b, TINY_A, 5)
+    nnis_amd.write_random_model(c, TINY_A, 6)
+    read = lambda d: open(os.path.join(d, "model.safetensors"), "rb").read()  # noqa: E731
+    assert read(a) == read(b) and read(a) != read(c)
+
+
+def test_load_keeps_stored_types_and_shares_a_tied_head(model_dirs):
+    w = load_weights(model_dirs["A"], _specs(TINY_A), "cpu", widen_to_float32=False)
+    assert all(t.dtype == torch.bfloat16 for t in w.values())
+    assert w["lm_head.weight"].data_ptr() == w["model.embed_tokens.weight"].data_ptr()
+    wide = load_weights(model_dirs["A"], _specs(TINY_A), "cpu", widen_to_float32=True)
+    assert all(t.dtype == torch.float32 for t in wide.values())
+    assert torch.equal(wide["model.norm.weight"], w["model.norm.weight"].float())  # widening is exact
+    # stored in 32-bit stays so
+    c = load_weights(model_dirs["C"], _specs(TINY_C), "cpu", widen_to_float32=False)
+    assert all(t.dtype == torch.float32 for t in c.values())
+
+
+def test_one_error_lists_everything(model_dirs, tmp_path):
+    folder = str(tmp_path / "broken")
+    shutil.copytree(model_dirs["B"], folder)
+    handle = SafetensorsFile(os.path.join(folder, "model.safetensors"))
+    tensors = []
+    for name in handle.names():
+        tensor = handle.tensor(name).clone()
+        if name == "model.layers.1.mlp.up_proj.weight":
+            continue  # missing
+        if name == "model.layers.0.self_attn.k_proj.weight":
+            tensor = tensor[:, :-1].contiguous()  # wrong shape
+        if name == "model.norm.weight":
+            tensor = tensor.to(torch.float16)  # unsupported stored type
+        tensors.append((name, tensor))
+    tensors.append(("model.layers.7.extra.weight", torch.zeros(2)))  # unexpected
+    tensors.append(("model.layers.0.self_attn.rotary_emb.inv_freq", torch.zeros(16)))  # a known buffer: ignored
+    write_safetensors(os.path.join(folder, "model.safetensors"), tensors)
+    with pytest.raises(WeightError) as info:
+        load_weights(folder, _specs(TINY_B), "cpu", widen_to_float32=False)
+    text = str(info.value)
+    assert "missing tensors (1)" in text and "model.layers.1.mlp.up_proj.weight [256, 96]" in text
+    assert "unexpected tensors (1)" in text and "model.layers.7.extra.weight" in text
+    assert "wrong shapes (1)" in text and "expected [32, 96], file has [32, 95]" in text
+    assert "unsupported stored types (1)" in text and "F16" in text
+    assert "inv_freq" not in text
+
+
+def test_untied_model_without_head_is_an_error(model_dirs, tmp_path):
+    folder = str(tmp_path / "nohead")
+    shutil.copytree(model_dirs["B"], folder)
+    handle = SafetensorsFile(os.path.join(folder, "model.safetensors"))
+    write_safetensors(os.path.join(folder, "model.safetensors"),
+                      [(n, handle.tensor(n).clone()) for n in handle.names() if n != "lm_head.weight"])
+    with pytest.raises(WeightError, match="lm_head.weight"):
+        load_weights(folder, _specs(TINY_B), "cpu", widen_to_float32=False)
+
+
+def test_head_in_file_wins_when_tied(model_dirs, tmp_path):
+    # /root/reference/crates/nnis-model/src/safetensors_loader.rs:755-786
+    folder = str(tmp_path / "tiedhead")
+    shutil.copytree(model_dirs["A"], folder)
+    handle = SafetensorsFile(os.path.join(folder, "model.safetensors"))
+    tensors = [(n, handle.tensor(n).clone()) for n in handle.names()]
+    head = torch.full((512, 64), 0.5, dtype=torch.bfloat16)
+    write_safetensors(os.path.join(folder, "model.safetensors"), tensors + [("lm_head.weight", head)])
+    w = load_weights(folder, _specs(TINY_A), "cpu", widen_to_float32=False)
+    assert torch.equal(w["lm_head.weight"], head)
+
+
+def test_folder_errors(model_dirs, tmp_path):
+    empty = tmp_path / "empty"
+    empty.mkdir()
+    with pytest.raises(WeightError, match="neither"):
+        load_weights(str(empty), _specs(TINY_A), "cpu", False)
+    both = str(tmp_path / "both")
+    shutil.copytree(model_dirs["A"], both)
+    with open(os.path.join(both, "model.safetensors.index.json"), "w") as f:
+        json.dump({"weight_map": {}}, f)
+    with pytest.raises(WeightError, match="both"):
+        load_weights(both, _specs(TINY_A), "cpu", False)
+    # shards named by an index; a path that leaves the folder is refused
+    sharded = tmp_path / "sharded"
+    sharded.mkdir()
+    handle = SafetensorsFile(os.path.join(model_dirs["A"], "model.safetensors"))
+    names = handle.names()
+    half = len(names) // 2
+    write_safetensors(str(sharded / "s1.safetensors"), [(n, handle.tensor(n).clone()) for n in names[:half]])
+    write_safetensors(str(sharded / "s2.safetensors"), [(n, handle.tensor(n).clone()) for n in names[half:]])
+    weight_map = {n: ("s1.safetensors" if i < half else "s2.safetensors") for i, n in enumerate(names)}
+    (sharded / "model.safetensors.index.json").write_text(json.dumps({"weight_map": weight_map}))
+    w = load_weights(str(sharded), _specs(TINY_A), "cpu", False)
+    assert torch.equal(w["model.norm.weight"], handle.tensor("model.norm.weight"))
+    (sharded / "model.safetensors.index.json").write_text(json.dumps({"weight_map": {"x": "../A/model.safetensors"}}))
+    with pytest.raises(WeightError, match="leaves"):
+        load_weights(str(sharded), _specs(TINY_A), "cpu", False)
+
+
+def test_malformed_container(tmp_path):
+    path = tmp_path / "bad.safetensors"
+    path.write_bytes(b"\x01\x02")
+    with pytest.raises(WeightError, match="too short"):
+        SafetensorsFile(str(path))
+    path.write_bytes(struct.pack("<Q", 1 << 40) + b"{}")
+    with pytest.raises(WeightError, match="header length"):
+        SafetensorsFile(str(path))
+    path.write_bytes(struct.pack("<Q", 4) + b"nope")
+    with pytest.raises(WeightError, match="malformed"):
+        SafetensorsFile(str(path))
+    header = json.dumps({"t": {"dtype": "F32", "shape": [4], "data_offsets": [0, 8]}}).encode()
+    path.write_bytes(struct.pack("<Q", len(header)) + header + b"\0" * 8)
+    with pytest.raises(WeightError, match="does not fit"):
+        SafetensorsFile(str(path))
