@@ -1,0 +1,173 @@
+"""Decode and prefill throughput of the Llama engine on one MI355X.
+
+    python bench.py --gpus 1 --steps K --warmup W
+
+Default run: the SmolLM2-135M layer sizes (30 layers, hidden 576, 9 query and 3
+key/value heads of 64, inner 1536, vocabulary 49152, tied head) with random
+weights, a batch of 8 sequences whose prompts are uniform in [128, 2048]
+tokens, in a cache sized for 8192 tokens per sequence.  A step is one decode
+step of the whole batch through the generation path: token ids in, the model,
+greedy selection on the device, token ids out.  ``value`` is decoded tokens per
+second.  The prefill figure is one step over a 2,048-token prompt.  Peaks used
+for the fractions are the published MI355X ones: HBM 8 TB/s; dense matrix
+rate 2.5 PFLOP/s for bfloat16, 157.3 TFLOP/s for 32-bit.
+"""
+
+import argparse
+import json
+import os
+import sys
+import tempfile
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+FLOP_PEAK = {"bfloat16": 2.5e15, "float32": 157.3e12}
+
+SHAPE = dict(layers=30, hidden=576, heads=9, kv_heads=3, head_dim=64, inner=1536, vocab=49152, rope_theta=100000.0,
+             rms_norm_eps=1e-5, context=8192)
+
+
+def model_config(layers):
+    return {
+        "architectures": ["LlamaForCausalLM"], "model_type": "llama", "hidden_act": "silu",
+        "num_hidden_layers": layers, "hidden_size": SHAPE["hidden"], "num_attention_heads": SHAPE["heads"],
+        "num_key_value_heads": SHAPE["kv_heads"], "head_dim": SHAPE["head_dim"], "intermediate_size": SHAPE["inner"],
+        "vocab_size": SHAPE["vocab"], "rope_theta": SHAPE["rope_theta"], "rms_norm_eps": SHAPE["rms_norm_eps"],
+        "tie_word_embeddings": True, "max_position_embeddings": SHAPE["context"], "torch_dtype": "bfloat16",
+        "eos_token_id": 0,
+    }
+
+
+def step_flops(layers, tokens_per_sequence, wanted_rows):
+    """Multiply-adds x2 of one step over whole prompts from empty slots."""
+    h, nq, nkv, hd, inner, vocab = (SHAPE[k] for k in ("hidden", "heads", "kv_heads", "head_dim", "inner", "vocab"))
+    per_token = 2 * ((nq + 2 * nkv) * hd * h + nq * hd * h + 3 * h * inner)
+    total = 0
+    for n in tokens_per_sequence:
+        total += layers * (per_token * n + 2 * 2 * nq * hd * n * (n + 1) // 2)
+    return total + 2 * wanted_rows * h * vocab
+
+
+def main() -> int:
+    parser = argparse.ArgumentParser()
+    parser.add_argument("--gpus", type=int, default=1)
+    parser.add_argument("--steps", type=int, default=64)
+    parser.add_argument("--warmup", type=int, default=8)
+    parser.add_argument("--batch", type=int, default=8)
+    parser.add_argument("--layers", type=int, default=SHAPE["layers"])
+    parser.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    parser.add_argument("--seed", type=int, default=0)
+    parser.add_argument("--no-points", action="store_true", help="skip the batch-1 and batch-64 decode points")
+    args = parser.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this library runs on one GPU; --gpus {args.gpus} is not supported")
+        return 2
+
+    import numpy as np
+    import torch
+
+    import nnis_amd
+    from nnis_amd.api import load_engine
+    from nnis_amd.engine.batch import StepEntry
+    from nnis_amd.sampling.device import DeviceSelector
+
+    rng = np.random.default_rng(args.seed)
+    with tempfile.TemporaryDirectory() as folder:
+        nnis_amd.write_random_model(folder, model_config(args.layers), seed=args.seed)
+        sync = torch.cuda.synchronize
+
+        def decode_run(batch, steps, warmup):
+            """Prefills ``batch`` prompts in one step, then times ``steps`` decode steps."""
+            lengths = rng.integers(128, 2049, size=batch).tolist()
+            room = sum(((n + warmup + steps + 63) // 64) * 64 for n in lengths)
+            engine = load_engine(folder, dtype=args.dtype, max_tokens=room)
+            selector = DeviceSelector(engine)
+            slots = [engine.start_sequence() for _ in range(batch)]
+            prompts = [rng.integers(0, SHAPE["vocab"], size=n).tolist() for n in lengths]
+            logits = engine.step([StepEntry(s, p, None) for s, p in zip(slots, prompts)])
+            tokens = selector.select(logits, slots, [None] * batch)
+
+            def one_step(tokens):
+                logits = engine.step([StepEntry(s, [t], None) for s, t in zip(slots, tokens)])
+                return selector.select(logits, slots, [None] * batch)
+
+            for _ in range(warmup):
+                tokens = one_step(tokens)
+            sync()
+            start = time.perf_counter()
+            for _ in range(steps):
+                tokens = one_step(tokens)
+            sync()
+            seconds = time.perf_counter() - start
+            context_tokens = sum(engine.length(s) for s in slots) - batch * steps / 2.0  # mean over the timed steps
+            step_bytes = engine.model.step_weight_bytes() + engine.cache.bytes_per_token() * context_tokens
+            del engine
+            torch.cuda.empty_cache()
+            return seconds, step_bytes, lengths
+
+        seconds, step_bytes, lengths = decode_run(args.batch, args.steps, args.warmup)
+        ms_per_step = 1000.0 * seconds / args.steps
+        value = args.batch * args.steps / seconds
+        achieved = step_bytes / (seconds / args.steps) / 1e9
+
+        # prefill: 2,048 tokens of one sequence in one step, logits at the last place
+        prefill_tokens = 2048
+        engine = load_engine(folder, dtype=args.dtype, max_tokens=prefill_tokens)
+        prompt = rng.integers(0, SHAPE["vocab"], size=prefill_tokens).tolist()
+        times = []
+        for _ in range(4):
+            slot = engine.start_sequence()
+            sync()
+            start = time.perf_counter()
+            engine.step([StepEntry(slot, prompt, None)])
+            sync()
+            times.append(time.perf_counter() - start)
+            engine.end_sequence(slot)
+        prefill_seconds = min(times[1:])
+        del engine
+        torch.cuda.empty_cache()
+        flops = step_flops(args.layers, [prefill_tokens], 1)
+
+        points = {}
+        if not args.no_points:
+            for batch in (1, 64):
+                s, _, _ = decode_run(batch, max(8, args.steps // 2), max(2, args.warmup // 2))
+                points[f"decode_b{batch}"] = round(batch * max(8, args.steps // 2) / s, 1)
+
+    record = {
+        "metric": "decode tok/s at batch 8 (SmolLM2-135M shape); prefill tok/s at 2048 tokens; decode at batch 1 and 64 in points",
+        "value": round(value, 1),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+        "data": "synthetic: random weights N(0, 0.02) from a seed, uniform-random token ids",
+        "config": {
+            "model": "SmolLM2-135M shape (Llama)", "layers": args.layers, "layers_of_model": SHAPE["layers"],
+            "hidden": SHAPE["hidden"], "heads": SHAPE["heads"], "kv_heads": SHAPE["kv_heads"], "head_dim": SHAPE["head_dim"],
+            "inner": SHAPE["inner"], "vocab": SHAPE["vocab"], "tied_head": True, "context": SHAPE["context"],
+            "global_batch": args.batch, "seq_len": SHAPE["context"], "prompt_min": 128, "prompt_max": 2048,
+            "mean_prompt": round(float(np.mean(lengths)), 1), "parallelism": "single GPU", "sampling": "greedy on device",
+        },
+        "prefill": {
+            "value": round(prefill_tokens / prefill_seconds, 1), "tokens": prefill_tokens,
+            "ms": round(1000.0 * prefill_seconds, 3), "frac": round(flops / prefill_seconds / FLOP_PEAK[args.dtype], 5),
+        },
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 5)},
+        "points": points,
+    }
+    print(json.dumps(record))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

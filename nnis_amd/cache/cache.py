@@ -53,8 +53,9 @@ class KVGroup:
         # prompt can be written before its scores are taken
         per_slot = min(pages, pages_for(max_positions))
         self.table = PageTable(pages, slots, per_slot)
-        self.k = torch.empty((len(entries), pages, request.kv_heads, PAGE_TOKENS, request.head_dim), dtype=dtype, device=device)
-        self.v = torch.empty((len(entries), pages, request.kv_heads, request.head_dim, PAGE_TOKENS), dtype=dtype, device=device)
+        # zero at first: a page's unwritten tail is multiplied by zero weights, so it must hold numbers
+        self.k = torch.zeros((len(entries), pages, request.kv_heads, PAGE_TOKENS, request.head_dim), dtype=dtype, device=device)
+        self.v = torch.zeros((len(entries), pages, request.kv_heads, request.head_dim, PAGE_TOKENS), dtype=dtype, device=device)
         pinned = torch.device(device).type == "cuda"
         self.block_table_host = torch.zeros((slots, per_slot), dtype=torch.int32, pin_memory=pinned)
         self.block_table = torch.zeros((slots, per_slot), dtype=torch.int32, device=device)

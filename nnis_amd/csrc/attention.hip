@@ -113,6 +113,352 @@ __global__ __launch_bounds__(256) void attention_rows_kernel(AttnArgs a) {
   }
 }
 
+
+// =============================================================================
+// bfloat16 on the matrix cores (head sizes in steps of 16)
+//
+// Scores are taken transposed, S^T[key][column] = K[key][:] . Q[column][:], with
+// v_mfma_f32_16x16x32_bf16: first operand a tile of 16 keys, second a tile of
+// 16 "columns".  A column is one (query token, query head) pair; the columns of
+// a wave all read the same key/value head, so a key tile loaded once serves up
+// to C column tiles (the heads of a group, or further query positions).  The
+// result lies with lane l as S^T[key 4*(l/16)+e][column l%16]: a column's
+// softmax state lives in the lanes l%16 == column, its running maximum kept
+// equal over the four lane groups.  The output is taken transposed too,
+// O^T[d][column] += V^T[d][key] . P^T[key][column]: first operand a tile of 16
+// channels from the value page (stored with keys contiguous per channel),
+// second the probabilities, which are already in the lanes that need them --
+// key (group g, element e) of the instruction's 32 is key 4g+e of the first
+// score tile for e < 4 and of the second for e >= 4, and the value operand is
+// loaded in that order.  Softmax is in 32-bit (base-2 exponentials of scores
+// scaled by log2 e); probabilities are rounded to bfloat16 for the product
+// with the bfloat16 values.
+// =============================================================================
+#if NNIS_HEAD_DIM % 16 == 0
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+constexpr int kFullD = HD / 32;       // steps of 32 channels in a score
+constexpr bool kTailD = (HD % 32) != 0;  // plus one of 16
+constexpr int kTilesD = HD / 16;      // output tiles of 16 channels
+constexpr float kLog2e = 1.4426950408889634f;
+
+struct QFrag {
+  bf16x8 full[kFullD > 0 ? kFullD : 1];
+  bf16x4 tail;
+};
+
+__device__ __forceinline__ bf16x4 zero4() {
+  bf16x4 z;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) z[i] = (__bf16)0.0f;
+  return z;
+}
+
+// the operand of one row (a key, or a column's query) of HD channels
+__device__ __forceinline__ QFrag load_row_operand(const bf16_t* row, int g) {
+  QFrag f;
+#pragma unroll
+  for (int c = 0; c < kFullD; ++c) f.full[c] = *(const bf16x8*)(row + 32 * c + 8 * g);
+  f.tail = kTailD ? *(const bf16x4*)(row + 32 * kFullD + 4 * g) : zero4();
+  return f;
+}
+
+__device__ __forceinline__ f32x4 score_tile(const QFrag& keys, const QFrag& query) {
+  f32x4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+  for (int c = 0; c < kFullD; ++c) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(keys.full[c], query.full[c], acc, 0, 0, 0);
+  if (kTailD) {
+    // the 16-channel remainder is a sum of its own, added afterwards: the two
+    // instruction shapes never feed each other's accumulator
+    const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
+    const f32x4 rest = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(keys.tail, query.tail, zero, 0, 0, 0);
+    acc = kFullD > 0 ? acc + rest : rest;
+  }
+  return acc;
+}
+
+// Softmax state of C column tiles and their outputs
+template <int C>
+struct AttnState {
+  float m[C];       // running maximum (base-2 scaled score) of this lane's column, equal over lane groups
+  float l[C];       // this lane's part of the running sum
+  f32x4 o[C][kTilesD];
+};
+
+template <int C>
+__device__ __forceinline__ void init_state(AttnState<C>& st) {
+#pragma unroll
+  for (int c = 0; c < C; ++c) {
+    st.m[c] = -INFINITY;
+    st.l[c] = 0.0f;
+#pragma unroll
+    for (int t = 0; t < kTilesD; ++t) st.o[c][t] = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
+  }
+}
+
+// One block of 32 keys (keys key0 .. key0+31, inside one page) for C column tiles.
+//   k_block: &K[page][kv_head][key0 % 64][0]      (row stride HD)
+//   v_block: &V[page][kv_head][0][key0 % 64]      (channel stride 64)
+//   lo[c], hi[c]: the column of this lane reads keys lo <= key <= hi
+template <int C>
+__device__ __forceinline__ void attend_block(AttnState<C>& st, const QFrag (&q)[C], const bf16_t* k_block,
+                                             const bf16_t* v_block, int key0, const int (&lo)[C], const int (&hi)[C],
+                                             float scale_log2, int r, int g) {
+  QFrag keys[2];
+#pragma unroll
+  for (int t = 0; t < 2; ++t) keys[t] = load_row_operand(k_block + (size_t)(16 * t + r) * HD, g);
+  bf16x4 v_lo[kTilesD], v_hi[kTilesD];
+#pragma unroll
+  for (int t = 0; t < kTilesD; ++t) {
+    const bf16_t* channel = v_block + (size_t)(16 * t + r) * kPageTokens + 4 * g;
+    v_lo[t] = *(const bf16x4*)channel;
+    v_hi[t] = *(const bf16x4*)(channel + 16);
+  }
+#pragma unroll
+  for (int c = 0; c < C; ++c) {
+    f32x4 s[2];
+    float block_max = -INFINITY;
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      s[t] = score_tile(keys[t], q[c]);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int key = key0 + 16 * t + 4 * g + e;
+        s[t][e] = (key >= lo[c] && key <= hi[c]) ? s[t][e] * scale_log2 : -INFINITY;
+        block_max = fmaxf(block_max, s[t][e]);
+      }
+    }
+    block_max = fmaxf(block_max, __shfl_xor(block_max, 16, kWave));
+    block_max = fmaxf(block_max, __shfl_xor(block_max, 32, kWave));
+    const float m_new = fmaxf(st.m[c], block_max);
+    const float m_safe = m_new == -INFINITY ? 0.0f : m_new;  // a column that has seen no key yet
+    const float alpha = __builtin_amdgcn_exp2f(st.m[c] - m_safe);
+    bf16x8 p;
+    float sum = 0.0f;
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float w = __builtin_amdgcn_exp2f(s[t][e] - m_safe);
+        sum += w;
+        p[4 * t + e] = (__bf16)w;
+      }
+    st.l[c] = st.l[c] * alpha + sum;
+    st.m[c] = m_new;
+    bf16x8 v_operand;
+#pragma unroll
+    for (int t = 0; t < kTilesD; ++t) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        v_operand[e] = v_lo[t][e];
+        v_operand[4 + e] = v_hi[t][e];
+      }
+      st.o[c][t] = st.o[c][t] * alpha;
+      st.o[c][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v_operand, p, st.o[c][t], 0, 0, 0);
+    }
+  }
+}
+
+struct MfmaArgs {
+  const bf16_t* q;  // [tokens, heads, HD]
+  bf16_t* out;      // [tokens, heads, HD]
+  const bf16_t* k_pages;
+  const bf16_t* v_pages;
+  const int* block_table;
+  int max_pages;
+  int heads, kv_heads;
+  int window;
+  float scale_log2;
+  // prefill: one work item per (sequence, tile of 16*QT query rows)
+  const int* tile_seq;    // [tiles] sequence of the tile
+  const int* tile_row0;   // [tiles] first row of the tile within its sequence's new tokens
+  const int* seq_slot;    // [batch]
+  const int* seq_start;   // [batch + 1] first packed row of each sequence
+  const int* seq_pos0;    // [batch] position of a sequence's first new token
+  // decode: one token per sequence
+  const int* tok_slot;    // [tokens]
+  const int* tok_pos;     // [tokens]
+  int splits;
+  float* partial;         // [tokens, heads, splits, HD + 2] when splits > 1
+};
+
+__device__ __forceinline__ const bf16_t* k_page_ptr(const MfmaArgs& a, int page, int kv_head) {
+  return a.k_pages + ((size_t)page * a.kv_heads + kv_head) * kPageTokens * HD;
+}
+__device__ __forceinline__ const bf16_t* v_page_ptr(const MfmaArgs& a, int page, int kv_head) {
+  return a.v_pages + ((size_t)page * a.kv_heads + kv_head) * HD * kPageTokens;
+}
+
+// ---- prefill: a wave = (query tile, kv head, chunk of GH query heads); C = QT * GH column tiles --------
+template <int QT, int GH>
+__global__ __launch_bounds__(kWave) void attention_prefill_kernel(MfmaArgs a) {
+  constexpr int C = QT * GH;
+  const int lane = threadIdx.x, r = lane % 16, g = lane / 16;
+  const int tile = blockIdx.x;
+  const int group = a.heads / a.kv_heads;
+  const int chunks = (group + GH - 1) / GH;
+  const int kv_head = blockIdx.y / chunks;
+  const int head0 = kv_head * group + (blockIdx.y % chunks) * GH;
+  const int seq = a.tile_seq[tile];
+  const int row0 = a.tile_row0[tile];
+  const int slot = a.seq_slot[seq];
+  const int start = a.seq_start[seq];
+  const int rows = a.seq_start[seq + 1] - start;
+  const int pos0 = a.seq_pos0[seq];
+  const int* pages = a.block_table + (size_t)slot * a.max_pages;
+
+  QFrag q[C];
+  int lo[C], hi[C];
+  bool live[C];
+  int last = -1;
+#pragma unroll
+  for (int qt = 0; qt < QT; ++qt)
+#pragma unroll
+    for (int gh = 0; gh < GH; ++gh) {
+      const int c = qt * GH + gh;
+      const int row = row0 + 16 * qt + r;
+      const int head = head0 + gh;
+      live[c] = row < rows && head < kv_head * group + group;
+      const int safe_row = row < rows ? row : rows - 1;
+      const int safe_head = head < a.heads ? head : a.heads - 1;
+      q[c] = load_row_operand(a.q + ((size_t)(start + safe_row) * a.heads + safe_head) * HD, g);
+      hi[c] = live[c] ? pos0 + row : -1;
+      lo[c] = (a.window > 0 && hi[c] + 1 > a.window) ? hi[c] + 1 - a.window : 0;
+      last = hi[c] > last ? hi[c] : last;
+    }
+  // the wave runs to the farthest key any of its columns reads, from the nearest
+  int first = 0x7fffffff;
+#pragma unroll
+  for (int c = 0; c < C; ++c) first = (live[c] && lo[c] < first) ? lo[c] : first;
+#pragma unroll
+  for (int offset = kWave / 2; offset > 0; offset >>= 1) {
+    last = max(last, __shfl_xor(last, offset, kWave));
+    first = min(first, __shfl_xor(first, offset, kWave));
+  }
+  AttnState<C> st;
+  init_state(st);
+  if (last >= 0) {
+    for (int key0 = (first / 32) * 32; key0 <= last; key0 += 32) {
+      const int page = pages[key0 / kPageTokens];
+      const int inside = key0 % kPageTokens;
+      attend_block<C>(st, q, k_page_ptr(a, page, kv_head) + (size_t)inside * HD, v_page_ptr(a, page, kv_head) + inside,
+                      key0, lo, hi, a.scale_log2, r, g);
+    }
+  }
+#pragma unroll
+  for (int qt = 0; qt < QT; ++qt)
+#pragma unroll
+    for (int gh = 0; gh < GH; ++gh) {
+      const int c = qt * GH + gh;
+      float total = st.l[c];
+      total += __shfl_xor(total, 16, kWave);
+      total += __shfl_xor(total, 32, kWave);
+      if (!live[c]) continue;
+      const float inv = 1.0f / total;
+      bf16_t* dst = a.out + ((size_t)(start + row0 + 16 * qt + r) * a.heads + head0 + gh) * HD;
+#pragma unroll
+      for (int t = 0; t < kTilesD; ++t) {
+        bf16x4 packed;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) packed[e] = (__bf16)(st.o[c][t][e] * inv);
+        *(bf16x4*)(dst + 16 * t + 4 * g) = packed;
+      }
+    }
+}
+
+// ---- decode: a wave = (token, kv head, split of the keys); columns are the heads of the group ---------
+template <int C>
+__global__ __launch_bounds__(kWave) void attention_decode_kernel(MfmaArgs a) {
+  const int lane = threadIdx.x, r = lane % 16, g = lane / 16;
+  const int token = blockIdx.x, kv_head = blockIdx.y, split = blockIdx.z;
+  const int slot = a.tok_slot[token];
+  if (slot < 0) return;  // a padding row: its output is never read
+  const int group = a.heads / a.kv_heads;
+  const int pos = a.tok_pos[token];
+  const int first_key = (a.window > 0 && pos + 1 > a.window) ? pos + 1 - a.window : 0;
+  const int* pages = a.block_table + (size_t)slot * a.max_pages;
+
+  QFrag q[C];
+  int lo[C], hi[C];
+  bool live[C];
+#pragma unroll
+  for (int c = 0; c < C; ++c) {
+    const int member = 16 * c + r;
+    live[c] = member < group;
+    const int head = kv_head * group + (live[c] ? member : 0);
+    q[c] = load_row_operand(a.q + ((size_t)token * a.heads + head) * HD, g);
+    lo[c] = first_key;
+    hi[c] = live[c] ? pos : -1;
+  }
+  // blocks of 32 keys are dealt to the splits in contiguous runs
+  const int block_first = first_key / 32, block_count = pos / 32 + 1 - block_first;
+  const int per_split = (block_count + a.splits - 1) / a.splits;
+  const int begin = block_first + split * per_split;
+  const int end = min(begin + per_split, block_first + block_count);
+  AttnState<C> st;
+  init_state(st);
+  for (int block = begin; block < end; ++block) {
+    const int key0 = block * 32;
+    const int page = pages[key0 / kPageTokens];
+    const int inside = key0 % kPageTokens;
+    attend_block<C>(st, q, k_page_ptr(a, page, kv_head) + (size_t)inside * HD, v_page_ptr(a, page, kv_head) + inside, key0,
+                    lo, hi, a.scale_log2, r, g);
+  }
+#pragma unroll
+  for (int c = 0; c < C; ++c) {
+    float total = st.l[c];
+    total += __shfl_xor(total, 16, kWave);
+    total += __shfl_xor(total, 32, kWave);
+    if (!live[c]) continue;
+    const int head = kv_head * group + 16 * c + r;
+    if (a.splits == 1) {
+      const float inv = 1.0f / total;
+      bf16_t* dst = a.out + ((size_t)token * a.heads + head) * HD;
+#pragma unroll
+      for (int t = 0; t < kTilesD; ++t) {
+        bf16x4 packed;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) packed[e] = (__bf16)(st.o[c][t][e] * inv);
+        *(bf16x4*)(dst + 16 * t + 4 * g) = packed;
+      }
+    } else {
+      float* dst = a.partial + (((size_t)token * a.heads + head) * a.splits + split) * (HD + 2);
+#pragma unroll
+      for (int t = 0; t < kTilesD; ++t) *(f32x4*)(dst + 16 * t + 4 * g) = st.o[c][t];
+      if (g == 0) {
+        dst[HD] = st.m[c];
+        dst[HD + 1] = total;
+      }
+    }
+  }
+}
+
+// sums the splits of one (token, head): out = sum_s O_s 2^(m_s - M) / sum_s l_s 2^(m_s - M)
+__global__ void attention_combine_kernel(const float* __restrict__ partial, bf16_t* __restrict__ out,
+                                         const int* __restrict__ tok_slot, int heads, int splits) {
+  const int token = blockIdx.x, head = blockIdx.y;
+  if (tok_slot[token] < 0) return;
+  const float* base = partial + ((size_t)token * heads + head) * splits * (HD + 2);
+  float m_all = -INFINITY;
+  for (int s = 0; s < splits; ++s) m_all = fmaxf(m_all, base[(size_t)s * (HD + 2) + HD]);
+  for (int d = threadIdx.x; d < HD; d += blockDim.x) {
+    float num = 0.0f, den = 0.0f;
+    for (int s = 0; s < splits; ++s) {
+      const float* p = base + (size_t)s * (HD + 2);
+      const float m = p[HD];
+      const float w = m == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(m - m_all);
+      num += p[d] * w;
+      den += p[HD + 1] * w;
+    }
+    out[((size_t)token * heads + head) * HD + d] = (bf16_t)(num / den);
+  }
+}
+
+#endif  // NNIS_HEAD_DIM % 16 == 0
+
 }  // namespace
 
 extern "C" int nnis_attention_rows(const void* q, int q_dtype, void* out, int out_dtype, const void* k_pages,
@@ -141,3 +487,102 @@ extern "C" int nnis_attention_rows(const void* q, int q_dtype, void* out, int ou
   NNIS_LAUNCH_CHECK("attention_rows");
   return 0;
 }
+
+
+#if NNIS_HEAD_DIM % 16 == 0
+namespace {
+constexpr int kMaxColumns = HD <= 64 ? 4 : (HD <= 128 ? 2 : 1);  // column tiles a wave carries (registers)
+
+int fill_common(MfmaArgs& a, const void* q, void* out, const void* k_pages, const void* v_pages, const int* block_table,
+                int max_pages, int heads, int kv_heads, int head_dim, int window, float scale) {
+  NNIS_REQUIRE(head_dim == HD, "attention: this module is compiled for head_dim %d, got %d", HD, head_dim);
+  NNIS_REQUIRE(heads > 0 && kv_heads > 0 && heads % kv_heads == 0, "attention: %d heads do not divide into %d kv heads",
+               heads, kv_heads);
+  NNIS_REQUIRE(window >= 0 && max_pages > 0, "attention: bad window %d or block table width %d", window, max_pages);
+  NNIS_REQUIRE(((uintptr_t)q % 16 == 0) && ((uintptr_t)out % 16 == 0) && ((uintptr_t)k_pages % 16 == 0) &&
+                   ((uintptr_t)v_pages % 16 == 0),
+               "attention: operands must be 16-byte aligned");
+  a.q = (const bf16_t*)q; a.out = (bf16_t*)out; a.k_pages = (const bf16_t*)k_pages; a.v_pages = (const bf16_t*)v_pages;
+  a.block_table = block_table; a.max_pages = max_pages; a.heads = heads; a.kv_heads = kv_heads; a.window = window;
+  a.scale_log2 = scale * kLog2e;
+  a.tile_seq = a.tile_row0 = a.seq_slot = a.seq_start = a.seq_pos0 = a.tok_slot = a.tok_pos = nullptr;
+  a.splits = 1; a.partial = nullptr;
+  return 0;
+}
+}  // namespace
+
+// rows of 16*QT queries per tile, as the host must cut them
+extern "C" int nnis_attention_prefill_tile_rows(int heads, int kv_heads) {
+  const int group = heads / (kv_heads > 0 ? kv_heads : 1);
+  const int gh = group < kMaxColumns ? group : kMaxColumns;
+  return 16 * (kMaxColumns / (gh > 0 ? gh : 1));
+}
+
+extern "C" int nnis_attention_prefill_bf16(const void* q, void* out, const void* k_pages, const void* v_pages,
+                                           const int* block_table, int max_pages, const int* tile_seq,
+                                           const int* tile_row0, int tiles, const int* seq_slot, const int* seq_start,
+                                           const int* seq_pos0, int heads, int kv_heads, int head_dim, int window,
+                                           float scale, void* stream) {
+  MfmaArgs a;
+  if (fill_common(a, q, out, k_pages, v_pages, block_table, max_pages, heads, kv_heads, head_dim, window, scale)) return 1;
+  if (tiles <= 0) return 0;
+  a.tile_seq = tile_seq; a.tile_row0 = tile_row0; a.seq_slot = seq_slot; a.seq_start = seq_start; a.seq_pos0 = seq_pos0;
+  const int group = heads / kv_heads;
+  const int gh = group < kMaxColumns ? group : kMaxColumns;
+  const int qt = kMaxColumns / gh;
+  const int chunks = (group + gh - 1) / gh;
+  const dim3 grid(tiles, kv_heads * chunks);
+  NNIS_REQUIRE(grid.y <= 65535, "attention: %d head chunks exceed the grid limit", grid.y);
+  hipStream_t s = (hipStream_t)stream;
+  if (qt == 4 && gh == 1) hipLaunchKernelGGL((attention_prefill_kernel<4, 1>), grid, dim3(kWave), 0, s, a);
+  else if (qt == 2 && gh == 2) hipLaunchKernelGGL((attention_prefill_kernel<2, 2>), grid, dim3(kWave), 0, s, a);
+  else if (qt == 2 && gh == 1) hipLaunchKernelGGL((attention_prefill_kernel<2, 1>), grid, dim3(kWave), 0, s, a);
+  else if (qt == 1 && gh == 3) hipLaunchKernelGGL((attention_prefill_kernel<1, 3>), grid, dim3(kWave), 0, s, a);
+  else if (qt == 1 && gh == 4) hipLaunchKernelGGL((attention_prefill_kernel<1, 4>), grid, dim3(kWave), 0, s, a);
+  else if (qt == 1 && gh == 2) hipLaunchKernelGGL((attention_prefill_kernel<1, 2>), grid, dim3(kWave), 0, s, a);
+  else if (qt == 1 && gh == 1) hipLaunchKernelGGL((attention_prefill_kernel<1, 1>), grid, dim3(kWave), 0, s, a);
+  else return nnis_fail("attention: no kernel for %d query tiles x %d heads", qt, gh);
+  NNIS_LAUNCH_CHECK("attention_prefill");
+  return 0;
+}
+
+// partial: float32 scratch of at least tokens * heads * splits * (head_dim + 2), needed when splits > 1
+extern "C" int nnis_attention_decode_bf16(const void* q, void* out, const void* k_pages, const void* v_pages,
+                                          const int* block_table, int max_pages, const int* tok_slot, const int* tok_pos,
+                                          int tokens, int heads, int kv_heads, int head_dim, int window, float scale,
+                                          int splits, float* partial, void* stream) {
+  MfmaArgs a;
+  if (fill_common(a, q, out, k_pages, v_pages, block_table, max_pages, heads, kv_heads, head_dim, window, scale)) return 1;
+  NNIS_REQUIRE(splits >= 1 && splits <= 65535, "attention: bad number of splits %d", splits);
+  NNIS_REQUIRE(splits == 1 || partial != nullptr, "attention: splits need scratch memory");
+  NNIS_REQUIRE(kv_heads <= 65535, "attention: %d kv heads exceed the grid limit", kv_heads);
+  if (tokens <= 0) return 0;
+  const int group = heads / kv_heads;
+  NNIS_REQUIRE(group <= 16 * kMaxColumns, "attention: a group of %d query heads is more than this head size's decode kernel carries (%d)",
+               group, 16 * kMaxColumns);
+  a.tok_slot = tok_slot; a.tok_pos = tok_pos; a.splits = splits; a.partial = partial;
+  const dim3 grid(tokens, kv_heads, splits);
+  hipStream_t s = (hipStream_t)stream;
+  const int tiles = (group + 15) / 16;
+  if (tiles == 1) hipLaunchKernelGGL((attention_decode_kernel<1>), grid, dim3(kWave), 0, s, a);
+  else if (tiles == 2 && kMaxColumns >= 2) hipLaunchKernelGGL((attention_decode_kernel<(kMaxColumns >= 2 ? 2 : 1)>), grid, dim3(kWave), 0, s, a);
+  else hipLaunchKernelGGL((attention_decode_kernel<kMaxColumns>), grid, dim3(kWave), 0, s, a);
+  NNIS_LAUNCH_CHECK("attention_decode");
+  if (splits > 1) {
+    hipLaunchKernelGGL(attention_combine_kernel, dim3(tokens, heads), dim3(HD < 64 ? 64 : (HD > 256 ? 256 : HD)), 0, s, partial,
+                       (bf16_t*)out, tok_slot, heads, splits);
+    NNIS_LAUNCH_CHECK("attention_combine");
+  }
+  return 0;
+}
+#else
+extern "C" int nnis_attention_prefill_tile_rows(int, int) { return 0; }
+extern "C" int nnis_attention_prefill_bf16(const void*, void*, const void*, const void*, const int*, int, const int*, const int*,
+                                           int, const int*, const int*, const int*, int, int, int, int, float, void*) {
+  return nnis_fail("attention: the matrix-core kernels need a head size in steps of 16; this module has %d", NNIS_HEAD_DIM);
+}
+extern "C" int nnis_attention_decode_bf16(const void*, void*, const void*, const void*, const int*, int, const int*, const int*,
+                                          int, int, int, int, int, float, int, float*, void*) {
+  return nnis_fail("attention: the matrix-core kernels need a head size in steps of 16; this module has %d", NNIS_HEAD_DIM);
+}
+#endif

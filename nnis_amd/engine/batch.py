@@ -33,3 +33,5 @@ class StepContext:
     host_slots: List[int] = field(default_factory=list)
     host_new: List[int] = field(default_factory=list)
     host_pos0: List[int] = field(default_factory=list)
+    splits: int = 0  # runs the keys of a decode step are cut into; 0: chosen by the kernel's wrapper
+    tiles: dict = field(default_factory=dict)  # work lists of prefill kernels, by tile size, made on first use

@@ -28,11 +28,17 @@ _CORE_SIGNATURES = {
     "nnis_silu_mul": [_VOID, _INT, _VOID, _INT, _INT, _INT, _VOID],
     "nnis_argmax": [_VOID, _VOID, _INT, _INT, _VOID],
     "nnis_gemm_ordered": [_VOID, _INT, _VOID, _INT, _VOID, _INT, _INT, _INT, _INT, _VOID],
+    "nnis_gemm_bf16": [_VOID, _VOID, _VOID, _INT, _INT, _INT, _INT, _VOID],
     "nnis_sample": [_VOID, _VOID, _INT, _INT, _VOID, _VOID, _VOID, _VOID, _VOID, _VOID, _VOID],
 }
 _ATTN_SIGNATURES = {
     "nnis_attention_rows": [_VOID, _INT, _VOID, _INT, _VOID, _VOID, _INT, _VOID, _INT, _VOID, _VOID, _INT, _INT, _INT,
                             _INT, _INT, _FLT, _VOID],
+    "nnis_attention_prefill_tile_rows": [_INT, _INT],
+    "nnis_attention_prefill_bf16": [_VOID, _VOID, _VOID, _VOID, _VOID, _INT, _VOID, _VOID, _INT, _VOID, _VOID, _VOID, _INT,
+                                    _INT, _INT, _INT, _FLT, _VOID],
+    "nnis_attention_decode_bf16": [_VOID, _VOID, _VOID, _VOID, _VOID, _INT, _VOID, _VOID, _INT, _INT, _INT, _INT, _INT, _FLT,
+                                   _INT, _VOID, _VOID],
 }
 
 _DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1}
@@ -241,15 +247,140 @@ def attention_rows(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_
 # dispatch by operand types
 # ---------------------------------------------------------------------------
 
+def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[M, N] = x[M, K] @ w[N, K]^T on the matrix cores: bfloat16 operands,
+    32-bit accumulation, bfloat16 or float32 output.  K must be a multiple of 8."""
+    _dev(x, "x"), _dev(w, "weight"), _dev(out, "out")
+    m, k = x.shape
+    n = w.shape[0]
+    if w.shape[1] != k or out.shape != (m, n):
+        raise KernelError(f"gemm: x {tuple(x.shape)} w {tuple(w.shape)} out {tuple(out.shape)} do not fit")
+    if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
+        raise KernelError(f"gemm_bf16 takes bfloat16 operands, got {x.dtype} and {w.dtype}")
+    lib = core()
+    _check(lib, lib.nnis_gemm_bf16(x.data_ptr(), w.data_ptr(), out.data_ptr(), _code(out), m, n, k, _stream()))
+    return out
+
+
+def _mfma_ok(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> bool:
+    return (x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and x.shape[1] % 8 == 0
+            and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0 and out.data_ptr() % 16 == 0)
+
+
 def linear(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
-    """out = x @ weight^T.  32-bit operands take the ordered 32-bit product;
-    bfloat16 operands take the matrix-core kernels."""
+    """out = x @ weight^T.  bfloat16 operands take the matrix-core kernels;
+    32-bit operands (and widths the 16-byte loads cannot take) the ordered
+    32-bit product."""
+    if _mfma_ok(x, weight, out):
+        return gemm_bf16(x, weight, out)
     return gemm_ordered(x, weight, out)
+
+
+def _check_pages(q, out, k_pages, v_pages, block_table, heads, kv_heads, head_dim):
+    tokens = q.shape[0]
+    if q.shape != (tokens, heads * head_dim) or out.shape != q.shape:
+        raise KernelError(f"attention: q {tuple(q.shape)} / out {tuple(out.shape)} do not fit {heads} heads of {head_dim}")
+    if tuple(k_pages.shape[1:]) != (kv_heads, PAGE_TOKENS, head_dim) or tuple(v_pages.shape[1:]) != (kv_heads, head_dim, PAGE_TOKENS):
+        raise KernelError(f"attention: page shapes {tuple(k_pages.shape)} / {tuple(v_pages.shape)} do not fit")
+    if block_table.dtype != torch.int32 or block_table.dim() != 2:
+        raise KernelError("attention: block_table must be int32 [slots, pages]")
+    for t, what in ((q, "q"), (out, "out"), (k_pages, "k_pages"), (v_pages, "v_pages")):
+        _dev(t, what)
+        if t.dtype != torch.bfloat16:
+            raise KernelError(f"attention: the matrix-core kernels take bfloat16, {what} is {t.dtype}")
+
+
+def prefill_tile_rows(heads: int, kv_heads: int, head_dim: int) -> int:
+    """Query rows per work item of ``attention_prefill_bf16`` for these sizes."""
+    return attention_module(head_dim).nnis_attention_prefill_tile_rows(heads, kv_heads)
+
+
+def attention_prefill_bf16(q, out, k_pages, v_pages, block_table, tile_seq, tile_row0, seq_slot, seq_start, seq_pos0,
+                           heads, kv_heads, head_dim, scale, window=0):
+    """Causal attention of whole runs of new tokens over the cache, on the
+    matrix cores.  ``tile_seq``/``tile_row0`` (int32) name, per work item, a
+    sequence of the step and the first of ``prefill_tile_rows`` rows of its
+    new tokens; ``seq_start`` [batch + 1] gives each sequence's packed rows."""
+    _check_pages(q, out, k_pages, v_pages, block_table, heads, kv_heads, head_dim)
+    for t in (tile_seq, tile_row0, seq_slot, seq_start, seq_pos0):
+        _dev(t, "step metadata")
+        if t.dtype != torch.int32:
+            raise KernelError("attention: step metadata must be int32")
+    tiles = tile_seq.numel()
+    if tile_row0.numel() != tiles or seq_start.numel() != seq_slot.numel() + 1 or seq_pos0.numel() != seq_slot.numel():
+        raise KernelError("attention: step metadata arrays do not fit each other")
+    lib = attention_module(head_dim)
+    _check(lib, lib.nnis_attention_prefill_bf16(q.data_ptr(), out.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(),
+                                                block_table.data_ptr(), block_table.shape[1], tile_seq.data_ptr(),
+                                                tile_row0.data_ptr(), tiles, seq_slot.data_ptr(), seq_start.data_ptr(),
+                                                seq_pos0.data_ptr(), heads, kv_heads, head_dim, int(window), float(scale),
+                                                _stream()))
+    return out
+
+
+def attention_decode_bf16(q, out, k_pages, v_pages, block_table, tok_slot, tok_pos, heads, kv_heads, head_dim, scale,
+                          window=0, splits=1, partial=None):
+    """One query token per sequence over its cached keys, the keys cut into
+    ``splits`` runs that are summed afterwards.  ``partial``: float32 scratch of
+    tokens * heads * splits * (head_dim + 2) when splits > 1."""
+    _check_pages(q, out, k_pages, v_pages, block_table, heads, kv_heads, head_dim)
+    tokens = q.shape[0]
+    for t in (tok_slot, tok_pos):
+        _dev(t, "step metadata")
+        if t.dtype != torch.int32 or t.numel() < tokens:
+            raise KernelError("attention: tok_slot / tok_pos must be int32 with one entry per token")
+    if splits > 1:
+        if partial is None or partial.dtype != torch.float32 or partial.numel() < tokens * heads * splits * (head_dim + 2):
+            raise KernelError("attention: splits need float32 scratch of tokens * heads * splits * (head_dim + 2)")
+        _dev(partial, "partial")
+    lib = attention_module(head_dim)
+    _check(lib, lib.nnis_attention_decode_bf16(q.data_ptr(), out.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(),
+                                               block_table.data_ptr(), block_table.shape[1], tok_slot.data_ptr(),
+                                               tok_pos.data_ptr(), tokens, heads, kv_heads, head_dim, int(window),
+                                               float(scale), int(splits), _ptr(partial) if splits > 1 else None, _stream()))
+    return out
+
+
+def decode_splits(batch: int, kv_heads: int, longest: int) -> int:
+    """Runs the keys of a decode step are cut into: enough waves to fill the
+    chip (about four a compute unit), at least two blocks of 32 keys a run, a
+    power of two."""
+    blocks = (longest + 31) // 32
+    want = max(1, 1024 // max(1, batch * kv_heads))
+    splits = max(1, min(want, blocks // 2))
+    return 1 << (splits.bit_length() - 1)
+
+
+def _prefill_tiles(ctx, rows: int, device):
+    """Work items of a prefill step for tiles of ``rows`` query rows, longest first."""
+    cached = ctx.tiles.get(rows)
+    if cached is None:
+        items = [(pos0 + min(row0 + rows, count), seq, row0)
+                 for seq, (count, pos0) in enumerate(zip(ctx.host_new, ctx.host_pos0)) for row0 in range(0, count, rows)]
+        items.sort(reverse=True)
+        packed = torch.tensor([[seq for _, seq, _ in items], [row0 for _, _, row0 in items]], dtype=torch.int32)
+        packed = packed.to(device, non_blocking=True)
+        cached = ctx.tiles[rows] = (packed[0], packed[1])
+    return cached
 
 
 def attention(q: torch.Tensor, out: torch.Tensor, view, ctx, heads: int, kv_heads: int, head_dim: int, scale: float,
               window: int = 0) -> torch.Tensor:
-    """Attention of the step's tokens over the cache ``view``."""
+    """Attention of the step's tokens over the cache ``view``: bfloat16 with a
+    head size in steps of 16 runs on the matrix cores (one kernel for single
+    tokens, one for runs of tokens); anything else takes the 32-bit kernel."""
+    fast = (q.dtype == torch.bfloat16 and view.k_pages.dtype == torch.bfloat16 and head_dim % 16 == 0)
+    if fast and ctx.decode and heads // kv_heads <= 16 * (4 if head_dim <= 64 else (2 if head_dim <= 128 else 1)):
+        splits = ctx.splits or decode_splits(ctx.batch, kv_heads, ctx.max_len)
+        partial = None
+        if splits > 1:
+            partial = torch.empty(q.shape[0] * heads * splits * (head_dim + 2), dtype=torch.float32, device=q.device)
+        return attention_decode_bf16(q, out, view.k_pages, view.v_pages, view.block_table, ctx.tok_slot, ctx.tok_pos, heads,
+                                     kv_heads, head_dim, scale, window, splits, partial)
+    if fast and not ctx.decode:
+        tile_seq, tile_row0 = _prefill_tiles(ctx, prefill_tile_rows(heads, kv_heads, head_dim), q.device)
+        return attention_prefill_bf16(q, out, view.k_pages, view.v_pages, view.block_table, tile_seq, tile_row0,
+                                      ctx.seq_slot, ctx.seq_start, ctx.seq_pos0, heads, kv_heads, head_dim, scale, window)
     return attention_rows(q, out, view.k_pages, view.v_pages, view.block_table, ctx.tok_slot, ctx.tok_pos, heads,
                           kv_heads, head_dim, scale, window)
 

@@ -82,6 +82,130 @@ def test_gemm_ordered(m, n, k, x_dtype, w_dtype, y_dtype):
         assert torch.equal(alone[0], y[m - 1])
 
 
+@pytest.mark.parametrize("m", [1, 8, 16, 17, 40, 64, 65, 130, 300])
+@pytest.mark.parametrize("n, k", [(576, 576), (960, 576), (1000, 96), (70, 176), (3072, 64), (64, 1536), (17, 8), (200, 1096)])
+@pytest.mark.parametrize("y_dtype", ["bfloat16", "float32"])
+def test_gemm_bf16_on_the_matrix_cores(m, n, k, y_dtype):
+    """Skinny (M <= 64) and tiled kernels at sizes with tails in every
+    dimension.  Integer-valued operands make the 32-bit sums exact, so any
+    misplaced or dropped product shows as a whole-number error."""
+    ops = _ops()
+    torch.manual_seed(m + n + k)
+    x = torch.randint(-3, 4, (m, k)).to(torch.bfloat16)
+    w = torch.randint(-3, 4, (n, k)).to(torch.bfloat16)
+    y = torch.full((m, n), 7.0, dtype=DT[y_dtype], device="cuda")
+    ops.gemm_bf16(x.cuda(), w.cuda(), y)
+    want = x.double() @ w.double().t()
+    if y_dtype == "float32":
+        assert torch.equal(y.cpu().double(), want)
+    else:
+        assert torch.equal(y.cpu(), want.to(torch.bfloat16))
+    # and with ordinary values, against the 64-bit product
+    x = torch.randn(m, k).to(torch.bfloat16)
+    w = torch.randn(n, k).to(torch.bfloat16)
+    ops.gemm_bf16(x.cuda(), w.cuda(), y)
+    want = x.double() @ w.double().t()
+    scale = x.double().abs() @ w.double().abs().t()
+    tol = 1e-6 * math.sqrt(k) if y_dtype == "float32" else 4e-3
+    assert ((y.cpu().double() - want).abs() <= tol * scale + 1e-30).all()
+
+
+def test_gemm_bf16_refuses_what_it_cannot_load():
+    ops = _ops()
+    x = torch.zeros(4, 12, dtype=torch.bfloat16, device="cuda")
+    w = torch.zeros(6, 12, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(KernelError, match="multiple of 8"):
+        ops.gemm_bf16(x, w, torch.zeros(4, 6, dtype=torch.bfloat16, device="cuda"))
+    out = torch.zeros(4, 6, dtype=torch.bfloat16, device="cuda")
+    ops.linear(x + 1, w + 1, out)  # the dispatcher falls back to the ordered product
+    assert (out == 12).all()
+
+
+MFMA_SHAPES = [(4, 2, 16), (3, 3, 16), (3, 1, 32), (6, 2, 48), (6, 6, 48), (4, 2, 48), (9, 3, 64), (2, 2, 64), (5, 5, 80),
+               (4, 1, 112), (8, 2, 128), (32, 1, 64), (40, 2, 16)]
+
+
+def _plain_rows(q_rows, ks, vs, scale, window=0):
+    """q_rows: list of (slot, pos, q[heads, hd]) -> plain attention output per row."""
+    out = []
+    for slot, pos, q in q_rows:
+        lo = max(0, pos + 1 - window) if window else 0
+        full_q = torch.zeros(pos + 1 - lo, *q.shape)
+        full_q[-1] = q
+        out.append(P.causal_attention(full_q, ks[slot][lo:pos + 1], vs[slot][lo:pos + 1], scale)[-1])
+    return torch.stack(out)
+
+
+@pytest.mark.parametrize("heads, kv_heads, head_dim", MFMA_SHAPES)
+@pytest.mark.parametrize("splits", [1, 4, 16])
+def test_decode_attention_on_the_matrix_cores(heads, kv_heads, head_dim, splits):
+    ops = _ops()
+    torch.manual_seed(heads + head_dim)
+    lengths = [700, 1, 65, 33]
+    ks = [torch.randn(n, kv_heads, head_dim).bfloat16().float() for n in lengths]
+    vs = [torch.randn(n, kv_heads, head_dim).bfloat16().float() for n in lengths]
+    scale = 1.0 / math.sqrt(head_dim)
+    q_last = torch.randn(heads, head_dim)
+    ks[0][3, 0] = (q_last[0] * (12.0 / scale / q_last[0].pow(2).sum())).bfloat16().float()  # a far key among hundreds
+    k_pages, v_pages, table = _paged(ks, vs, torch.bfloat16, kv_heads, head_dim)
+    rows = [(0, 699, q_last), (1, 0, torch.randn(heads, head_dim)), (-1, 9, torch.randn(heads, head_dim)),
+            (2, 64, torch.randn(heads, head_dim)), (3, 31, torch.randn(heads, head_dim))]
+    rows = [(s, p, q.bfloat16().float()) for s, p, q in rows]
+    q = torch.stack([q for _, _, q in rows]).bfloat16().reshape(len(rows), -1).cuda()
+    out = torch.full((len(rows), heads * head_dim), 3.0, dtype=torch.bfloat16, device="cuda")
+    partial = torch.empty(len(rows) * heads * splits * (head_dim + 2), dtype=torch.float32, device="cuda")
+    ops.attention_decode_bf16(q, out, k_pages, v_pages, table, _i32([s for s, _, _ in rows]), _i32([p for _, p, _ in rows]),
+                              heads, kv_heads, head_dim, scale, 0, splits, partial)
+    got = out.cpu().float().view(len(rows), heads, head_dim)
+    live = [i for i, (s, _, _) in enumerate(rows) if s >= 0]
+    want = _plain_rows([rows[i] for i in live], ks, vs, scale)
+    assert (got[live] - want).abs().max().item() <= 2e-2
+    assert (got[2] == 3.0).all()  # the padding row is left alone
+    assert (got[0, 0] - vs[0][3, 0]).abs().max().item() < 0.05
+    # a window: the row at position 699 reads keys 600..699 only
+    ops.attention_decode_bf16(q, out, k_pages, v_pages, table, _i32([s for s, _, _ in rows]), _i32([p for _, p, _ in rows]),
+                              heads, kv_heads, head_dim, scale, 100, splits, partial)
+    got = out.cpu().float().view(len(rows), heads, head_dim)
+    want = _plain_rows([rows[i] for i in live], ks, vs, scale, window=100)
+    assert (got[live] - want).abs().max().item() <= 2e-2
+
+
+@pytest.mark.parametrize("heads, kv_heads, head_dim", MFMA_SHAPES)
+def test_prefill_attention_on_the_matrix_cores(heads, kv_heads, head_dim):
+    """Three sequences in one step: a whole prompt, a continuation that starts
+    at position 70, and a single token; every new row against the plain
+    attention over its sequence's keys up to its own position."""
+    ops = _ops()
+    torch.manual_seed(heads * 3 + head_dim)
+    sequences = [(2, 0, 130), (0, 70, 37), (1, 0, 1)]  # (slot, first new position, new tokens)
+    total = {slot: pos0 + n for slot, pos0, n in sequences}
+    ks = [torch.randn(total[s], kv_heads, head_dim).bfloat16().float() for s in range(3)]
+    vs = [torch.randn(total[s], kv_heads, head_dim).bfloat16().float() for s in range(3)]
+    scale = 1.0 / math.sqrt(head_dim)
+    k_pages, v_pages, table = _paged(ks, vs, torch.bfloat16, kv_heads, head_dim)
+    rows = [(slot, pos0 + i, torch.randn(heads, head_dim).bfloat16().float()) for slot, pos0, n in sequences for i in range(n)]
+    # one loud key: row 100 of the first sequence must find key 17 (head 0)
+    loud_q = rows[100][2][0]
+    ks[2][17, 0] = (loud_q * (12.0 / scale / loud_q.pow(2).sum())).bfloat16().float()
+    k_pages, v_pages, table = _paged(ks, vs, torch.bfloat16, kv_heads, head_dim)
+    q = torch.stack([q for _, _, q in rows]).bfloat16().reshape(len(rows), -1).cuda()
+    out = torch.full((len(rows), heads * head_dim), 3.0, dtype=torch.bfloat16, device="cuda")
+    tile = ops.prefill_tile_rows(heads, kv_heads, head_dim)
+    assert tile in (16, 32, 64)
+    items = [(seq, row0) for seq, (_, _, n) in enumerate(sequences) for row0 in range(0, n, tile)]
+    starts = [0, 130, 167, 168]
+    for window in (0, 40):
+        ops.attention_prefill_bf16(q, out, k_pages, v_pages, table, _i32([s for s, _ in items]), _i32([r for _, r in items]),
+                                   _i32([s for s, _, _ in sequences]), _i32(starts), _i32([p for _, p, _ in sequences]),
+                                   heads, kv_heads, head_dim, scale, window)
+        got = out.cpu().float().view(len(rows), heads, head_dim)
+        want = _plain_rows(rows, ks, vs, scale, window=window)
+        error = (got - want).abs().amax(dim=(1, 2))
+        assert error.max().item() <= 2e-2, (window, int(error.argmax()), error.max().item())
+        if window == 0:
+            assert (got[100, 0] - vs[2][17, 0]).abs().max().item() < 0.05
+
+
 def _paged(k_seqs, v_seqs, dtype, kv_heads, head_dim, page_order=None, pages=32, max_pages=12):
     """Lays sequences out in pages the way the cache does.  k_seqs[i]: [len, kv_heads, head_dim]."""
     k_pages = torch.full((pages, kv_heads, 64, head_dim), 77.0, dtype=dtype)
