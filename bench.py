@@ -91,7 +91,7 @@ def main() -> int:
             tokens = selector.select(logits, slots, [None] * batch)
 
             def one_step(tokens):
-                logits = engine.step([StepEntry(s, [t], None) for s, t in zip(slots, tokens)])
+                logits = engine.step_view([StepEntry(s, [t], None) for s, t in zip(slots, tokens)])
                 return selector.select(logits, slots, [None] * batch)
 
             for _ in range(warmup):

@@ -199,31 +199,37 @@ __device__ __forceinline__ void init_state(AttnState<C>& st) {
   }
 }
 
-// One block of 32 keys (keys key0 .. key0+31, inside one page) for C column tiles.
+// One block of 32 keys (keys key0 .. key0+31, inside one page): its operands.
 //   k_block: &K[page][kv_head][key0 % 64][0]      (row stride HD)
 //   v_block: &V[page][kv_head][0][key0 % 64]      (channel stride 64)
-//   lo[c], hi[c]: the column of this lane reads keys lo <= key <= hi
-template <int C>
-__device__ __forceinline__ void attend_block(AttnState<C>& st, const QFrag (&q)[C], const bf16_t* k_block,
-                                             const bf16_t* v_block, int key0, const int (&lo)[C], const int (&hi)[C],
-                                             float scale_log2, int r, int g) {
+struct BlockFrags {
   QFrag keys[2];
-#pragma unroll
-  for (int t = 0; t < 2; ++t) keys[t] = load_row_operand(k_block + (size_t)(16 * t + r) * HD, g);
   bf16x4 v_lo[kTilesD], v_hi[kTilesD];
+};
+
+__device__ __forceinline__ void load_block(BlockFrags& f, const bf16_t* k_block, const bf16_t* v_block, int r, int g) {
+#pragma unroll
+  for (int t = 0; t < 2; ++t) f.keys[t] = load_row_operand(k_block + (size_t)(16 * t + r) * HD, g);
 #pragma unroll
   for (int t = 0; t < kTilesD; ++t) {
     const bf16_t* channel = v_block + (size_t)(16 * t + r) * kPageTokens + 4 * g;
-    v_lo[t] = *(const bf16x4*)channel;
-    v_hi[t] = *(const bf16x4*)(channel + 16);
+    f.v_lo[t] = *(const bf16x4*)channel;
+    f.v_hi[t] = *(const bf16x4*)(channel + 16);
   }
+}
+
+// Scores, softmax update and output update of one loaded block for C column tiles.
+//   lo[c], hi[c]: the column of this lane reads keys lo <= key <= hi
+template <int C>
+__device__ __forceinline__ void attend_block(AttnState<C>& st, const QFrag (&q)[C], const BlockFrags& f, int key0,
+                                             const int (&lo)[C], const int (&hi)[C], float scale_log2, int g) {
 #pragma unroll
   for (int c = 0; c < C; ++c) {
     f32x4 s[2];
     float block_max = -INFINITY;
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
-      s[t] = score_tile(keys[t], q[c]);
+      s[t] = score_tile(f.keys[t], q[c]);
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         const int key = key0 + 16 * t + 4 * g + e;
@@ -253,14 +259,29 @@ __device__ __forceinline__ void attend_block(AttnState<C>& st, const QFrag (&q)[
     for (int t = 0; t < kTilesD; ++t) {
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        v_operand[e] = v_lo[t][e];
-        v_operand[4 + e] = v_hi[t][e];
+        v_operand[e] = f.v_lo[t][e];
+        v_operand[4 + e] = f.v_hi[t][e];
       }
       st.o[c][t] = st.o[c][t] * alpha;
       st.o[c][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v_operand, p, st.o[c][t], 0, 0, 0);
     }
   }
 }
+
+// The pages of a run of key blocks, 64 at a time in the lanes of the wave: a
+// block's page is a lane broadcast, not a dependent load in front of every block.
+struct PageRun {
+  const int* pages;
+  int max_pages;
+  int first, stride;  // lane i holds the page of block index first + i * stride (in units of 32 keys)
+  int cached;
+  __device__ __forceinline__ void fill(int lane) {
+    int index = (first + lane * stride) / 2;  // two blocks of 32 keys a page
+    index = index < max_pages ? index : max_pages - 1;
+    cached = pages[index];
+  }
+  __device__ __forceinline__ int page(int i) const { return __shfl(cached, i, kWave); }
+};
 
 struct MfmaArgs {
   const bf16_t* q;  // [tokens, heads, HD]
@@ -292,11 +313,89 @@ __device__ __forceinline__ const bf16_t* v_page_ptr(const MfmaArgs& a, int page,
   return a.v_pages + ((size_t)page * a.kv_heads + kv_head) * HD * kPageTokens;
 }
 
+// Waves of a block that dealt a run of key blocks among themselves: waves 1.. leave
+// their states in LDS, wave 0 folds them into its own.  Returns false for the
+// waves that are done.  `merge` holds [waves - 1][C][kTilesD * 4 + 2][64] floats.
+template <int C>
+__device__ __forceinline__ bool merge_waves(AttnState<C>& st, float* merge, int wave, int waves, int lane) {
+  constexpr int kValues = kTilesD * 4 + 2;
+  if (waves == 1) return true;
+  if (wave > 0) {
+    float* mine = merge + (size_t)(wave - 1) * C * kValues * kWave;
+#pragma unroll
+    for (int c = 0; c < C; ++c) {
+      float* col = mine + (size_t)c * kValues * kWave + lane;
+#pragma unroll
+      for (int t = 0; t < kTilesD; ++t)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) col[(4 * t + e) * kWave] = st.o[c][t][e];
+      col[(kTilesD * 4) * kWave] = st.m[c];
+      col[(kTilesD * 4 + 1) * kWave] = st.l[c];
+    }
+  }
+  __syncthreads();
+  if (wave > 0) return false;
+  for (int other = 0; other < waves - 1; ++other) {
+    const float* theirs = merge + (size_t)other * C * kValues * kWave;
+#pragma unroll
+    for (int c = 0; c < C; ++c) {
+      const float* col = theirs + (size_t)c * kValues * kWave + lane;
+      const float m_other = col[(kTilesD * 4) * kWave];
+      const float m_new = fmaxf(st.m[c], m_other);
+      const float m_safe = m_new == -INFINITY ? 0.0f : m_new;
+      const float mine_w = __builtin_amdgcn_exp2f(st.m[c] - m_safe);
+      const float their_w = __builtin_amdgcn_exp2f(m_other - m_safe);
+      st.l[c] = st.l[c] * mine_w + col[(kTilesD * 4 + 1) * kWave] * their_w;
+      st.m[c] = m_new;
+#pragma unroll
+      for (int t = 0; t < kTilesD; ++t)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) st.o[c][t][e] = st.o[c][t][e] * mine_w + col[(4 * t + e) * kWave] * their_w;
+    }
+  }
+  return true;
+}
+
+// Runs the key blocks first + wave, first + wave + waves, ... (count of them: `mine`)
+// through the softmax state, the next block's operands in flight while one is worked on.
+template <int C>
+__device__ __forceinline__ void attend_run(AttnState<C>& st, const QFrag (&q)[C], const MfmaArgs& a, const int* pages,
+                                           int kv_head, int first, int stride, int mine, const int (&lo)[C],
+                                           const int (&hi)[C], int lane) {
+  if (mine <= 0) return;
+  const int r = lane % 16, g = lane / 16;
+  const bf16_t* k_base = k_page_ptr(a, 0, kv_head);
+  const bf16_t* v_base = v_page_ptr(a, 0, kv_head);
+  const size_t k_page_stride = (size_t)a.kv_heads * kPageTokens * HD, v_page_stride = (size_t)a.kv_heads * HD * kPageTokens;
+  PageRun run = {pages, a.max_pages, first, stride, 0};
+  run.fill(lane);
+  BlockFrags current, next;
+  {
+    const int page = run.page(0);
+    const int inside = (first * 32) % kPageTokens;
+    load_block(current, k_base + page * k_page_stride + (size_t)inside * HD, v_base + page * v_page_stride + inside, r, g);
+  }
+  for (int i = 0; i < mine; ++i) {
+    if (i + 1 < mine) {
+      if (((i + 1) & 63) == 0) {
+        run.first = first + (i + 1) * stride;
+        run.fill(lane);
+      }
+      const int page = run.page((i + 1) & 63);
+      const int inside = ((first + (i + 1) * stride) * 32) % kPageTokens;
+      load_block(next, k_base + page * k_page_stride + (size_t)inside * HD, v_base + page * v_page_stride + inside, r, g);
+    }
+    attend_block<C>(st, q, current, (first + i * stride) * 32, lo, hi, a.scale_log2, g);
+    current = next;
+  }
+}
+
 // ---- prefill: a wave = (query tile, kv head, chunk of GH query heads); C = QT * GH column tiles --------
 template <int QT, int GH>
-__global__ __launch_bounds__(kWave) void attention_prefill_kernel(MfmaArgs a) {
+__global__ __launch_bounds__(256) void attention_prefill_kernel(MfmaArgs a, int waves) {
+  extern __shared__ float merge[];
   constexpr int C = QT * GH;
-  const int lane = threadIdx.x, r = lane % 16, g = lane / 16;
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave, r = lane % 16, g = lane / 16;
   const int tile = blockIdx.x;
   const int group = a.heads / a.kv_heads;
   const int chunks = (group + GH - 1) / GH;
@@ -341,13 +440,11 @@ __global__ __launch_bounds__(kWave) void attention_prefill_kernel(MfmaArgs a) {
   AttnState<C> st;
   init_state(st);
   if (last >= 0) {
-    for (int key0 = (first / 32) * 32; key0 <= last; key0 += 32) {
-      const int page = pages[key0 / kPageTokens];
-      const int inside = key0 % kPageTokens;
-      attend_block<C>(st, q, k_page_ptr(a, page, kv_head) + (size_t)inside * HD, v_page_ptr(a, page, kv_head) + inside,
-                      key0, lo, hi, a.scale_log2, r, g);
-    }
+    const int first_block = first / 32, blocks = last / 32 + 1 - first_block;
+    const int mine = blocks > wave ? (blocks - wave + waves - 1) / waves : 0;
+    attend_run<C>(st, q, a, pages, kv_head, first_block + wave, waves, mine, lo, hi, lane);
   }
+  if (!merge_waves<C>(st, merge, wave, waves, lane)) return;
 #pragma unroll
   for (int qt = 0; qt < QT; ++qt)
 #pragma unroll
@@ -369,13 +466,15 @@ __global__ __launch_bounds__(kWave) void attention_prefill_kernel(MfmaArgs a) {
     }
 }
 
-// ---- decode: a wave = (token, kv head, split of the keys); columns are the heads of the group ---------
+// ---- decode: a block = (token, kv head, split of the keys); columns are the heads of the group; ------
+// the block's waves deal the split's key blocks among themselves and merge their states through LDS
 template <int C>
-__global__ __launch_bounds__(kWave) void attention_decode_kernel(MfmaArgs a) {
-  const int lane = threadIdx.x, r = lane % 16, g = lane / 16;
+__global__ __launch_bounds__(512) void attention_decode_kernel(MfmaArgs a, int waves) {
+  extern __shared__ float merge[];  // [waves - 1][C][kTilesD * 4 + 2][64]
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave, r = lane % 16, g = lane / 16;
   const int token = blockIdx.x, kv_head = blockIdx.y, split = blockIdx.z;
   const int slot = a.tok_slot[token];
-  if (slot < 0) return;  // a padding row: its output is never read
+  if (slot < 0) return;  // a padding row (the whole block leaves): its output is never read
   const int group = a.heads / a.kv_heads;
   const int pos = a.tok_pos[token];
   const int first_key = (a.window > 0 && pos + 1 > a.window) ? pos + 1 - a.window : 0;
@@ -393,20 +492,16 @@ __global__ __launch_bounds__(kWave) void attention_decode_kernel(MfmaArgs a) {
     lo[c] = first_key;
     hi[c] = live[c] ? pos : -1;
   }
-  // blocks of 32 keys are dealt to the splits in contiguous runs
+  // blocks of 32 keys are dealt to the splits in contiguous runs, and within a split to the waves in turn
   const int block_first = first_key / 32, block_count = pos / 32 + 1 - block_first;
   const int per_split = (block_count + a.splits - 1) / a.splits;
   const int begin = block_first + split * per_split;
   const int end = min(begin + per_split, block_first + block_count);
   AttnState<C> st;
   init_state(st);
-  for (int block = begin; block < end; ++block) {
-    const int key0 = block * 32;
-    const int page = pages[key0 / kPageTokens];
-    const int inside = key0 % kPageTokens;
-    attend_block<C>(st, q, k_page_ptr(a, page, kv_head) + (size_t)inside * HD, v_page_ptr(a, page, kv_head) + inside, key0,
-                    lo, hi, a.scale_log2, r, g);
-  }
+  const int mine = end > begin + wave ? (end - begin - wave + waves - 1) / waves : 0;  // key blocks of this wave
+  attend_run<C>(st, q, a, pages, kv_head, begin + wave, waves, mine, lo, hi, lane);
+  if (!merge_waves<C>(st, merge, wave, waves, lane)) return;
 #pragma unroll
   for (int c = 0; c < C; ++c) {
     float total = st.l[c];
@@ -518,11 +613,21 @@ extern "C" int nnis_attention_prefill_tile_rows(int heads, int kv_heads) {
   return 16 * (kMaxColumns / (gh > 0 ? gh : 1));
 }
 
+// waves a block of the prefill kernel may have for these sizes (LDS of the merge)
+extern "C" int nnis_attention_prefill_max_waves(int heads, int kv_heads) {
+  const int group = heads / (kv_heads > 0 ? kv_heads : 1);
+  const int gh = group < kMaxColumns ? group : kMaxColumns;
+  const int columns = (kMaxColumns / (gh > 0 ? gh : 1)) * gh;
+  const size_t per_wave = (size_t)columns * (kTilesD * 4 + 2) * kWave * sizeof(float);
+  int waves = 1 + (int)(65536 / per_wave);
+  return waves >= 4 ? 4 : (waves >= 2 ? 2 : 1);
+}
+
 extern "C" int nnis_attention_prefill_bf16(const void* q, void* out, const void* k_pages, const void* v_pages,
                                            const int* block_table, int max_pages, const int* tile_seq,
                                            const int* tile_row0, int tiles, const int* seq_slot, const int* seq_start,
                                            const int* seq_pos0, int heads, int kv_heads, int head_dim, int window,
-                                           float scale, void* stream) {
+                                           float scale, int waves, void* stream) {
   MfmaArgs a;
   if (fill_common(a, q, out, k_pages, v_pages, block_table, max_pages, heads, kv_heads, head_dim, window, scale)) return 1;
   if (tiles <= 0) return 0;
@@ -533,29 +638,45 @@ extern "C" int nnis_attention_prefill_bf16(const void* q, void* out, const void*
   const int chunks = (group + gh - 1) / gh;
   const dim3 grid(tiles, kv_heads * chunks);
   NNIS_REQUIRE(grid.y <= 65535, "attention: %d head chunks exceed the grid limit", grid.y);
+  const size_t per_wave = (size_t)qt * gh * (kTilesD * 4 + 2) * kWave * sizeof(float);
+  NNIS_REQUIRE(waves >= 1 && waves <= 4 && (waves - 1) * per_wave <= 65536,
+               "attention: %d waves a block do not fit this head size (LDS)", waves);
+  const size_t lds = (waves - 1) * per_wave;
+  const dim3 block(kWave * waves);
   hipStream_t s = (hipStream_t)stream;
-  if (qt == 4 && gh == 1) hipLaunchKernelGGL((attention_prefill_kernel<4, 1>), grid, dim3(kWave), 0, s, a);
-  else if (qt == 2 && gh == 2) hipLaunchKernelGGL((attention_prefill_kernel<2, 2>), grid, dim3(kWave), 0, s, a);
-  else if (qt == 2 && gh == 1) hipLaunchKernelGGL((attention_prefill_kernel<2, 1>), grid, dim3(kWave), 0, s, a);
-  else if (qt == 1 && gh == 3) hipLaunchKernelGGL((attention_prefill_kernel<1, 3>), grid, dim3(kWave), 0, s, a);
-  else if (qt == 1 && gh == 4) hipLaunchKernelGGL((attention_prefill_kernel<1, 4>), grid, dim3(kWave), 0, s, a);
-  else if (qt == 1 && gh == 2) hipLaunchKernelGGL((attention_prefill_kernel<1, 2>), grid, dim3(kWave), 0, s, a);
-  else if (qt == 1 && gh == 1) hipLaunchKernelGGL((attention_prefill_kernel<1, 1>), grid, dim3(kWave), 0, s, a);
+  if (qt == 4 && gh == 1) hipLaunchKernelGGL((attention_prefill_kernel<4, 1>), grid, block, lds, s, a, waves);
+  else if (qt == 2 && gh == 2) hipLaunchKernelGGL((attention_prefill_kernel<2, 2>), grid, block, lds, s, a, waves);
+  else if (qt == 2 && gh == 1) hipLaunchKernelGGL((attention_prefill_kernel<2, 1>), grid, block, lds, s, a, waves);
+  else if (qt == 1 && gh == 3) hipLaunchKernelGGL((attention_prefill_kernel<1, 3>), grid, block, lds, s, a, waves);
+  else if (qt == 1 && gh == 4) hipLaunchKernelGGL((attention_prefill_kernel<1, 4>), grid, block, lds, s, a, waves);
+  else if (qt == 1 && gh == 2) hipLaunchKernelGGL((attention_prefill_kernel<1, 2>), grid, block, lds, s, a, waves);
+  else if (qt == 1 && gh == 1) hipLaunchKernelGGL((attention_prefill_kernel<1, 1>), grid, block, lds, s, a, waves);
   else return nnis_fail("attention: no kernel for %d query tiles x %d heads", qt, gh);
   NNIS_LAUNCH_CHECK("attention_prefill");
   return 0;
 }
 
 // partial: float32 scratch of at least tokens * heads * splits * (head_dim + 2), needed when splits > 1
+extern "C" int nnis_attention_decode_max_waves(int heads, int kv_heads) {
+  const int group = heads / (kv_heads > 0 ? kv_heads : 1);
+  const int tiles = (group + 15) / 16;
+  const int per_wave = tiles * (kTilesD * 4 + 2) * kWave * 4;  // bytes of LDS a wave beyond the first needs
+  int waves = 1 + 65536 / per_wave;
+  return waves > 8 ? 8 : (waves >= 4 ? 4 : (waves >= 2 ? 2 : 1));
+}
+
 extern "C" int nnis_attention_decode_bf16(const void* q, void* out, const void* k_pages, const void* v_pages,
                                           const int* block_table, int max_pages, const int* tok_slot, const int* tok_pos,
                                           int tokens, int heads, int kv_heads, int head_dim, int window, float scale,
-                                          int splits, float* partial, void* stream) {
+                                          int splits, int waves, float* partial, void* stream) {
   MfmaArgs a;
   if (fill_common(a, q, out, k_pages, v_pages, block_table, max_pages, heads, kv_heads, head_dim, window, scale)) return 1;
   NNIS_REQUIRE(splits >= 1 && splits <= 65535, "attention: bad number of splits %d", splits);
   NNIS_REQUIRE(splits == 1 || partial != nullptr, "attention: splits need scratch memory");
   NNIS_REQUIRE(kv_heads <= 65535, "attention: %d kv heads exceed the grid limit", kv_heads);
+  NNIS_REQUIRE(waves >= 1 && waves <= nnis_attention_decode_max_waves(heads, kv_heads),
+               "attention: %d waves a block; this head size and group take at most %d", waves,
+               nnis_attention_decode_max_waves(heads, kv_heads));
   if (tokens <= 0) return 0;
   const int group = heads / kv_heads;
   NNIS_REQUIRE(group <= 16 * kMaxColumns, "attention: a group of %d query heads is more than this head size's decode kernel carries (%d)",
@@ -564,9 +685,10 @@ extern "C" int nnis_attention_decode_bf16(const void* q, void* out, const void* 
   const dim3 grid(tokens, kv_heads, splits);
   hipStream_t s = (hipStream_t)stream;
   const int tiles = (group + 15) / 16;
-  if (tiles == 1) hipLaunchKernelGGL((attention_decode_kernel<1>), grid, dim3(kWave), 0, s, a);
-  else if (tiles == 2 && kMaxColumns >= 2) hipLaunchKernelGGL((attention_decode_kernel<(kMaxColumns >= 2 ? 2 : 1)>), grid, dim3(kWave), 0, s, a);
-  else hipLaunchKernelGGL((attention_decode_kernel<kMaxColumns>), grid, dim3(kWave), 0, s, a);
+  const size_t lds = (size_t)(waves - 1) * tiles * (kTilesD * 4 + 2) * kWave * sizeof(float);
+  if (tiles == 1) hipLaunchKernelGGL((attention_decode_kernel<1>), grid, dim3(kWave * waves), lds, s, a, waves);
+  else if (tiles == 2) hipLaunchKernelGGL((attention_decode_kernel<(kMaxColumns >= 2 ? 2 : 1)>), grid, dim3(kWave * waves), lds, s, a, waves);
+  else hipLaunchKernelGGL((attention_decode_kernel<kMaxColumns>), grid, dim3(kWave * waves), lds, s, a, waves);
   NNIS_LAUNCH_CHECK("attention_decode");
   if (splits > 1) {
     hipLaunchKernelGGL(attention_combine_kernel, dim3(tokens, heads), dim3(HD < 64 ? 64 : (HD > 256 ? 256 : HD)), 0, s, partial,
@@ -577,12 +699,14 @@ extern "C" int nnis_attention_decode_bf16(const void* q, void* out, const void* 
 }
 #else
 extern "C" int nnis_attention_prefill_tile_rows(int, int) { return 0; }
+extern "C" int nnis_attention_prefill_max_waves(int, int) { return 1; }
 extern "C" int nnis_attention_prefill_bf16(const void*, void*, const void*, const void*, const int*, int, const int*, const int*,
-                                           int, const int*, const int*, const int*, int, int, int, int, float, void*) {
+                                           int, const int*, const int*, const int*, int, int, int, int, float, int, void*) {
   return nnis_fail("attention: the matrix-core kernels need a head size in steps of 16; this module has %d", NNIS_HEAD_DIM);
 }
+extern "C" int nnis_attention_decode_max_waves(int, int) { return 1; }
 extern "C" int nnis_attention_decode_bf16(const void*, void*, const void*, const void*, const int*, int, const int*, const int*,
-                                          int, int, int, int, int, float, int, float*, void*) {
+                                          int, int, int, int, int, float, int, int, float*, void*) {
   return nnis_fail("attention: the matrix-core kernels need a head size in steps of 16; this module has %d", NNIS_HEAD_DIM);
 }
 #endif

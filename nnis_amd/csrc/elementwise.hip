@@ -73,6 +73,76 @@ __global__ void rmsnorm_kernel(void* __restrict__ x, int x_dtype, const void* __
   }
 }
 
+// One wave per row, the row held in registers: a single pass over memory and no
+// block barrier.  Needs width % 4 == 0 (16-byte accesses) and width <= 256 * CH.
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4_t;
+
+__device__ __forceinline__ f32x4_t load4_as_f32(const void* base, int dtype, size_t index) {
+  if (dtype == NNIS_F32) return *(const f32x4_t*)((const float*)base + index);
+  const bf16x4_t v = *(const bf16x4_t*)((const bf16_t*)base + index);
+  return (f32x4_t){(float)v[0], (float)v[1], (float)v[2], (float)v[3]};
+}
+
+__device__ __forceinline__ void store4_from_f32(void* base, int dtype, size_t index, f32x4_t v) {
+  if (dtype == NNIS_F32) {
+    *(f32x4_t*)((float*)base + index) = v;
+  } else {
+    bf16x4_t packed;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) packed[e] = (__bf16)v[e];
+    *(bf16x4_t*)((bf16_t*)base + index) = packed;
+  }
+}
+
+template <int CH>
+__global__ __launch_bounds__(256) void rmsnorm_wave_kernel(void* __restrict__ x, int x_dtype, const void* __restrict__ delta,
+                                                           int delta_dtype, const void* __restrict__ weight, int weight_dtype,
+                                                           void* __restrict__ out, int out_dtype, const int* __restrict__ rows,
+                                                           int out_rows, int width, float inv_width, float eps) {
+  const int lane = threadIdx.x % kWave;
+  const int out_row = blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
+  if (out_row >= out_rows) return;
+  const int in_row = rows ? rows[out_row] : out_row;
+  const size_t in_base = (size_t)in_row * width;
+  const size_t out_base = (size_t)out_row * width;
+  const bool write_back = delta != nullptr && rows == nullptr;
+  f32x4_t v[CH];
+  float sumsq = 0.0f;
+#pragma unroll
+  for (int c = 0; c < CH; ++c) {
+    const int col = 4 * (lane + kWave * c);
+    if (col < width) {
+      v[c] = load4_as_f32(x, x_dtype, in_base + col);
+      if (delta) {
+        v[c] += load4_as_f32(delta, delta_dtype, in_base + col);
+        if (write_back) *(f32x4_t*)((float*)x + in_base + col) = v[c];
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) sumsq = fmaf(v[c][e], v[c][e], sumsq);
+    }
+  }
+  const float scale = 1.0f / sqrtf(wave_sum(sumsq) * inv_width + eps);
+#pragma unroll
+  for (int c = 0; c < CH; ++c) {
+    const int col = 4 * (lane + kWave * c);
+    if (col < width) {
+      const f32x4_t w = load4_as_f32(weight, weight_dtype, col);
+      store4_from_f32(out, out_dtype, out_base + col, (v[c] * scale) * w);
+    }
+  }
+}
+
+template <int CH>
+static void launch_rmsnorm_wave(void* x, int x_dtype, const void* delta, int delta_dtype, const void* weight, int weight_dtype,
+                                void* out, int out_dtype, const int* rows, int out_rows, int width, float eps,
+                                hipStream_t stream) {
+  const int waves = out_rows >= 1024 ? 4 : 1;  // few rows: one wave a block, spread over the chip
+  hipLaunchKernelGGL(rmsnorm_wave_kernel<CH>, dim3((out_rows + waves - 1) / waves), dim3(waves * kWave), 0, stream, x,
+                     x_dtype, delta, delta_dtype, weight, weight_dtype, out, out_dtype, rows, out_rows, width,
+                     1.0f / (float)width, eps);
+}
+
 extern "C" int nnis_rmsnorm(void* x, int x_dtype, const void* delta, int delta_dtype, const void* weight,
                             int weight_dtype, void* out, int out_dtype, const int* rows, int out_rows, int width,
                             float eps, void* stream) {
@@ -84,8 +154,27 @@ extern "C" int nnis_rmsnorm(void* x, int x_dtype, const void* delta, int delta_d
   NNIS_REQUIRE(out_rows >= 0 && width > 0, "rmsnorm: bad sizes rows=%d width=%d", out_rows, width);
   NNIS_REQUIRE(eps > 0.0f, "rmsnorm: eps must be positive, got %g", (double)eps);
   if (out_rows == 0) return 0;
+  hipStream_t s = (hipStream_t)stream;
+  const bool aligned = ((uintptr_t)x % 16 == 0) && ((uintptr_t)out % 16 == 0) && ((uintptr_t)weight % 16 == 0) &&
+                       (delta == nullptr || (uintptr_t)delta % 16 == 0);
+  if (width % 4 == 0 && aligned && width <= 256 * 32) {
+    const int chunks = (width + 255) / 256;
+#define NNIS_NORM_CASE(CH)                                                                                          \
+  launch_rmsnorm_wave<CH>(x, x_dtype, delta, delta_dtype, weight, weight_dtype, out, out_dtype, rows, out_rows, width, \
+                          eps, s)
+    if (chunks <= 1) NNIS_NORM_CASE(1);
+    else if (chunks <= 2) NNIS_NORM_CASE(2);
+    else if (chunks <= 3) NNIS_NORM_CASE(3);
+    else if (chunks <= 4) NNIS_NORM_CASE(4);
+    else if (chunks <= 8) NNIS_NORM_CASE(8);
+    else if (chunks <= 16) NNIS_NORM_CASE(16);
+    else NNIS_NORM_CASE(32);
+#undef NNIS_NORM_CASE
+    NNIS_LAUNCH_CHECK("rmsnorm_wave");
+    return 0;
+  }
   const int threads = width >= 1024 ? 256 : (width >= 256 ? 128 : 64);
-  hipLaunchKernelGGL(rmsnorm_kernel, dim3(out_rows), dim3(threads), 0, (hipStream_t)stream, x, x_dtype, delta,
+  hipLaunchKernelGGL(rmsnorm_kernel, dim3(out_rows), dim3(threads), 0, s, x, x_dtype, delta,
                      delta_dtype, weight, weight_dtype, out, out_dtype, rows, width, 1.0f / (float)width, eps);
   NNIS_LAUNCH_CHECK("rmsnorm");
   return 0;

@@ -64,13 +64,20 @@ __device__ __forceinline__ void store4<bf16_t>(bf16_t* y, size_t index, f32x4 v,
 }
 
 // -----------------------------------------------------------------------------
-// skinny: MT token tiles of 16 (M <= 16 * MT), KSPLIT waves share one strip
+// skinny: MT token tiles of 16 (M <= 16 * MT); KSPLIT waves share one strip's K.
+// A decode-sized product is bound by memory latency, not bandwidth: a wave
+// issues the loads of DEPTH steps of 64 k (weights and activations) before the
+// first multiply, so its whole share of K is usually one round trip.
 // -----------------------------------------------------------------------------
 template <int MT, int KSPLIT, typename OutT>
-__global__ __launch_bounds__(256) void gemm_skinny_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
-                                                          OutT* __restrict__ y, int m, int n, int k) {
-  constexpr int kStrips = 4 / KSPLIT;  // strips of 16 weight rows per block
-  __shared__ float partial[KSPLIT > 1 ? 4 : 1][MT][kWave][4];
+__global__ __launch_bounds__(KSPLIT > 4 ? 64 * KSPLIT : 256) void gemm_skinny_kernel(const bf16_t* __restrict__ x,
+                                                                                   const bf16_t* __restrict__ w,
+                                                                                   OutT* __restrict__ y, int m, int n,
+                                                                                   int k) {
+  constexpr int kWaves = KSPLIT > 4 ? KSPLIT : 4;
+  constexpr int kStrips = kWaves / KSPLIT;  // strips of 16 weight rows per block
+  constexpr int DEPTH = MT <= 2 ? 4 : 2;
+  __shared__ float partial[KSPLIT > 1 ? kWaves : 1][MT][kWave][4];
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
   const int strip = blockIdx.x * kStrips + wave / KSPLIT;
   const int part = wave % KSPLIT;
@@ -93,19 +100,28 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const bf16_t* __restri
       token = token < m ? token : m - 1;
       x_ptr[t] = x + (size_t)token * k;
     }
-#pragma unroll 2
-    for (int k0 = part * 64; k0 < k; k0 += 64 * KSPLIT) {
-      const int ka = k0 + g * 16, kb = ka + 8;
-      const bool in_a = ka + 8 <= k, in_b = kb + 8 <= k;
-      const bf16x8 wa = in_a ? load_chunk(w_ptr + ka) : zero_chunk();
-      const bf16x8 wb = in_b ? load_chunk(w_ptr + kb) : zero_chunk();
+    const int chunks = (k + 63) / 64;
+    for (int base = part; base < chunks; base += KSPLIT * DEPTH) {
+      bf16x8 wa[DEPTH], wb[DEPTH], xa[DEPTH][MT], xb[DEPTH][MT];
 #pragma unroll
-      for (int t = 0; t < MT; ++t) {
-        const bf16x8 xa = in_a ? load_chunk(x_ptr[t] + ka) : zero_chunk();
-        const bf16x8 xb = in_b ? load_chunk(x_ptr[t] + kb) : zero_chunk();
-        acc[t] = mfma(wa, xa, acc[t]);
-        acc[t] = mfma(wb, xb, acc[t]);
+      for (int d = 0; d < DEPTH; ++d) {
+        const int ka = (base + d * KSPLIT) * 64 + g * 16, kb = ka + 8;
+        const bool in_a = ka + 8 <= k, in_b = kb + 8 <= k;  // false also for steps beyond the last
+        wa[d] = in_a ? load_chunk(w_ptr + ka) : zero_chunk();
+        wb[d] = in_b ? load_chunk(w_ptr + kb) : zero_chunk();
+#pragma unroll
+        for (int t = 0; t < MT; ++t) {
+          xa[d][t] = in_a ? load_chunk(x_ptr[t] + ka) : zero_chunk();
+          xb[d][t] = in_b ? load_chunk(x_ptr[t] + kb) : zero_chunk();
+        }
       }
+#pragma unroll
+      for (int d = 0; d < DEPTH; ++d)
+#pragma unroll
+        for (int t = 0; t < MT; ++t) {
+          acc[t] = mfma(wa[d], xa[d][t], acc[t]);
+          acc[t] = mfma(wb[d], xb[d][t], acc[t]);
+        }
     }
   }
 
@@ -240,14 +256,16 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
 template <int MT, int KSPLIT, typename OutT>
 void launch_skinny(const bf16_t* x, const bf16_t* w, OutT* y, int m, int n, int k, hipStream_t stream) {
   const int strips = (n + 15) / 16;
-  const int per_block = 4 / KSPLIT;
-  hipLaunchKernelGGL((gemm_skinny_kernel<MT, KSPLIT, OutT>), dim3((strips + per_block - 1) / per_block), dim3(256), 0,
-                     stream, x, w, y, m, n, k);
+  const int waves = KSPLIT > 4 ? KSPLIT : 4;
+  const int per_block = waves / KSPLIT;
+  hipLaunchKernelGGL((gemm_skinny_kernel<MT, KSPLIT, OutT>), dim3((strips + per_block - 1) / per_block),
+                     dim3(64 * waves), 0, stream, x, w, y, m, n, k);
 }
 
 template <int MT, typename OutT>
 void dispatch_skinny_split(const bf16_t* x, const bf16_t* w, OutT* y, int m, int n, int k, int split, hipStream_t stream) {
-  if (split == 4) launch_skinny<MT, 4, OutT>(x, w, y, m, n, k, stream);
+  if (split == 8) launch_skinny<MT, 8, OutT>(x, w, y, m, n, k, stream);
+  else if (split == 4) launch_skinny<MT, 4, OutT>(x, w, y, m, n, k, stream);
   else if (split == 2) launch_skinny<MT, 2, OutT>(x, w, y, m, n, k, stream);
   else launch_skinny<MT, 1, OutT>(x, w, y, m, n, k, stream);
 }
@@ -291,11 +309,16 @@ extern "C" int nnis_gemm_bf16(const void* x, const void* w, void* y, int y_dtype
   const bf16_t* xp = (const bf16_t*)x;
   const bf16_t* wp = (const bf16_t*)w;
   if (m <= 64) {
-    // waves of a block share a strip's K when there are too few strips to fill the chip
+    // With few strips the waves of a block share a strip's K, so that each wave's
+    // share is one round of loads (4 steps of 64 for up to 32 tokens, 2 beyond);
+    // with thousands of strips there are waves enough to hide the latency.
     const int strips = (n + 15) / 16;
+    const int chunks = (k + 63) / 64;
+    const int depth = m <= 32 ? 4 : 2;
     int split = 1;
-    if (strips < 1024 && k >= 256) split = 2;
-    if (strips < 512 && k >= 512) split = 4;
+    if (strips < 2048) {
+      while (split < 8 && chunks > split * depth) split *= 2;
+    }
     if (y_dtype == NNIS_F32) dispatch_skinny<float>(xp, wp, (float*)y, m, n, k, split, stream);
     else dispatch_skinny<bf16_t>(xp, wp, (bf16_t*)y, m, n, k, split, stream);
     NNIS_LAUNCH_CHECK("gemm_skinny");

@@ -34,4 +34,5 @@ class StepContext:
     host_new: List[int] = field(default_factory=list)
     host_pos0: List[int] = field(default_factory=list)
     splits: int = 0  # runs the keys of a decode step are cut into; 0: chosen by the kernel's wrapper
+    waves: int = 1  # waves of a block of the decode attention kernel (used when splits is given)
     tiles: dict = field(default_factory=dict)  # work lists of prefill kernels, by tile size, made on first use

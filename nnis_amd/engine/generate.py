@@ -112,6 +112,7 @@ def generate(engine, requests: Sequence[GenerationRequest], selector=None, max_b
     if limit <= 0:
         raise CacheFull("the cache has no free slot")
 
+    step = getattr(engine, "step_view", engine.step)  # the logits are read at once: no copy needed
     for batch in plan_batches(needs, engine.free_pages(), limit):
         live = list(batch)
         slot_of = {}
@@ -121,7 +122,7 @@ def generate(engine, requests: Sequence[GenerationRequest], selector=None, max_b
                 selector.start(slot_of[index], requests[index].sampling)
             feed = {index: list(requests[index].prompt) for index in live}
             while live:
-                logits = engine.step([StepEntry(slot_of[i], feed[i], None) for i in live])
+                logits = step([StepEntry(slot_of[i], feed[i], None) for i in live])
                 tokens = selector.select(logits, [slot_of[i] for i in live], [requests[i].sampling for i in live])
                 still = []
                 for index, token in zip(live, tokens):

@@ -20,7 +20,7 @@ from .batch import StepContext, StepEntry
 
 
 class Engine:
-    def __init__(self, model, rt, max_tokens: int, max_slots: Optional[int] = None):
+    def __init__(self, model, rt, max_tokens: int, max_slots: Optional[int] = None, use_graphs: Optional[bool] = None):
         if not model.bound:
             raise InvalidInput("the model has no weights bound; load it first")
         self.model = model
@@ -31,6 +31,11 @@ class Engine:
         self.cache = SequenceCache(requests, shared, max_tokens, model.spec.max_positions, rt.dtype, rt.device, max_slots)
         self._staging = None
         self._staging_dev = None
+        # decode steps are replayed from HIP graphs when every part of the model
+        # runs only kernels that read the step's metadata from device memory
+        self._borrowed = False
+        self.use_graphs = model.graph_safe() if use_graphs is None else (use_graphs and model.graph_safe())
+        self._graphs = None
 
     # ---- sequences -----------------------------------------------------------
     def start_sequence(self) -> int:
@@ -96,7 +101,14 @@ class Engine:
 
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
         """Returns float32 logits [wanted places, vocab], in the order of the
-        entries and of each entry's ``want``."""
+        entries and of each entry's ``want``.  The result is the caller's to keep."""
+        logits = self.step_view(entries)
+        return logits.clone() if self._borrowed else logits
+
+    def step_view(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        """As ``step``, but the rows may view a buffer that the next step
+        overwrites: for callers that read them at once (the generation loop)."""
+        self._borrowed = False
         growth = self._validate(entries)
         pos0 = [self.cache.length(e.slot) for e in entries]
         counts = [len(e.tokens) for e in entries]
@@ -117,6 +129,9 @@ class Engine:
             row += n
             seq_start[index + 1] = row
         self.cache.grow(growth)
+
+        if self.use_graphs and all(n == 1 for n in counts):
+            return self._graph_step(entries, pos0)
 
         # the staging buffer is reused: wait until the previous step's copy has left it
         torch.cuda.current_stream().synchronize() if self._staging is not None else None
@@ -141,3 +156,19 @@ class Engine:
             host_pos0=pos0,
         )
         return self.model.forward(dev[0], ctx, self.cache, dev[6], self.rt)
+
+    def _graph_step(self, entries: Sequence[StepEntry], pos0: List[int]) -> torch.Tensor:
+        """A step of single tokens, replayed from a captured graph.  The rows
+        returned view the graph's output buffer: read them before the next step."""
+        from .graph import DecodeGraphs
+
+        if self._graphs is None:
+            self._graphs = DecodeGraphs(self)
+        plan = self.model.decode_plan(len(entries), max(p + 1 for p in pos0), self.rt)
+        graph = self._graphs.get(len(entries), plan)
+        logits = graph.run([int(e.tokens[0]) for e in entries], [e.slot for e in entries], pos0)
+        wanted = [i for i, e in enumerate(entries) if e.want is None or len(e.want) > 0]
+        if len(wanted) == len(entries):
+            self._borrowed = True
+            return logits[: len(entries)]
+        return logits[torch.tensor(wanted, dtype=torch.long, device=logits.device)]

@@ -36,9 +36,11 @@ _ATTN_SIGNATURES = {
                             _INT, _INT, _FLT, _VOID],
     "nnis_attention_prefill_tile_rows": [_INT, _INT],
     "nnis_attention_prefill_bf16": [_VOID, _VOID, _VOID, _VOID, _VOID, _INT, _VOID, _VOID, _INT, _VOID, _VOID, _VOID, _INT,
-                                    _INT, _INT, _INT, _FLT, _VOID],
+                                    _INT, _INT, _INT, _FLT, _INT, _VOID],
+    "nnis_attention_prefill_max_waves": [_INT, _INT],
     "nnis_attention_decode_bf16": [_VOID, _VOID, _VOID, _VOID, _VOID, _INT, _VOID, _VOID, _INT, _INT, _INT, _INT, _INT, _FLT,
-                                   _INT, _VOID, _VOID],
+                                   _INT, _INT, _VOID, _VOID],
+    "nnis_attention_decode_max_waves": [_INT, _INT],
 }
 
 _DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1}
@@ -295,8 +297,12 @@ def prefill_tile_rows(heads: int, kv_heads: int, head_dim: int) -> int:
     return attention_module(head_dim).nnis_attention_prefill_tile_rows(heads, kv_heads)
 
 
+def prefill_max_waves(heads: int, kv_heads: int, head_dim: int) -> int:
+    return attention_module(head_dim).nnis_attention_prefill_max_waves(heads, kv_heads)
+
+
 def attention_prefill_bf16(q, out, k_pages, v_pages, block_table, tile_seq, tile_row0, seq_slot, seq_start, seq_pos0,
-                           heads, kv_heads, head_dim, scale, window=0):
+                           heads, kv_heads, head_dim, scale, window=0, waves=1):
     """Causal attention of whole runs of new tokens over the cache, on the
     matrix cores.  ``tile_seq``/``tile_row0`` (int32) name, per work item, a
     sequence of the step and the first of ``prefill_tile_rows`` rows of its
@@ -314,15 +320,17 @@ def attention_prefill_bf16(q, out, k_pages, v_pages, block_table, tile_seq, tile
                                                 block_table.data_ptr(), block_table.shape[1], tile_seq.data_ptr(),
                                                 tile_row0.data_ptr(), tiles, seq_slot.data_ptr(), seq_start.data_ptr(),
                                                 seq_pos0.data_ptr(), heads, kv_heads, head_dim, int(window), float(scale),
-                                                _stream()))
+                                                int(waves), _stream()))
     return out
 
 
 def attention_decode_bf16(q, out, k_pages, v_pages, block_table, tok_slot, tok_pos, heads, kv_heads, head_dim, scale,
-                          window=0, splits=1, partial=None):
-    """One query token per sequence over its cached keys, the keys cut into
-    ``splits`` runs that are summed afterwards.  ``partial``: float32 scratch of
-    tokens * heads * splits * (head_dim + 2) when splits > 1."""
+                          window=0, splits=1, partial=None, waves=1):
+    """One query token per sequence over its cached keys.  The keys are cut
+    into ``splits`` runs, each a block of ``waves`` waves that deal its keys
+    among themselves and merge in LDS; the runs are summed by a second kernel.
+    ``partial``: float32 scratch of tokens * heads * splits * (head_dim + 2)
+    when splits > 1."""
     _check_pages(q, out, k_pages, v_pages, block_table, heads, kv_heads, head_dim)
     tokens = q.shape[0]
     for t in (tok_slot, tok_pos):
@@ -337,18 +345,28 @@ def attention_decode_bf16(q, out, k_pages, v_pages, block_table, tok_slot, tok_p
     _check(lib, lib.nnis_attention_decode_bf16(q.data_ptr(), out.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(),
                                                block_table.data_ptr(), block_table.shape[1], tok_slot.data_ptr(),
                                                tok_pos.data_ptr(), tokens, heads, kv_heads, head_dim, int(window),
-                                               float(scale), int(splits), _ptr(partial) if splits > 1 else None, _stream()))
+                                               float(scale), int(splits), int(waves), _ptr(partial) if splits > 1 else None,
+                                               _stream()))
     return out
 
 
-def decode_splits(batch: int, kv_heads: int, longest: int) -> int:
-    """Runs the keys of a decode step are cut into: enough waves to fill the
-    chip (about four a compute unit), at least two blocks of 32 keys a run, a
-    power of two."""
+def decode_max_waves(heads: int, kv_heads: int, head_dim: int) -> int:
+    return attention_module(head_dim).nnis_attention_decode_max_waves(heads, kv_heads)
+
+
+def decode_plan(batch: int, kv_heads: int, longest: int, max_waves: int = 8):
+    """(splits, waves) of a decode step's attention.  The kernel is bound by
+    memory latency: a wave has one block of 32 keys in flight beside the one it
+    works on, so the keys are spread over as many waves as the chip holds
+    (about two thousand), down to two blocks a wave.  Waves of a block merge in
+    LDS; beyond 8 waves the keys are also cut into runs that a second kernel
+    sums.  Powers of two."""
     blocks = (longest + 31) // 32
-    want = max(1, 1024 // max(1, batch * kv_heads))
-    splits = max(1, min(want, blocks // 2))
-    return 1 << (splits.bit_length() - 1)
+    parallel = max(1, min(blocks // 2, 2048 // max(1, batch * kv_heads)))
+    waves = min(max_waves, 1 << (parallel.bit_length() - 1))
+    rest = parallel // waves
+    splits = 1 << (rest.bit_length() - 1) if rest >= 2 else 1
+    return splits, waves
 
 
 def _prefill_tiles(ctx, rows: int, device):
@@ -371,16 +389,23 @@ def attention(q: torch.Tensor, out: torch.Tensor, view, ctx, heads: int, kv_head
     tokens, one for runs of tokens); anything else takes the 32-bit kernel."""
     fast = (q.dtype == torch.bfloat16 and view.k_pages.dtype == torch.bfloat16 and head_dim % 16 == 0)
     if fast and ctx.decode and heads // kv_heads <= 16 * (4 if head_dim <= 64 else (2 if head_dim <= 128 else 1)):
-        splits = ctx.splits or decode_splits(ctx.batch, kv_heads, ctx.max_len)
+        if ctx.splits:
+            splits, waves = ctx.splits, ctx.waves
+        else:
+            splits, waves = decode_plan(ctx.batch, kv_heads, ctx.max_len)
+        waves = min(waves, decode_max_waves(heads, kv_heads, head_dim))
         partial = None
         if splits > 1:
             partial = torch.empty(q.shape[0] * heads * splits * (head_dim + 2), dtype=torch.float32, device=q.device)
         return attention_decode_bf16(q, out, view.k_pages, view.v_pages, view.block_table, ctx.tok_slot, ctx.tok_pos, heads,
-                                     kv_heads, head_dim, scale, window, splits, partial)
+                                     kv_heads, head_dim, scale, window, splits, partial, waves)
     if fast and not ctx.decode:
         tile_seq, tile_row0 = _prefill_tiles(ctx, prefill_tile_rows(heads, kv_heads, head_dim), q.device)
+        # the waves of a block deal a tile's key blocks among themselves: worth it once a tile reads many
+        waves = min(prefill_max_waves(heads, kv_heads, head_dim), 4 if ctx.max_len >= 512 else (2 if ctx.max_len >= 128 else 1))
         return attention_prefill_bf16(q, out, view.k_pages, view.v_pages, view.block_table, tile_seq, tile_row0,
-                                      ctx.seq_slot, ctx.seq_start, ctx.seq_pos0, heads, kv_heads, head_dim, scale, window)
+                                      ctx.seq_slot, ctx.seq_start, ctx.seq_pos0, heads, kv_heads, head_dim, scale, window,
+                                      waves)
     return attention_rows(q, out, view.k_pages, view.v_pages, view.block_table, ctx.tok_slot, ctx.tok_pos, heads,
                           kv_heads, head_dim, scale, window)
 

@@ -49,6 +49,16 @@ class DecoderModel:
         total = sum(self.layers[entry.layer].weight_bytes() for entry in self.spec.schedule)
         return total + self.final_norm.weight_bytes() + self.head.weight_bytes()
 
+    def graph_safe(self) -> bool:
+        """True when a step's kernels read tokens, slots and positions from
+        device memory only, so that a captured step can be replayed."""
+        return all(getattr(part, "graph_safe", False) for part in self.parts())
+
+    def decode_plan(self, batch: int, longest: int, rt):
+        """(splits, waves) of a decode step's attention kernels, one plan for all layers."""
+        kv_heads = [request.kv_heads for _, request in self.cache_requests()[0] if hasattr(request, "kv_heads")]
+        return rt.ops.decode_plan(batch, min(kv_heads), longest) if kv_heads else (1, 1)
+
     # ---- cache ---------------------------------------------------------------
     def cache_requests(self) -> Tuple[List[Tuple[int, Any]], Dict[int, int]]:
         requests, shared = [], {}

@@ -18,6 +18,8 @@ from .linear import Projection
 
 
 class CausalSelfAttention(Mixer):
+    graph_safe = True
+
     def __init__(self, width, heads, kv_heads, head_dim, q, k, v, o, position=None, window=None, positions=None):
         if heads % kv_heads != 0:
             raise InvalidInput(f"{heads} query heads do not divide into {kv_heads} key/value heads")

@@ -75,7 +75,14 @@ class StateRequest:
 
 
 class Part:
-    """Common base: tensors in, bound device weights out."""
+    """Common base: tensors in, bound device weights out.
+
+    ``graph_safe`` says that ``forward`` only launches kernels that read the
+    step's tokens, slots and positions from the context's device tensors (no
+    host-side branching on them), so that a captured step can be replayed.  A
+    part has to say so itself; the default is no."""
+
+    graph_safe = False
 
     def tensors(self) -> List[TensorSpec]:
         return []

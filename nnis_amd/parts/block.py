@@ -20,6 +20,7 @@ class PreNormBlock(Block):
         self.norm2 = build_part("norm", norm2)
         self.feed_forward = build_part("feed_forward", feed_forward)
         self._parts = [self.norm1, self.mixer, self.norm2, self.feed_forward]
+        self.graph_safe = all(getattr(part, "graph_safe", False) for part in self._parts)
 
     def tensors(self):
         return [spec for part in self._parts for spec in part.tensors()]

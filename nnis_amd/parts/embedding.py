@@ -13,6 +13,8 @@ from .linear import Projection
 
 
 class TokenEmbedding(Part):
+    graph_safe = True
+
     def __init__(self, vocab_size, width, weight):
         self.vocab_size, self.width, self.weight_name = int(vocab_size), int(width), weight
         self.table = None
@@ -29,6 +31,8 @@ class TokenEmbedding(Part):
 
 
 class LinearHead(Part):
+    graph_safe = True
+
     def __init__(self, vocab_size, width, weight, tied_to=None):
         self.vocab_size, self.width, self.weight_name, self.tied_to = int(vocab_size), int(width), weight, tied_to
         self.projection = None

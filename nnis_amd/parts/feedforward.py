@@ -13,6 +13,8 @@ from .linear import Projection
 
 
 class GatedFeedForward(FeedForward):
+    graph_safe = True
+
     def __init__(self, width, inner, gate, up, down, activation="silu"):
         if activation != "silu":
             raise Unsupported(f"gated feed-forward activation {activation!r}; only silu is built")

@@ -7,6 +7,8 @@ from .base import Norm, TensorSpec, register_part
 
 
 class RMSNorm(Norm):
+    graph_safe = True
+
     def __init__(self, width: int, eps: float, weight: str):
         self.width = int(width)
         self.eps = float(eps)

@@ -28,6 +28,8 @@ def rotary_tables(positions: int, rot_dim: int, theta: float):
 
 
 class RotaryHalf(PositionEncoding):
+    graph_safe = True
+
     def __init__(self, rot_dim: int, theta: float, max_positions: int):
         if rot_dim <= 0 or rot_dim % 2 != 0:
             raise InvalidInput(f"rotary dimension must be even and positive; got {rot_dim}")

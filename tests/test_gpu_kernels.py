@@ -37,7 +37,7 @@ def test_embed(dtype):
     assert torch.equal(out.cpu(), want)
 
 
-@pytest.mark.parametrize("width", [5, 576, 4100])
+@pytest.mark.parametrize("width", [5, 64, 576, 1020, 4100, 8192, 9000])
 @pytest.mark.parametrize("x_dtype, w_dtype, out_dtype", [("float32", "float32", "float32"), ("float32", "bfloat16", "bfloat16"),
                                                          ("bfloat16", "float32", "bfloat16"), ("float32", "float32", "bfloat16")])
 def test_rmsnorm(width, x_dtype, w_dtype, out_dtype):
@@ -137,8 +137,8 @@ def _plain_rows(q_rows, ks, vs, scale, window=0):
 
 
 @pytest.mark.parametrize("heads, kv_heads, head_dim", MFMA_SHAPES)
-@pytest.mark.parametrize("splits", [1, 4, 16])
-def test_decode_attention_on_the_matrix_cores(heads, kv_heads, head_dim, splits):
+@pytest.mark.parametrize("splits, waves", [(1, 1), (4, 1), (16, 2), (1, 8), (2, 4)])
+def test_decode_attention_on_the_matrix_cores(heads, kv_heads, head_dim, splits, waves):
     ops = _ops()
     torch.manual_seed(heads + head_dim)
     lengths = [700, 1, 65, 33]
@@ -154,8 +154,9 @@ def test_decode_attention_on_the_matrix_cores(heads, kv_heads, head_dim, splits)
     q = torch.stack([q for _, _, q in rows]).bfloat16().reshape(len(rows), -1).cuda()
     out = torch.full((len(rows), heads * head_dim), 3.0, dtype=torch.bfloat16, device="cuda")
     partial = torch.empty(len(rows) * heads * splits * (head_dim + 2), dtype=torch.float32, device="cuda")
+    waves = min(waves, ops.decode_max_waves(heads, kv_heads, head_dim))
     ops.attention_decode_bf16(q, out, k_pages, v_pages, table, _i32([s for s, _, _ in rows]), _i32([p for _, p, _ in rows]),
-                              heads, kv_heads, head_dim, scale, 0, splits, partial)
+                              heads, kv_heads, head_dim, scale, 0, splits, partial, waves)
     got = out.cpu().float().view(len(rows), heads, head_dim)
     live = [i for i, (s, _, _) in enumerate(rows) if s >= 0]
     want = _plain_rows([rows[i] for i in live], ks, vs, scale)
@@ -164,7 +165,7 @@ def test_decode_attention_on_the_matrix_cores(heads, kv_heads, head_dim, splits)
     assert (got[0, 0] - vs[0][3, 0]).abs().max().item() < 0.05
     # a window: the row at position 699 reads keys 600..699 only
     ops.attention_decode_bf16(q, out, k_pages, v_pages, table, _i32([s for s, _, _ in rows]), _i32([p for _, p, _ in rows]),
-                              heads, kv_heads, head_dim, scale, 100, splits, partial)
+                              heads, kv_heads, head_dim, scale, 100, splits, partial, waves)
     got = out.cpu().float().view(len(rows), heads, head_dim)
     want = _plain_rows([rows[i] for i in live], ks, vs, scale, window=100)
     assert (got[live] - want).abs().max().item() <= 2e-2
@@ -194,10 +195,11 @@ def test_prefill_attention_on_the_matrix_cores(heads, kv_heads, head_dim):
     assert tile in (16, 32, 64)
     items = [(seq, row0) for seq, (_, _, n) in enumerate(sequences) for row0 in range(0, n, tile)]
     starts = [0, 130, 167, 168]
-    for window in (0, 40):
+    most = ops.prefill_max_waves(heads, kv_heads, head_dim)
+    for window, waves in ((0, 1), (40, 1), (0, most), (40, min(2, most))):
         ops.attention_prefill_bf16(q, out, k_pages, v_pages, table, _i32([s for s, _ in items]), _i32([r for _, r in items]),
                                    _i32([s for s, _, _ in sequences]), _i32(starts), _i32([p for _, p, _ in sequences]),
-                                   heads, kv_heads, head_dim, scale, window)
+                                   heads, kv_heads, head_dim, scale, window, waves)
         got = out.cpu().float().view(len(rows), heads, head_dim)
         want = _plain_rows(rows, ks, vs, scale, window=window)
         error = (got - want).abs().amax(dim=(1, 2))
