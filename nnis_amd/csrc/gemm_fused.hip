@@ -1,0 +1,361 @@
+// Decode-sized projections (M <= 64 tokens) fused with what stands before and
+// after them in a pre-norm block, so that a layer is five kernels, not eleven:
+//
+//   prologue   v = x + delta            residual sum in 32-bit, written once to x_out
+//              operand = bf16(v * g)    g: the norm's weight
+//              ss += v * v              while K streams by anyway
+//   product    acc = W . operand        v_mfma_f32_16x16x32_bf16, weights streamed once
+//   epilogue   y = acc / sqrt(ss / K + eps)   the row's scale commutes with the product
+//              then one of: store | SiLU(gate) * up | rotate-half RoPE and cache write
+//
+// RMSNorm as in /root/reference/crates/nnis-model/src/kernels.rs:15-48 (eps inside
+// the root, mean over the row); SiLU-multiply as fused_swiglu.rs:14-28; RoPE as
+// runtime_kernels.rs:38-66; keys stored rotated, values as they are
+// (runtime.rs:997-1016).  Statistics, the scale, the activation and the rotation
+// are 32-bit; the only rounding before the product is that of its bfloat16 operand.
+//
+// A wave owns one unit of output: a strip of 16 weight rows, or a pair of strips
+// that the epilogue needs together (gate and up rows of the same channels; the
+// two halves of a head that rotate into each other).  KSPLIT waves share a
+// unit's K and add their parts, and their partial sums of squares, through LDS.
+#include "common.h"
+
+namespace {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+enum : int { EPI_STORE = 0, EPI_SILU = 1, EPI_ROPE = 2 };
+
+struct FusedArgs {
+  const float* x_in;    // [m, k]
+  const bf16_t* delta;  // [m, k] or null
+  float* x_out;         // [m, k], written when delta != null
+  const void* norm_w;   // [k]
+  int norm_w_dtype;
+  float eps;
+  const bf16_t* w;  // [n, k]
+  int m, n, k;
+  bf16_t* y;  // store: [m, n]; silu: [m, n / 2]; rope: queries [m, heads * head_dim]
+  // rope + cache write
+  const float* cos_table;
+  const float* sin_table;
+  const int* tok_slot;
+  const int* tok_pos;
+  bf16_t* k_pages;  // null: this run keeps no cache of its own
+  bf16_t* v_pages;
+  const int* block_table;
+  int max_pages;
+  int heads, kv_heads, head_dim;
+};
+
+__device__ __forceinline__ bf16x8 zero8() {
+  bf16x8 z;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) z[i] = (__bf16)0.0f;
+  return z;
+}
+
+// eight consecutive floats of the norm weight, whatever its storage type
+__device__ __forceinline__ void load_gain8(const void* base, int dtype, int index, float (&out)[8]) {
+  if (dtype == NNIS_F32) {
+    const f32x4 a = *(const f32x4*)((const float*)base + index);
+    const f32x4 b = *(const f32x4*)((const float*)base + index + 4);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      out[e] = a[e];
+      out[4 + e] = b[e];
+    }
+  } else {
+    const bf16x8 v = *(const bf16x8*)((const bf16_t*)base + index);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) out[e] = (float)v[e];
+  }
+}
+
+template <int MT, int KSPLIT, int EPI>
+__global__ __launch_bounds__(KSPLIT > 4 ? 64 * KSPLIT : 256) void gemm_fused_kernel(FusedArgs a) {
+  constexpr bool PAIR = EPI != EPI_STORE;
+  constexpr int NACC = PAIR ? 2 : 1;
+  constexpr int kWaves = KSPLIT > 4 ? KSPLIT : 4;
+  constexpr int kUnits = kWaves / KSPLIT;  // units per block
+  __shared__ float part_acc[KSPLIT > 1 ? kWaves : 1][NACC][MT][kWave][4];
+  __shared__ float part_ss[KSPLIT > 1 ? kWaves : 1][MT][kWave];
+
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  const int unit = blockIdx.x * kUnits + wave / KSPLIT;
+  const int part = wave % KSPLIT;
+  const int r = lane % 16, g = lane / 16;
+  const int k = a.k, m = a.m, n = a.n;
+
+  // rows of the weight this unit multiplies
+  int units, row0, row1 = 0;
+  if (EPI == EPI_STORE) {
+    units = (n + 15) / 16;
+    row0 = unit * 16;
+  } else if (EPI == EPI_SILU) {
+    units = (n / 2 + 15) / 16;
+    row0 = unit * 16;
+    row1 = n / 2 + unit * 16;
+  } else {
+    const int per_head = a.head_dim / 32;
+    units = (a.heads + 2 * a.kv_heads) * per_head;
+    row0 = (unit / per_head) * a.head_dim + (unit % per_head) * 16;
+    row1 = row0 + a.head_dim / 2;
+  }
+  const bool active = unit < units;
+  const int row_limit = EPI == EPI_SILU ? n / 2 : n;  // rows0 beyond this are padding of the last strip
+
+  f32x4 acc[NACC][MT];
+  float ss[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    ss[t] = 0.0f;
+#pragma unroll
+    for (int j = 0; j < NACC; ++j) acc[j][t] = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
+  }
+
+  if (active) {
+    int wr0 = row0 + r, wr1 = row1 + r;
+    wr0 = wr0 < row_limit ? wr0 : row_limit - 1;
+    wr1 = wr1 < n ? wr1 : n - 1;
+    const bf16_t* w0 = a.w + (size_t)wr0 * k;
+    const bf16_t* w1 = a.w + (size_t)wr1 * k;
+    size_t x_row[MT];
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+      int token = t * 16 + r;
+      token = token < m ? token : m - 1;
+      x_row[t] = (size_t)token * k;
+    }
+    const bool writes_x = a.delta != nullptr && unit == 0;  // the first unit's waves cover every k once
+    const int chunks = (k + 63) / 64;
+    for (int chunk = part; chunk < chunks; chunk += KSPLIT) {
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        // A matrix instruction runs for the whole wave whatever lanes a branch
+        // has switched off: a lane whose 8 k lie beyond K feeds it zeros, it
+        // never skips it.  K is a multiple of 8: a group is whole or absent.
+        const int kk = chunk * 64 + g * 16 + half * 8;
+        const bool in = kk + 8 <= k;
+        const bf16x8 wa = in ? *(const bf16x8*)(w0 + kk) : zero8();
+        const bf16x8 wb = (PAIR && in) ? *(const bf16x8*)(w1 + kk) : zero8();
+        float gain[8];
+        if (in) {
+          load_gain8(a.norm_w, a.norm_w_dtype, kk, gain);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) gain[e] = 0.0f;
+        }
+#pragma unroll
+        for (int t = 0; t < MT; ++t) {
+          float v[8];
+#pragma unroll
+          for (int e = 0; e < 8; ++e) v[e] = 0.0f;
+          if (in) {
+            const f32x4 xa = *(const f32x4*)(a.x_in + x_row[t] + kk);
+            const f32x4 xb = *(const f32x4*)(a.x_in + x_row[t] + kk + 4);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              v[e] = xa[e];
+              v[4 + e] = xb[e];
+            }
+            if (a.delta) {
+              const bf16x8 d = *(const bf16x8*)(a.delta + x_row[t] + kk);
+#pragma unroll
+              for (int e = 0; e < 8; ++e) v[e] += (float)d[e];
+              if (writes_x && t * 16 + r < m) {
+                *(f32x4*)(a.x_out + x_row[t] + kk) = (f32x4){v[0], v[1], v[2], v[3]};
+                *(f32x4*)(a.x_out + x_row[t] + kk + 4) = (f32x4){v[4], v[5], v[6], v[7]};
+              }
+            }
+          }
+          bf16x8 operand;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            ss[t] = fmaf(v[e], v[e], ss[t]);
+            operand[e] = (__bf16)(v[e] * gain[e]);
+          }
+          acc[0][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa, operand, acc[0][t], 0, 0, 0);
+          if (PAIR) acc[1][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wb, operand, acc[1][t], 0, 0, 0);
+        }
+      }
+    }
+  }
+  // a token's sum of squares: over the four lane groups of this wave, then over the waves that share K
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    ss[t] += __shfl_xor(ss[t], 16, kWave);
+    ss[t] += __shfl_xor(ss[t], 32, kWave);
+  }
+  if constexpr (KSPLIT > 1) {
+    if (part != 0) {
+#pragma unroll
+      for (int t = 0; t < MT; ++t) {
+        part_ss[wave][t][lane] = ss[t];
+#pragma unroll
+        for (int j = 0; j < NACC; ++j)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) part_acc[wave][j][t][lane][e] = acc[j][t][e];
+      }
+    }
+    __syncthreads();
+    if (part != 0) return;
+#pragma unroll
+    for (int other = 1; other < KSPLIT; ++other)
+#pragma unroll
+      for (int t = 0; t < MT; ++t) {
+        ss[t] += part_ss[wave + other][t][lane];
+#pragma unroll
+        for (int j = 0; j < NACC; ++j)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) acc[j][t][e] += part_acc[wave + other][j][t][lane][e];
+      }
+  }
+  if (!active) return;
+
+  // lane holds D[row 4g + e][token r] of each strip
+  const float inv_k = 1.0f / (float)k;
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    const int token = t * 16 + r;
+    if (token >= m) continue;
+    const float scale = 1.0f / sqrtf(ss[t] * inv_k + a.eps);
+    if (EPI == EPI_STORE) {
+      const int n0 = row0 + g * 4;
+      for (int e = 0; e < 4; ++e)
+        if (n0 + e < n) a.y[(size_t)token * n + n0 + e] = (bf16_t)(acc[0][t][e] * scale);
+    } else if (EPI == EPI_SILU) {
+      const int inner = n / 2;
+      const int n0 = row0 + g * 4;
+      for (int e = 0; e < 4; ++e) {
+        if (n0 + e >= inner) continue;
+        const float gate = acc[0][t][e] * scale, up = acc[1][t][e] * scale;
+        a.y[(size_t)token * inner + n0 + e] = (bf16_t)(gate / (1.0f + expf(-gate)) * up);
+      }
+    } else {
+      const int hd = a.head_dim, half = hd / 2;
+      const int head = row0 / hd;
+      const int f0 = row0 % hd + g * 4;  // feature in the lower half; its partner is f0 + half
+      const int slot = a.tok_slot[token];
+      const int pos = a.tok_pos[token];
+      float lo[4], hi[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        lo[e] = acc[0][t][e] * scale;
+        hi[e] = acc[1][t][e] * scale;
+      }
+      if (head < a.heads + a.kv_heads) {  // queries and keys rotate
+        const f32x4 c = *(const f32x4*)(a.cos_table + (size_t)pos * half + f0);
+        const f32x4 s = *(const f32x4*)(a.sin_table + (size_t)pos * half + f0);
+        bf16x4 out_lo, out_hi;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          out_lo[e] = (__bf16)(lo[e] * c[e] - hi[e] * s[e]);
+          out_hi[e] = (__bf16)(hi[e] * c[e] + lo[e] * s[e]);
+        }
+        if (head < a.heads) {
+          bf16_t* dst = a.y + ((size_t)token * a.heads + head) * hd;
+          *(bf16x4*)(dst + f0) = out_lo;
+          *(bf16x4*)(dst + f0 + half) = out_hi;
+        } else if (slot >= 0 && a.k_pages) {
+          const int page = a.block_table[(size_t)slot * a.max_pages + pos / kPageTokens];
+          bf16_t* dst = a.k_pages + (((size_t)page * a.kv_heads + (head - a.heads)) * kPageTokens + pos % kPageTokens) * hd;
+          *(bf16x4*)(dst + f0) = out_lo;
+          *(bf16x4*)(dst + f0 + half) = out_hi;
+        }
+      } else if (slot >= 0 && a.v_pages) {  // values are stored as they are, keys contiguous per channel
+        const int page = a.block_table[(size_t)slot * a.max_pages + pos / kPageTokens];
+        bf16_t* dst = a.v_pages + ((size_t)page * a.kv_heads + (head - a.heads - a.kv_heads)) * hd * kPageTokens +
+                      pos % kPageTokens;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          dst[(size_t)(f0 + e) * kPageTokens] = (bf16_t)lo[e];
+          dst[(size_t)(f0 + half + e) * kPageTokens] = (bf16_t)hi[e];
+        }
+      }
+    }
+  }
+}
+
+template <int MT, int KSPLIT, int EPI>
+void launch_fused(const FusedArgs& a, int units, hipStream_t stream) {
+  constexpr int kWaves = KSPLIT > 4 ? KSPLIT : 4;
+  constexpr int kUnits = kWaves / KSPLIT;
+  hipLaunchKernelGGL((gemm_fused_kernel<MT, KSPLIT, EPI>), dim3((units + kUnits - 1) / kUnits), dim3(64 * kWaves), 0,
+                     stream, a);
+}
+
+template <int MT, int EPI>
+void dispatch_fused_split(const FusedArgs& a, int units, int split, hipStream_t stream) {
+  if (split == 8 && MT <= 2) launch_fused<MT, (MT <= 2 ? 8 : 4), EPI>(a, units, stream);
+  else if (split >= 4) launch_fused<MT, 4, EPI>(a, units, stream);
+  else if (split == 2) launch_fused<MT, 2, EPI>(a, units, stream);
+  else launch_fused<MT, 1, EPI>(a, units, stream);
+}
+
+template <int EPI>
+void dispatch_fused(const FusedArgs& a, int units, int split, hipStream_t stream) {
+  const int tiles = (a.m + 15) / 16;
+  if (tiles == 1) dispatch_fused_split<1, EPI>(a, units, split, stream);
+  else if (tiles == 2) dispatch_fused_split<2, EPI>(a, units, split, stream);
+  else if (tiles == 3) dispatch_fused_split<3, EPI>(a, units, split, stream);
+  else dispatch_fused_split<4, EPI>(a, units, split, stream);
+}
+
+}  // namespace
+
+// epilogue: 0 store [m, n]; 1 SiLU(gate) * up -> [m, n / 2] (gate rows first); 2 RoPE + cache write,
+// queries -> y [m, heads * head_dim].  delta may be null (then x_out is not written).
+extern "C" int nnis_gemm_fused(const float* x_in, const void* delta, float* x_out, const void* norm_w, int norm_w_dtype,
+                               float eps, const void* w, int m, int n, int k, int epilogue, void* y, const float* cos_table,
+                               const float* sin_table, int table_positions, const int* tok_slot, const int* tok_pos,
+                               void* k_pages, void* v_pages, const int* block_table, int max_pages, int heads, int kv_heads,
+                               int head_dim, void* stream_ptr) {
+  NNIS_REQUIRE(m > 0 && m <= 64, "gemm_fused: takes 1 to 64 tokens, got %d", m);
+  NNIS_REQUIRE(n > 0 && k > 0 && k % 8 == 0, "gemm_fused: bad sizes n=%d k=%d (K must be a multiple of 8)", n, k);
+  NNIS_REQUIRE(nnis_dtype_ok(norm_w_dtype), "gemm_fused: unknown norm weight dtype %d", norm_w_dtype);
+  NNIS_REQUIRE(eps > 0.0f, "gemm_fused: eps must be positive");
+  NNIS_REQUIRE(delta == nullptr || x_out != nullptr, "gemm_fused: a pending sum needs a place for the new residual");
+  NNIS_REQUIRE(x_out != x_in, "gemm_fused: the new residual must not overwrite the one being read");
+  for (const void* p : {(const void*)x_in, delta, (const void*)x_out, norm_w, w, (const void*)y})
+    NNIS_REQUIRE((uintptr_t)p % 16 == 0, "gemm_fused: operands must be 16-byte aligned");
+  FusedArgs a;
+  a.x_in = x_in; a.delta = (const bf16_t*)delta; a.x_out = x_out; a.norm_w = norm_w; a.norm_w_dtype = norm_w_dtype;
+  a.eps = eps; a.w = (const bf16_t*)w; a.m = m; a.n = n; a.k = k; a.y = (bf16_t*)y;
+  a.cos_table = cos_table; a.sin_table = sin_table; a.tok_slot = tok_slot; a.tok_pos = tok_pos;
+  a.k_pages = (bf16_t*)k_pages; a.v_pages = (bf16_t*)v_pages; a.block_table = block_table; a.max_pages = max_pages;
+  a.heads = heads; a.kv_heads = kv_heads; a.head_dim = head_dim;
+  int units;
+  if (epilogue == EPI_STORE) {
+    units = (n + 15) / 16;
+  } else if (epilogue == EPI_SILU) {
+    NNIS_REQUIRE(n % 2 == 0, "gemm_fused: gate and up rows must be as many (n=%d)", n);
+    units = (n / 2 + 15) / 16;
+  } else if (epilogue == EPI_ROPE) {
+    NNIS_REQUIRE(heads > 0 && kv_heads > 0 && head_dim > 0 && head_dim % 32 == 0,
+                 "gemm_fused: the rotating epilogue needs a head size in steps of 32, got %d", head_dim);
+    NNIS_REQUIRE(n == (heads + 2 * kv_heads) * head_dim, "gemm_fused: %d weight rows for %d+2*%d heads of %d", n, heads,
+                 kv_heads, head_dim);
+    NNIS_REQUIRE(cos_table && sin_table && tok_slot && tok_pos, "gemm_fused: the rotating epilogue needs tables and positions");
+    NNIS_REQUIRE((k_pages == nullptr) == (v_pages == nullptr), "gemm_fused: key and value pages must come together");
+    NNIS_REQUIRE(k_pages == nullptr || (block_table && max_pages > 0), "gemm_fused: cache without a block table");
+    NNIS_REQUIRE(table_positions > 0, "gemm_fused: empty rotation tables");
+    units = (heads + 2 * kv_heads) * (head_dim / 32);
+  } else {
+    return nnis_fail("gemm_fused: unknown epilogue %d", epilogue);
+  }
+  // few units: their waves share K so that each wave's share is a step or two of 64
+  const int chunks = (k + 63) / 64;
+  int split = 1;
+  if (units < 2048) {
+    while (split < 8 && chunks > split * 2) split *= 2;
+  }
+  hipStream_t stream = (hipStream_t)stream_ptr;
+  if (epilogue == EPI_STORE) dispatch_fused<EPI_STORE>(a, units, split, stream);
+  else if (epilogue == EPI_SILU) dispatch_fused<EPI_SILU>(a, units, split, stream);
+  else dispatch_fused<EPI_ROPE>(a, units, split, stream);
+  NNIS_LAUNCH_CHECK("gemm_fused");
+  return 0;
+}

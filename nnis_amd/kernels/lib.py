@@ -42,7 +42,7 @@ FLAGS = [
     "-Wno-unused-command-line-argument",
 ]
 HEADERS = ["common.h"]
-CORE_SOURCES = ["elementwise.hip", "gemm.hip", "gemm_mfma.hip", "sampling.hip"]
+CORE_SOURCES = ["elementwise.hip", "gemm.hip", "gemm_mfma.hip", "gemm_fused.hip", "sampling.hip"]
 ATTENTION_SOURCES = ["attention.hip"]
 PREBUILT_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 112, 128)
 

@@ -29,6 +29,8 @@ _CORE_SIGNATURES = {
     "nnis_argmax": [_VOID, _VOID, _INT, _INT, _VOID],
     "nnis_gemm_ordered": [_VOID, _INT, _VOID, _INT, _VOID, _INT, _INT, _INT, _INT, _VOID],
     "nnis_gemm_bf16": [_VOID, _VOID, _VOID, _INT, _INT, _INT, _INT, _VOID],
+    "nnis_gemm_fused": [_VOID, _VOID, _VOID, _VOID, _INT, _FLT, _VOID, _INT, _INT, _INT, _INT, _VOID, _VOID, _VOID, _INT,
+                        _VOID, _VOID, _VOID, _VOID, _VOID, _INT, _INT, _INT, _INT, _VOID],
     "nnis_sample": [_VOID, _VOID, _INT, _INT, _VOID, _VOID, _VOID, _VOID, _VOID, _VOID, _VOID],
 }
 _ATTN_SIGNATURES = {
@@ -262,6 +264,58 @@ def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tens
     lib = core()
     _check(lib, lib.nnis_gemm_bf16(x.data_ptr(), w.data_ptr(), out.data_ptr(), _code(out), m, n, k, _stream()))
     return out
+
+
+EPILOGUE_STORE, EPILOGUE_SILU, EPILOGUE_ROPE = 0, 1, 2
+FUSED_MAX_TOKENS = 16  # beyond a tile of 16 tokens every wave re-reads too much of x: the separate kernels win
+
+
+def gemm_fused(x_in: torch.Tensor, delta: Optional[torch.Tensor], x_out: Optional[torch.Tensor], norm_weight: torch.Tensor,
+               eps: float, w: torch.Tensor, y: torch.Tensor, epilogue: int = EPILOGUE_STORE, rope: Optional[dict] = None):
+    """y = epilogue( W . rmsnorm(x_in + delta) ) for up to 64 tokens, in one
+    kernel; ``x_out`` receives x_in + delta.  ``epilogue``: store; SiLU(gate) *
+    up for a weight of gate rows followed by up rows; or rotate-half RoPE with
+    the write of keys and values into the cache (``rope``: cos, sin, tok_slot,
+    tok_pos, k_pages, v_pages, block_table, heads, kv_heads, head_dim)."""
+    m, k = x_in.shape
+    n = w.shape[0]
+    _dev(x_in, "x"), _dev(norm_weight, "norm weight"), _dev(w, "weight"), _dev(y, "y")
+    if x_in.dtype != torch.float32 or w.dtype != torch.bfloat16 or y.dtype != torch.bfloat16 or w.shape[1] != k:
+        raise KernelError("gemm_fused: x must be float32 [m, k], the weight bfloat16 [n, k] and y bfloat16")
+    if norm_weight.numel() != k:
+        raise KernelError(f"gemm_fused: norm weight of {norm_weight.numel()} for width {k}")
+    if delta is not None:
+        _dev(delta, "delta"), _dev(x_out, "x_out")
+        if delta.shape != x_in.shape or delta.dtype != torch.bfloat16 or x_out.shape != x_in.shape or x_out.dtype != torch.float32:
+            raise KernelError("gemm_fused: delta must be bfloat16 and x_out float32, both shaped like x")
+    expect = {EPILOGUE_STORE: (m, n), EPILOGUE_SILU: (m, n // 2)}.get(epilogue)
+    r = rope or {}
+    if epilogue == EPILOGUE_ROPE:
+        expect = (m, r["heads"] * r["head_dim"])
+        for name in ("cos", "sin", "tok_slot", "tok_pos"):
+            _dev(r[name], name)
+        if r["cos"].dtype != torch.float32 or r["cos"].shape != r["sin"].shape or r["cos"].shape[1] != r["head_dim"] // 2:
+            raise KernelError("gemm_fused: rotation tables must be float32 [positions, head_dim / 2]")
+        if r["tok_slot"].dtype != torch.int32 or r["tok_pos"].dtype != torch.int32 or min(r["tok_slot"].numel(), r["tok_pos"].numel()) < m:
+            raise KernelError("gemm_fused: tok_slot / tok_pos must be int32 with one entry per token")
+        if r.get("k_pages") is not None:
+            kp, vp, bt = r["k_pages"], r["v_pages"], r["block_table"]
+            _dev(kp, "k_pages"), _dev(vp, "v_pages"), _dev(bt, "block_table")
+            if (kp.dtype != torch.bfloat16 or vp.dtype != torch.bfloat16 or bt.dtype != torch.int32
+                    or tuple(kp.shape[1:]) != (r["kv_heads"], PAGE_TOKENS, r["head_dim"])
+                    or tuple(vp.shape[1:]) != (r["kv_heads"], r["head_dim"], PAGE_TOKENS)):
+                raise KernelError("gemm_fused: cache pages must be bfloat16 in the cache's layout, the block table int32")
+    if expect is None or tuple(y.shape) != expect:
+        raise KernelError(f"gemm_fused: y {tuple(y.shape)} does not fit epilogue {epilogue} (expected {expect})")
+    lib = core()
+    bt = r.get("block_table")
+    _check(lib, lib.nnis_gemm_fused(
+        x_in.data_ptr(), _ptr(delta), _ptr(x_out) if delta is not None else None, norm_weight.data_ptr(), _code(norm_weight),
+        float(eps), w.data_ptr(), m, n, k, int(epilogue), y.data_ptr(), _ptr(r.get("cos")), _ptr(r.get("sin")),
+        r["cos"].shape[0] if r.get("cos") is not None else 0, _ptr(r.get("tok_slot")), _ptr(r.get("tok_pos")),
+        _ptr(r.get("k_pages")), _ptr(r.get("v_pages")), _ptr(bt), bt.shape[1] if bt is not None else 0,
+        r.get("heads", 0), r.get("kv_heads", 0), r.get("head_dim", 0), _stream()))
+    return y
 
 
 def _mfma_ok(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> bool:

@@ -55,12 +55,28 @@ class CausalSelfAttention(Mixer):
     def cache_request(self):
         return KVRequest(self.kv_heads, self.head_dim, self.window)
 
-    def forward(self, x, ctx, view, rt):
+    takes_pending_norm = True
+
+    def _project_rotate_store(self, x, ctx, view, rt):
+        """Queries [tokens, heads * head_dim], rotated; keys and values of the
+        step's tokens in the cache."""
+        from .lazy import PendingNorm
+
+        tables = self.position.rotary() if self.position is not None else None
+        writes = not view.read_only
+        if isinstance(x, PendingNorm):
+            if (x.can_fuse(self.qkv.weight) and tables is not None and tables.rot_dim == self.head_dim
+                    and self.head_dim % 32 == 0 and view.k_pages.dtype == torch.bfloat16):
+                # residual sum, norm, the three projections, the rotation and the cache write in one kernel
+                rope = dict(cos=tables.cos, sin=tables.sin, tok_slot=ctx.tok_slot, tok_pos=ctx.tok_pos,
+                            k_pages=view.k_pages if writes else None, v_pages=view.v_pages if writes else None,
+                            block_table=view.block_table if writes else None, heads=self.heads,
+                            kv_heads=self.kv_heads, head_dim=self.head_dim)
+                return x.fused(self.qkv.weight, rt.empty(x.rows, self.heads * self.head_dim), rt.ops.EPILOGUE_ROPE, rope)
+            x = x.materialize()
         tokens = x.shape[0]
         qkv = self.qkv(x, rt)
         q = rt.empty(tokens, self.heads * self.head_dim)
-        tables = self.position.rotary() if self.position is not None else None
-        writes = not view.read_only
         rt.ops.rope_kv_write(
             qkv, q,
             tables.cos if tables else None, tables.sin if tables else None, tables.rot_dim if tables else 0,
@@ -68,6 +84,11 @@ class CausalSelfAttention(Mixer):
             view.k_pages if writes else None, view.v_pages if writes else None, view.block_table if writes else None,
             self.heads, self.kv_heads, self.head_dim,
         )
+        return q
+
+    def forward(self, x, ctx, view, rt):
+        q = self._project_rotate_store(x, ctx, view, rt)
+        tokens = q.shape[0]
         attn = rt.empty(tokens, self.heads * self.head_dim)
         rt.ops.attention(q, attn, view, ctx, self.heads, self.kv_heads, self.head_dim, self.scale, self.window or 0)
         return self.out(attn, rt)

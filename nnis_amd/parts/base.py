@@ -23,9 +23,12 @@ The interfaces:
     in the schedule (``KVRequest``, ``StateRequest`` or ``None``);
     ``forward(x, ctx, view, rt)`` -> y, where ``x`` is ``[tokens, width]`` in
     the activation type, ``ctx`` is the step's ``StepContext`` and ``view``
-    is the cache's view for this schedule entry.
+    is the cache's view for this schedule entry.  A mixer that sets
+    ``takes_pending_norm = True`` is handed a ``PendingNorm`` instead of ``x``
+    and must consume it (``materialize()`` or ``fused(...)``).
 ``FeedForward``
-    ``forward(x, ctx, rt)`` -> y, row-wise over the packed tokens.
+    ``forward(x, ctx, rt)`` -> y, row-wise over the packed tokens; the same
+    ``takes_pending_norm`` option.
 ``Block``
     ``forward(stream, ctx, view, rt)`` -> stream; the block owns the
     arrangement of norm, mixer and feed-forward around the residual stream.
@@ -103,6 +106,12 @@ class Norm(Part):
 
     def add_forward(self, residual, delta, rt, rows=None):
         raise NotImplementedError
+
+    def defer(self, x, delta, rt):
+        """The norm of x (+ delta) as a value not computed yet; see ``PendingNorm``."""
+        from .lazy import PendingNorm
+
+        return PendingNorm(self, x, delta, rt)
 
 
 @dataclass

@@ -4,7 +4,9 @@ x += mixer(norm1(x)); x += feed_forward(norm2(x))
 
 The residual stream is kept in 32-bit as a pair (x, pending): ``pending`` is a
 part's output not yet added.  The sum is taken by the next norm in the same
-kernel that normalises, so the stream is read and written once per part.
+kernel that normalises, and a mixer or feed-forward that starts with a
+projection may take sum and norm into that projection's kernel
+(``PendingNorm``), so the stream is read and written once per part.
 """
 
 from __future__ import annotations
@@ -37,10 +39,17 @@ class PreNormBlock(Block):
 
     def forward(self, stream, ctx, view, rt):
         x, pending = stream
-        normed = self.norm1.forward(x, rt) if pending is None else self.norm1.add_forward(x, pending, rt)
-        mixed = self.mixer.forward(normed, ctx, view, rt)
-        normed = self.norm2.add_forward(x, mixed, rt)
-        return x, self.feed_forward.forward(normed, ctx, rt)
+        normed = self.norm1.defer(x, pending, rt)
+        if getattr(self.mixer, "takes_pending_norm", False):
+            mixed = self.mixer.forward(normed, ctx, view, rt)
+        else:
+            mixed = self.mixer.forward(normed.materialize(), ctx, view, rt)
+        normed = self.norm2.defer(normed.residual, mixed, rt)
+        if getattr(self.feed_forward, "takes_pending_norm", False):
+            out = self.feed_forward.forward(normed, ctx, rt)
+        else:
+            out = self.feed_forward.forward(normed.materialize(), ctx, rt)
+        return normed.residual, out
 
 
 register_part("block", "pre_norm", PreNormBlock)

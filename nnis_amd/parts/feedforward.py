@@ -37,7 +37,17 @@ class GatedFeedForward(FeedForward):
     def weight_bytes(self):
         return self.gate_up.weight_bytes() + self.down.weight_bytes()
 
+    takes_pending_norm = True
+
     def forward(self, x, ctx, rt):
+        from .lazy import PendingNorm
+
+        if isinstance(x, PendingNorm):
+            if x.can_fuse(self.gate_up.weight):
+                # residual sum, norm, both projections and the gating in one kernel
+                hidden = x.fused(self.gate_up.weight, rt.empty(x.rows, self.inner), rt.ops.EPILOGUE_SILU)
+                return self.down(hidden, rt)
+            x = x.materialize()
         gate_up = self.gate_up(x, rt)
         hidden = rt.ops.silu_mul(gate_up, rt.empty(x.shape[0], self.inner))
         return self.down(hidden, rt)

@@ -8,6 +8,7 @@ from .base import Norm, TensorSpec, register_part
 
 class RMSNorm(Norm):
     graph_safe = True
+    fusable_rms = True  # ``weight`` and ``eps`` are all a projection kernel needs to apply this norm itself
 
     def __init__(self, width: int, eps: float, weight: str):
         self.width = int(width)

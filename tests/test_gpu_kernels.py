@@ -208,6 +208,72 @@ def test_prefill_attention_on_the_matrix_cores(heads, kv_heads, head_dim):
             assert (got[100, 0] - vs[2][17, 0]).abs().max().item() < 0.05
 
 
+@pytest.mark.parametrize("m", [1, 8, 16, 17, 40, 64])
+@pytest.mark.parametrize("k", [64, 96, 576, 1096])
+@pytest.mark.parametrize("with_delta", [False, True])
+@pytest.mark.parametrize("gain_dtype", ["bfloat16", "float32"])
+def test_fused_norm_projection(m, k, with_delta, gain_dtype):
+    """Residual sum + RMSNorm + projection in one kernel, with each epilogue,
+    against the plain functions one after another."""
+    ops = _ops()
+    torch.manual_seed(m * 7 + k)
+    eps = 2e-5
+    x = torch.randn(m, k) * 2
+    delta = torch.randn(m, k).bfloat16() if with_delta else None
+    gain = (1 + 0.3 * torch.randn(k)).to(DT[gain_dtype])
+    summed = x + (delta.float() if with_delta else 0)
+    normed = P.rms_norm(summed.double(), gain.double(), eps)
+
+    def run(w, y, epilogue, rope=None):
+        x_out = torch.full((m, k), 9.0, device="cuda") if with_delta else None
+        ops.gemm_fused(x.cuda(), delta.cuda() if with_delta else None, x_out, gain.cuda(), eps, w.cuda(), y, epilogue, rope)
+        if with_delta:
+            assert torch.equal(x_out.cpu(), summed)  # the residual sum, exactly, written once
+        return y.cpu().double()
+
+    def close(got, want, what):
+        assert ((got - want).abs() <= 2e-2 * (1 + want.abs())).all(), (what, (got - want).abs().max().item())
+
+    # store, with a ragged last strip
+    n = 70
+    w = (torch.randn(n, k) / math.sqrt(k)).bfloat16()
+    close(run(w, torch.empty(m, n, dtype=torch.bfloat16, device="cuda"), ops.EPILOGUE_STORE), normed @ w.double().t(), "store")
+    # gate rows, then up rows
+    inner = 88
+    w = (torch.randn(2 * inner, k) / math.sqrt(k)).bfloat16()
+    both = normed @ w.double().t()
+    close(run(w, torch.empty(m, inner, dtype=torch.bfloat16, device="cuda"), ops.EPILOGUE_SILU),
+          P.silu(both[:, :inner]) * both[:, inner:], "silu")
+    # queries, keys, values: rotation and the cache
+    heads, kv_heads, head_dim = 3, 2, 32
+    w = (torch.randn((heads + 2 * kv_heads) * head_dim, k) / math.sqrt(k)).bfloat16()
+    qkv = (normed @ w.double().t()).view(m, heads + 2 * kv_heads, head_dim)
+    cos_np, sin_np = P.rope_tables(512, head_dim, 10000.0)
+    slots = [(i * 5) % 7 - (1 if i % 9 == 4 else 0) * 100 for i in range(m)]  # some padding rows
+    slots = [s if s >= 0 else -1 for s in slots]
+    positions = [(i * 37) % 300 for i in range(m)]
+    table = torch.arange(7 * 5, dtype=torch.int32).view(7, 5).flip(0).contiguous()
+    k_pages = torch.full((35, kv_heads, 64, head_dim), 7.0, dtype=torch.bfloat16, device="cuda")
+    v_pages = torch.full((35, kv_heads, head_dim, 64), 7.0, dtype=torch.bfloat16, device="cuda")
+    rope = dict(cos=torch.from_numpy(cos_np).cuda(), sin=torch.from_numpy(sin_np).cuda(), tok_slot=_i32(slots),
+                tok_pos=_i32(positions), k_pages=k_pages, v_pages=v_pages, block_table=table.cuda(), heads=heads,
+                kv_heads=kv_heads, head_dim=head_dim)
+    got_q = run(w, torch.empty(m, heads * head_dim, dtype=torch.bfloat16, device="cuda"), ops.EPILOGUE_ROPE, rope)
+    pos = torch.tensor(positions)
+    turned = P.rope_rotate_half(qkv[:, :heads + kv_heads], torch.from_numpy(cos_np)[pos].double(), torch.from_numpy(sin_np)[pos].double())
+    close(got_q.view(m, heads, head_dim), turned[:, :heads], "queries")
+    seen = {}
+    for t in range(m):  # a later token of the same slot and position overwrites an earlier one
+        if slots[t] >= 0:
+            seen[(slots[t], positions[t])] = t
+    for (slot, position), t in seen.items():
+        page, inside = table[slot, position // 64].item(), position % 64
+        close(k_pages[page, :, inside, :].cpu().double(), turned[t, heads:], "keys")
+        close(v_pages[page, :, :, inside].cpu().double(), qkv[t, heads + kv_heads:], "values")
+    written = sum(1 for _ in seen)
+    assert int((k_pages.cpu().float() != 7.0).any(dim=-1).sum()) <= written * kv_heads
+
+
 def _paged(k_seqs, v_seqs, dtype, kv_heads, head_dim, page_order=None, pages=32, max_pages=12):
     """Lays sequences out in pages the way the cache does.  k_seqs[i]: [len, kv_heads, head_dim]."""
     k_pages = torch.full((pages, kv_heads, 64, head_dim), 77.0, dtype=dtype)
