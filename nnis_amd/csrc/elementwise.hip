@@ -278,6 +278,68 @@ __global__ void rope_kv_write_kernel(RopeWriteArgs a) {
   }
 }
 
+// The same for bfloat16 throughout with rot_dim / 2 and head_dim - rot_dim multiples of 4: a
+// thread takes 4 consecutive pairs (or 4 pass-through or value channels), 8- and 16-byte accesses.
+__global__ void rope_kv_write_bf16_kernel(RopeWriteArgs a) {
+  const int token = blockIdx.x;
+  const int slot = a.tok_slot[token];
+  if (slot < 0) return;
+  const int pos = a.tok_pos[token];
+  const int hd = a.head_dim;
+  const int half = a.rot_dim / 2;
+  const int row_width = (a.heads + 2 * a.kv_heads) * hd;
+  const bf16_t* src = (const bf16_t*)a.qkv + (size_t)token * row_width;
+  const bool rotate = a.cos_table != nullptr && pos < a.table_positions;
+  int page = -1;
+  if (a.k_pages) page = a.block_table[(size_t)slot * a.max_pages + pos / kPageTokens];
+  const int in_page = pos % kPageTokens;
+  const int rot_heads = a.heads + a.kv_heads;
+  const int groups_per_head = (hd - half) / 4;  // half/4 groups of pairs, then (hd - rot_dim)/4 pass-through groups
+  const int rot_items = rot_heads * groups_per_head;
+  const int v_items = page >= 0 ? a.kv_heads * (hd / 4) : 0;
+  for (int item = threadIdx.x; item < rot_items + v_items; item += blockDim.x) {
+    if (item < rot_items) {
+      const int head = item / groups_per_head;
+      const int e = (item % groups_per_head) * 4;
+      bf16_t* dst;
+      if (head < a.heads) {
+        dst = (bf16_t*)a.q_out + ((size_t)token * a.heads + head) * hd;
+      } else {
+        if (page < 0) continue;
+        dst = (bf16_t*)a.k_pages + (((size_t)page * a.kv_heads + (head - a.heads)) * kPageTokens + in_page) * hd;
+      }
+      const bf16_t* x = src + (size_t)head * hd;
+      if (e < half) {
+        const bf16x4_t x0 = *(const bf16x4_t*)(x + e), x1 = *(const bf16x4_t*)(x + e + half);
+        f32x4_t c = {1.0f, 1.0f, 1.0f, 1.0f}, sn = {0.0f, 0.0f, 0.0f, 0.0f};
+        if (rotate) {
+          c = *(const f32x4_t*)(a.cos_table + (size_t)pos * half + e);
+          sn = *(const f32x4_t*)(a.sin_table + (size_t)pos * half + e);
+        }
+        bf16x4_t lo, hi;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float f0 = (float)x0[j], f1 = (float)x1[j];
+          lo[j] = (__bf16)(f0 * c[j] - f1 * sn[j]);
+          hi[j] = (__bf16)(f1 * c[j] + f0 * sn[j]);
+        }
+        *(bf16x4_t*)(dst + e) = lo;
+        *(bf16x4_t*)(dst + e + half) = hi;
+      } else {
+        *(bf16x4_t*)(dst + e + half) = *(const bf16x4_t*)(x + e + half);  // channels at and beyond rot_dim
+      }
+    } else {
+      const int v_item = item - rot_items;
+      const int kv_head = v_item / (hd / 4);
+      const int d = (v_item % (hd / 4)) * 4;
+      const bf16x4_t v = *(const bf16x4_t*)(src + (size_t)(a.heads + a.kv_heads + kv_head) * hd + d);
+      bf16_t* dst = (bf16_t*)a.v_pages + (((size_t)page * a.kv_heads + kv_head) * hd + d) * kPageTokens + in_page;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) dst[(size_t)j * kPageTokens] = v[j];
+    }
+  }
+}
+
 extern "C" int nnis_rope_kv_write(const void* qkv, int qkv_dtype, void* q_out, int q_dtype, const float* cos_table,
                                   const float* sin_table, int table_positions, int rot_dim, const int* tok_slot,
                                   const int* tok_pos, void* k_pages, void* v_pages, int cache_dtype,
@@ -299,6 +361,16 @@ extern "C" int nnis_rope_kv_write(const void* qkv, int qkv_dtype, void* q_out, i
   a.tok_slot = tok_slot; a.tok_pos = tok_pos; a.k_pages = k_pages; a.v_pages = v_pages;
   a.cache_dtype = cache_dtype; a.block_table = block_table; a.max_pages = max_pages;
   a.heads = heads; a.kv_heads = kv_heads; a.head_dim = head_dim;
+  const bool all_bf16 = qkv_dtype == NNIS_BF16 && q_dtype == NNIS_BF16 && (k_pages == nullptr || cache_dtype == NNIS_BF16);
+  const bool aligned = ((uintptr_t)qkv % 16 == 0) && ((uintptr_t)q_out % 16 == 0) && ((uintptr_t)k_pages % 16 == 0) &&
+                       ((uintptr_t)v_pages % 16 == 0) && ((uintptr_t)cos_table % 16 == 0) && ((uintptr_t)sin_table % 16 == 0);
+  if (all_bf16 && aligned && head_dim % 4 == 0 && (a.rot_dim / 2) % 4 == 0) {
+    const int items = (heads + kv_heads) * (head_dim - a.rot_dim / 2) / 4 + kv_heads * head_dim / 4;
+    const int threads = items > 128 ? 256 : (items > 64 ? 128 : 64);
+    hipLaunchKernelGGL(rope_kv_write_bf16_kernel, dim3(tokens), dim3(threads), 0, (hipStream_t)stream, a);
+    NNIS_LAUNCH_CHECK("rope_kv_write_bf16");
+    return 0;
+  }
   const int work = (heads + 2 * kv_heads) * head_dim / 2;
   const int threads = work >= 512 ? 256 : (work >= 128 ? 128 : 64);
   hipLaunchKernelGGL(rope_kv_write_kernel, dim3(tokens), dim3(threads), 0, (hipStream_t)stream, a);
@@ -323,11 +395,41 @@ __global__ void silu_mul_kernel(const void* __restrict__ gate_up, int in_dtype, 
   }
 }
 
+// the same on bfloat16 rows whose width is a multiple of 8: 16-byte accesses, 8 channels a thread
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+
+__global__ void silu_mul_bf16_kernel(const bf16_t* __restrict__ gate_up, bf16_t* __restrict__ out, int inner, size_t groups) {
+  const int per_row = inner / 8;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < groups; i += (size_t)gridDim.x * blockDim.x) {
+    const size_t row = i / per_row;
+    const int col = (int)(i % per_row) * 8;
+    const bf16x8_t g = *(const bf16x8_t*)(gate_up + row * 2 * inner + col);
+    const bf16x8_t u = *(const bf16x8_t*)(gate_up + row * 2 * inner + inner + col);
+    bf16x8_t y;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float gate = (float)g[e];
+      y[e] = (__bf16)(gate / (1.0f + expf(-gate)) * (float)u[e]);
+    }
+    *(bf16x8_t*)(out + row * inner + col) = y;
+  }
+}
+
 extern "C" int nnis_silu_mul(const void* gate_up, int in_dtype, void* out, int out_dtype, int tokens, int inner,
                              void* stream) {
   NNIS_REQUIRE(nnis_dtype_ok(in_dtype) && nnis_dtype_ok(out_dtype), "silu_mul: unknown dtype");
   NNIS_REQUIRE(tokens >= 0 && inner > 0, "silu_mul: bad sizes tokens=%d inner=%d", tokens, inner);
   if (tokens == 0) return 0;
+  if (in_dtype == NNIS_BF16 && out_dtype == NNIS_BF16 && inner % 8 == 0 && (uintptr_t)gate_up % 16 == 0 &&
+      (uintptr_t)out % 16 == 0) {
+    const size_t groups = (size_t)tokens * (inner / 8);
+    size_t blocks = (groups + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    hipLaunchKernelGGL(silu_mul_bf16_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                       (const bf16_t*)gate_up, (bf16_t*)out, inner, groups);
+    NNIS_LAUNCH_CHECK("silu_mul_bf16");
+    return 0;
+  }
   const size_t total = (size_t)tokens * inner;
   size_t blocks = (total + 255) / 256;
   if (blocks > 65536) blocks = 65536;

@@ -80,6 +80,7 @@ __global__ __launch_bounds__(KSPLIT > 4 ? 64 * KSPLIT : 256) void gemm_fused_ker
   constexpr int NACC = PAIR ? 2 : 1;
   constexpr int kWaves = KSPLIT > 4 ? KSPLIT : 4;
   constexpr int kUnits = kWaves / KSPLIT;  // units per block
+  constexpr int DEPTH = MT == 1 ? 2 : 1;   // steps of 64 k whose loads are in flight together
   __shared__ float part_acc[KSPLIT > 1 ? kWaves : 1][NACC][MT][kWave][4];
   __shared__ float part_ss[KSPLIT > 1 ? kWaves : 1][MT][kWave];
 
@@ -107,6 +108,29 @@ __global__ __launch_bounds__(KSPLIT > 4 ? 64 * KSPLIT : 256) void gemm_fused_ker
   const bool active = unit < units;
   const int row_limit = EPI == EPI_SILU ? n / 2 : n;  // rows0 beyond this are padding of the last strip
 
+  // what the rotating epilogue needs of each token is asked for now, so that it
+  // has arrived when the product is done
+  int tok_slot[MT], tok_pos[MT], tok_page[MT];
+  f32x4 tok_cos[MT], tok_sin[MT];
+  if (EPI == EPI_ROPE && active && part == 0) {
+    const int head = row0 / a.head_dim;
+    const int f0 = row0 % a.head_dim + g * 4;
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+      int token = t * 16 + r;
+      token = token < m ? token : m - 1;
+      tok_slot[t] = a.tok_slot[token];
+      tok_pos[t] = a.tok_pos[token];
+      tok_page[t] = -1;
+      if (head < a.heads + a.kv_heads) {
+        tok_cos[t] = *(const f32x4*)(a.cos_table + (size_t)tok_pos[t] * (a.head_dim / 2) + f0);
+        tok_sin[t] = *(const f32x4*)(a.sin_table + (size_t)tok_pos[t] * (a.head_dim / 2) + f0);
+      }
+      if (head >= a.heads && tok_slot[t] >= 0 && a.k_pages)
+        tok_page[t] = a.block_table[(size_t)tok_slot[t] * a.max_pages + tok_pos[t] / kPageTokens];
+    }
+  }
+
   f32x4 acc[NACC][MT];
   float ss[MT];
 #pragma unroll
@@ -130,57 +154,92 @@ __global__ __launch_bounds__(KSPLIT > 4 ? 64 * KSPLIT : 256) void gemm_fused_ker
       x_row[t] = (size_t)token * k;
     }
     const bool writes_x = a.delta != nullptr && unit == 0;  // the first unit's waves cover every k once
+    const bool gain_f32 = a.norm_w_dtype == NNIS_F32;
     const int chunks = (k + 63) / 64;
-    for (int chunk = part; chunk < chunks; chunk += KSPLIT) {
+    // The product is bound by memory latency: a wave asks for everything its next
+    // DEPTH steps of 64 k need (weights, residual, pending sum, gain) before it
+    // touches any of it, so its share of K is one round trip, not one per step.
+    // A matrix instruction runs for the whole wave whatever lanes a branch has
+    // switched off: a lane whose 8 k lie beyond K feeds it zeros, it never skips
+    // it.  K is a multiple of 8: a group of 8 is whole or absent.
+    for (int base = part; base < chunks; base += KSPLIT * DEPTH) {
+      bf16x8 wa[DEPTH][2], wb[DEPTH][2], dl[DEPTH][2][MT];
+      f32x4 xr[DEPTH][2][MT][2], gr[DEPTH][2][2];
 #pragma unroll
-      for (int half = 0; half < 2; ++half) {
-        // A matrix instruction runs for the whole wave whatever lanes a branch
-        // has switched off: a lane whose 8 k lie beyond K feeds it zeros, it
-        // never skips it.  K is a multiple of 8: a group is whole or absent.
-        const int kk = chunk * 64 + g * 16 + half * 8;
-        const bool in = kk + 8 <= k;
-        const bf16x8 wa = in ? *(const bf16x8*)(w0 + kk) : zero8();
-        const bf16x8 wb = (PAIR && in) ? *(const bf16x8*)(w1 + kk) : zero8();
-        float gain[8];
-        if (in) {
-          load_gain8(a.norm_w, a.norm_w_dtype, kk, gain);
-        } else {
+      for (int d = 0; d < DEPTH; ++d)
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+          const int kk = (base + d * KSPLIT) * 64 + g * 16 + half * 8;
+          const bool in = kk + 8 <= k;
+          wa[d][half] = in ? *(const bf16x8*)(w0 + kk) : zero8();
+          wb[d][half] = (PAIR && in) ? *(const bf16x8*)(w1 + kk) : zero8();
+          if (in) {
+            if (gain_f32) {
+              gr[d][half][0] = *(const f32x4*)((const float*)a.norm_w + kk);
+              gr[d][half][1] = *(const f32x4*)((const float*)a.norm_w + kk + 4);
+            } else {
+              gr[d][half][0] = *(const f32x4*)((const bf16_t*)a.norm_w + kk);  // 8 bfloat16, unpacked below
+            }
+#pragma unroll
+            for (int t = 0; t < MT; ++t) {
+              xr[d][half][t][0] = *(const f32x4*)(a.x_in + x_row[t] + kk);
+              xr[d][half][t][1] = *(const f32x4*)(a.x_in + x_row[t] + kk + 4);
+              if (a.delta) dl[d][half][t] = *(const bf16x8*)(a.delta + x_row[t] + kk);
+            }
+          }
+        }
+#pragma unroll
+      for (int d = 0; d < DEPTH; ++d)
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+          const int kk = (base + d * KSPLIT) * 64 + g * 16 + half * 8;
+          const bool in = kk + 8 <= k;
+          float gain[8];
 #pragma unroll
           for (int e = 0; e < 8; ++e) gain[e] = 0.0f;
-        }
-#pragma unroll
-        for (int t = 0; t < MT; ++t) {
-          float v[8];
-#pragma unroll
-          for (int e = 0; e < 8; ++e) v[e] = 0.0f;
           if (in) {
-            const f32x4 xa = *(const f32x4*)(a.x_in + x_row[t] + kk);
-            const f32x4 xb = *(const f32x4*)(a.x_in + x_row[t] + kk + 4);
+            if (gain_f32) {
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              v[e] = xa[e];
-              v[4 + e] = xb[e];
+              for (int e = 0; e < 4; ++e) {
+                gain[e] = gr[d][half][0][e];
+                gain[4 + e] = gr[d][half][1][e];
+              }
+            } else {
+              const bf16x8 packed = __builtin_bit_cast(bf16x8, gr[d][half][0]);
+#pragma unroll
+              for (int e = 0; e < 8; ++e) gain[e] = (float)packed[e];
             }
-            if (a.delta) {
-              const bf16x8 d = *(const bf16x8*)(a.delta + x_row[t] + kk);
+          }
 #pragma unroll
-              for (int e = 0; e < 8; ++e) v[e] += (float)d[e];
-              if (writes_x && t * 16 + r < m) {
-                *(f32x4*)(a.x_out + x_row[t] + kk) = (f32x4){v[0], v[1], v[2], v[3]};
-                *(f32x4*)(a.x_out + x_row[t] + kk + 4) = (f32x4){v[4], v[5], v[6], v[7]};
+          for (int t = 0; t < MT; ++t) {
+            float v[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[e] = 0.0f;
+            if (in) {
+#pragma unroll
+              for (int e = 0; e < 4; ++e) {
+                v[e] = xr[d][half][t][0][e];
+                v[4 + e] = xr[d][half][t][1][e];
+              }
+              if (a.delta) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) v[e] += (float)dl[d][half][t][e];
+                if (writes_x && t * 16 + r < m) {
+                  *(f32x4*)(a.x_out + x_row[t] + kk) = (f32x4){v[0], v[1], v[2], v[3]};
+                  *(f32x4*)(a.x_out + x_row[t] + kk + 4) = (f32x4){v[4], v[5], v[6], v[7]};
+                }
               }
             }
-          }
-          bf16x8 operand;
+            bf16x8 operand;
 #pragma unroll
-          for (int e = 0; e < 8; ++e) {
-            ss[t] = fmaf(v[e], v[e], ss[t]);
-            operand[e] = (__bf16)(v[e] * gain[e]);
+            for (int e = 0; e < 8; ++e) {
+              ss[t] = fmaf(v[e], v[e], ss[t]);
+              operand[e] = (__bf16)(v[e] * gain[e]);
+            }
+            acc[0][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[d][half], operand, acc[0][t], 0, 0, 0);
+            if (PAIR) acc[1][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wb[d][half], operand, acc[1][t], 0, 0, 0);
           }
-          acc[0][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa, operand, acc[0][t], 0, 0, 0);
-          if (PAIR) acc[1][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wb, operand, acc[1][t], 0, 0, 0);
         }
-      }
     }
   }
   // a token's sum of squares: over the four lane groups of this wave, then over the waves that share K
@@ -238,8 +297,8 @@ __global__ __launch_bounds__(KSPLIT > 4 ? 64 * KSPLIT : 256) void gemm_fused_ker
       const int hd = a.head_dim, half = hd / 2;
       const int head = row0 / hd;
       const int f0 = row0 % hd + g * 4;  // feature in the lower half; its partner is f0 + half
-      const int slot = a.tok_slot[token];
-      const int pos = a.tok_pos[token];
+      const int pos = tok_pos[t];
+      const int page = tok_page[t];
       float lo[4], hi[4];
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
@@ -247,8 +306,7 @@ __global__ __launch_bounds__(KSPLIT > 4 ? 64 * KSPLIT : 256) void gemm_fused_ker
         hi[e] = acc[1][t][e] * scale;
       }
       if (head < a.heads + a.kv_heads) {  // queries and keys rotate
-        const f32x4 c = *(const f32x4*)(a.cos_table + (size_t)pos * half + f0);
-        const f32x4 s = *(const f32x4*)(a.sin_table + (size_t)pos * half + f0);
+        const f32x4 c = tok_cos[t], s = tok_sin[t];
         bf16x4 out_lo, out_hi;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
@@ -259,14 +317,12 @@ __global__ __launch_bounds__(KSPLIT > 4 ? 64 * KSPLIT : 256) void gemm_fused_ker
           bf16_t* dst = a.y + ((size_t)token * a.heads + head) * hd;
           *(bf16x4*)(dst + f0) = out_lo;
           *(bf16x4*)(dst + f0 + half) = out_hi;
-        } else if (slot >= 0 && a.k_pages) {
-          const int page = a.block_table[(size_t)slot * a.max_pages + pos / kPageTokens];
+        } else if (page >= 0) {
           bf16_t* dst = a.k_pages + (((size_t)page * a.kv_heads + (head - a.heads)) * kPageTokens + pos % kPageTokens) * hd;
           *(bf16x4*)(dst + f0) = out_lo;
           *(bf16x4*)(dst + f0 + half) = out_hi;
         }
-      } else if (slot >= 0 && a.v_pages) {  // values are stored as they are, keys contiguous per channel
-        const int page = a.block_table[(size_t)slot * a.max_pages + pos / kPageTokens];
+      } else if (page >= 0) {  // values are stored as they are, keys contiguous per channel
         bf16_t* dst = a.v_pages + ((size_t)page * a.kv_heads + (head - a.heads - a.kv_heads)) * hd * kPageTokens +
                       pos % kPageTokens;
 #pragma unroll
@@ -307,12 +363,13 @@ void dispatch_fused(const FusedArgs& a, int units, int split, hipStream_t stream
 }  // namespace
 
 // epilogue: 0 store [m, n]; 1 SiLU(gate) * up -> [m, n / 2] (gate rows first); 2 RoPE + cache write,
-// queries -> y [m, heads * head_dim].  delta may be null (then x_out is not written).
+// queries -> y [m, heads * head_dim].  delta may be null (then x_out is not written).  split_hint: 0, or the
+// number of waves (1, 2, 4, 8) that share a unit's K, overriding the choice made here.
 extern "C" int nnis_gemm_fused(const float* x_in, const void* delta, float* x_out, const void* norm_w, int norm_w_dtype,
                                float eps, const void* w, int m, int n, int k, int epilogue, void* y, const float* cos_table,
                                const float* sin_table, int table_positions, const int* tok_slot, const int* tok_pos,
                                void* k_pages, void* v_pages, const int* block_table, int max_pages, int heads, int kv_heads,
-                               int head_dim, void* stream_ptr) {
+                               int head_dim, int split_hint, void* stream_ptr) {
   NNIS_REQUIRE(m > 0 && m <= 64, "gemm_fused: takes 1 to 64 tokens, got %d", m);
   NNIS_REQUIRE(n > 0 && k > 0 && k % 8 == 0, "gemm_fused: bad sizes n=%d k=%d (K must be a multiple of 8)", n, k);
   NNIS_REQUIRE(nnis_dtype_ok(norm_w_dtype), "gemm_fused: unknown norm weight dtype %d", norm_w_dtype);
@@ -352,6 +409,7 @@ extern "C" int nnis_gemm_fused(const float* x_in, const void* delta, float* x_ou
   if (units < 2048) {
     while (split < 8 && chunks > split * 2) split *= 2;
   }
+  if (split_hint == 1 || split_hint == 2 || split_hint == 4 || split_hint == 8) split = split_hint;  // for tuning runs
   hipStream_t stream = (hipStream_t)stream_ptr;
   if (epilogue == EPI_STORE) dispatch_fused<EPI_STORE>(a, units, split, stream);
   else if (epilogue == EPI_SILU) dispatch_fused<EPI_SILU>(a, units, split, stream);

@@ -297,8 +297,10 @@ void dispatch_tiled(const bf16_t* x, const bf16_t* w, OutT* y, int m, int n, int
 
 }  // namespace
 
-// y_dtype: NNIS_BF16 or NNIS_F32.  Picks the skinny kernel for M <= 64.
-extern "C" int nnis_gemm_bf16(const void* x, const void* w, void* y, int y_dtype, int m, int n, int k, void* stream_ptr) {
+// y_dtype: NNIS_BF16 or NNIS_F32.  Picks the skinny kernel for M <= 64.  split_hint: 0, or the number of
+// waves (1, 2, 4, 8) that share a strip's K in the skinny kernel, overriding the choice made here.
+extern "C" int nnis_gemm_bf16(const void* x, const void* w, void* y, int y_dtype, int m, int n, int k, int split_hint,
+                              void* stream_ptr) {
   NNIS_REQUIRE(nnis_dtype_ok(y_dtype), "gemm_bf16: unknown output dtype %d", y_dtype);
   NNIS_REQUIRE(m >= 0 && n > 0 && k > 0, "gemm_bf16: bad sizes m=%d n=%d k=%d", m, n, k);
   NNIS_REQUIRE(k % 8 == 0, "gemm_bf16: K=%d is not a multiple of 8 (16-byte loads); use the ordered kernel", k);
@@ -319,6 +321,7 @@ extern "C" int nnis_gemm_bf16(const void* x, const void* w, void* y, int y_dtype
     if (strips < 2048) {
       while (split < 8 && chunks > split * depth) split *= 2;
     }
+    if (split_hint == 1 || split_hint == 2 || split_hint == 4 || split_hint == 8) split = split_hint;  // for tuning runs
     if (y_dtype == NNIS_F32) dispatch_skinny<float>(xp, wp, (float*)y, m, n, k, split, stream);
     else dispatch_skinny<bf16_t>(xp, wp, (bf16_t*)y, m, n, k, split, stream);
     NNIS_LAUNCH_CHECK("gemm_skinny");
