@@ -143,6 +143,39 @@ def test_command_line(model_dirs):
     assert run.returncode == 1 and run.stderr.startswith("nnis generate:")
 
 
+def test_command_line_with_text(model_dirs, tmp_path):
+    """Text in and out through a tokenizer.json in the model folder (a word-level
+    one made here), and the process entry point around the command line."""
+    import json
+    import shutil
+
+    from tokenizers import Tokenizer
+    from tokenizers.models import WordLevel
+    from tokenizers.pre_tokenizers import Whitespace
+
+    folder = str(tmp_path / "with_tokenizer")
+    shutil.copytree(model_dirs["B"], folder)
+    vocab = {f"w{i}": i for i in range(1000)}
+    tokenizer = Tokenizer(WordLevel(vocab, unk_token="w0"))
+    tokenizer.pre_tokenizer = Whitespace()
+    tokenizer.save(folder + "/tokenizer.json")
+    plain = P.PlainLlama(folder)
+    prompt = [3, 141, 59, 26]
+    want = " ".join(f"w{t}" for t in plain.greedy(prompt, 5))
+    run = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "nnis"), "generate", "--model", folder, "--prompt",
+                          " ".join(f"w{t}" for t in prompt), "--max-new-tokens", "5", "--dtype", "float32"],
+                         capture_output=True, text=True, timeout=300)
+    assert run.returncode == 0, run.stderr[-2000:]
+    assert run.stdout.strip() == want
+    result = str(tmp_path / "result.json")
+    run = subprocess.run([sys.executable, "-m", "nnis_amd.process", "--model", folder, "--prompt",
+                          " ".join(f"w{t}" for t in prompt), "--max-new-tokens", "5", "--dtype", "float32", "--result", result],
+                         capture_output=True, text=True, timeout=300, cwd=ROOT)
+    assert run.returncode == 0, run.stderr[-2000:]
+    record = json.load(open(result))
+    assert record["status"] == "generated" and record["stdout"]["utf8"].strip() == want
+
+
 @pytest.mark.parametrize("options", [dict(), dict(temperature=0.8), dict(top_k=40), dict(top_p=0.7),
                                      dict(temperature=1.3, top_k=200, top_p=0.95), dict(top_k=1)])
 def test_device_sampling_matches_the_host_sampler(options):
