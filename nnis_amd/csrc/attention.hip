@@ -273,10 +273,10 @@ __device__ __forceinline__ void attend_block(AttnState<C>& st, const QFrag (&q)[
 struct PageRun {
   const int* pages;
   int max_pages;
-  int first, stride;  // lane i holds the page of block index first + i * stride (in units of 32 keys)
+  int first, stride;  // lane i holds the page at index first + i * stride of the sequence's block-table row
   int cached;
   __device__ __forceinline__ void fill(int lane) {
-    int index = (first + lane * stride) / 2;  // two blocks of 32 keys a page
+    int index = first + lane * stride;
     index = index < max_pages ? index : max_pages - 1;
     cached = pages[index];
   }
@@ -356,12 +356,14 @@ __device__ __forceinline__ bool merge_waves(AttnState<C>& st, float* merge, int 
   return true;
 }
 
-// Runs the key blocks first + wave, first + wave + waves, ... (count of them: `mine`)
-// through the softmax state, the next block's operands in flight while one is worked on.
+// Runs the pages first, first + stride, ... (`mine` of them) of a sequence through the
+// softmax state, each as two blocks of 32 keys one after the other (so both halves of a
+// value line are used while it is near), the next block's operands in flight while one is
+// worked on.  Blocks that start beyond `last_key` are left out.
 template <int C>
 __device__ __forceinline__ void attend_run(AttnState<C>& st, const QFrag (&q)[C], const MfmaArgs& a, const int* pages,
-                                           int kv_head, int first, int stride, int mine, const int (&lo)[C],
-                                           const int (&hi)[C], int lane) {
+                                           int kv_head, int first, int stride, int mine, int last_key,
+                                           const int (&lo)[C], const int (&hi)[C], int lane) {
   if (mine <= 0) return;
   const int r = lane % 16, g = lane / 16;
   const bf16_t* k_base = k_page_ptr(a, 0, kv_head);
@@ -369,30 +371,32 @@ __device__ __forceinline__ void attend_run(AttnState<C>& st, const QFrag (&q)[C]
   const size_t k_page_stride = (size_t)a.kv_heads * kPageTokens * HD, v_page_stride = (size_t)a.kv_heads * HD * kPageTokens;
   PageRun run = {pages, a.max_pages, first, stride, 0};
   run.fill(lane);
+  // block b of the run: page index first + (b / 2) * stride, half b % 2
+  int blocks = 2 * mine;
+  if ((first + (mine - 1) * stride) * kPageTokens + 32 > last_key) --blocks;  // the last page's second half is beyond the keys
   BlockFrags current, next;
   {
     const int page = run.page(0);
-    const int inside = (first * 32) % kPageTokens;
-    load_block(current, k_base + page * k_page_stride + (size_t)inside * HD, v_base + page * v_page_stride + inside, r, g);
+    load_block(current, k_base + page * k_page_stride, v_base + page * v_page_stride, r, g);
   }
-  for (int i = 0; i < mine; ++i) {
-    if (i + 1 < mine) {
-      if (((i + 1) & 63) == 0) {
-        run.first = first + (i + 1) * stride;
+  for (int b = 0; b < blocks; ++b) {
+    if (b + 1 < blocks) {
+      const int n = (b + 1) >> 1, inside = ((b + 1) & 1) * 32;
+      if (inside == 0 && (n & 63) == 0) {
+        run.first = first + n * stride;
         run.fill(lane);
       }
-      const int page = run.page((i + 1) & 63);
-      const int inside = ((first + (i + 1) * stride) * 32) % kPageTokens;
+      const int page = run.page(n & 63);
       load_block(next, k_base + page * k_page_stride + (size_t)inside * HD, v_base + page * v_page_stride + inside, r, g);
     }
-    attend_block<C>(st, q, current, (first + i * stride) * 32, lo, hi, a.scale_log2, g);
+    attend_block<C>(st, q, current, (first + (b >> 1) * stride) * kPageTokens + (b & 1) * 32, lo, hi, a.scale_log2, g);
     current = next;
   }
 }
 
 // ---- prefill: a wave = (query tile, kv head, chunk of GH query heads); C = QT * GH column tiles --------
 template <int QT, int GH>
-__global__ __launch_bounds__(256) void attention_prefill_kernel(MfmaArgs a, int waves) {
+__global__ __launch_bounds__(512) void attention_prefill_kernel(MfmaArgs a, int waves) {
   extern __shared__ float merge[];
   constexpr int C = QT * GH;
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave, r = lane % 16, g = lane / 16;
@@ -440,9 +444,9 @@ __global__ __launch_bounds__(256) void attention_prefill_kernel(MfmaArgs a, int 
   AttnState<C> st;
   init_state(st);
   if (last >= 0) {
-    const int first_block = first / 32, blocks = last / 32 + 1 - first_block;
-    const int mine = blocks > wave ? (blocks - wave + waves - 1) / waves : 0;
-    attend_run<C>(st, q, a, pages, kv_head, first_block + wave, waves, mine, lo, hi, lane);
+    const int first_page = first / kPageTokens, page_count = last / kPageTokens + 1 - first_page;
+    const int mine = page_count > wave ? (page_count - wave + waves - 1) / waves : 0;  // pages of this wave
+    attend_run<C>(st, q, a, pages, kv_head, first_page + wave, waves, mine, last, lo, hi, lane);
   }
   if (!merge_waves<C>(st, merge, wave, waves, lane)) return;
 #pragma unroll
@@ -492,15 +496,15 @@ __global__ __launch_bounds__(512) void attention_decode_kernel(MfmaArgs a, int w
     lo[c] = first_key;
     hi[c] = live[c] ? pos : -1;
   }
-  // blocks of 32 keys are dealt to the splits in contiguous runs, and within a split to the waves in turn
-  const int block_first = first_key / 32, block_count = pos / 32 + 1 - block_first;
-  const int per_split = (block_count + a.splits - 1) / a.splits;
-  const int begin = block_first + split * per_split;
-  const int end = min(begin + per_split, block_first + block_count);
+  // pages are dealt to the splits in contiguous runs, and within a split to the waves in turn
+  const int page_first = first_key / kPageTokens, page_count = pos / kPageTokens + 1 - page_first;
+  const int per_split = (page_count + a.splits - 1) / a.splits;
+  const int begin = page_first + split * per_split;
+  const int end = min(begin + per_split, page_first + page_count);
   AttnState<C> st;
   init_state(st);
-  const int mine = end > begin + wave ? (end - begin - wave + waves - 1) / waves : 0;  // key blocks of this wave
-  attend_run<C>(st, q, a, pages, kv_head, begin + wave, waves, mine, lo, hi, lane);
+  const int mine = end > begin + wave ? (end - begin - wave + waves - 1) / waves : 0;  // pages of this wave
+  attend_run<C>(st, q, a, pages, kv_head, begin + wave, waves, mine, pos, lo, hi, lane);
   if (!merge_waves<C>(st, merge, wave, waves, lane)) return;
 #pragma unroll
   for (int c = 0; c < C; ++c) {
@@ -607,39 +611,49 @@ int fill_common(MfmaArgs& a, const void* q, void* out, const void* k_pages, cons
 }  // namespace
 
 // rows of 16*QT queries per tile, as the host must cut them
-extern "C" int nnis_attention_prefill_tile_rows(int heads, int kv_heads) {
+// `columns`: the most column tiles a wave carries, 1 .. kMaxColumns (0: as many as the head size allows).
+// Fewer columns mean more, lighter blocks and more waves to deal a tile's keys to.
+static void prefill_shape(int heads, int kv_heads, int columns, int* qt, int* gh) {
   const int group = heads / (kv_heads > 0 ? kv_heads : 1);
-  const int gh = group < kMaxColumns ? group : kMaxColumns;
-  return 16 * (kMaxColumns / (gh > 0 ? gh : 1));
+  const int most = (columns >= 1 && columns < kMaxColumns) ? columns : kMaxColumns;
+  *gh = group < most ? group : most;
+  if (*gh < 1) *gh = 1;
+  *qt = most / *gh;
+  if (*qt == 3) *qt = 2;  // query tiles come in 1, 2 or 4
+}
+
+extern "C" int nnis_attention_prefill_tile_rows(int heads, int kv_heads, int columns) {
+  int qt, gh;
+  prefill_shape(heads, kv_heads, columns, &qt, &gh);
+  return 16 * qt;
 }
 
 // waves a block of the prefill kernel may have for these sizes (LDS of the merge)
-extern "C" int nnis_attention_prefill_max_waves(int heads, int kv_heads) {
-  const int group = heads / (kv_heads > 0 ? kv_heads : 1);
-  const int gh = group < kMaxColumns ? group : kMaxColumns;
-  const int columns = (kMaxColumns / (gh > 0 ? gh : 1)) * gh;
-  const size_t per_wave = (size_t)columns * (kTilesD * 4 + 2) * kWave * sizeof(float);
-  int waves = 1 + (int)(65536 / per_wave);
-  return waves >= 4 ? 4 : (waves >= 2 ? 2 : 1);
+extern "C" int nnis_attention_prefill_max_waves(int heads, int kv_heads, int columns) {
+  int qt, gh;
+  prefill_shape(heads, kv_heads, columns, &qt, &gh);
+  const size_t per_wave = (size_t)qt * gh * (kTilesD * 4 + 2) * kWave * sizeof(float);
+  const int waves = 1 + (int)(65536 / per_wave);
+  return waves >= 8 ? 8 : (waves >= 4 ? 4 : (waves >= 2 ? 2 : 1));
 }
 
 extern "C" int nnis_attention_prefill_bf16(const void* q, void* out, const void* k_pages, const void* v_pages,
                                            const int* block_table, int max_pages, const int* tile_seq,
                                            const int* tile_row0, int tiles, const int* seq_slot, const int* seq_start,
                                            const int* seq_pos0, int heads, int kv_heads, int head_dim, int window,
-                                           float scale, int waves, void* stream) {
+                                           float scale, int waves, int columns, void* stream) {
   MfmaArgs a;
   if (fill_common(a, q, out, k_pages, v_pages, block_table, max_pages, heads, kv_heads, head_dim, window, scale)) return 1;
   if (tiles <= 0) return 0;
   a.tile_seq = tile_seq; a.tile_row0 = tile_row0; a.seq_slot = seq_slot; a.seq_start = seq_start; a.seq_pos0 = seq_pos0;
   const int group = heads / kv_heads;
-  const int gh = group < kMaxColumns ? group : kMaxColumns;
-  const int qt = kMaxColumns / gh;
+  int qt, gh;
+  prefill_shape(heads, kv_heads, columns, &qt, &gh);
   const int chunks = (group + gh - 1) / gh;
   const dim3 grid(tiles, kv_heads * chunks);
   NNIS_REQUIRE(grid.y <= 65535, "attention: %d head chunks exceed the grid limit", grid.y);
   const size_t per_wave = (size_t)qt * gh * (kTilesD * 4 + 2) * kWave * sizeof(float);
-  NNIS_REQUIRE(waves >= 1 && waves <= 4 && (waves - 1) * per_wave <= 65536,
+  NNIS_REQUIRE(waves >= 1 && waves <= 8 && (waves - 1) * per_wave <= 65536,
                "attention: %d waves a block do not fit this head size (LDS)", waves);
   const size_t lds = (waves - 1) * per_wave;
   const dim3 block(kWave * waves);
@@ -698,10 +712,10 @@ extern "C" int nnis_attention_decode_bf16(const void* q, void* out, const void* 
   return 0;
 }
 #else
-extern "C" int nnis_attention_prefill_tile_rows(int, int) { return 0; }
-extern "C" int nnis_attention_prefill_max_waves(int, int) { return 1; }
+extern "C" int nnis_attention_prefill_tile_rows(int, int, int) { return 0; }
+extern "C" int nnis_attention_prefill_max_waves(int, int, int) { return 1; }
 extern "C" int nnis_attention_prefill_bf16(const void*, void*, const void*, const void*, const int*, int, const int*, const int*,
-                                           int, const int*, const int*, const int*, int, int, int, int, float, int, void*) {
+                                           int, const int*, const int*, const int*, int, int, int, int, float, int, int, void*) {
   return nnis_fail("attention: the matrix-core kernels need a head size in steps of 16; this module has %d", NNIS_HEAD_DIM);
 }
 extern "C" int nnis_attention_decode_max_waves(int, int) { return 1; }

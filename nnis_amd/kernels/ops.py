@@ -36,10 +36,10 @@ _CORE_SIGNATURES = {
 _ATTN_SIGNATURES = {
     "nnis_attention_rows": [_VOID, _INT, _VOID, _INT, _VOID, _VOID, _INT, _VOID, _INT, _VOID, _VOID, _INT, _INT, _INT,
                             _INT, _INT, _FLT, _VOID],
-    "nnis_attention_prefill_tile_rows": [_INT, _INT],
+    "nnis_attention_prefill_tile_rows": [_INT, _INT, _INT],
     "nnis_attention_prefill_bf16": [_VOID, _VOID, _VOID, _VOID, _VOID, _INT, _VOID, _VOID, _INT, _VOID, _VOID, _VOID, _INT,
-                                    _INT, _INT, _INT, _FLT, _INT, _VOID],
-    "nnis_attention_prefill_max_waves": [_INT, _INT],
+                                    _INT, _INT, _INT, _FLT, _INT, _INT, _VOID],
+    "nnis_attention_prefill_max_waves": [_INT, _INT, _INT],
     "nnis_attention_decode_bf16": [_VOID, _VOID, _VOID, _VOID, _VOID, _INT, _VOID, _VOID, _INT, _INT, _INT, _INT, _INT, _FLT,
                                    _INT, _INT, _VOID, _VOID],
     "nnis_attention_decode_max_waves": [_INT, _INT],
@@ -347,17 +347,19 @@ def _check_pages(q, out, k_pages, v_pages, block_table, heads, kv_heads, head_di
             raise KernelError(f"attention: the matrix-core kernels take bfloat16, {what} is {t.dtype}")
 
 
-def prefill_tile_rows(heads: int, kv_heads: int, head_dim: int) -> int:
-    """Query rows per work item of ``attention_prefill_bf16`` for these sizes."""
-    return attention_module(head_dim).nnis_attention_prefill_tile_rows(heads, kv_heads)
+def prefill_tile_rows(heads: int, kv_heads: int, head_dim: int, columns: int = 0) -> int:
+    """Query rows per work item of ``attention_prefill_bf16`` for these sizes.
+    ``columns``: the most 16-column tiles (query tiles x heads of a group) a
+    wave carries; 0 for as many as the head size allows."""
+    return attention_module(head_dim).nnis_attention_prefill_tile_rows(heads, kv_heads, columns)
 
 
-def prefill_max_waves(heads: int, kv_heads: int, head_dim: int) -> int:
-    return attention_module(head_dim).nnis_attention_prefill_max_waves(heads, kv_heads)
+def prefill_max_waves(heads: int, kv_heads: int, head_dim: int, columns: int = 0) -> int:
+    return attention_module(head_dim).nnis_attention_prefill_max_waves(heads, kv_heads, columns)
 
 
 def attention_prefill_bf16(q, out, k_pages, v_pages, block_table, tile_seq, tile_row0, seq_slot, seq_start, seq_pos0,
-                           heads, kv_heads, head_dim, scale, window=0, waves=1):
+                           heads, kv_heads, head_dim, scale, window=0, waves=1, columns=0):
     """Causal attention of whole runs of new tokens over the cache, on the
     matrix cores.  ``tile_seq``/``tile_row0`` (int32) name, per work item, a
     sequence of the step and the first of ``prefill_tile_rows`` rows of its
@@ -375,7 +377,7 @@ def attention_prefill_bf16(q, out, k_pages, v_pages, block_table, tile_seq, tile
                                                 block_table.data_ptr(), block_table.shape[1], tile_seq.data_ptr(),
                                                 tile_row0.data_ptr(), tiles, seq_slot.data_ptr(), seq_start.data_ptr(),
                                                 seq_pos0.data_ptr(), heads, kv_heads, head_dim, int(window), float(scale),
-                                                int(waves), _stream()))
+                                                int(waves), int(columns), _stream()))
     return out
 
 
@@ -412,16 +414,23 @@ def decode_max_waves(heads: int, kv_heads: int, head_dim: int) -> int:
 def decode_plan(batch: int, kv_heads: int, longest: int, max_waves: int = 4):
     """(splits, waves) of a decode step's attention.  The kernel is bound by
     memory latency (a wave has one block of 32 keys in flight beside the one it
-    works on), so the keys are spread over about a thousand waves, down to two
-    blocks a wave.  Four waves of a block merge in LDS; beyond that the keys are
+    works on), so the keys are spread over about a thousand waves, down to one
+    page of 64 keys a wave.  Four waves of a block merge in LDS; beyond that the keys are
     cut into runs that a second kernel sums.  Powers of two.  Measured on the
     SmolLM2-135M shape: batch 8 at 1.7k keys runs 1.11 ms a step with (4, 4)
     against 1.41 with (1, 8) and 2.78 with (1, 1)."""
-    blocks = (longest + 31) // 32
-    parallel = max(1, min(blocks // 2, 1024 // max(1, batch * kv_heads)))
+    pages = (longest + 63) // 64
+    parallel = max(1, min(pages, 1024 // max(1, batch * kv_heads)))
     parallel = 1 << (parallel.bit_length() - 1)
     waves = min(max_waves, parallel)
     return parallel // waves, waves
+
+
+# One column tile a wave (and so up to 8 waves a block) for long sequences was measured slower than the full
+# group a wave with 4 waves (2,048 tokens, 9/3 heads of 64: 5.5 ms a step against 4.6): keys and values are read
+# once per query head then.  The switch stays for other shapes; 0 is off.
+PREFILL_NARROW_FROM = 1024
+PREFILL_COLUMNS = 0
 
 
 def _prefill_tiles(ctx, rows: int, device):
@@ -455,12 +464,15 @@ def attention(q: torch.Tensor, out: torch.Tensor, view, ctx, heads: int, kv_head
         return attention_decode_bf16(q, out, view.k_pages, view.v_pages, view.block_table, ctx.tok_slot, ctx.tok_pos, heads,
                                      kv_heads, head_dim, scale, window, splits, partial, waves)
     if fast and not ctx.decode:
-        tile_seq, tile_row0 = _prefill_tiles(ctx, prefill_tile_rows(heads, kv_heads, head_dim), q.device)
-        # the waves of a block deal a tile's key blocks among themselves: worth it once a tile reads many
-        waves = min(prefill_max_waves(heads, kv_heads, head_dim), 4 if ctx.max_len >= 512 else (2 if ctx.max_len >= 128 else 1))
+        # A tile's keys are a chain of dependent loads: the longest tile sets the kernel's time.  The waves of
+        # a block deal the keys among themselves (their merge lives in LDS).
+        columns = PREFILL_COLUMNS if ctx.max_len >= PREFILL_NARROW_FROM else 0
+        most = prefill_max_waves(heads, kv_heads, head_dim, columns)
+        waves = min(most, 8 if ctx.max_len >= 1024 else (4 if ctx.max_len >= 512 else (2 if ctx.max_len >= 128 else 1)))
+        tile_seq, tile_row0 = _prefill_tiles(ctx, prefill_tile_rows(heads, kv_heads, head_dim, columns), q.device)
         return attention_prefill_bf16(q, out, view.k_pages, view.v_pages, view.block_table, tile_seq, tile_row0,
                                       ctx.seq_slot, ctx.seq_start, ctx.seq_pos0, heads, kv_heads, head_dim, scale, window,
-                                      waves)
+                                      waves, columns)
     return attention_rows(q, out, view.k_pages, view.v_pages, view.block_table, ctx.tok_slot, ctx.tok_pos, heads,
                           kv_heads, head_dim, scale, window)
 

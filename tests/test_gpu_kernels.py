@@ -195,11 +195,14 @@ def test_prefill_attention_on_the_matrix_cores(heads, kv_heads, head_dim):
     assert tile in (16, 32, 64)
     items = [(seq, row0) for seq, (_, _, n) in enumerate(sequences) for row0 in range(0, n, tile)]
     starts = [0, 130, 167, 168]
-    most = ops.prefill_max_waves(heads, kv_heads, head_dim)
-    for window, waves in ((0, 1), (40, 1), (0, most), (40, min(2, most))):
+    starts = [0, 130, 167, 168]
+    for window, waves, columns in ((0, 1, 0), (40, 1, 0), (0, 8, 0), (40, 2, 0), (0, 8, 1), (40, 4, 2)):
+        waves = min(waves, ops.prefill_max_waves(heads, kv_heads, head_dim, columns))
+        tile = ops.prefill_tile_rows(heads, kv_heads, head_dim, columns)
+        items = [(seq, row0) for seq, (_, _, n) in enumerate(sequences) for row0 in range(0, n, tile)]
         ops.attention_prefill_bf16(q, out, k_pages, v_pages, table, _i32([s for s, _ in items]), _i32([r for _, r in items]),
                                    _i32([s for s, _, _ in sequences]), _i32(starts), _i32([p for _, p, _ in sequences]),
-                                   heads, kv_heads, head_dim, scale, window, waves)
+                                   heads, kv_heads, head_dim, scale, window, waves, columns)
         got = out.cpu().float().view(len(rows), heads, head_dim)
         want = _plain_rows(rows, ks, vs, scale, window=window)
         error = (got - want).abs().amax(dim=(1, 2))
