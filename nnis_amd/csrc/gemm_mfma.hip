@@ -168,6 +168,10 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
   constexpr int WM = BM / 2, WN = BN / 2;  // a wave's part of the tile
   constexpr int TM = WM / 16, TN = WN / 16;
   constexpr int A_CHUNKS = BM * 8 / 256, B_CHUNKS = BN * 8 / 256;  // 16-byte chunks a thread stages per step
+  // Global loads run PF steps ahead of the multiply, in registers; the step after
+  // the current one lies in the other LDS buffer.  With few blocks on a compute
+  // unit nothing else hides the latency of a load, so short products need depth.
+  constexpr int PF = (BM * BN >= 128 * 128) ? 3 : 4;
   __shared__ bf16x8 a_tile[2][BM * 8];
   __shared__ bf16x8 b_tile[2][BN * 8];
 
@@ -183,60 +187,76 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
 #pragma unroll
     for (int j = 0; j < TN; ++j) acc[i][j] = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
 
-  bf16x8 a_stage[A_CHUNKS], b_stage[B_CHUNKS];
-  auto fetch = [&](int k0) {
+  // what this thread stages: rows and chunk of each of its 16-byte pieces
+  const bf16_t* a_src[A_CHUNKS];
+  const bf16_t* b_src[B_CHUNKS];
+  int a_dst[A_CHUNKS], b_dst[B_CHUNKS];
+  const int chunk_k = (tid % 8) * 8;
 #pragma unroll
-    for (int c = 0; c < A_CHUNKS; ++c) {
-      const int index = tid + c * 256;  // row = index / 8, chunk = index % 8
-      int row = row0 + index / 8;
-      row = row < m ? row : m - 1;
-      const int kk = k0 + (index % 8) * 8;
-      a_stage[c] = kk + 8 <= k ? load_chunk(x + (size_t)row * k + kk) : zero_chunk();
-    }
-#pragma unroll
-    for (int c = 0; c < B_CHUNKS; ++c) {
-      const int index = tid + c * 256;
-      int row = col0 + index / 8;
-      row = row < n ? row : n - 1;
-      const int kk = k0 + (index % 8) * 8;
-      b_stage[c] = kk + 8 <= k ? load_chunk(w + (size_t)row * k + kk) : zero_chunk();
-    }
-  };
-  auto stage = [&](int buffer) {
-#pragma unroll
-    for (int c = 0; c < A_CHUNKS; ++c) {
-      const int index = tid + c * 256;
-      a_tile[buffer][swizzled(index / 8, index % 8)] = a_stage[c];
-    }
-#pragma unroll
-    for (int c = 0; c < B_CHUNKS; ++c) {
-      const int index = tid + c * 256;
-      b_tile[buffer][swizzled(index / 8, index % 8)] = b_stage[c];
-    }
-  };
-
-  const int steps = (k + kBK - 1) / kBK;
-  fetch(0);
-  stage(0);
-  __syncthreads();
-  for (int step = 0; step < steps; ++step) {
-    const int buffer = step & 1;
-    if (step + 1 < steps) fetch((step + 1) * kBK);
-#pragma unroll
-    for (int half = 0; half < 2; ++half) {  // two instructions of 32 k per stage
-      bf16x8 a_frag[TM], b_frag[TN];
-#pragma unroll
-      for (int i = 0; i < TM; ++i) a_frag[i] = a_tile[buffer][swizzled(wave_m * WM + i * 16 + r, half * 4 + g)];
-#pragma unroll
-      for (int j = 0; j < TN; ++j) b_frag[j] = b_tile[buffer][swizzled(wave_n * WN + j * 16 + r, half * 4 + g)];
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j) acc[i][j] = mfma(b_frag[j], a_frag[i], acc[i][j]);
-    }
-    if (step + 1 < steps) stage(buffer ^ 1);
-    __syncthreads();
+  for (int c = 0; c < A_CHUNKS; ++c) {
+    const int index = tid + c * 256;  // row = index / 8, chunk = index % 8
+    int row = row0 + index / 8;
+    row = row < m ? row : m - 1;
+    a_src[c] = x + (size_t)row * k + chunk_k;
+    a_dst[c] = swizzled(index / 8, index % 8);
   }
+#pragma unroll
+  for (int c = 0; c < B_CHUNKS; ++c) {
+    const int index = tid + c * 256;
+    int row = col0 + index / 8;
+    row = row < n ? row : n - 1;
+    b_src[c] = w + (size_t)row * k + chunk_k;
+    b_dst[c] = swizzled(index / 8, index % 8);
+  }
+
+  bf16x8 a_stage[PF][A_CHUNKS], b_stage[PF][B_CHUNKS];
+  const int steps = (k + kBK - 1) / kBK;
+
+#define NNIS_FETCH(slot, step)                                                                   \
+  do {                                                                                           \
+    const int k0 = (step) * kBK;                                                                 \
+    const bool in = k0 + chunk_k + 8 <= k;                                                       \
+    _Pragma("unroll") for (int c = 0; c < A_CHUNKS; ++c) a_stage[slot][c] = in ? load_chunk(a_src[c] + k0) : zero_chunk(); \
+    _Pragma("unroll") for (int c = 0; c < B_CHUNKS; ++c) b_stage[slot][c] = in ? load_chunk(b_src[c] + k0) : zero_chunk(); \
+  } while (0)
+#define NNIS_STAGE(slot, buffer)                                                                 \
+  do {                                                                                           \
+    _Pragma("unroll") for (int c = 0; c < A_CHUNKS; ++c) a_tile[buffer][a_dst[c]] = a_stage[slot][c]; \
+    _Pragma("unroll") for (int c = 0; c < B_CHUNKS; ++c) b_tile[buffer][b_dst[c]] = b_stage[slot][c]; \
+  } while (0)
+
+#pragma unroll
+  for (int s = 0; s < PF; ++s)
+    if (s < steps) NNIS_FETCH(s, s);
+  NNIS_STAGE(0, 0);
+  __syncthreads();
+  for (int base = 0; base < steps; base += PF) {
+#pragma unroll
+    for (int j = 0; j < PF; ++j) {
+      const int step = base + j;
+      if (step < steps) {  // uniform over the block
+        const int buffer = step & 1;
+        // slot j went to LDS a step ago: refill it with the step PF ahead
+        if (step + PF < steps) NNIS_FETCH(j, step + PF);
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {  // two instructions of 32 k per stage
+          bf16x8 a_frag[TM], b_frag[TN];
+#pragma unroll
+          for (int i = 0; i < TM; ++i) a_frag[i] = a_tile[buffer][swizzled(wave_m * WM + i * 16 + r, half * 4 + g)];
+#pragma unroll
+          for (int jj = 0; jj < TN; ++jj) b_frag[jj] = b_tile[buffer][swizzled(wave_n * WN + jj * 16 + r, half * 4 + g)];
+#pragma unroll
+          for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int jj = 0; jj < TN; ++jj) acc[i][jj] = mfma(b_frag[jj], a_frag[i], acc[i][jj]);
+        }
+        if (step + 1 < steps) NNIS_STAGE((j + 1) % PF, buffer ^ 1);
+        __syncthreads();
+      }
+    }
+  }
+#undef NNIS_FETCH
+#undef NNIS_STAGE
 
   // first operand = weight rows: lane holds D[n = 4g + e][token = r]
   const bool vector_ok = (n % 4) == 0;
@@ -286,12 +306,14 @@ void launch_tiled(const bf16_t* x, const bf16_t* w, OutT* y, int m, int n, int k
 }
 
 template <typename OutT>
-void dispatch_tiled(const bf16_t* x, const bf16_t* w, OutT* y, int m, int n, int k, hipStream_t stream) {
+void dispatch_tiled(const bf16_t* x, const bf16_t* w, OutT* y, int m, int n, int k, int tile_hint, hipStream_t stream) {
   // the largest tile that still gives every compute unit a block or two
   const long long blocks_128 = (long long)((m + 127) / 128) * ((n + 127) / 128);
   const long long blocks_64_128 = (long long)((m + 63) / 64) * ((n + 127) / 128);
-  if (blocks_128 >= 384) launch_tiled<128, 128, OutT>(x, w, y, m, n, k, stream);
-  else if (blocks_64_128 >= 256) launch_tiled<64, 128, OutT>(x, w, y, m, n, k, stream);
+  int tile = blocks_128 >= 384 ? 1 : (blocks_64_128 >= 256 ? 2 : 3);
+  if (tile_hint >= 1 && tile_hint <= 3) tile = tile_hint;  // for tuning runs
+  if (tile == 1) launch_tiled<128, 128, OutT>(x, w, y, m, n, k, stream);
+  else if (tile == 2) launch_tiled<64, 128, OutT>(x, w, y, m, n, k, stream);
   else launch_tiled<64, 64, OutT>(x, w, y, m, n, k, stream);
 }
 
@@ -327,8 +349,9 @@ extern "C" int nnis_gemm_bf16(const void* x, const void* w, void* y, int y_dtype
     NNIS_LAUNCH_CHECK("gemm_skinny");
   } else {
     NNIS_REQUIRE((m + 63) / 64 <= 65535, "gemm_bf16: %d rows exceed the grid limit", m);
-    if (y_dtype == NNIS_F32) dispatch_tiled<float>(xp, wp, (float*)y, m, n, k, stream);
-    else dispatch_tiled<bf16_t>(xp, wp, (bf16_t*)y, m, n, k, stream);
+    const int tile_hint = split_hint >= 16 ? split_hint / 16 : 0;  // hints of 16, 32, 48 pick the tile: 128x128, 64x128, 64x64
+    if (y_dtype == NNIS_F32) dispatch_tiled<float>(xp, wp, (float*)y, m, n, k, tile_hint, stream);
+    else dispatch_tiled<bf16_t>(xp, wp, (bf16_t*)y, m, n, k, tile_hint, stream);
     NNIS_LAUNCH_CHECK("gemm_tiled");
   }
   return 0;
