@@ -26,8 +26,15 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0
 FLOP_PEAK = {"bfloat16": 2.5e15, "float32": 157.3e12}
 
-SHAPE = dict(layers=30, hidden=576, heads=9, kv_heads=3, head_dim=64, inner=1536, vocab=49152, rope_theta=100000.0,
-             rms_norm_eps=1e-5, context=8192)
+SHAPES = {
+    "smollm2-135m": dict(name="SmolLM2-135M", layers=30, hidden=576, heads=9, kv_heads=3, head_dim=64, inner=1536, vocab=49152,
+                         rope_theta=100000.0, rms_norm_eps=1e-5, context=8192, tied=True),
+    "smollm2-1.7b": dict(name="SmolLM2-1.7B", layers=24, hidden=2048, heads=32, kv_heads=32, head_dim=64, inner=8192, vocab=49152,
+                         rope_theta=130000.0, rms_norm_eps=1e-5, context=8192, tied=True),
+    "tinyllama-1.1b": dict(name="TinyLlama-1.1B", layers=22, hidden=2048, heads=32, kv_heads=4, head_dim=64, inner=5632,
+                           vocab=32000, rope_theta=10000.0, rms_norm_eps=1e-5, context=2048, tied=False),
+}
+SHAPE = dict(SHAPES["smollm2-135m"])  # the default run's; --shape puts another in its place
 
 
 def model_config(layers):
@@ -36,7 +43,7 @@ def model_config(layers):
         "num_hidden_layers": layers, "hidden_size": SHAPE["hidden"], "num_attention_heads": SHAPE["heads"],
         "num_key_value_heads": SHAPE["kv_heads"], "head_dim": SHAPE["head_dim"], "intermediate_size": SHAPE["inner"],
         "vocab_size": SHAPE["vocab"], "rope_theta": SHAPE["rope_theta"], "rms_norm_eps": SHAPE["rms_norm_eps"],
-        "tie_word_embeddings": True, "max_position_embeddings": SHAPE["context"], "torch_dtype": "bfloat16",
+        "tie_word_embeddings": SHAPE["tied"], "max_position_embeddings": SHAPE["context"], "torch_dtype": "bfloat16",
         "eos_token_id": 0,
     }
 
@@ -57,7 +64,8 @@ def main() -> int:
     parser.add_argument("--steps", type=int, default=64)
     parser.add_argument("--warmup", type=int, default=8)
     parser.add_argument("--batch", type=int, default=8)
-    parser.add_argument("--layers", type=int, default=SHAPE["layers"])
+    parser.add_argument("--shape", default="smollm2-135m", choices=sorted(SHAPES), help="layer sizes of the model")
+    parser.add_argument("--layers", type=int, default=0, help="fewer layers than the shape has (0: all of them)")
     parser.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     parser.add_argument("--seed", type=int, default=0)
     parser.add_argument("--no-points", action="store_true", help="skip the batch-1 and batch-64 decode points")
@@ -65,6 +73,10 @@ def main() -> int:
     if args.gpus != 1:
         print(f"bench.py: this library runs on one GPU; --gpus {args.gpus} is not supported")
         return 2
+    SHAPE.clear()
+    SHAPE.update(SHAPES[args.shape])
+    args.layers = args.layers or SHAPE["layers"]
+    longest_prompt = min(2048, SHAPE["context"] - args.steps - args.warmup - 1)
 
     import numpy as np
     import torch
@@ -81,7 +93,7 @@ def main() -> int:
 
         def decode_run(batch, steps, warmup):
             """Prefills ``batch`` prompts in one step, then times ``steps`` decode steps."""
-            lengths = rng.integers(128, 2049, size=batch).tolist()
+            lengths = rng.integers(128, longest_prompt + 1, size=batch).tolist()
             room = batch * SHAPE["context"]  # every sequence may grow to the model's context
             engine = load_engine(folder, dtype=args.dtype, max_tokens=room)
             selector = DeviceSelector(engine)
@@ -114,7 +126,7 @@ def main() -> int:
         achieved = step_bytes / (seconds / args.steps) / 1e9
 
         # prefill: 2,048 tokens of one sequence in one step, logits at the last place
-        prefill_tokens = 2048
+        prefill_tokens = min(2048, SHAPE["context"])
         engine = load_engine(folder, dtype=args.dtype, max_tokens=prefill_tokens)
         prompt = rng.integers(0, SHAPE["vocab"], size=prefill_tokens).tolist()
         times = []
@@ -138,7 +150,8 @@ def main() -> int:
                 points[f"decode_b{batch}"] = round(batch * max(8, args.steps // 2) / s, 1)
 
     record = {
-        "metric": "decode tok/s at batch 8 (SmolLM2-135M shape); prefill tok/s at 2048 tokens; decode at batch 1 and 64 in points",
+        "metric": f"decode tok/s at batch {args.batch} ({SHAPE['name']} shape); prefill tok/s at {prefill_tokens} tokens; "
+                  "decode at batch 1 and 64 in points",
         "value": round(value, 1),
         "unit": "tokens/s",
         "n_gpus": 1,
@@ -151,10 +164,10 @@ def main() -> int:
         "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
         "data": "synthetic: random weights N(0, 0.02) from a seed, uniform-random token ids",
         "config": {
-            "model": "SmolLM2-135M shape (Llama)", "layers": args.layers, "layers_of_model": SHAPE["layers"],
+            "model": f"{SHAPE['name']} shape (Llama)", "layers": args.layers, "layers_of_model": SHAPE["layers"],
             "hidden": SHAPE["hidden"], "heads": SHAPE["heads"], "kv_heads": SHAPE["kv_heads"], "head_dim": SHAPE["head_dim"],
-            "inner": SHAPE["inner"], "vocab": SHAPE["vocab"], "tied_head": True, "context": SHAPE["context"],
-            "global_batch": args.batch, "seq_len": SHAPE["context"], "prompt_min": 128, "prompt_max": 2048,
+            "inner": SHAPE["inner"], "vocab": SHAPE["vocab"], "tied_head": SHAPE["tied"], "context": SHAPE["context"],
+            "global_batch": args.batch, "seq_len": SHAPE["context"], "prompt_min": 128, "prompt_max": longest_prompt,
             "mean_prompt": round(float(np.mean(lengths)), 1), "parallelism": "single GPU", "sampling": "greedy on device",
         },
         "prefill": {

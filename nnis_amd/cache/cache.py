@@ -4,9 +4,11 @@ fixed-size state per slot.
 
 Layout of a key/value group (``entries`` = schedule entries that keep a cache
 in this group):
-    k  [entries, pages, kv_heads, 64, head_dim]   a token's key is a row
-    v  [entries, pages, kv_heads, head_dim, 64]   a page's keys are contiguous per channel
+    k  [entries, pages, kv_heads, head_dim / 8, 64, 8]       8 channels of a token together
+    v  [entries, pages, kv_heads, head_dim / 16, 2, 4, 16, 8] 8 tokens of a channel together
     block_table [slots, max_pages_per_slot] int32, on the device
+(``layout.py`` has the orders in full: they are those in which the attention
+kernels read.)
 The reference's cache is [layer][kv_head][capacity][head_dim] per session
 (/root/reference/crates/nnis-rt/src/kv_cache.rs:1-5,98-110); pages replace the
 fixed capacity so that the memory follows the tokens actually held.
@@ -22,14 +24,15 @@ import torch
 from ..errors import CacheFull, InvalidInput
 from ..parts.base import KVRequest, StateRequest
 from .allocator import PAGE_TOKENS, FreeList, PageTable, pages_for
+from .layout import k_page_shape, v_page_shape
 
 
 @dataclass
 class KVView:
     """What an attention-like mixer sees of the cache for one schedule entry."""
 
-    k_pages: torch.Tensor  # [pages, kv_heads, 64, head_dim]
-    v_pages: torch.Tensor  # [pages, kv_heads, head_dim, 64]
+    k_pages: torch.Tensor  # [pages, *k_page_shape(kv_heads, head_dim)]
+    v_pages: torch.Tensor  # [pages, *v_page_shape(kv_heads, head_dim)]
     block_table: torch.Tensor  # [slots, max_pages_per_slot]
     window: Optional[int]
     read_only: bool  # this run reads another entry's cache and writes nothing
@@ -54,8 +57,8 @@ class KVGroup:
         per_slot = min(pages, pages_for(max_positions))
         self.table = PageTable(pages, slots, per_slot)
         # zero at first: a page's unwritten tail is multiplied by zero weights, so it must hold numbers
-        self.k = torch.zeros((len(entries), pages, request.kv_heads, PAGE_TOKENS, request.head_dim), dtype=dtype, device=device)
-        self.v = torch.zeros((len(entries), pages, request.kv_heads, request.head_dim, PAGE_TOKENS), dtype=dtype, device=device)
+        self.k = torch.zeros((len(entries), pages) + k_page_shape(request.kv_heads, request.head_dim), dtype=dtype, device=device)
+        self.v = torch.zeros((len(entries), pages) + v_page_shape(request.kv_heads, request.head_dim), dtype=dtype, device=device)
         pinned = torch.device(device).type == "cuda"
         self.block_table_host = torch.zeros((slots, per_slot), dtype=torch.int32, pin_memory=pinned)
         self.block_table = torch.zeros((slots, per_slot), dtype=torch.int32, device=device)

@@ -81,18 +81,18 @@ __global__ __launch_bounds__(256) void attention_rows_kernel(AttnArgs a) {
   for (int j = lo + lane; j < kv_len; j += kWave) {
     const int page = pages[j / kPageTokens];
     const int r = j % kPageTokens;
-    const CacheT* krow = kp + (((size_t)page * a.kv_heads + kv_head) * kPageTokens + r) * HD;
+    const CacheT* keys = kp + ((size_t)page * a.kv_heads + kv_head) * nnis_k_page_elems(HD);
     float dot = 0.0f;
 #pragma unroll
-    for (int d = 0; d < HD; ++d) dot = fmaf(qs[d], to_f32(krow[d]), dot);
+    for (int d = 0; d < HD; ++d) dot = fmaf(qs[d], to_f32(keys[nnis_k_offset(r, d)]), dot);
     const float s = dot * a.scale;
     const float m_new = fmaxf(m, s);
     const float alpha = expf(m - m_new);  // exp(-inf) = 0 on the first key
     const float p = expf(s - m_new);
     l = l * alpha + p;
-    const CacheT* vcol = vp + ((size_t)page * a.kv_heads + kv_head) * HD * kPageTokens + r;
+    const CacheT* values = vp + ((size_t)page * a.kv_heads + kv_head) * nnis_v_page_elems(HD);
 #pragma unroll
-    for (int d = 0; d < HD; ++d) o[d] = o[d] * alpha + p * to_f32(vcol[(size_t)d * kPageTokens]);
+    for (int d = 0; d < HD; ++d) o[d] = o[d] * alpha + p * to_f32(values[nnis_v_offset(d, r)]);
     m = m_new;
   }
 
@@ -126,11 +126,11 @@ __global__ __launch_bounds__(256) void attention_rows_kernel(AttnArgs a) {
 // softmax state lives in the lanes l%16 == column, its running maximum kept
 // equal over the four lane groups.  The output is taken transposed too,
 // O^T[d][column] += V^T[d][key] . P^T[key][column]: first operand a tile of 16
-// channels from the value page (stored with keys contiguous per channel),
-// second the probabilities, which are already in the lanes that need them --
-// key (group g, element e) of the instruction's 32 is key 4g+e of the first
-// score tile for e < 4 and of the second for e >= 4, and the value operand is
-// loaded in that order.  Softmax is in 32-bit (base-2 exponentials of scores
+// channels from the value page, second the probabilities, which are already in
+// the lanes that need them -- the rows of the two score tiles of a block of 32
+// keys are dealt so that lane group g ends up with keys 8g .. 8g+7, and the
+// value page keeps 8 consecutive keys of a channel together, one 16-byte load
+// per lane and tile.  Softmax is in 32-bit (base-2 exponentials of scores
 // scaled by log2 e); probabilities are rounded to bfloat16 for the product
 // with the bfloat16 values.
 // =============================================================================
@@ -143,6 +143,17 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 constexpr int kFullD = HD / 32;       // steps of 32 channels in a score
 constexpr bool kTailD = (HD % 32) != 0;  // plus one of 16
 constexpr int kTilesD = HD / 16;      // output tiles of 16 channels
+// waves of a block: beyond 64 channels a wave needs more registers than a block of 8 waves leaves it
+constexpr int kBlockWaves = HD <= 64 ? 8 : 4;
+constexpr int kPartial = HD + 4;  // floats a split leaves per (token, head), rows 16-byte aligned
+// key blocks a decoding wave has in flight (its registers hold their operands)
+constexpr int kDecodeRing = HD <= 64 ? 4 : (HD <= 128 ? 2 : 1);
+// the kernel with keys on lanes: pages in flight, and how far a score may rise above the softmax's
+// reference (as a power of two) before the reference moves
+constexpr int kKeysRing = HD <= 64 ? 3 : 2;
+constexpr int kKeysWaves = 4;  // of a block of that kernel: a wave keeps kKeysRing pages in registers
+constexpr int kKeysMaxHD = 128;
+constexpr float kLazyRise = 8.0f;
 constexpr float kLog2e = 1.4426950408889634f;
 
 struct QFrag {
@@ -199,23 +210,25 @@ __device__ __forceinline__ void init_state(AttnState<C>& st) {
   }
 }
 
-// One block of 32 keys (keys key0 .. key0+31, inside one page): its operands.
-//   k_block: &K[page][kv_head][key0 % 64][0]      (row stride HD)
-//   v_block: &V[page][kv_head][0][key0 % 64]      (channel stride 64)
+// One block of 32 keys (half h of a page): its operands, read in the page's order.  Row i = 4g' + e of
+// score tile t is key 8g' + 4t + e of the block, so that a lane's eight probabilities (tile 0, then tile
+// 1) are those of keys 8g .. 8g+7, the order in which a value operand holds them.
 struct BlockFrags {
   QFrag keys[2];
-  bf16x4 v_lo[kTilesD], v_hi[kTilesD];
+  bf16x8 values[kTilesD];
 };
 
-__device__ __forceinline__ void load_block(BlockFrags& f, const bf16_t* k_block, const bf16_t* v_block, int r, int g) {
+// k_page, v_page: the page's keys and values of one kv head
+__device__ __forceinline__ void load_block(BlockFrags& f, const bf16_t* k_page, const bf16_t* v_page, int h, int r, int g) {
 #pragma unroll
-  for (int t = 0; t < 2; ++t) f.keys[t] = load_row_operand(k_block + (size_t)(16 * t + r) * HD, g);
+  for (int t = 0; t < 2; ++t) {
+    const int key = 32 * h + 8 * (r / 4) + 4 * t + r % 4;
 #pragma unroll
-  for (int t = 0; t < kTilesD; ++t) {
-    const bf16_t* channel = v_block + (size_t)(16 * t + r) * kPageTokens + 4 * g;
-    f.v_lo[t] = *(const bf16x4*)channel;
-    f.v_hi[t] = *(const bf16x4*)(channel + 16);
+    for (int c = 0; c < kFullD; ++c) f.keys[t].full[c] = *(const bf16x8*)(k_page + nnis_k_offset(key, 32 * c + 8 * g));
+    f.keys[t].tail = kTailD ? *(const bf16x4*)(k_page + nnis_k_offset(key, 32 * kFullD + 4 * g)) : zero4();
   }
+#pragma unroll
+  for (int t = 0; t < kTilesD; ++t) f.values[t] = *(const bf16x8*)(v_page + nnis_v_offset(16 * t + r, 32 * h + 8 * g));
 }
 
 // Scores, softmax update and output update of one loaded block for C column tiles.
@@ -232,7 +245,7 @@ __device__ __forceinline__ void attend_block(AttnState<C>& st, const QFrag (&q)[
       s[t] = score_tile(f.keys[t], q[c]);
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        const int key = key0 + 16 * t + 4 * g + e;
+        const int key = key0 + 8 * g + 4 * t + e;
         s[t][e] = (key >= lo[c] && key <= hi[c]) ? s[t][e] * scale_log2 : -INFINITY;
         block_max = fmaxf(block_max, s[t][e]);
       }
@@ -254,16 +267,10 @@ __device__ __forceinline__ void attend_block(AttnState<C>& st, const QFrag (&q)[
       }
     st.l[c] = st.l[c] * alpha + sum;
     st.m[c] = m_new;
-    bf16x8 v_operand;
 #pragma unroll
     for (int t = 0; t < kTilesD; ++t) {
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        v_operand[e] = f.v_lo[t][e];
-        v_operand[4 + e] = f.v_hi[t][e];
-      }
       st.o[c][t] = st.o[c][t] * alpha;
-      st.o[c][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v_operand, p, st.o[c][t], 0, 0, 0);
+      st.o[c][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.values[t], p, st.o[c][t], 0, 0, 0);
     }
   }
 }
@@ -303,14 +310,14 @@ struct MfmaArgs {
   const int* tok_slot;    // [tokens]
   const int* tok_pos;     // [tokens]
   int splits;
-  float* partial;         // [tokens, heads, splits, HD + 2] when splits > 1
+  float* partial;         // [tokens, heads, splits, kPartial] when splits > 1: HD outputs, maximum, sum
 };
 
 __device__ __forceinline__ const bf16_t* k_page_ptr(const MfmaArgs& a, int page, int kv_head) {
-  return a.k_pages + ((size_t)page * a.kv_heads + kv_head) * kPageTokens * HD;
+  return a.k_pages + ((size_t)page * a.kv_heads + kv_head) * nnis_k_page_elems(HD);
 }
 __device__ __forceinline__ const bf16_t* v_page_ptr(const MfmaArgs& a, int page, int kv_head) {
-  return a.v_pages + ((size_t)page * a.kv_heads + kv_head) * HD * kPageTokens;
+  return a.v_pages + ((size_t)page * a.kv_heads + kv_head) * nnis_v_page_elems(HD);
 }
 
 // Waves of a block that dealt a run of key blocks among themselves: waves 1.. leave
@@ -358,9 +365,10 @@ __device__ __forceinline__ bool merge_waves(AttnState<C>& st, float* merge, int 
 
 // Runs the pages first, first + stride, ... (`mine` of them) of a sequence through the
 // softmax state, each as two blocks of 32 keys one after the other (so both halves of a
-// value line are used while it is near), the next block's operands in flight while one is
-// worked on.  Blocks that start beyond `last_key` are left out.
-template <int C>
+// value line are used while it is near).  RING blocks' operands are in flight at a time:
+// a block's place is asked for again as soon as it has been worked on, so a wave with
+// up to RING blocks waits for memory once.  Blocks that start beyond `last_key` are left out.
+template <int C, int RING>
 __device__ __forceinline__ void attend_run(AttnState<C>& st, const QFrag (&q)[C], const MfmaArgs& a, const int* pages,
                                            int kv_head, int first, int stride, int mine, int last_key,
                                            const int (&lo)[C], const int (&hi)[C], int lane) {
@@ -368,35 +376,41 @@ __device__ __forceinline__ void attend_run(AttnState<C>& st, const QFrag (&q)[C]
   const int r = lane % 16, g = lane / 16;
   const bf16_t* k_base = k_page_ptr(a, 0, kv_head);
   const bf16_t* v_base = v_page_ptr(a, 0, kv_head);
-  const size_t k_page_stride = (size_t)a.kv_heads * kPageTokens * HD, v_page_stride = (size_t)a.kv_heads * HD * kPageTokens;
+  const size_t k_page_stride = (size_t)a.kv_heads * nnis_k_page_elems(HD), v_page_stride = (size_t)a.kv_heads * nnis_v_page_elems(HD);
   PageRun run = {pages, a.max_pages, first, stride, 0};
   run.fill(lane);
   // block b of the run: page index first + (b / 2) * stride, half b % 2
   int blocks = 2 * mine;
   if ((first + (mine - 1) * stride) * kPageTokens + 32 > last_key) --blocks;  // the last page's second half is beyond the keys
-  BlockFrags current, next;
-  {
-    const int page = run.page(0);
-    load_block(current, k_base + page * k_page_stride, v_base + page * v_page_stride, r, g);
-  }
-  for (int b = 0; b < blocks; ++b) {
-    if (b + 1 < blocks) {
-      const int n = (b + 1) >> 1, inside = ((b + 1) & 1) * 32;
-      if (inside == 0 && (n & 63) == 0) {
-        run.first = first + n * stride;
-        run.fill(lane);
-      }
-      const int page = run.page(n & 63);
-      load_block(next, k_base + page * k_page_stride + (size_t)inside * HD, v_base + page * v_page_stride + inside, r, g);
+  BlockFrags ring[RING];
+  // blocks are asked for in rising order, so the 64 cached page ids move on with them
+  auto ask = [&](BlockFrags& into, int b) {
+    const int n = b >> 1;
+    if ((b & 1) == 0 && n > 0 && (n & 63) == 0) {
+      run.first = first + n * stride;
+      run.fill(lane);
     }
-    attend_block<C>(st, q, current, (first + (b >> 1) * stride) * kPageTokens + (b & 1) * 32, lo, hi, a.scale_log2, g);
-    current = next;
+    const int page = run.page(n & 63);
+    load_block(into, k_base + page * k_page_stride, v_base + page * v_page_stride, b & 1, r, g);
+  };
+#pragma unroll
+  for (int i = 0; i < RING; ++i)
+    if (i < blocks) ask(ring[i], i);
+  for (int b0 = 0; b0 < blocks; b0 += RING) {
+#pragma unroll
+    for (int i = 0; i < RING; ++i) {
+      const int b = b0 + i;
+      if (b < blocks) {
+        attend_block<C>(st, q, ring[i], (first + (b >> 1) * stride) * kPageTokens + (b & 1) * 32, lo, hi, a.scale_log2, g);
+        if (b + RING < blocks) ask(ring[i], b + RING);
+      }
+    }
   }
 }
 
 // ---- prefill: a wave = (query tile, kv head, chunk of GH query heads); C = QT * GH column tiles --------
 template <int QT, int GH>
-__global__ __launch_bounds__(512) void attention_prefill_kernel(MfmaArgs a, int waves) {
+__global__ __launch_bounds__(64 * kBlockWaves) void attention_prefill_kernel(MfmaArgs a, int waves) {
   extern __shared__ float merge[];
   constexpr int C = QT * GH;
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave, r = lane % 16, g = lane / 16;
@@ -446,7 +460,7 @@ __global__ __launch_bounds__(512) void attention_prefill_kernel(MfmaArgs a, int 
   if (last >= 0) {
     const int first_page = first / kPageTokens, page_count = last / kPageTokens + 1 - first_page;
     const int mine = page_count > wave ? (page_count - wave + waves - 1) / waves : 0;  // pages of this wave
-    attend_run<C>(st, q, a, pages, kv_head, first_page + wave, waves, mine, last, lo, hi, lane);
+    attend_run<C, 2>(st, q, a, pages, kv_head, first_page + wave, waves, mine, last, lo, hi, lane);
   }
   if (!merge_waves<C>(st, merge, wave, waves, lane)) return;
 #pragma unroll
@@ -470,10 +484,55 @@ __global__ __launch_bounds__(512) void attention_prefill_kernel(MfmaArgs a, int 
     }
 }
 
-// ---- decode: a block = (token, kv head, split of the keys); columns are the heads of the group; ------
-// the block's waves deal the split's key blocks among themselves and merge their states through LDS
+// The end of a decode block: the waves' states merge in LDS; the wave that is left writes the output
+// (one split) or leaves its state in `partial` for the combine kernel.
 template <int C>
-__global__ __launch_bounds__(512) void attention_decode_kernel(MfmaArgs a, int waves) {
+__device__ __forceinline__ void finish_decode(AttnState<C>& st, const bool (&live)[C], const MfmaArgs& a, float* merge,
+                                              int token, int kv_head, int split, int wave, int waves, int lane) {
+  const int r = lane % 16, g = lane / 16;
+  const int group = a.heads / a.kv_heads;
+  if (!merge_waves<C>(st, merge, wave, waves, lane)) return;  // one wave is left
+  float total[C];
+#pragma unroll
+  for (int c = 0; c < C; ++c) {
+    total[c] = st.l[c];
+    total[c] += __shfl_xor(total[c], 16, kWave);
+    total[c] += __shfl_xor(total[c], 32, kWave);
+  }
+  if (a.splits == 1) {
+#pragma unroll
+    for (int c = 0; c < C; ++c) {
+      if (!live[c]) continue;
+      const float inv = 1.0f / total[c];
+      bf16_t* dst = a.out + ((size_t)token * a.heads + kv_head * group + 16 * c + r) * HD;
+#pragma unroll
+      for (int t = 0; t < kTilesD; ++t) {
+        bf16x4 packed;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) packed[e] = (__bf16)(st.o[c][t][e] * inv);
+        *(bf16x4*)(dst + 16 * t + 4 * g) = packed;
+      }
+    }
+    return;
+  }
+#pragma unroll
+  for (int c = 0; c < C; ++c) {
+    if (!live[c]) continue;
+    float* dst = a.partial + (((size_t)token * a.heads + kv_head * group + 16 * c + r) * a.splits + split) * kPartial;
+#pragma unroll
+    for (int t = 0; t < kTilesD; ++t) *(f32x4*)(dst + 16 * t + 4 * g) = st.o[c][t];
+    if (g == 0) {
+      dst[HD] = st.m[c];
+      dst[HD + 1] = total[c];
+    }
+  }
+}
+
+// ---- decode: a block = (token, kv head, split of the keys); columns are the heads of the group; ------
+// the block's waves deal the split's pages among themselves and merge their states through LDS.  With
+// more than one split every block leaves its state in `partial` for the combine kernel.
+template <int C>
+__global__ __launch_bounds__(64 * kBlockWaves) void attention_decode_kernel(MfmaArgs a, int waves) {
   extern __shared__ float merge[];  // [waves - 1][C][kTilesD * 4 + 2][64]
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave, r = lane % 16, g = lane / 16;
   const int token = blockIdx.x, kv_head = blockIdx.y, split = blockIdx.z;
@@ -504,49 +563,191 @@ __global__ __launch_bounds__(512) void attention_decode_kernel(MfmaArgs a, int w
   AttnState<C> st;
   init_state(st);
   const int mine = end > begin + wave ? (end - begin - wave + waves - 1) / waves : 0;  // pages of this wave
-  attend_run<C>(st, q, a, pages, kv_head, begin + wave, waves, mine, pos, lo, hi, lane);
-  if (!merge_waves<C>(st, merge, wave, waves, lane)) return;
+  attend_run<C, (kDecodeRing / C >= 2 ? kDecodeRing / C : 2)>(st, q, a, pages, kv_head, begin + wave, waves, mine, pos, lo, hi, lane);
+  finish_decode<C>(st, live, a, merge, token, kv_head, split, wave, waves, lane);
+}
+
+// ---- decode with keys on lanes, for groups of up to 4 query heads ------------------------------------
+// The kernel above spends a lane on every (key, column) pair of a 16-column tile, of which a small
+// group fills a few.  Here scores are taken with v_mfma_f32_4x4x4_16B_bf16, sixteen products of 4x4
+// at a time: block b of the instruction multiplies keys 4b .. 4b+3 of a page (first operand: lane l
+// holds 4 channels of key l) by the group's heads (second operand: lane 4b+j holds the same channels
+// of head j), so lane 4b+j ends up with the scores of its head for its four keys and the softmax
+// arithmetic of a page of 64 keys x 4 heads is four values a lane.  The probabilities go through LDS
+// into the columns operand of the 16x16x32 product with the value page, whose outputs and end are
+// those of the kernel above (heads in columns 0..3).  All lanes of a head share one reference of the
+// softmax, which moves only when a score rises more than kLazyRise above it (then every lane's
+// sums are scaled, as in the running maximum; until then they are sums of 2^(score - reference) with
+// terms up to 2^kLazyRise, which changes no result beyond rounding).
+#if NNIS_HEAD_DIM <= 128
+struct KeysPage {
+  bf16x8 k[HD / 8];        // this lane's key, all channels
+  bf16x8 v[2][kTilesD];    // value operands of the two halves of the page
+};
+
+__device__ __forceinline__ void load_keys_page(KeysPage& f, const bf16_t* k_page, const bf16_t* v_page, int lane) {
+  const int r = lane % 16, g = lane / 16;
 #pragma unroll
-  for (int c = 0; c < C; ++c) {
-    float total = st.l[c];
-    total += __shfl_xor(total, 16, kWave);
-    total += __shfl_xor(total, 32, kWave);
-    if (!live[c]) continue;
-    const int head = kv_head * group + 16 * c + r;
-    if (a.splits == 1) {
-      const float inv = 1.0f / total;
-      bf16_t* dst = a.out + ((size_t)token * a.heads + head) * HD;
+  for (int c = 0; c < HD / 8; ++c) f.k[c] = *(const bf16x8*)(k_page + nnis_k_offset(lane, 8 * c));
 #pragma unroll
-      for (int t = 0; t < kTilesD; ++t) {
-        bf16x4 packed;
+  for (int h = 0; h < 2; ++h)
 #pragma unroll
-        for (int e = 0; e < 4; ++e) packed[e] = (__bf16)(st.o[c][t][e] * inv);
-        *(bf16x4*)(dst + 16 * t + 4 * g) = packed;
-      }
-    } else {
-      float* dst = a.partial + (((size_t)token * a.heads + head) * a.splits + split) * (HD + 2);
+    for (int t = 0; t < kTilesD; ++t) f.v[h][t] = *(const bf16x8*)(v_page + nnis_v_offset(16 * t + r, 32 * h + 8 * g));
+}
+
+__device__ __forceinline__ bf16x4 low4(bf16x8 v) { return __builtin_shufflevector(v, v, 0, 1, 2, 3); }
+__device__ __forceinline__ bf16x4 high4(bf16x8 v) { return __builtin_shufflevector(v, v, 4, 5, 6, 7); }
+
+__global__ __launch_bounds__(64 * kKeysWaves) void attention_decode_keys_kernel(MfmaArgs a, int waves) {
+  extern __shared__ float merge[];  // [waves - 1][kTilesD * 4 + 2][64]
+  constexpr int kStageRow = kPageTokens + 8;  // bfloat16 per head: a page's probabilities, rows apart in the banks
+  __shared__ __attribute__((aligned(16))) bf16_t stage[kKeysWaves][4][kStageRow];
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave, r = lane % 16, g = lane / 16;
+  const int blk = lane / 4, j = lane % 4;  // the scores' layout: keys 4 blk .. 4 blk + 3 of a page, head j of the group
+  const int token = blockIdx.x, kv_head = blockIdx.y, split = blockIdx.z;
+  const int slot = a.tok_slot[token];
+  if (slot < 0) return;  // a padding row (the whole block leaves): its output is never read
+  const int group = a.heads / a.kv_heads;
+  const int pos = a.tok_pos[token];
+  const int first_key = (a.window > 0 && pos + 1 > a.window) ? pos + 1 - a.window : 0;
+  const int* pages = a.block_table + (size_t)slot * a.max_pages;
+
+  // the query of head j, all channels (heads beyond the group: zeros, their columns are never written)
+  bf16x8 q[HD / 8];
+  {
+    const bf16_t* row = a.q + ((size_t)token * a.heads + kv_head * group + (j < group ? j : 0)) * HD;
 #pragma unroll
-      for (int t = 0; t < kTilesD; ++t) *(f32x4*)(dst + 16 * t + 4 * g) = st.o[c][t];
-      if (g == 0) {
-        dst[HD] = st.m[c];
-        dst[HD + 1] = total;
+    for (int c = 0; c < HD / 8; ++c) {
+      q[c] = *(const bf16x8*)(row + 8 * c);
+      if (j >= group) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) q[c][e] = (__bf16)0.0f;
       }
     }
   }
-}
+  const int page_first = first_key / kPageTokens, page_count = pos / kPageTokens + 1 - page_first;
+  const int per_split = (page_count + a.splits - 1) / a.splits;
+  const int begin = page_first + split * per_split;
+  const int end = min(begin + per_split, page_first + page_count);
+  const int mine = end > begin + wave ? (end - begin - wave + waves - 1) / waves : 0;  // pages of this wave
+  const int first = begin + wave, stride = waves;
 
-// sums the splits of one (token, head): out = sum_s O_s 2^(m_s - M) / sum_s l_s 2^(m_s - M)
+  AttnState<1> st;
+  init_state(st);
+  float reference = -INFINITY;  // of head j; equal in all lanes of the head
+  float sum = 0.0f;             // this lane's part of the head's sum
+  if (mine > 0) {
+    const bf16_t* k_base = k_page_ptr(a, 0, kv_head);
+    const bf16_t* v_base = v_page_ptr(a, 0, kv_head);
+    const size_t k_page_stride = (size_t)a.kv_heads * nnis_k_page_elems(HD), v_page_stride = (size_t)a.kv_heads * nnis_v_page_elems(HD);
+    PageRun run = {pages, a.max_pages, first, stride, 0};
+    run.fill(lane);
+    KeysPage ring[kKeysRing];
+    auto ask = [&](KeysPage& into, int n) {
+      if (n > 0 && (n & 63) == 0) {
+        run.first = first + n * stride;
+        run.fill(lane);
+      }
+      const int page = run.page(n & 63);
+      load_keys_page(into, k_base + page * k_page_stride, v_base + page * v_page_stride, lane);
+    };
+    bf16_t* mine_stage = &stage[wave][0][0];
+#pragma unroll
+    for (int i = 0; i < kKeysRing; ++i)
+      if (i < mine) ask(ring[i], i);
+    for (int n0 = 0; n0 < mine; n0 += kKeysRing) {
+#pragma unroll
+      for (int i = 0; i < kKeysRing; ++i) {
+        const int n = n0 + i;
+        if (n >= mine) continue;
+        const KeysPage& f = ring[i];
+        const int key0 = (first + n * stride) * kPageTokens;
+        // scores of this lane's head for keys key0 + 4 blk + (0..3): two chains of products, added
+        f32x4 s0 = {0.0f, 0.0f, 0.0f, 0.0f}, s1 = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int c = 0; c < HD / 8; ++c) {
+          s0 = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(low4(f.k[c]), low4(q[c]), s0, 0, 0, 0);
+          s1 = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(high4(f.k[c]), high4(q[c]), s1, 0, 0, 0);
+        }
+        f32x4 s = s0 + s1;
+        const bool inside = key0 >= first_key && key0 + kPageTokens - 1 <= pos;  // every key of the page is read
+        float top = -INFINITY;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int key = key0 + 4 * blk + e;
+          s[e] = (inside || (key >= first_key && key <= pos)) ? s[e] * a.scale_log2 : -INFINITY;
+          top = fmaxf(top, s[e]);
+        }
+        if (__any(top > reference + kLazyRise)) {  // also the first page, whose reference is -inf
+          float moved = fmaxf(reference, top);
+#pragma unroll
+          for (int offset = 4; offset < kWave; offset <<= 1) moved = fmaxf(moved, __shfl_xor(moved, offset, kWave));
+          // the lanes 16 g + r with r < 4 hold head r in both layouts: the outputs are scaled by the same factor
+          const float shrink = reference == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(reference - moved);
+          sum *= shrink;
+#pragma unroll
+          for (int t = 0; t < kTilesD; ++t) st.o[0][t] = st.o[0][t] * shrink;
+          reference = moved;
+        }
+        const float base = reference == -INFINITY ? 0.0f : reference;
+        bf16x4 p;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float w = __builtin_amdgcn_exp2f(s[e] - base);
+          sum += w;
+          p[e] = (__bf16)w;
+        }
+        // through LDS into the columns operand: column = head, 8 consecutive keys a lane
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();  // the reads of the page before are done
+        *(bf16x4*)(mine_stage + j * kStageRow + 4 * blk) = p;
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          bf16x8 columns = *(const bf16x8*)(mine_stage + (r < 4 ? r : 0) * kStageRow + 32 * h + 8 * g);
+          if (r >= 4) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) columns[e] = (__bf16)0.0f;
+          }
+#pragma unroll
+          for (int t = 0; t < kTilesD; ++t)
+            st.o[0][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.v[h][t], columns, st.o[0][t], 0, 0, 0);
+        }
+        if (n + kKeysRing < mine) ask(ring[i], n + kKeysRing);
+      }
+    }
+  }
+  // into the state the end works on: a column's maximum in its lanes, and parts of its sum that add up over
+  // the lane groups g -- the lanes 16 g + r, r < 4, take the sums of the blocks 4 g .. 4 g + 3 of head r
+  sum += __shfl_xor(sum, 4, kWave);
+  sum += __shfl_xor(sum, 8, kWave);
+  st.m[0] = reference;
+  st.l[0] = sum;
+  bool live[1] = {r < group && r < 4};
+  if (r >= 4) {  // columns that hold no head
+    st.m[0] = -INFINITY;
+    st.l[0] = 0.0f;
+  }
+  finish_decode<1>(st, live, a, merge, token, kv_head, split, wave, waves, lane);
+}
+#endif  // NNIS_HEAD_DIM <= 128
+
+// sums the splits of one (token, head): out = sum_s O_s 2^(m_s - M) / sum_s l_s 2^(m_s - M).
+// A kernel of its own: letting the last block of a (token, kv head) do it needs a device-wide fence in
+// every block, which was measured several times dearer than this launch.
 __global__ void attention_combine_kernel(const float* __restrict__ partial, bf16_t* __restrict__ out,
                                          const int* __restrict__ tok_slot, int heads, int splits) {
   const int token = blockIdx.x, head = blockIdx.y;
   if (tok_slot[token] < 0) return;
-  const float* base = partial + ((size_t)token * heads + head) * splits * (HD + 2);
+  const float* base = partial + ((size_t)token * heads + head) * splits * kPartial;
   float m_all = -INFINITY;
-  for (int s = 0; s < splits; ++s) m_all = fmaxf(m_all, base[(size_t)s * (HD + 2) + HD]);
+  for (int s = 0; s < splits; ++s) m_all = fmaxf(m_all, base[(size_t)s * kPartial + HD]);
   for (int d = threadIdx.x; d < HD; d += blockDim.x) {
     float num = 0.0f, den = 0.0f;
     for (int s = 0; s < splits; ++s) {
-      const float* p = base + (size_t)s * (HD + 2);
+      const float* p = base + (size_t)s * kPartial;
       const float m = p[HD];
       const float w = m == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(m - m_all);
       num += p[d] * w;
@@ -634,7 +835,8 @@ extern "C" int nnis_attention_prefill_max_waves(int heads, int kv_heads, int col
   prefill_shape(heads, kv_heads, columns, &qt, &gh);
   const size_t per_wave = (size_t)qt * gh * (kTilesD * 4 + 2) * kWave * sizeof(float);
   const int waves = 1 + (int)(65536 / per_wave);
-  return waves >= 8 ? 8 : (waves >= 4 ? 4 : (waves >= 2 ? 2 : 1));
+  const int fit = waves >= 8 ? 8 : (waves >= 4 ? 4 : (waves >= 2 ? 2 : 1));
+  return fit < kBlockWaves ? fit : kBlockWaves;
 }
 
 extern "C" int nnis_attention_prefill_bf16(const void* q, void* out, const void* k_pages, const void* v_pages,
@@ -653,40 +855,62 @@ extern "C" int nnis_attention_prefill_bf16(const void* q, void* out, const void*
   const dim3 grid(tiles, kv_heads * chunks);
   NNIS_REQUIRE(grid.y <= 65535, "attention: %d head chunks exceed the grid limit", grid.y);
   const size_t per_wave = (size_t)qt * gh * (kTilesD * 4 + 2) * kWave * sizeof(float);
-  NNIS_REQUIRE(waves >= 1 && waves <= 8 && (waves - 1) * per_wave <= 65536,
+  NNIS_REQUIRE(waves >= 1 && waves <= kBlockWaves && (waves - 1) * per_wave <= 65536,
                "attention: %d waves a block do not fit this head size (LDS)", waves);
   const size_t lds = (waves - 1) * per_wave;
   const dim3 block(kWave * waves);
   hipStream_t s = (hipStream_t)stream;
-  if (qt == 4 && gh == 1) hipLaunchKernelGGL((attention_prefill_kernel<4, 1>), grid, block, lds, s, a, waves);
-  else if (qt == 2 && gh == 2) hipLaunchKernelGGL((attention_prefill_kernel<2, 2>), grid, block, lds, s, a, waves);
-  else if (qt == 2 && gh == 1) hipLaunchKernelGGL((attention_prefill_kernel<2, 1>), grid, block, lds, s, a, waves);
-  else if (qt == 1 && gh == 3) hipLaunchKernelGGL((attention_prefill_kernel<1, 3>), grid, block, lds, s, a, waves);
-  else if (qt == 1 && gh == 4) hipLaunchKernelGGL((attention_prefill_kernel<1, 4>), grid, block, lds, s, a, waves);
-  else if (qt == 1 && gh == 2) hipLaunchKernelGGL((attention_prefill_kernel<1, 2>), grid, block, lds, s, a, waves);
-  else if (qt == 1 && gh == 1) hipLaunchKernelGGL((attention_prefill_kernel<1, 1>), grid, block, lds, s, a, waves);
-  else return nnis_fail("attention: no kernel for %d query tiles x %d heads", qt, gh);
+  bool launched = true;
+  if constexpr (kMaxColumns >= 4) {
+    if (qt == 4 && gh == 1) hipLaunchKernelGGL((attention_prefill_kernel<4, 1>), grid, block, lds, s, a, waves);
+    else if (qt == 2 && gh == 2) hipLaunchKernelGGL((attention_prefill_kernel<2, 2>), grid, block, lds, s, a, waves);
+    else if (qt == 1 && gh == 3) hipLaunchKernelGGL((attention_prefill_kernel<1, 3>), grid, block, lds, s, a, waves);
+    else if (qt == 1 && gh == 4) hipLaunchKernelGGL((attention_prefill_kernel<1, 4>), grid, block, lds, s, a, waves);
+    else launched = false;
+  } else {
+    launched = false;
+  }
+  if (!launched) {
+    launched = true;
+    if constexpr (kMaxColumns >= 2) {
+      if (qt == 2 && gh == 1) hipLaunchKernelGGL((attention_prefill_kernel<2, 1>), grid, block, lds, s, a, waves);
+      else if (qt == 1 && gh == 2) hipLaunchKernelGGL((attention_prefill_kernel<1, 2>), grid, block, lds, s, a, waves);
+      else launched = false;
+    } else {
+      launched = false;
+    }
+  }
+  if (!launched) {
+    if (qt == 1 && gh == 1) hipLaunchKernelGGL((attention_prefill_kernel<1, 1>), grid, block, lds, s, a, waves);
+    else return nnis_fail("attention: no kernel for %d query tiles x %d heads", qt, gh);
+  }
   NNIS_LAUNCH_CHECK("attention_prefill");
   return 0;
 }
 
-// partial: float32 scratch of at least tokens * heads * splits * (head_dim + 2), needed when splits > 1
 extern "C" int nnis_attention_decode_max_waves(int heads, int kv_heads) {
   const int group = heads / (kv_heads > 0 ? kv_heads : 1);
   const int tiles = (group + 15) / 16;
   const int per_wave = tiles * (kTilesD * 4 + 2) * kWave * 4;  // bytes of LDS a wave beyond the first needs
-  int waves = 1 + 65536 / per_wave;
-  return waves > 8 ? 8 : (waves >= 4 ? 4 : (waves >= 2 ? 2 : 1));
+  const int waves = 1 + 65536 / per_wave;
+  const int fit = waves >= 8 ? 8 : (waves >= 4 ? 4 : (waves >= 2 ? 2 : 1));
+  const int most = (group <= 4 && HD <= kKeysMaxHD && kKeysWaves < kBlockWaves) ? kKeysWaves : kBlockWaves;
+  return fit < most ? fit : most;
 }
 
+// With splits > 1 the call needs scratch memory: `partial`, float32 of at least tokens * heads * splits *
+// (head_dim + 4), contents of no matter.  Two calls that run at the same time must not share it.
+// kind: 0 picks the kernel (keys on lanes for groups of up to 4 heads, else heads in columns); 1 and 2 ask
+// for columns or keys on lanes and fail where that kernel does not take the sizes.
 extern "C" int nnis_attention_decode_bf16(const void* q, void* out, const void* k_pages, const void* v_pages,
                                           const int* block_table, int max_pages, const int* tok_slot, const int* tok_pos,
                                           int tokens, int heads, int kv_heads, int head_dim, int window, float scale,
-                                          int splits, int waves, float* partial, void* stream) {
+                                          int splits, int waves, float* partial, int kind, void* stream) {
   MfmaArgs a;
   if (fill_common(a, q, out, k_pages, v_pages, block_table, max_pages, heads, kv_heads, head_dim, window, scale)) return 1;
   NNIS_REQUIRE(splits >= 1 && splits <= 65535, "attention: bad number of splits %d", splits);
   NNIS_REQUIRE(splits == 1 || partial != nullptr, "attention: splits need scratch memory");
+  NNIS_REQUIRE((uintptr_t)partial % 16 == 0, "attention: scratch memory must be 16-byte aligned");
   NNIS_REQUIRE(kv_heads <= 65535, "attention: %d kv heads exceed the grid limit", kv_heads);
   NNIS_REQUIRE(waves >= 1 && waves <= nnis_attention_decode_max_waves(heads, kv_heads),
                "attention: %d waves a block; this head size and group take at most %d", waves,
@@ -695,14 +919,32 @@ extern "C" int nnis_attention_decode_bf16(const void* q, void* out, const void* 
   const int group = heads / kv_heads;
   NNIS_REQUIRE(group <= 16 * kMaxColumns, "attention: a group of %d query heads is more than this head size's decode kernel carries (%d)",
                group, 16 * kMaxColumns);
+  NNIS_REQUIRE(kind >= 0 && kind <= 2, "attention: unknown decode kernel %d", kind);
+  const bool keys_fit = group <= 4 && HD <= kKeysMaxHD;
+  NNIS_REQUIRE(kind != 2 || keys_fit, "attention: the kernel with keys on lanes takes groups of up to 4 heads of up to %d channels",
+               kKeysMaxHD);
   a.tok_slot = tok_slot; a.tok_pos = tok_pos; a.splits = splits; a.partial = partial;
   const dim3 grid(tokens, kv_heads, splits);
   hipStream_t s = (hipStream_t)stream;
   const int tiles = (group + 15) / 16;
   const size_t lds = (size_t)(waves - 1) * tiles * (kTilesD * 4 + 2) * kWave * sizeof(float);
+#if NNIS_HEAD_DIM <= 128
+  {
+    if (kind == 2 || (kind == 0 && keys_fit)) {
+      hipLaunchKernelGGL(attention_decode_keys_kernel, grid, dim3(kWave * waves), lds, s, a, waves);
+      NNIS_LAUNCH_CHECK("attention_decode");
+      if (splits > 1) {
+        hipLaunchKernelGGL(attention_combine_kernel, dim3(tokens, heads), dim3(HD < 64 ? 64 : (HD > 256 ? 256 : HD)), 0, s,
+                           partial, (bf16_t*)out, tok_slot, heads, splits);
+        NNIS_LAUNCH_CHECK("attention_combine");
+      }
+      return 0;
+    }
+  }
+#endif
   if (tiles == 1) hipLaunchKernelGGL((attention_decode_kernel<1>), grid, dim3(kWave * waves), lds, s, a, waves);
   else if (tiles == 2) hipLaunchKernelGGL((attention_decode_kernel<(kMaxColumns >= 2 ? 2 : 1)>), grid, dim3(kWave * waves), lds, s, a, waves);
-  else hipLaunchKernelGGL((attention_decode_kernel<kMaxColumns>), grid, dim3(kWave * waves), lds, s, a, waves);
+  else hipLaunchKernelGGL((attention_decode_kernel<kMaxColumns>), grid, dim3(kWave * waves), lds, s, a, waves);  // 3 or 4 tiles
   NNIS_LAUNCH_CHECK("attention_decode");
   if (splits > 1) {
     hipLaunchKernelGGL(attention_combine_kernel, dim3(tokens, heads), dim3(HD < 64 ? 64 : (HD > 256 ? 256 : HD)), 0, s, partial,
@@ -720,7 +962,7 @@ extern "C" int nnis_attention_prefill_bf16(const void*, void*, const void*, cons
 }
 extern "C" int nnis_attention_decode_max_waves(int, int) { return 1; }
 extern "C" int nnis_attention_decode_bf16(const void*, void*, const void*, const void*, const int*, int, const int*, const int*,
-                                          int, int, int, int, int, float, int, int, float*, void*) {
+                                          int, int, int, int, int, float, int, int, float*, int, void*) {
   return nnis_fail("attention: the matrix-core kernels need a head size in steps of 16; this module has %d", NNIS_HEAD_DIM);
 }
 #endif

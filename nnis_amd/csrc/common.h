@@ -17,6 +17,20 @@ enum : int { NNIS_F32 = 0, NNIS_BF16 = 1 };
 constexpr int kWave = 64;        // lanes of a gfx950 wavefront
 constexpr int kPageTokens = 64;  // tokens a cache page holds
 
+// Where a page keeps its 64 tokens of one key/value head, in elements.  Both orders are those in which the
+// attention kernels' wave-wide 16-byte loads read: consecutive lanes, consecutive memory.
+//   keys    [chunk of 8 channels][token][8 channels]
+//   values  [tile of 16 channels][half of 32 tokens][group of 8 tokens][channel of the tile][8 tokens]
+// A head size that is no multiple of 8 (16) leaves the last chunk (tile) partly unused.
+__host__ __device__ constexpr size_t nnis_k_page_elems(int head_dim) { return (size_t)((head_dim + 7) / 8) * kPageTokens * 8; }
+__host__ __device__ constexpr size_t nnis_v_page_elems(int head_dim) { return (size_t)((head_dim + 15) / 16) * kPageTokens * 16; }
+__host__ __device__ constexpr size_t nnis_k_offset(int token, int channel) {
+  return (size_t)(channel / 8) * (kPageTokens * 8) + (size_t)token * 8 + channel % 8;
+}
+__host__ __device__ constexpr size_t nnis_v_offset(int channel, int token) {
+  return ((((size_t)(channel / 16) * 2 + token / 32) * 4 + (token % 32) / 8) * 16 + channel % 16) * 8 + token % 8;
+}
+
 extern thread_local char g_nnis_error[512];
 
 static inline int nnis_fail(const char* fmt, ...) {

@@ -260,19 +260,19 @@ __global__ void rope_kv_write_kernel(RopeWriteArgs a) {
       if (hi_index >= 0) store_from_f32(a.q_out, a.q_dtype, dst + hi_index, hi);
     } else if (page >= 0) {
       const int kv_head = head - a.heads;
-      const size_t dst = (((size_t)page * a.kv_heads + kv_head) * kPageTokens + in_page) * hd;
-      store_from_f32(a.k_pages, a.cache_dtype, dst + lo_index, lo);
-      if (hi_index >= 0) store_from_f32(a.k_pages, a.cache_dtype, dst + hi_index, hi);
+      const size_t dst = ((size_t)page * a.kv_heads + kv_head) * nnis_k_page_elems(hd);
+      store_from_f32(a.k_pages, a.cache_dtype, dst + nnis_k_offset(in_page, lo_index), lo);
+      if (hi_index >= 0) store_from_f32(a.k_pages, a.cache_dtype, dst + nnis_k_offset(in_page, hi_index), hi);
     }
   }
-  // values: copied, transposed into the page
+  // values: copied into the page's order
   if (page >= 0) {
     const size_t v_src = in_base + (size_t)(a.heads + a.kv_heads) * hd;
     for (int item = threadIdx.x; item < a.kv_heads * hd; item += blockDim.x) {
       const int kv_head = item / hd;
       const int d = item % hd;
       const float v = load_as_f32(a.qkv, a.qkv_dtype, v_src + item);
-      const size_t dst = (((size_t)page * a.kv_heads + kv_head) * hd + d) * kPageTokens + in_page;
+      const size_t dst = ((size_t)page * a.kv_heads + kv_head) * nnis_v_page_elems(hd) + nnis_v_offset(d, in_page);
       store_from_f32(a.v_pages, a.cache_dtype, dst, v);
     }
   }
@@ -301,13 +301,16 @@ __global__ void rope_kv_write_bf16_kernel(RopeWriteArgs a) {
     if (item < rot_items) {
       const int head = item / groups_per_head;
       const int e = (item % groups_per_head) * 4;
-      bf16_t* dst;
+      // where 4 channels from channel `ch` on go: a query row, or the key page (4 channels lie within a chunk of 8)
+      bf16_t* q_row = nullptr;
+      bf16_t* k_page = nullptr;
       if (head < a.heads) {
-        dst = (bf16_t*)a.q_out + ((size_t)token * a.heads + head) * hd;
+        q_row = (bf16_t*)a.q_out + ((size_t)token * a.heads + head) * hd;
       } else {
         if (page < 0) continue;
-        dst = (bf16_t*)a.k_pages + (((size_t)page * a.kv_heads + (head - a.heads)) * kPageTokens + in_page) * hd;
+        k_page = (bf16_t*)a.k_pages + ((size_t)page * a.kv_heads + (head - a.heads)) * nnis_k_page_elems(hd);
       }
+      auto place = [&](int ch) { return q_row ? q_row + ch : k_page + nnis_k_offset(in_page, ch); };
       const bf16_t* x = src + (size_t)head * hd;
       if (e < half) {
         const bf16x4_t x0 = *(const bf16x4_t*)(x + e), x1 = *(const bf16x4_t*)(x + e + half);
@@ -323,19 +326,19 @@ __global__ void rope_kv_write_bf16_kernel(RopeWriteArgs a) {
           lo[j] = (__bf16)(f0 * c[j] - f1 * sn[j]);
           hi[j] = (__bf16)(f1 * c[j] + f0 * sn[j]);
         }
-        *(bf16x4_t*)(dst + e) = lo;
-        *(bf16x4_t*)(dst + e + half) = hi;
+        *(bf16x4_t*)place(e) = lo;
+        *(bf16x4_t*)place(e + half) = hi;
       } else {
-        *(bf16x4_t*)(dst + e + half) = *(const bf16x4_t*)(x + e + half);  // channels at and beyond rot_dim
+        *(bf16x4_t*)place(e + half) = *(const bf16x4_t*)(x + e + half);  // channels at and beyond rot_dim
       }
     } else {
       const int v_item = item - rot_items;
       const int kv_head = v_item / (hd / 4);
       const int d = (v_item % (hd / 4)) * 4;
       const bf16x4_t v = *(const bf16x4_t*)(src + (size_t)(a.heads + a.kv_heads + kv_head) * hd + d);
-      bf16_t* dst = (bf16_t*)a.v_pages + (((size_t)page * a.kv_heads + kv_head) * hd + d) * kPageTokens + in_page;
+      bf16_t* dst = (bf16_t*)a.v_pages + ((size_t)page * a.kv_heads + kv_head) * nnis_v_page_elems(hd);
 #pragma unroll
-      for (int j = 0; j < 4; ++j) dst[(size_t)j * kPageTokens] = v[j];
+      for (int j = 0; j < 4; ++j) dst[nnis_v_offset(d + j, in_page)] = v[j];
     }
   }
 }

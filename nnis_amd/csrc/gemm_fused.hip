@@ -318,17 +318,16 @@ __global__ __launch_bounds__(KSPLIT > 4 ? 64 * KSPLIT : 256) void gemm_fused_ker
           *(bf16x4*)(dst + f0) = out_lo;
           *(bf16x4*)(dst + f0 + half) = out_hi;
         } else if (page >= 0) {
-          bf16_t* dst = a.k_pages + (((size_t)page * a.kv_heads + (head - a.heads)) * kPageTokens + pos % kPageTokens) * hd;
-          *(bf16x4*)(dst + f0) = out_lo;
-          *(bf16x4*)(dst + f0 + half) = out_hi;
+          bf16_t* dst = a.k_pages + ((size_t)page * a.kv_heads + (head - a.heads)) * nnis_k_page_elems(hd);
+          *(bf16x4*)(dst + nnis_k_offset(pos % kPageTokens, f0)) = out_lo;  // 4 channels lie within a chunk of 8
+          *(bf16x4*)(dst + nnis_k_offset(pos % kPageTokens, f0 + half)) = out_hi;
         }
-      } else if (page >= 0) {  // values are stored as they are, keys contiguous per channel
-        bf16_t* dst = a.v_pages + ((size_t)page * a.kv_heads + (head - a.heads - a.kv_heads)) * hd * kPageTokens +
-                      pos % kPageTokens;
+      } else if (page >= 0) {  // values are stored as they are
+        bf16_t* dst = a.v_pages + ((size_t)page * a.kv_heads + (head - a.heads - a.kv_heads)) * nnis_v_page_elems(hd);
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          dst[(size_t)(f0 + e) * kPageTokens] = (bf16_t)lo[e];
-          dst[(size_t)(f0 + half + e) * kPageTokens] = (bf16_t)hi[e];
+          dst[nnis_v_offset(f0 + e, pos % kPageTokens)] = (bf16_t)lo[e];
+          dst[nnis_v_offset(f0 + half + e, pos % kPageTokens)] = (bf16_t)hi[e];
         }
       }
     }

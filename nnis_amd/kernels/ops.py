@@ -10,6 +10,7 @@ from typing import Optional
 
 import torch
 
+from ..cache.layout import k_page_shape, v_page_shape
 from ..errors import KernelError
 from . import lib as _lib
 
@@ -41,11 +42,17 @@ _ATTN_SIGNATURES = {
                                     _INT, _INT, _INT, _FLT, _INT, _INT, _VOID],
     "nnis_attention_prefill_max_waves": [_INT, _INT, _INT],
     "nnis_attention_decode_bf16": [_VOID, _VOID, _VOID, _VOID, _VOID, _INT, _VOID, _VOID, _INT, _INT, _INT, _INT, _INT, _FLT,
-                                   _INT, _INT, _VOID, _VOID],
+                                   _INT, _INT, _VOID, _INT, _VOID],
     "nnis_attention_decode_max_waves": [_INT, _INT],
 }
 
 _DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1}
+
+
+def _pages_fit(k_pages: torch.Tensor, v_pages: torch.Tensor, kv_heads: int, head_dim: int) -> bool:
+    """Key and value pages [pages, ...] in the cache's layout for these sizes, contiguous."""
+    return (tuple(k_pages.shape[1:]) == k_page_shape(kv_heads, head_dim) and tuple(v_pages.shape[1:]) == v_page_shape(kv_heads, head_dim)
+            and k_pages.is_contiguous() and v_pages.is_contiguous() and k_pages.shape[0] == v_pages.shape[0])
 
 
 def _code(t: torch.Tensor) -> int:
@@ -176,7 +183,7 @@ def rope_kv_write(qkv: torch.Tensor, q_out: torch.Tensor, cos: Optional[torch.Te
     cache_code = 0
     if k_pages is not None:
         _dev(k_pages, "k_pages"), _dev(v_pages, "v_pages"), _dev(block_table, "block_table")
-        if tuple(k_pages.shape[1:]) != (kv_heads, PAGE_TOKENS, head_dim) or tuple(v_pages.shape[1:]) != (kv_heads, head_dim, PAGE_TOKENS):
+        if not _pages_fit(k_pages, v_pages, kv_heads, head_dim):
             raise KernelError(f"rope_kv_write: page shapes {tuple(k_pages.shape)} / {tuple(v_pages.shape)} do not fit")
         if block_table.dtype != torch.int32 or block_table.dim() != 2:
             raise KernelError("rope_kv_write: block_table must be int32 [slots, pages]")
@@ -233,7 +240,7 @@ def attention_rows(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_
     tokens = q.shape[0]
     if q.shape != (tokens, heads * head_dim) or out.shape != q.shape:
         raise KernelError(f"attention: q {tuple(q.shape)} / out {tuple(out.shape)} do not fit {heads} heads of {head_dim}")
-    if tuple(k_pages.shape[1:]) != (kv_heads, PAGE_TOKENS, head_dim) or tuple(v_pages.shape[1:]) != (kv_heads, head_dim, PAGE_TOKENS):
+    if not _pages_fit(k_pages, v_pages, kv_heads, head_dim):
         raise KernelError(f"attention: page shapes {tuple(k_pages.shape)} / {tuple(v_pages.shape)} do not fit")
     if k_pages.dtype != v_pages.dtype:
         raise KernelError("attention: key and value pages differ in type")
@@ -303,8 +310,7 @@ def gemm_fused(x_in: torch.Tensor, delta: Optional[torch.Tensor], x_out: Optiona
             kp, vp, bt = r["k_pages"], r["v_pages"], r["block_table"]
             _dev(kp, "k_pages"), _dev(vp, "v_pages"), _dev(bt, "block_table")
             if (kp.dtype != torch.bfloat16 or vp.dtype != torch.bfloat16 or bt.dtype != torch.int32
-                    or tuple(kp.shape[1:]) != (r["kv_heads"], PAGE_TOKENS, r["head_dim"])
-                    or tuple(vp.shape[1:]) != (r["kv_heads"], r["head_dim"], PAGE_TOKENS)):
+                    or not _pages_fit(kp, vp, r["kv_heads"], r["head_dim"])):
                 raise KernelError("gemm_fused: cache pages must be bfloat16 in the cache's layout, the block table int32")
     if expect is None or tuple(y.shape) != expect:
         raise KernelError(f"gemm_fused: y {tuple(y.shape)} does not fit epilogue {epilogue} (expected {expect})")
@@ -337,7 +343,7 @@ def _check_pages(q, out, k_pages, v_pages, block_table, heads, kv_heads, head_di
     tokens = q.shape[0]
     if q.shape != (tokens, heads * head_dim) or out.shape != q.shape:
         raise KernelError(f"attention: q {tuple(q.shape)} / out {tuple(out.shape)} do not fit {heads} heads of {head_dim}")
-    if tuple(k_pages.shape[1:]) != (kv_heads, PAGE_TOKENS, head_dim) or tuple(v_pages.shape[1:]) != (kv_heads, head_dim, PAGE_TOKENS):
+    if not _pages_fit(k_pages, v_pages, kv_heads, head_dim):
         raise KernelError(f"attention: page shapes {tuple(k_pages.shape)} / {tuple(v_pages.shape)} do not fit")
     if block_table.dtype != torch.int32 or block_table.dim() != 2:
         raise KernelError("attention: block_table must be int32 [slots, pages]")
@@ -382,12 +388,15 @@ def attention_prefill_bf16(q, out, k_pages, v_pages, block_table, tile_seq, tile
 
 
 def attention_decode_bf16(q, out, k_pages, v_pages, block_table, tok_slot, tok_pos, heads, kv_heads, head_dim, scale,
-                          window=0, splits=1, partial=None, waves=1):
+                          window=0, splits=1, partial=None, waves=1, kernel="auto"):
     """One query token per sequence over its cached keys.  The keys are cut
-    into ``splits`` runs, each a block of ``waves`` waves that deal its keys
+    into ``splits`` runs, each a block of ``waves`` waves that deal its pages
     among themselves and merge in LDS; the runs are summed by a second kernel.
-    ``partial``: float32 scratch of tokens * heads * splits * (head_dim + 2)
-    when splits > 1."""
+    ``partial``: float32 scratch of tokens * heads * splits * (head_dim + 4)
+    when splits > 1 (``decode_scratch`` keeps one per device).  ``kernel``:
+    "keys" (keys on lanes; groups of up to 4 heads of up to 128 channels),
+    "columns" (heads in the columns of a tile; any group the head size
+    carries) or "auto", which takes "keys" where it fits."""
     _check_pages(q, out, k_pages, v_pages, block_table, heads, kv_heads, head_dim)
     tokens = q.shape[0]
     for t in (tok_slot, tok_pos):
@@ -395,16 +404,35 @@ def attention_decode_bf16(q, out, k_pages, v_pages, block_table, tok_slot, tok_p
         if t.dtype != torch.int32 or t.numel() < tokens:
             raise KernelError("attention: tok_slot / tok_pos must be int32 with one entry per token")
     if splits > 1:
-        if partial is None or partial.dtype != torch.float32 or partial.numel() < tokens * heads * splits * (head_dim + 2):
-            raise KernelError("attention: splits need float32 scratch of tokens * heads * splits * (head_dim + 2)")
+        if partial is None or partial.dtype != torch.float32 or partial.numel() < tokens * heads * splits * (head_dim + 4):
+            raise KernelError("attention: splits need float32 scratch of tokens * heads * splits * (head_dim + 4)")
         _dev(partial, "partial")
     lib = attention_module(head_dim)
     _check(lib, lib.nnis_attention_decode_bf16(q.data_ptr(), out.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(),
                                                block_table.data_ptr(), block_table.shape[1], tok_slot.data_ptr(),
                                                tok_pos.data_ptr(), tokens, heads, kv_heads, head_dim, int(window),
                                                float(scale), int(splits), int(waves), _ptr(partial) if splits > 1 else None,
-                                               _stream()))
+                                               _DECODE_KERNELS[kernel], _stream()))
     return out
+
+
+_DECODE_KERNELS = {"auto": 0, "columns": 1, "keys": 2}
+_decode_scratch = {}
+
+
+def decode_scratch(device, floats: int) -> torch.Tensor:
+    """Scratch of the split decode attention, kept per device and grown when a
+    call needs more.  Calls on one device share it, so they must follow one
+    another on one stream; it grows outside a graph capture only (the run that
+    warms a graph up sizes it)."""
+    key = (device.type, device.index)
+    held = _decode_scratch.get(key)
+    if held is None or held.numel() < floats:
+        if torch.cuda.is_current_stream_capturing():
+            raise KernelError("attention: the decode scratch would have to grow inside a graph capture")
+        held = torch.empty(max(floats, 2 * held.numel() if held is not None else 1 << 16), dtype=torch.float32, device=device)
+        _decode_scratch[key] = held
+    return held
 
 
 def decode_max_waves(heads: int, kv_heads: int, head_dim: int) -> int:
@@ -460,7 +488,7 @@ def attention(q: torch.Tensor, out: torch.Tensor, view, ctx, heads: int, kv_head
         waves = min(waves, decode_max_waves(heads, kv_heads, head_dim))
         partial = None
         if splits > 1:
-            partial = torch.empty(q.shape[0] * heads * splits * (head_dim + 2), dtype=torch.float32, device=q.device)
+            partial = decode_scratch(q.device, q.shape[0] * heads * splits * (head_dim + 4))
         return attention_decode_bf16(q, out, view.k_pages, view.v_pages, view.block_table, ctx.tok_slot, ctx.tok_pos, heads,
                                      kv_heads, head_dim, scale, window, splits, partial, waves)
     if fast and not ctx.decode:

@@ -66,8 +66,9 @@ def test_groups_have_storage_of_their_own():
     cache = _cache(extra=[(4, StateRequest((3, 5)))])
     assert len(cache.kv_groups) == 2  # all keys / a window of them
     full, windowed = cache.kv_groups
-    assert full.k.shape == (2, 8, 2, 64, 16) and full.v.shape == (2, 8, 2, 16, 64)
-    assert windowed.k.shape == (1, 8, 1, 64, 32) and windowed.request.window == 100
+    # [entries, pages, kv_heads, ...]: keys in chunks of 8 channels, values in tiles of 16 channels
+    assert full.k.shape == (2, 8, 2, 2, 64, 8) and full.v.shape == (2, 8, 2, 1, 2, 4, 16, 8)
+    assert windowed.k.shape == (1, 8, 1, 4, 64, 8) and windowed.request.window == 100
     assert cache.view(0).k_pages.data_ptr() != cache.view(1).k_pages.data_ptr()
     shared = cache.view(3)  # reads entry 1's cache
     assert shared.read_only and shared.k_pages.data_ptr() == cache.view(1).k_pages.data_ptr()
@@ -116,3 +117,33 @@ def test_state_starts_at_zero():
     assert cache.view(4).state[slot].abs().sum() == 0 and region[slot] == 0
     with pytest.raises(InvalidInput):
         cache.add_state_region("extra", (), torch.int64)
+
+
+@pytest.mark.parametrize("head_dim", [16, 24, 64, 80])
+def test_a_page_holds_every_key_and_value_once(head_dim):
+    """The page orders are one-to-one: every (token, channel) has a place of
+    its own inside the page, 8 channels of a key lie together and so do 8
+    tokens of a value channel."""
+    from nnis_amd.cache.layout import k_offset, k_page_shape, v_offset, v_page_shape
+
+    k_size = 1
+    for n in k_page_shape(1, head_dim):
+        k_size *= n
+    v_size = 1
+    for n in v_page_shape(1, head_dim):
+        v_size *= n
+    k_places = {k_offset(t, c) for t in range(64) for c in range(head_dim)}
+    v_places = {v_offset(c, t) for t in range(64) for c in range(head_dim)}
+    assert len(k_places) == len(v_places) == 64 * head_dim
+    assert max(k_places) < k_size and max(v_places) < v_size
+    assert k_size == 64 * 8 * ((head_dim + 7) // 8) and v_size == 64 * 16 * ((head_dim + 15) // 16)
+    for t in (0, 37, 63):
+        for c in range(0, head_dim - 7, 8):
+            assert [k_offset(t, c + i) - k_offset(t, c) for i in range(8)] == list(range(8))
+    for c in (0, head_dim - 1):
+        for t in range(0, 64, 8):
+            assert [v_offset(c, t + i) - v_offset(c, t) for i in range(8)] == list(range(8))
+    # a wave's loads: lane = token reads 16 consecutive bytes of a chunk after its neighbour's
+    assert k_offset(5, 8) - k_offset(4, 8) == 8
+    # lane (r, g) of a value load: channel 16 t + r, tokens 32 h + 8 g ..; consecutive lanes r, then g
+    assert v_offset(1, 0) - v_offset(0, 0) == 8 and v_offset(0, 8) - v_offset(15, 0) == 8

@@ -122,7 +122,14 @@ def test_gemm_bf16_refuses_what_it_cannot_load():
 
 
 MFMA_SHAPES = [(4, 2, 16), (3, 3, 16), (3, 1, 32), (6, 2, 48), (6, 6, 48), (4, 2, 48), (9, 3, 64), (2, 2, 64), (5, 5, 80),
-               (4, 1, 112), (8, 2, 128), (32, 1, 64), (40, 2, 16)]
+               (4, 1, 112), (8, 2, 128), (32, 1, 64), (40, 2, 16), (8, 1, 64), (12, 2, 32)]
+
+
+def _small_decode_call(heads, kv_heads, head_dim):
+    """Arguments of a one-token decode call over one page (for calls that are to be refused)."""
+    k_pages, v_pages = _empty_pages(1, kv_heads, head_dim, torch.bfloat16, 0.0, 0.0, "cuda")
+    q = torch.zeros(1, heads * head_dim, dtype=torch.bfloat16, device="cuda")
+    return (q, torch.empty_like(q), k_pages, v_pages, _i32([[0]]), _i32([0]), _i32([0]), heads, kv_heads, head_dim, 1.0)
 
 
 def _plain_rows(q_rows, ks, vs, scale, window=0):
@@ -138,8 +145,13 @@ def _plain_rows(q_rows, ks, vs, scale, window=0):
 
 @pytest.mark.parametrize("heads, kv_heads, head_dim", MFMA_SHAPES)
 @pytest.mark.parametrize("splits, waves", [(1, 1), (4, 1), (16, 2), (1, 8), (2, 4)])
-def test_decode_attention_on_the_matrix_cores(heads, kv_heads, head_dim, splits, waves):
+@pytest.mark.parametrize("kernel", ["columns", "keys"])
+def test_decode_attention_on_the_matrix_cores(heads, kv_heads, head_dim, splits, waves, kernel):
     ops = _ops()
+    if kernel == "keys" and heads // kv_heads > 4:
+        with pytest.raises(Exception, match="keys on lanes"):
+            ops.attention_decode_bf16(*_small_decode_call(heads, kv_heads, head_dim), kernel="keys")
+        return
     torch.manual_seed(heads + head_dim)
     lengths = [700, 1, 65, 33]
     ks = [torch.randn(n, kv_heads, head_dim).bfloat16().float() for n in lengths]
@@ -153,10 +165,10 @@ def test_decode_attention_on_the_matrix_cores(heads, kv_heads, head_dim, splits,
     rows = [(s, p, q.bfloat16().float()) for s, p, q in rows]
     q = torch.stack([q for _, _, q in rows]).bfloat16().reshape(len(rows), -1).cuda()
     out = torch.full((len(rows), heads * head_dim), 3.0, dtype=torch.bfloat16, device="cuda")
-    partial = torch.empty(len(rows) * heads * splits * (head_dim + 2), dtype=torch.float32, device="cuda")
+    partial = torch.full((len(rows) * heads * splits * (head_dim + 4),), float("nan"), dtype=torch.float32, device="cuda")
     waves = min(waves, ops.decode_max_waves(heads, kv_heads, head_dim))
     ops.attention_decode_bf16(q, out, k_pages, v_pages, table, _i32([s for s, _, _ in rows]), _i32([p for _, p, _ in rows]),
-                              heads, kv_heads, head_dim, scale, 0, splits, partial, waves)
+                              heads, kv_heads, head_dim, scale, 0, splits, partial, waves, kernel)
     got = out.cpu().float().view(len(rows), heads, head_dim)
     live = [i for i, (s, _, _) in enumerate(rows) if s >= 0]
     want = _plain_rows([rows[i] for i in live], ks, vs, scale)
@@ -165,7 +177,7 @@ def test_decode_attention_on_the_matrix_cores(heads, kv_heads, head_dim, splits,
     assert (got[0, 0] - vs[0][3, 0]).abs().max().item() < 0.05
     # a window: the row at position 699 reads keys 600..699 only
     ops.attention_decode_bf16(q, out, k_pages, v_pages, table, _i32([s for s, _, _ in rows]), _i32([p for _, p, _ in rows]),
-                              heads, kv_heads, head_dim, scale, 100, splits, partial, waves)
+                              heads, kv_heads, head_dim, scale, 100, splits, partial, waves, kernel)
     got = out.cpu().float().view(len(rows), heads, head_dim)
     want = _plain_rows([rows[i] for i in live], ks, vs, scale, window=100)
     assert (got[live] - want).abs().max().item() <= 2e-2
@@ -256,8 +268,7 @@ def test_fused_norm_projection(m, k, with_delta, gain_dtype):
     slots = [s if s >= 0 else -1 for s in slots]
     positions = [(i * 37) % 300 for i in range(m)]
     table = torch.arange(7 * 5, dtype=torch.int32).view(7, 5).flip(0).contiguous()
-    k_pages = torch.full((35, kv_heads, 64, head_dim), 7.0, dtype=torch.bfloat16, device="cuda")
-    v_pages = torch.full((35, kv_heads, head_dim, 64), 7.0, dtype=torch.bfloat16, device="cuda")
+    k_pages, v_pages = _empty_pages(35, kv_heads, head_dim, torch.bfloat16, 7.0, 7.0, "cuda")
     rope = dict(cos=torch.from_numpy(cos_np).cuda(), sin=torch.from_numpy(sin_np).cuda(), tok_slot=_i32(slots),
                 tok_pos=_i32(positions), k_pages=k_pages, v_pages=v_pages, block_table=table.cuda(), heads=heads,
                 kv_heads=kv_heads, head_dim=head_dim)
@@ -269,18 +280,48 @@ def test_fused_norm_projection(m, k, with_delta, gain_dtype):
     for t in range(m):  # a later token of the same slot and position overwrites an earlier one
         if slots[t] >= 0:
             seen[(slots[t], positions[t])] = t
+    k_plain, v_plain = _read_pages(k_pages, v_pages, head_dim)
     for (slot, position), t in seen.items():
         page, inside = table[slot, position // 64].item(), position % 64
-        close(k_pages[page, :, inside, :].cpu().double(), turned[t, heads:], "keys")
-        close(v_pages[page, :, :, inside].cpu().double(), qkv[t, heads + kv_heads:], "values")
+        close(k_plain[page, :, inside, :].double(), turned[t, heads:], "keys")
+        close(v_plain[page, :, inside, :].double(), qkv[t, heads + kv_heads:], "values")
     written = sum(1 for _ in seen)
-    assert int((k_pages.cpu().float() != 7.0).any(dim=-1).sum()) <= written * kv_heads
+    assert int((k_plain != 7.0).any(dim=-1).sum()) <= written * kv_heads
+    assert int((v_plain != 7.0).any(dim=-1).sum()) <= written * kv_heads
+
+
+def _k_index(head_dim):
+    """[64 tokens, head_dim] -> offset of each (token, channel) in a page's keys of one head."""
+    t = torch.arange(64).view(64, 1)
+    c = torch.arange(head_dim).view(1, head_dim)
+    return (c // 8) * 512 + t * 8 + c % 8
+
+
+def _v_index(head_dim):
+    t = torch.arange(64).view(64, 1)
+    c = torch.arange(head_dim).view(1, head_dim)
+    return ((((c // 16) * 2 + t // 32) * 4 + (t % 32) // 8) * 16 + c % 16) * 8 + t % 8
+
+
+def _empty_pages(pages, kv_heads, head_dim, dtype, k_fill, v_fill, device="cpu"):
+    k_pages = torch.full((pages, kv_heads, (head_dim + 7) // 8, 64, 8), k_fill, dtype=dtype, device=device)
+    v_pages = torch.full((pages, kv_heads, (head_dim + 15) // 16, 2, 4, 16, 8), v_fill, dtype=dtype, device=device)
+    return k_pages, v_pages
+
+
+def _read_pages(k_pages, v_pages, head_dim):
+    """Pages back in plain order: keys and values as [pages, kv_heads, 64 tokens, head_dim]."""
+    pages, kv_heads = k_pages.shape[:2]
+    k = k_pages.cpu().float().reshape(pages, kv_heads, -1)[:, :, _k_index(head_dim)]
+    v = v_pages.cpu().float().reshape(pages, kv_heads, -1)[:, :, _v_index(head_dim)]
+    return k, v
 
 
 def _paged(k_seqs, v_seqs, dtype, kv_heads, head_dim, page_order=None, pages=32, max_pages=12):
     """Lays sequences out in pages the way the cache does.  k_seqs[i]: [len, kv_heads, head_dim]."""
-    k_pages = torch.full((pages, kv_heads, 64, head_dim), 77.0, dtype=dtype)
-    v_pages = torch.full((pages, kv_heads, head_dim, 64), -55.0, dtype=dtype)
+    k_pages, v_pages = _empty_pages(pages, kv_heads, head_dim, dtype, 77.0, -55.0)
+    k_flat, v_flat = k_pages.view(pages, kv_heads, -1), v_pages.view(pages, kv_heads, -1)
+    k_index, v_index = _k_index(head_dim), _v_index(head_dim)
     table = torch.zeros(len(k_seqs), max_pages, dtype=torch.int32)
     order = list(page_order or range(pages))
     for slot, (k, v) in enumerate(zip(k_seqs, v_seqs)):
@@ -289,8 +330,8 @@ def _paged(k_seqs, v_seqs, dtype, kv_heads, head_dim, page_order=None, pages=32,
             table[slot, page_index] = page
             chunk = slice(page_index * 64, min(k.shape[0], page_index * 64 + 64))
             n = chunk.stop - chunk.start
-            k_pages[page, :, :n, :] = k[chunk].transpose(0, 1).to(dtype)
-            v_pages[page, :, :, :n] = v[chunk].permute(1, 2, 0).to(dtype)
+            k_flat[page][:, k_index[:n]] = k[chunk].transpose(0, 1).to(dtype)
+            v_flat[page][:, v_index[:n]] = v[chunk].transpose(0, 1).to(dtype)
     return k_pages.cuda(), v_pages.cuda(), table.cuda()
 
 
@@ -371,8 +412,7 @@ def test_rope_and_cache_write(dtype, heads, kv_heads, head_dim, rot_dim):
     width = (heads + 2 * kv_heads) * head_dim
     qkv = torch.randn(tokens, width).to(DT[dtype])
     table = torch.tensor([[3, 0, 0, 0], [9, 4, 6, 0], [1, 7, 2, 5]], dtype=torch.int32)
-    k_pages = torch.full((10, kv_heads, 64, head_dim), 7.0, dtype=DT[dtype], device="cuda")
-    v_pages = torch.full((10, kv_heads, head_dim, 64), 7.0, dtype=DT[dtype], device="cuda")
+    k_pages, v_pages = _empty_pages(10, kv_heads, head_dim, DT[dtype], 7.0, 7.0, "cuda")
     q_out = torch.full((tokens, heads * head_dim), 5.0, dtype=DT[dtype], device="cuda")
     cos = sin = None
     if rot_dim:
@@ -388,6 +428,7 @@ def test_rope_and_cache_write(dtype, heads, kv_heads, head_dim, rot_dim):
         rotated = torch.cat([turned, rotated[..., rot_dim:]], dim=-1)
     tol = 1e-6 if dtype == "float32" else 1e-2
     touched_k = torch.zeros(10, 64, dtype=torch.bool)
+    k_plain, v_plain = _read_pages(k_pages, v_pages, head_dim)  # [pages, kv_heads, 64, head_dim]
     for t in range(tokens):
         if slots[t] < 0:
             assert (q_out[t] == 5.0).all()
@@ -395,11 +436,13 @@ def test_rope_and_cache_write(dtype, heads, kv_heads, head_dim, rot_dim):
         assert (q_out[t].cpu().float().view(heads, head_dim) - rotated[t, :heads]).abs().max() <= tol
         page, inside = table[slots[t], positions[t] // 64].item(), positions[t] % 64
         touched_k[page, inside] = True
-        assert (k_pages[page, :, inside, :].cpu().float() - rotated[t, heads:]).abs().max() <= tol
-        assert torch.equal(v_pages[page, :, :, inside].cpu().float(), x[t, heads + kv_heads:])  # values are copied as they are
-    # nothing else in the cache was written
-    assert (k_pages.cpu().float()[~touched_k.unsqueeze(1).expand(-1, kv_heads, -1)] == 7.0).all()
-    assert (v_pages.cpu().float().transpose(2, 3)[~touched_k.unsqueeze(1).expand(-1, kv_heads, -1)] == 7.0).all()
+        assert (k_plain[page, :, inside, :] - rotated[t, heads:]).abs().max() <= tol
+        assert torch.equal(v_plain[page, :, inside, :], x[t, heads + kv_heads:])  # values are copied as they are
+    # nothing else in the cache was written (padding of a page's last chunk included)
+    assert (k_plain[~touched_k.unsqueeze(1).expand(-1, kv_heads, -1)] == 7.0).all()
+    assert (v_plain[~touched_k.unsqueeze(1).expand(-1, kv_heads, -1)] == 7.0).all()
+    assert int((k_pages != 7.0).sum()) <= int(touched_k.sum()) * kv_heads * head_dim
+    assert int((v_pages != 7.0).sum()) <= int(touched_k.sum()) * kv_heads * head_dim
     # a run that keeps no cache rotates the queries only
     q_only = torch.empty_like(q_out)
     ops.rope_kv_write(qkv.cuda(), q_only, cos, sin, rot_dim, _i32([0] * tokens), _i32(positions), None, None, None,
