@@ -460,7 +460,7 @@ __global__ __launch_bounds__(64 * kBlockWaves) void attention_prefill_kernel(Mfm
   if (last >= 0) {
     const int first_page = first / kPageTokens, page_count = last / kPageTokens + 1 - first_page;
     const int mine = page_count > wave ? (page_count - wave + waves - 1) / waves : 0;  // pages of this wave
-    attend_run<C, 2>(st, q, a, pages, kv_head, first_page + wave, waves, mine, last, lo, hi, lane);
+    attend_run<C, (HD > 64 ? 2 : (C <= 2 ? 4 : (C == 3 ? 3 : 2)))>(st, q, a, pages, kv_head, first_page + wave, waves, mine, last, lo, hi, lane);
   }
   if (!merge_waves<C>(st, merge, wave, waves, lane)) return;
 #pragma unroll

@@ -8,6 +8,9 @@
 //   epilogue   y = acc / sqrt(ss / K + eps)   the row's scale commutes with the product
 //              then one of: store | SiLU(gate) * up | rotate-half RoPE and cache write
 //
+// When the projection before (nnis_gemm_residual) has taken the sum and left bf16(v * g) and parts of ss
+// behind, the prologue is a plain operand load and a sum of those parts (PREP).
+//
 // RMSNorm as in /root/reference/crates/nnis-model/src/kernels.rs:15-48 (eps inside
 // the root, mean over the row); SiLU-multiply as fused_swiglu.rs:14-28; RoPE as
 // runtime_kernels.rs:38-66; keys stored rotated, values as they are
@@ -19,6 +22,7 @@
 // two halves of a head that rotate into each other).  KSPLIT waves share a
 // unit's K and add their parts, and their partial sums of squares, through LDS.
 #include "common.h"
+#include "epilogue.h"
 
 namespace {
 
@@ -26,9 +30,12 @@ typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
-enum : int { EPI_STORE = 0, EPI_SILU = 1, EPI_ROPE = 2 };
-
 struct FusedArgs {
+  // prepared by the projection before: the operand and parts of each row's sum of squares
+  const bf16_t* scaled;  // [m, k]
+  const float* ss_parts;  // [parts, m]
+  int parts;
+  // or taken here:
   const float* x_in;    // [m, k]
   const bf16_t* delta;  // [m, k] or null
   float* x_out;         // [m, k], written when delta != null
@@ -37,17 +44,8 @@ struct FusedArgs {
   float eps;
   const bf16_t* w;  // [n, k]
   int m, n, k;
-  bf16_t* y;  // store: [m, n]; silu: [m, n / 2]; rope: queries [m, heads * head_dim]
-  // rope + cache write
-  const float* cos_table;
-  const float* sin_table;
-  const int* tok_slot;
-  const int* tok_pos;
-  bf16_t* k_pages;  // null: this run keeps no cache of its own
-  bf16_t* v_pages;
-  const int* block_table;
-  int max_pages;
-  int heads, kv_heads, head_dim;
+  bf16_t* y;  // store: [m, n]; silu: [m, n / 2]; rope: queries [m, heads * head_dim] (= rope.q_out)
+  RopeTarget rope;
 };
 
 __device__ __forceinline__ bf16x8 zero8() {
@@ -74,13 +72,14 @@ __device__ __forceinline__ void load_gain8(const void* base, int dtype, int inde
   }
 }
 
-template <int MT, int KSPLIT, int EPI>
+template <int MT, int KSPLIT, int EPI, bool PREP>
 __global__ __launch_bounds__(KSPLIT > 4 ? 64 * KSPLIT : 256) void gemm_fused_kernel(FusedArgs a) {
   constexpr bool PAIR = EPI != EPI_STORE;
   constexpr int NACC = PAIR ? 2 : 1;
   constexpr int kWaves = KSPLIT > 4 ? KSPLIT : 4;
   constexpr int kUnits = kWaves / KSPLIT;  // units per block
-  constexpr int DEPTH = MT == 1 ? 2 : 1;   // steps of 64 k whose loads are in flight together
+  // steps of 64 k whose loads are in flight together
+  constexpr int DEPTH = PREP ? (MT <= 2 ? 4 : 2) : (MT == 1 ? 2 : 1);
   __shared__ float part_acc[KSPLIT > 1 ? kWaves : 1][NACC][MT][kWave][4];
   __shared__ float part_ss[KSPLIT > 1 ? kWaves : 1][MT][kWave];
 
@@ -100,36 +99,60 @@ __global__ __launch_bounds__(KSPLIT > 4 ? 64 * KSPLIT : 256) void gemm_fused_ker
     row0 = unit * 16;
     row1 = n / 2 + unit * 16;
   } else {
-    const int per_head = a.head_dim / 32;
-    units = (a.heads + 2 * a.kv_heads) * per_head;
-    row0 = (unit / per_head) * a.head_dim + (unit % per_head) * 16;
-    row1 = row0 + a.head_dim / 2;
+    const int per_head = a.rope.head_dim / 32;
+    units = (a.rope.heads + 2 * a.rope.kv_heads) * per_head;
+    row0 = (unit / per_head) * a.rope.head_dim + (unit % per_head) * 16;
+    row1 = row0 + a.rope.head_dim / 2;
   }
   const bool active = unit < units;
   const int row_limit = EPI == EPI_SILU ? n / 2 : n;  // rows0 beyond this are padding of the last strip
 
-  // what the rotating epilogue needs of each token is asked for now, so that it
-  // has arrived when the product is done
+  // What the rotating epilogue needs of each token hangs on the token's position and slot, which are
+  // asked for here; the loads that depend on them (`dependent` below) are issued after the first
+  // round of weight loads, so that the wave that ends the unit does not wait for them before it
+  // has asked for its weights.  The same goes for the parts of a prepared norm's sums of squares.
   int tok_slot[MT], tok_pos[MT], tok_page[MT];
   f32x4 tok_cos[MT], tok_sin[MT];
-  if (EPI == EPI_ROPE && active && part == 0) {
-    const int head = row0 / a.head_dim;
-    const int f0 = row0 % a.head_dim + g * 4;
+  constexpr int kPartRegs = 8;  // parts of a row's sum of squares a lane keeps in flight (4 lane groups share a row)
+  float ss_held[MT][kPartRegs];
+  const bool ends_unit = active && part == 0;
+  if (EPI == EPI_ROPE && ends_unit) {
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
       int token = t * 16 + r;
       token = token < m ? token : m - 1;
-      tok_slot[t] = a.tok_slot[token];
-      tok_pos[t] = a.tok_pos[token];
+      tok_slot[t] = a.rope.tok_slot[token];
+      tok_pos[t] = a.rope.tok_pos[token];
       tok_page[t] = -1;
-      if (head < a.heads + a.kv_heads) {
-        tok_cos[t] = *(const f32x4*)(a.cos_table + (size_t)tok_pos[t] * (a.head_dim / 2) + f0);
-        tok_sin[t] = *(const f32x4*)(a.sin_table + (size_t)tok_pos[t] * (a.head_dim / 2) + f0);
-      }
-      if (head >= a.heads && tok_slot[t] >= 0 && a.k_pages)
-        tok_page[t] = a.block_table[(size_t)tok_slot[t] * a.max_pages + tok_pos[t] / kPageTokens];
     }
   }
+  auto dependent = [&]() {
+    if (EPI == EPI_ROPE && ends_unit) {
+      const int head = row0 / a.rope.head_dim;
+      const int f0 = row0 % a.rope.head_dim + g * 4;
+#pragma unroll
+      for (int t = 0; t < MT; ++t) {
+        if (head < a.rope.heads + a.rope.kv_heads) {
+          tok_cos[t] = *(const f32x4*)(a.rope.cos_table + (size_t)tok_pos[t] * (a.rope.head_dim / 2) + f0);
+          tok_sin[t] = *(const f32x4*)(a.rope.sin_table + (size_t)tok_pos[t] * (a.rope.head_dim / 2) + f0);
+        }
+        if (head >= a.rope.heads && tok_slot[t] >= 0 && a.rope.k_pages)
+          tok_page[t] = a.rope.block_table[(size_t)tok_slot[t] * a.rope.max_pages + tok_pos[t] / kPageTokens];
+      }
+    }
+    if (PREP && ends_unit) {
+      // lane group g takes every fourth part; the groups are added with the sums of squares below
+#pragma unroll
+      for (int t = 0; t < MT; ++t) {
+        const int token = t * 16 + r;
+#pragma unroll
+        for (int i = 0; i < kPartRegs; ++i) {
+          const int p = g + 4 * i;
+          ss_held[t][i] = (token < m && p < a.parts) ? a.ss_parts[(size_t)p * m + token] : 0.0f;
+        }
+      }
+    }
+  };
 
   f32x4 acc[NACC][MT];
   float ss[MT];
@@ -139,7 +162,6 @@ __global__ __launch_bounds__(KSPLIT > 4 ? 64 * KSPLIT : 256) void gemm_fused_ker
 #pragma unroll
     for (int j = 0; j < NACC; ++j) acc[j][t] = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
   }
-
   if (active) {
     int wr0 = row0 + r, wr1 = row1 + r;
     wr0 = wr0 < row_limit ? wr0 : row_limit - 1;
@@ -153,9 +175,35 @@ __global__ __launch_bounds__(KSPLIT > 4 ? 64 * KSPLIT : 256) void gemm_fused_ker
       token = token < m ? token : m - 1;
       x_row[t] = (size_t)token * k;
     }
-    const bool writes_x = a.delta != nullptr && unit == 0;  // the first unit's waves cover every k once
+    const bool writes_x = !PREP && a.delta != nullptr && unit == 0;  // the first unit's waves cover every k once
     const bool gain_f32 = a.norm_w_dtype == NNIS_F32;
     const int chunks = (k + 63) / 64;
+    if constexpr (PREP) {
+      for (int base = part; base < chunks; base += KSPLIT * DEPTH) {
+        bf16x8 wa[DEPTH][2], wb[DEPTH][2], xs[DEPTH][2][MT];
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d)
+#pragma unroll
+          for (int half = 0; half < 2; ++half) {
+            const int kk = (base + d * KSPLIT) * 64 + g * 16 + half * 8;
+            const bool in = kk + 8 <= k;
+            wa[d][half] = in ? *(const bf16x8*)(w0 + kk) : zero8();
+            wb[d][half] = (PAIR && in) ? *(const bf16x8*)(w1 + kk) : zero8();
+#pragma unroll
+            for (int t = 0; t < MT; ++t) xs[d][half][t] = in ? *(const bf16x8*)(a.scaled + x_row[t] + kk) : zero8();
+          }
+        if (base == part) dependent();
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d)
+#pragma unroll
+          for (int half = 0; half < 2; ++half)
+#pragma unroll
+            for (int t = 0; t < MT; ++t) {
+              acc[0][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[d][half], xs[d][half][t], acc[0][t], 0, 0, 0);
+              if (PAIR) acc[1][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wb[d][half], xs[d][half][t], acc[1][t], 0, 0, 0);
+            }
+      }
+    } else
     // The product is bound by memory latency: a wave asks for everything its next
     // DEPTH steps of 64 k need (weights, residual, pending sum, gain) before it
     // touches any of it, so its share of K is one round trip, not one per step.
@@ -188,6 +236,7 @@ __global__ __launch_bounds__(KSPLIT > 4 ? 64 * KSPLIT : 256) void gemm_fused_ker
             }
           }
         }
+      if (base == part) dependent();
 #pragma unroll
       for (int d = 0; d < DEPTH; ++d)
 #pragma unroll
@@ -242,6 +291,16 @@ __global__ __launch_bounds__(KSPLIT > 4 ? 64 * KSPLIT : 256) void gemm_fused_ker
         }
     }
   }
+  if (PREP && ends_unit) {
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+#pragma unroll
+      for (int i = 0; i < kPartRegs; ++i) ss[t] += ss_held[t][i];
+      const int token = t * 16 + r;
+      if (token < m)
+        for (int p = g + 4 * kPartRegs; p < a.parts; p += 4) ss[t] += a.ss_parts[(size_t)p * m + token];  // wide rows
+    }
+  }
   // a token's sum of squares: over the four lane groups of this wave, then over the waves that share K
 #pragma unroll
   for (int t = 0; t < MT; ++t) {
@@ -285,50 +344,18 @@ __global__ __launch_bounds__(KSPLIT > 4 ? 64 * KSPLIT : 256) void gemm_fused_ker
       const int n0 = row0 + g * 4;
       for (int e = 0; e < 4; ++e)
         if (n0 + e < n) a.y[(size_t)token * n + n0 + e] = (bf16_t)(acc[0][t][e] * scale);
-    } else if (EPI == EPI_SILU) {
-      const int inner = n / 2;
-      const int n0 = row0 + g * 4;
-      for (int e = 0; e < 4; ++e) {
-        if (n0 + e >= inner) continue;
-        const float gate = acc[0][t][e] * scale, up = acc[1][t][e] * scale;
-        a.y[(size_t)token * inner + n0 + e] = (bf16_t)(gate / (1.0f + expf(-gate)) * up);
-      }
     } else {
-      const int hd = a.head_dim, half = hd / 2;
-      const int head = row0 / hd;
-      const int f0 = row0 % hd + g * 4;  // feature in the lower half; its partner is f0 + half
-      const int pos = tok_pos[t];
-      const int page = tok_page[t];
       float lo[4], hi[4];
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         lo[e] = acc[0][t][e] * scale;
         hi[e] = acc[1][t][e] * scale;
       }
-      if (head < a.heads + a.kv_heads) {  // queries and keys rotate
-        const f32x4 c = tok_cos[t], s = tok_sin[t];
-        bf16x4 out_lo, out_hi;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          out_lo[e] = (__bf16)(lo[e] * c[e] - hi[e] * s[e]);
-          out_hi[e] = (__bf16)(hi[e] * c[e] + lo[e] * s[e]);
-        }
-        if (head < a.heads) {
-          bf16_t* dst = a.y + ((size_t)token * a.heads + head) * hd;
-          *(bf16x4*)(dst + f0) = out_lo;
-          *(bf16x4*)(dst + f0 + half) = out_hi;
-        } else if (page >= 0) {
-          bf16_t* dst = a.k_pages + ((size_t)page * a.kv_heads + (head - a.heads)) * nnis_k_page_elems(hd);
-          *(bf16x4*)(dst + nnis_k_offset(pos % kPageTokens, f0)) = out_lo;  // 4 channels lie within a chunk of 8
-          *(bf16x4*)(dst + nnis_k_offset(pos % kPageTokens, f0 + half)) = out_hi;
-        }
-      } else if (page >= 0) {  // values are stored as they are
-        bf16_t* dst = a.v_pages + ((size_t)page * a.kv_heads + (head - a.heads - a.kv_heads)) * nnis_v_page_elems(hd);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          dst[nnis_v_offset(f0 + e, pos % kPageTokens)] = (bf16_t)lo[e];
-          dst[nnis_v_offset(f0 + half + e, pos % kPageTokens)] = (bf16_t)hi[e];
-        }
+      if (EPI == EPI_SILU) {
+        epilogue_silu(a.y, token, n / 2, row0 + g * 4, lo, hi);
+      } else {
+        const int hd = a.rope.head_dim;
+        epilogue_rope(a.rope, token, tok_pos[t], tok_page[t], row0 / hd, row0 % hd + g * 4, lo, hi, tok_cos[t], tok_sin[t]);
       }
     }
   }
@@ -338,8 +365,9 @@ template <int MT, int KSPLIT, int EPI>
 void launch_fused(const FusedArgs& a, int units, hipStream_t stream) {
   constexpr int kWaves = KSPLIT > 4 ? KSPLIT : 4;
   constexpr int kUnits = kWaves / KSPLIT;
-  hipLaunchKernelGGL((gemm_fused_kernel<MT, KSPLIT, EPI>), dim3((units + kUnits - 1) / kUnits), dim3(64 * kWaves), 0,
-                     stream, a);
+  const dim3 grid((units + kUnits - 1) / kUnits), block(64 * kWaves);
+  if (a.scaled) hipLaunchKernelGGL((gemm_fused_kernel<MT, KSPLIT, EPI, true>), grid, block, 0, stream, a);
+  else hipLaunchKernelGGL((gemm_fused_kernel<MT, KSPLIT, EPI, false>), grid, block, 0, stream, a);
 }
 
 template <int MT, int EPI>
@@ -357,6 +385,48 @@ void dispatch_fused(const FusedArgs& a, int units, int split, hipStream_t stream
   else if (tiles == 2) dispatch_fused_split<2, EPI>(a, units, split, stream);
   else if (tiles == 3) dispatch_fused_split<3, EPI>(a, units, split, stream);
   else dispatch_fused_split<4, EPI>(a, units, split, stream);
+}
+
+// checks what the epilogue needs, picks the split of K and launches; a.scaled tells the prologue
+int run_fused(FusedArgs& a, int epilogue, int table_positions, int split_hint, hipStream_t stream) {
+  const int n = a.n, k = a.k;
+  int units;
+  if (epilogue == EPI_STORE) {
+    units = (n + 15) / 16;
+  } else if (epilogue == EPI_SILU) {
+    NNIS_REQUIRE(n % 2 == 0, "gemm_fused: gate and up rows must be as many (n=%d)", n);
+    units = (n / 2 + 15) / 16;
+  } else if (epilogue == EPI_ROPE) {
+    NNIS_REQUIRE(a.rope.heads > 0 && a.rope.kv_heads > 0 && a.rope.head_dim > 0 && a.rope.head_dim % 32 == 0,
+                 "gemm_fused: the rotating epilogue needs a head size in steps of 32, got %d", a.rope.head_dim);
+    NNIS_REQUIRE(n == (a.rope.heads + 2 * a.rope.kv_heads) * a.rope.head_dim, "gemm_fused: %d weight rows for %d+2*%d heads of %d", n, a.rope.heads,
+                 a.rope.kv_heads, a.rope.head_dim);
+    NNIS_REQUIRE(a.rope.cos_table && a.rope.sin_table && a.rope.tok_slot && a.rope.tok_pos, "gemm_fused: the rotating epilogue needs tables and positions");
+    NNIS_REQUIRE((a.rope.k_pages == nullptr) == (a.rope.v_pages == nullptr), "gemm_fused: key and value pages must come together");
+    NNIS_REQUIRE(a.rope.k_pages == nullptr || (a.rope.block_table && a.rope.max_pages > 0), "gemm_fused: cache without a block table");
+    NNIS_REQUIRE(table_positions > 0, "gemm_fused: empty rotation tables");
+    units = (a.rope.heads + 2 * a.rope.kv_heads) * (a.rope.head_dim / 32);
+  } else {
+    return nnis_fail("gemm_fused: unknown epilogue %d", epilogue);
+  }
+  if (a.m > 64) {
+    NNIS_REQUIRE(a.scaled != nullptr, "gemm_fused: takes 1 to 64 tokens, got %d", a.m);
+    const int tile_hint = split_hint >= 16 ? split_hint / 16 : 0;
+    return nnis_gemm_scaled_tiled(a.scaled, a.ss_parts, a.parts, a.eps, a.w, a.m, n, k, epilogue, a.y, a.rope, tile_hint, stream);
+  }
+  // few units: their waves share K so that each wave's share is one round of loads
+  const int chunks = (k + 63) / 64;
+  const int depth = a.scaled ? (a.m <= 32 ? 4 : 2) : 2;
+  int split = 1;
+  if (units < 2048) {
+    while (split < 8 && chunks > split * depth) split *= 2;
+  }
+  if (split_hint == 1 || split_hint == 2 || split_hint == 4 || split_hint == 8) split = split_hint;  // for tuning runs
+  if (epilogue == EPI_STORE) dispatch_fused<EPI_STORE>(a, units, split, stream);
+  else if (epilogue == EPI_SILU) dispatch_fused<EPI_SILU>(a, units, split, stream);
+  else dispatch_fused<EPI_ROPE>(a, units, split, stream);
+  NNIS_LAUNCH_CHECK("gemm_fused");
+  return 0;
 }
 
 }  // namespace
@@ -378,41 +448,34 @@ extern "C" int nnis_gemm_fused(const float* x_in, const void* delta, float* x_ou
   for (const void* p : {(const void*)x_in, delta, (const void*)x_out, norm_w, w, (const void*)y})
     NNIS_REQUIRE((uintptr_t)p % 16 == 0, "gemm_fused: operands must be 16-byte aligned");
   FusedArgs a;
+  a.scaled = nullptr; a.ss_parts = nullptr; a.parts = 0;
   a.x_in = x_in; a.delta = (const bf16_t*)delta; a.x_out = x_out; a.norm_w = norm_w; a.norm_w_dtype = norm_w_dtype;
   a.eps = eps; a.w = (const bf16_t*)w; a.m = m; a.n = n; a.k = k; a.y = (bf16_t*)y;
-  a.cos_table = cos_table; a.sin_table = sin_table; a.tok_slot = tok_slot; a.tok_pos = tok_pos;
-  a.k_pages = (bf16_t*)k_pages; a.v_pages = (bf16_t*)v_pages; a.block_table = block_table; a.max_pages = max_pages;
-  a.heads = heads; a.kv_heads = kv_heads; a.head_dim = head_dim;
-  int units;
-  if (epilogue == EPI_STORE) {
-    units = (n + 15) / 16;
-  } else if (epilogue == EPI_SILU) {
-    NNIS_REQUIRE(n % 2 == 0, "gemm_fused: gate and up rows must be as many (n=%d)", n);
-    units = (n / 2 + 15) / 16;
-  } else if (epilogue == EPI_ROPE) {
-    NNIS_REQUIRE(heads > 0 && kv_heads > 0 && head_dim > 0 && head_dim % 32 == 0,
-                 "gemm_fused: the rotating epilogue needs a head size in steps of 32, got %d", head_dim);
-    NNIS_REQUIRE(n == (heads + 2 * kv_heads) * head_dim, "gemm_fused: %d weight rows for %d+2*%d heads of %d", n, heads,
-                 kv_heads, head_dim);
-    NNIS_REQUIRE(cos_table && sin_table && tok_slot && tok_pos, "gemm_fused: the rotating epilogue needs tables and positions");
-    NNIS_REQUIRE((k_pages == nullptr) == (v_pages == nullptr), "gemm_fused: key and value pages must come together");
-    NNIS_REQUIRE(k_pages == nullptr || (block_table && max_pages > 0), "gemm_fused: cache without a block table");
-    NNIS_REQUIRE(table_positions > 0, "gemm_fused: empty rotation tables");
-    units = (heads + 2 * kv_heads) * (head_dim / 32);
-  } else {
-    return nnis_fail("gemm_fused: unknown epilogue %d", epilogue);
-  }
-  // few units: their waves share K so that each wave's share is a step or two of 64
-  const int chunks = (k + 63) / 64;
-  int split = 1;
-  if (units < 2048) {
-    while (split < 8 && chunks > split * 2) split *= 2;
-  }
-  if (split_hint == 1 || split_hint == 2 || split_hint == 4 || split_hint == 8) split = split_hint;  // for tuning runs
-  hipStream_t stream = (hipStream_t)stream_ptr;
-  if (epilogue == EPI_STORE) dispatch_fused<EPI_STORE>(a, units, split, stream);
-  else if (epilogue == EPI_SILU) dispatch_fused<EPI_SILU>(a, units, split, stream);
-  else dispatch_fused<EPI_ROPE>(a, units, split, stream);
-  NNIS_LAUNCH_CHECK("gemm_fused");
-  return 0;
+  a.rope.q_out = (bf16_t*)y; a.rope.cos_table = cos_table; a.rope.sin_table = sin_table; a.rope.tok_slot = tok_slot; a.rope.tok_pos = tok_pos;
+  a.rope.k_pages = (bf16_t*)k_pages; a.rope.v_pages = (bf16_t*)v_pages; a.rope.block_table = block_table; a.rope.max_pages = max_pages;
+  a.rope.heads = heads; a.rope.kv_heads = kv_heads; a.rope.head_dim = head_dim;
+  return run_fused(a, epilogue, table_positions, split_hint, (hipStream_t)stream_ptr);
+}
+
+// The same product and epilogues on an operand that nnis_gemm_residual prepared: scaled = bf16(v * g)
+// [m, k] and ss_parts [parts, m], whose sum over the parts is a row's sum of squares.
+extern "C" int nnis_gemm_scaled(const void* scaled, const float* ss_parts, int parts, float eps, const void* w, int m, int n,
+                                int k, int epilogue, void* y, const float* cos_table, const float* sin_table,
+                                int table_positions, const int* tok_slot, const int* tok_pos, void* k_pages, void* v_pages,
+                                const int* block_table, int max_pages, int heads, int kv_heads, int head_dim, int split_hint,
+                                void* stream_ptr) {
+  NNIS_REQUIRE(m > 0, "gemm_scaled: no tokens");
+  NNIS_REQUIRE(n > 0 && k > 0 && k % 8 == 0, "gemm_scaled: bad sizes n=%d k=%d (K must be a multiple of 8)", n, k);
+  NNIS_REQUIRE(scaled && ss_parts && parts > 0, "gemm_scaled: the prepared operand is missing");
+  NNIS_REQUIRE(eps > 0.0f, "gemm_scaled: eps must be positive");
+  for (const void* p : {scaled, w, (const void*)y})
+    NNIS_REQUIRE((uintptr_t)p % 16 == 0, "gemm_scaled: operands must be 16-byte aligned");
+  FusedArgs a;
+  a.scaled = (const bf16_t*)scaled; a.ss_parts = ss_parts; a.parts = parts;
+  a.x_in = nullptr; a.delta = nullptr; a.x_out = nullptr; a.norm_w = nullptr; a.norm_w_dtype = NNIS_F32;
+  a.eps = eps; a.w = (const bf16_t*)w; a.m = m; a.n = n; a.k = k; a.y = (bf16_t*)y;
+  a.rope.q_out = (bf16_t*)y; a.rope.cos_table = cos_table; a.rope.sin_table = sin_table; a.rope.tok_slot = tok_slot; a.rope.tok_pos = tok_pos;
+  a.rope.k_pages = (bf16_t*)k_pages; a.rope.v_pages = (bf16_t*)v_pages; a.rope.block_table = block_table; a.rope.max_pages = max_pages;
+  a.rope.heads = heads; a.rope.kv_heads = kv_heads; a.rope.head_dim = head_dim;
+  return run_fused(a, epilogue, table_positions, split_hint, (hipStream_t)stream_ptr);
 }

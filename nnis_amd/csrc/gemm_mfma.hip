@@ -19,6 +19,9 @@
 // Both need K % 8 == 0 and 16-byte aligned operands (the host checks) and take
 // any M and N.
 #include "common.h"
+#include "epilogue.h"
+
+#include <type_traits>
 
 namespace {
 
@@ -38,11 +41,7 @@ __device__ __forceinline__ f32x4 mfma(bf16x8 a, bf16x8 b, f32x4 c) {
   return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
 }
 
-template <typename OutT>
-__device__ __forceinline__ void store4(OutT* y, size_t index, f32x4 v, int valid, bool vector_ok);
-
-template <>
-__device__ __forceinline__ void store4<float>(float* y, size_t index, f32x4 v, int valid, bool vector_ok) {
+__device__ __forceinline__ void store4(float* y, size_t index, f32x4 v, int valid, bool vector_ok) {
   if (valid == 4 && vector_ok) {
     *(f32x4*)(y + index) = v;
   } else {
@@ -50,8 +49,7 @@ __device__ __forceinline__ void store4<float>(float* y, size_t index, f32x4 v, i
   }
 }
 
-template <>
-__device__ __forceinline__ void store4<bf16_t>(bf16_t* y, size_t index, f32x4 v, int valid, bool vector_ok) {
+__device__ __forceinline__ void store4(bf16_t* y, size_t index, f32x4 v, int valid, bool vector_ok) {
   if (valid == 4 && vector_ok) {
     typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
     bf16x4 packed;
@@ -69,11 +67,91 @@ __device__ __forceinline__ void store4<bf16_t>(bf16_t* y, size_t index, f32x4 v,
 // issues the loads of DEPTH steps of 64 k (weights and activations) before the
 // first multiply, so its whole share of K is usually one round trip.
 // -----------------------------------------------------------------------------
+// What a projection that ends a part of a pre-norm block does with its result instead of storing it
+// (OutT = ResidualOut): the residual stream takes it in, and the norm that follows is prepared.
+//   v = resid + y (32-bit, in place);  scaled = bf16(v * gain);  ss[part][token] = sum over the part's
+//   columns of v * v.  The norm's 1 / sqrt(mean + eps) is left to the kernel that reads `scaled`: it needs
+//   the whole row, and the parts of a row are spread over the blocks.  Statistics as in
+//   /root/reference/crates/nnis-model/src/kernels.rs:15-48.
+struct ResidualOut {
+  float* resid;      // [m, n]
+  const void* gain;  // [n], the following norm's weight
+  int gain_dtype;
+  bf16_t* scaled;    // [m, n]
+  float* ss;         // [parts, m]; a part is 16 columns (skinny kernel) or a wave's columns (tiled kernel)
+};
+
+// four consecutive columns of a token: the lane's accumulator acc
+__device__ __forceinline__ float residual_take(const ResidualOut& o, size_t index, int column, f32x4 acc, int valid, bool vector_ok) {
+  typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+  float sq = 0.0f;
+  if (valid == 4 && vector_ok) {
+    f32x4 v = *(const f32x4*)(o.resid + index);
+    f32x4 g;
+    if (o.gain_dtype == NNIS_F32) {
+      g = *(const f32x4*)((const float*)o.gain + column);
+    } else {
+      const bf16x4 packed = *(const bf16x4*)((const bf16_t*)o.gain + column);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) g[e] = (float)packed[e];
+    }
+    bf16x4 scaled;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      v[e] += acc[e];
+      sq = fmaf(v[e], v[e], sq);
+      scaled[e] = (__bf16)(v[e] * g[e]);
+    }
+    *(f32x4*)(o.resid + index) = v;
+    *(bf16x4*)(o.scaled + index) = scaled;
+  } else {
+    for (int e = 0; e < valid; ++e) {
+      const float v = o.resid[index + e] + acc[e];
+      sq = fmaf(v, v, sq);
+      o.resid[index + e] = v;
+      o.scaled[index + e] = (bf16_t)(v * load_as_f32(o.gain, o.gain_dtype, column + e));
+    }
+  }
+  return sq;
+}
+
+// What the tiled kernel does for a projection that starts a part of a pre-norm block (OutT = ScaledOut<EPI>):
+// its operand is the `scaled` that a ResidualOut left, the row's 1 / sqrt(mean of squares + eps) is taken
+// from the parts of ss and applied to the product, then the epilogue stores, gates or rotates.  For the
+// two epilogues that need pairs of weight rows in one lane (gate and up of the same channels; the two
+// halves of a head that rotate into each other), the tile's strips of 16 weight rows alternate between the
+// two: strips 2u and 2u+1 of a wave are the lower and upper rows of pair unit u.
+template <int EPI>
+struct ScaledOut {
+  bf16_t* y;  // store: [m, n]; silu: [m, n / 2]; rope: the queries (= rope.q_out)
+  const float* ss_parts;  // [parts, m]
+  int parts;
+  float eps;
+  RopeTarget rope;
+};
+template <typename T> struct scaled_epilogue { static constexpr int value = -1; };
+template <int EPI> struct scaled_epilogue<ScaledOut<EPI>> { static constexpr int value = EPI; };
+
+// the weight row that strip row `tile_row` (0 .. BN-1) of column block `block` multiplies; -1 beyond the end
+template <int EPI, int BN>
+__device__ __forceinline__ int paired_weight_row(const RopeTarget& rope, int block, int tile_row, int n) {
+  constexpr int WN = BN / 2;
+  const int wave_n = tile_row / WN, strip = (tile_row % WN) / 16, rr = tile_row % 16;
+  const int unit = block * (BN / 32) + wave_n * (WN / 32) + strip / 2;
+  const bool upper = strip % 2;
+  if (EPI == EPI_SILU) {
+    const int inner = n / 2, channel = unit * 16 + rr;
+    return channel < inner ? (upper ? inner : 0) + channel : -1;
+  }
+  const int per_head = rope.head_dim / 32;
+  if (unit >= (rope.heads + 2 * rope.kv_heads) * per_head) return -1;
+  return (unit / per_head) * rope.head_dim + (unit % per_head) * 16 + rr + (upper ? rope.head_dim / 2 : 0);
+}
+
 template <int MT, int KSPLIT, typename OutT>
 __global__ __launch_bounds__(KSPLIT > 4 ? 64 * KSPLIT : 256) void gemm_skinny_kernel(const bf16_t* __restrict__ x,
                                                                                    const bf16_t* __restrict__ w,
-                                                                                   OutT* __restrict__ y, int m, int n,
-                                                                                   int k) {
+                                                                                   OutT y, int m, int n, int k) {
   constexpr int kWaves = KSPLIT > 4 ? KSPLIT : 4;
   constexpr int kStrips = kWaves / KSPLIT;  // strips of 16 weight rows per block
   constexpr int DEPTH = MT <= 2 ? 4 : 2;
@@ -150,30 +228,38 @@ __global__ __launch_bounds__(KSPLIT > 4 ? 64 * KSPLIT : 256) void gemm_skinny_ke
 #pragma unroll
   for (int t = 0; t < MT; ++t) {
     const int token = t * 16 + r;
-    if (token < m && valid > 0) store4<OutT>(y, (size_t)token * n + n0, acc[t], valid, vector_ok);
+    if constexpr (std::is_same<OutT, ResidualOut>::value) {
+      float sq = 0.0f;
+      if (token < m && valid > 0) sq = residual_take(y, (size_t)token * n + n0, n0, acc[t], valid, vector_ok);
+      sq += __shfl_xor(sq, 16, kWave);
+      sq += __shfl_xor(sq, 32, kWave);
+      if (g == 0 && token < m) y.ss[(size_t)strip * m + token] = sq;
+    } else {
+      if (token < m && valid > 0) store4(y, (size_t)token * n + n0, acc[t], valid, vector_ok);
+    }
   }
 }
 
 // -----------------------------------------------------------------------------
-// tiled: BM x BN output tile per block of 4 waves (2 x 2), K in steps of 64
+// tiled: BM x BN output tile per block of 4 waves (2 x 2), K in steps of BK (64 or 128)
 // -----------------------------------------------------------------------------
-constexpr int kBK = 64;  // k per stage: 8 chunks of 16 bytes per row
+// chunk c of row `row` of a staged tile (CHUNKS chunks of 16 bytes a row) lives at chunk c ^ (row % CHUNKS)
+template <int CHUNKS>
+__device__ __forceinline__ int swizzled(int row, int chunk) { return row * CHUNKS + (chunk ^ (row & (CHUNKS - 1))); }
 
-// chunk c (0..7) of row `row` of a staged tile lives at chunk (c ^ (row & 7))
-__device__ __forceinline__ int swizzled(int row, int chunk) { return row * 8 + (chunk ^ (row & 7)); }
-
-template <int BM, int BN, typename OutT>
+template <int BM, int BN, int BK, typename OutT>
 __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
-                                                         OutT* __restrict__ y, int m, int n, int k) {
+                                                         OutT y, int m, int n, int k) {
   constexpr int WM = BM / 2, WN = BN / 2;  // a wave's part of the tile
   constexpr int TM = WM / 16, TN = WN / 16;
-  constexpr int A_CHUNKS = BM * 8 / 256, B_CHUNKS = BN * 8 / 256;  // 16-byte chunks a thread stages per step
+  constexpr int CH = BK / 8;  // 16-byte chunks per staged row
+  constexpr int A_CHUNKS = BM * CH / 256, B_CHUNKS = BN * CH / 256;  // chunks a thread stages per step
   // Global loads run PF steps ahead of the multiply, in registers; the step after
   // the current one lies in the other LDS buffer.  With few blocks on a compute
   // unit nothing else hides the latency of a load, so short products need depth.
-  constexpr int PF = (BM * BN >= 128 * 128) ? 3 : 4;
-  __shared__ bf16x8 a_tile[2][BM * 8];
-  __shared__ bf16x8 b_tile[2][BN * 8];
+  constexpr int PF = (BM * BN * BK >= 128 * 128 * 64) ? 3 : 4;
+  __shared__ bf16x8 a_tile[2][BM * CH];
+  __shared__ bf16x8 b_tile[2][BN * CH];
 
   const int tid = threadIdx.x;
   const int wave = tid / kWave, lane = tid % kWave;
@@ -191,30 +277,60 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
   const bf16_t* a_src[A_CHUNKS];
   const bf16_t* b_src[B_CHUNKS];
   int a_dst[A_CHUNKS], b_dst[B_CHUNKS];
-  const int chunk_k = (tid % 8) * 8;
+  const int chunk_k = (tid % CH) * 8;
 #pragma unroll
   for (int c = 0; c < A_CHUNKS; ++c) {
-    const int index = tid + c * 256;  // row = index / 8, chunk = index % 8
-    int row = row0 + index / 8;
+    const int index = tid + c * 256;  // row = index / CH, chunk = index % CH
+    int row = row0 + index / CH;
     row = row < m ? row : m - 1;
     a_src[c] = x + (size_t)row * k + chunk_k;
-    a_dst[c] = swizzled(index / 8, index % 8);
+    a_dst[c] = swizzled<CH>(index / CH, index % CH);
   }
+  constexpr int EPI = scaled_epilogue<OutT>::value;  // -1: the product is stored or added as it is
+  constexpr bool kPaired = EPI == EPI_SILU || EPI == EPI_ROPE;
 #pragma unroll
   for (int c = 0; c < B_CHUNKS; ++c) {
     const int index = tid + c * 256;
-    int row = col0 + index / 8;
-    row = row < n ? row : n - 1;
+    int row;
+    if constexpr (kPaired) {
+      row = paired_weight_row<EPI, BN>(y.rope, blockIdx.x, index / CH, n);
+      row = row >= 0 ? row : 0;  // rows beyond the end read a valid row and are not stored
+    } else {
+      row = col0 + index / CH;
+      row = row < n ? row : n - 1;
+    }
     b_src[c] = w + (size_t)row * k + chunk_k;
-    b_dst[c] = swizzled(index / 8, index % 8);
+    b_dst[c] = swizzled<CH>(index / CH, index % CH);
+  }
+  // a prepared operand: the rows' scales, for the epilogue; and what the rotation needs of each token
+  __shared__ float row_scale[EPI >= 0 ? BM : 1];
+  int tok_pos[TM], tok_page[TM];
+  if constexpr (EPI >= 0) {
+    if (tid < BM) {
+      const int token = row0 + tid;
+      float total = 0.0f;
+      if (token < m)
+        for (int p = 0; p < y.parts; ++p) total += y.ss_parts[(size_t)p * m + token];
+      row_scale[tid] = 1.0f / sqrtf(total / (float)k + y.eps);
+    }
+    if constexpr (EPI == EPI_ROPE) {
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        int token = row0 + wave_m * WM + i * 16 + r;
+        token = token < m ? token : m - 1;
+        const int slot = y.rope.tok_slot[token];
+        tok_pos[i] = y.rope.tok_pos[token];
+        tok_page[i] = (slot >= 0 && y.rope.k_pages) ? y.rope.block_table[(size_t)slot * y.rope.max_pages + tok_pos[i] / kPageTokens] : -1;
+      }
+    }
   }
 
   bf16x8 a_stage[PF][A_CHUNKS], b_stage[PF][B_CHUNKS];
-  const int steps = (k + kBK - 1) / kBK;
+  const int steps = (k + BK - 1) / BK;
 
 #define NNIS_FETCH(slot, step)                                                                   \
   do {                                                                                           \
-    const int k0 = (step) * kBK;                                                                 \
+    const int k0 = (step) * BK;                                                                  \
     const bool in = k0 + chunk_k + 8 <= k;                                                       \
     _Pragma("unroll") for (int c = 0; c < A_CHUNKS; ++c) a_stage[slot][c] = in ? load_chunk(a_src[c] + k0) : zero_chunk(); \
     _Pragma("unroll") for (int c = 0; c < B_CHUNKS; ++c) b_stage[slot][c] = in ? load_chunk(b_src[c] + k0) : zero_chunk(); \
@@ -239,12 +355,12 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
         // slot j went to LDS a step ago: refill it with the step PF ahead
         if (step + PF < steps) NNIS_FETCH(j, step + PF);
 #pragma unroll
-        for (int half = 0; half < 2; ++half) {  // two instructions of 32 k per stage
+        for (int half = 0; half < BK / 32; ++half) {  // an instruction takes 32 k
           bf16x8 a_frag[TM], b_frag[TN];
 #pragma unroll
-          for (int i = 0; i < TM; ++i) a_frag[i] = a_tile[buffer][swizzled(wave_m * WM + i * 16 + r, half * 4 + g)];
+          for (int i = 0; i < TM; ++i) a_frag[i] = a_tile[buffer][swizzled<CH>(wave_m * WM + i * 16 + r, half * 4 + g)];
 #pragma unroll
-          for (int jj = 0; jj < TN; ++jj) b_frag[jj] = b_tile[buffer][swizzled(wave_n * WN + jj * 16 + r, half * 4 + g)];
+          for (int jj = 0; jj < TN; ++jj) b_frag[jj] = b_tile[buffer][swizzled<CH>(wave_n * WN + jj * 16 + r, half * 4 + g)];
 #pragma unroll
           for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -260,21 +376,64 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
 
   // first operand = weight rows: lane holds D[n = 4g + e][token = r]
   const bool vector_ok = (n % 4) == 0;
+  if constexpr (kPaired) {
+    // strips 2u and 2u+1 of this wave: lower and upper rows of a pair unit
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      const int token = row0 + wave_m * WM + i * 16 + r;
+      if (token >= m) continue;
+      const float scale = row_scale[wave_m * WM + i * 16 + r];
+#pragma unroll
+      for (int u = 0; u < TN / 2; ++u) {
+        const int first = paired_weight_row<EPI, BN>(y.rope, blockIdx.x, wave_n * WN + 32 * u, n);  // the unit's first lower row
+        if (first < 0) continue;
+        float lo[4], hi[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          lo[e] = acc[i][2 * u][e] * scale;
+          hi[e] = acc[i][2 * u + 1][e] * scale;
+        }
+        if constexpr (EPI == EPI_SILU) {
+          epilogue_silu(y.y, token, n / 2, first + 4 * g, lo, hi);
+        } else {
+          const int hd = y.rope.head_dim, head = first / hd, f0 = first % hd + 4 * g;
+          epi_f32x4 c = {1.0f, 1.0f, 1.0f, 1.0f}, sn = {0.0f, 0.0f, 0.0f, 0.0f};
+          if (head < y.rope.heads + y.rope.kv_heads) {
+            c = *(const epi_f32x4*)(y.rope.cos_table + (size_t)tok_pos[i] * (hd / 2) + f0);
+            sn = *(const epi_f32x4*)(y.rope.sin_table + (size_t)tok_pos[i] * (hd / 2) + f0);
+          }
+          epilogue_rope(y.rope, token, tok_pos[i], head >= y.rope.heads ? tok_page[i] : -1, head, f0, lo, hi, c, sn);
+        }
+      }
+    }
+  } else {
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
     const int token = row0 + wave_m * WM + i * 16 + r;
-    if (token >= m) continue;
+    float sq = 0.0f;
+    float scale = 1.0f;
+    if constexpr (EPI == EPI_STORE) scale = row_scale[wave_m * WM + i * 16 + r];
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
       const int n0 = col0 + wave_n * WN + j * 16 + g * 4;
       const int valid = n - n0 >= 4 ? 4 : (n - n0 > 0 ? n - n0 : 0);
-      if (valid > 0) store4<OutT>(y, (size_t)token * n + n0, acc[i][j], valid, vector_ok);
+      if (token >= m || valid <= 0) continue;
+      if constexpr (std::is_same<OutT, ResidualOut>::value) sq += residual_take(y, (size_t)token * n + n0, n0, acc[i][j], valid, vector_ok);
+      else if constexpr (EPI == EPI_STORE) store4(y.y, (size_t)token * n + n0, acc[i][j] * scale, valid, vector_ok);
+      else store4(y, (size_t)token * n + n0, acc[i][j], valid, vector_ok);
     }
+    if constexpr (std::is_same<OutT, ResidualOut>::value) {
+      // a part of the row's sum of squares: this wave's columns
+      sq += __shfl_xor(sq, 16, kWave);
+      sq += __shfl_xor(sq, 32, kWave);
+      if (g == 0 && token < m) y.ss[(size_t)(blockIdx.x * 2 + wave_n) * m + token] = sq;
+    }
+  }
   }
 }
 
 template <int MT, int KSPLIT, typename OutT>
-void launch_skinny(const bf16_t* x, const bf16_t* w, OutT* y, int m, int n, int k, hipStream_t stream) {
+void launch_skinny(const bf16_t* x, const bf16_t* w, OutT y, int m, int n, int k, hipStream_t stream) {
   const int strips = (n + 15) / 16;
   const int waves = KSPLIT > 4 ? KSPLIT : 4;
   const int per_block = waves / KSPLIT;
@@ -283,7 +442,7 @@ void launch_skinny(const bf16_t* x, const bf16_t* w, OutT* y, int m, int n, int 
 }
 
 template <int MT, typename OutT>
-void dispatch_skinny_split(const bf16_t* x, const bf16_t* w, OutT* y, int m, int n, int k, int split, hipStream_t stream) {
+void dispatch_skinny_split(const bf16_t* x, const bf16_t* w, OutT y, int m, int n, int k, int split, hipStream_t stream) {
   if (split == 8) launch_skinny<MT, 8, OutT>(x, w, y, m, n, k, stream);
   else if (split == 4) launch_skinny<MT, 4, OutT>(x, w, y, m, n, k, stream);
   else if (split == 2) launch_skinny<MT, 2, OutT>(x, w, y, m, n, k, stream);
@@ -291,7 +450,7 @@ void dispatch_skinny_split(const bf16_t* x, const bf16_t* w, OutT* y, int m, int
 }
 
 template <typename OutT>
-void dispatch_skinny(const bf16_t* x, const bf16_t* w, OutT* y, int m, int n, int k, int split, hipStream_t stream) {
+void dispatch_skinny(const bf16_t* x, const bf16_t* w, OutT y, int m, int n, int k, int split, hipStream_t stream) {
   const int tiles = (m + 15) / 16;
   if (tiles == 1) dispatch_skinny_split<1, OutT>(x, w, y, m, n, k, split, stream);
   else if (tiles == 2) dispatch_skinny_split<2, OutT>(x, w, y, m, n, k, split, stream);
@@ -299,25 +458,62 @@ void dispatch_skinny(const bf16_t* x, const bf16_t* w, OutT* y, int m, int n, in
   else dispatch_skinny_split<4, OutT>(x, w, y, m, n, k, split, stream);
 }
 
-template <int BM, int BN, typename OutT>
-void launch_tiled(const bf16_t* x, const bf16_t* w, OutT* y, int m, int n, int k, hipStream_t stream) {
-  hipLaunchKernelGGL((gemm_tiled_kernel<BM, BN, OutT>), dim3((n + BN - 1) / BN, (m + BM - 1) / BM), dim3(256), 0, stream,
-                     x, w, y, m, n, k);
+// `columns`: the weight rows the grid covers (n, or the rows of all pair units)
+template <int BM, int BN, int BK, typename OutT>
+void launch_tiled(const bf16_t* x, const bf16_t* w, OutT y, int m, int n, int k, int columns, hipStream_t stream) {
+  hipLaunchKernelGGL((gemm_tiled_kernel<BM, BN, BK, OutT>), dim3((columns + BN - 1) / BN, (m + BM - 1) / BM), dim3(256), 0,
+                     stream, x, w, y, m, n, k);
 }
 
+// returns the number of wave columns (parts of a row that a residual epilogue sums by itself)
 template <typename OutT>
-void dispatch_tiled(const bf16_t* x, const bf16_t* w, OutT* y, int m, int n, int k, int tile_hint, hipStream_t stream) {
+int dispatch_tiled(const bf16_t* x, const bf16_t* w, OutT y, int m, int n, int k, int tile_hint, hipStream_t stream,
+                   int columns = 0) {
+  if (columns <= 0) columns = n;
   // the largest tile that still gives every compute unit a block or two
-  const long long blocks_128 = (long long)((m + 127) / 128) * ((n + 127) / 128);
-  const long long blocks_64_128 = (long long)((m + 63) / 64) * ((n + 127) / 128);
+  const long long blocks_128 = (long long)((m + 127) / 128) * ((columns + 127) / 128);
+  const long long blocks_64_128 = (long long)((m + 63) / 64) * ((columns + 127) / 128);
   int tile = blocks_128 >= 384 ? 1 : (blocks_64_128 >= 256 ? 2 : 3);
-  if (tile_hint >= 1 && tile_hint <= 3) tile = tile_hint;  // for tuning runs
-  if (tile == 1) launch_tiled<128, 128, OutT>(x, w, y, m, n, k, stream);
-  else if (tile == 2) launch_tiled<64, 128, OutT>(x, w, y, m, n, k, stream);
-  else launch_tiled<64, 64, OutT>(x, w, y, m, n, k, stream);
+  if (tile_hint >= 1 && tile_hint <= 4) tile = tile_hint;  // for tuning runs
+  if (tile == 1) launch_tiled<128, 128, 64, OutT>(x, w, y, m, n, k, columns, stream);
+  else if (tile == 2) launch_tiled<64, 128, 64, OutT>(x, w, y, m, n, k, columns, stream);
+  else if (tile == 3) launch_tiled<64, 64, 64, OutT>(x, w, y, m, n, k, columns, stream);
+  else launch_tiled<64, 64, 128, OutT>(x, w, y, m, n, k, columns, stream);
+  const int width = tile <= 2 ? 128 : 64;
+  return 2 * ((columns + width - 1) / width);
+}
+
+// With few strips the waves of a block share a strip's K, so that each wave's
+// share is one round of loads (4 steps of 64 for up to 32 tokens, 2 beyond);
+// with thousands of strips there are waves enough to hide the latency.
+int skinny_split(int m, int n, int k, int split_hint) {
+  const int strips = (n + 15) / 16;
+  const int chunks = (k + 63) / 64;
+  const int depth = m <= 32 ? 4 : 2;
+  int split = 1;
+  if (strips < 2048) {
+    while (split < 8 && chunks > split * depth) split *= 2;
+  }
+  if (split_hint == 1 || split_hint == 2 || split_hint == 4 || split_hint == 8) split = split_hint;  // for tuning runs
+  return split;
 }
 
 }  // namespace
+
+int nnis_gemm_scaled_tiled(const bf16_t* scaled, const float* ss_parts, int parts, float eps, const bf16_t* w, int m, int n,
+                           int k, int epilogue, bf16_t* y, const RopeTarget& rope, int tile_hint, hipStream_t stream) {
+  NNIS_REQUIRE((m + 63) / 64 <= 65535, "gemm_scaled: %d rows exceed the grid limit", m);
+  if (epilogue == EPI_STORE) {
+    dispatch_tiled<ScaledOut<EPI_STORE>>(scaled, w, {y, ss_parts, parts, eps, rope}, m, n, k, tile_hint, stream);
+  } else if (epilogue == EPI_SILU) {
+    dispatch_tiled<ScaledOut<EPI_SILU>>(scaled, w, {y, ss_parts, parts, eps, rope}, m, n, k, tile_hint, stream,
+                                        32 * ((n / 2 + 15) / 16));
+  } else {
+    dispatch_tiled<ScaledOut<EPI_ROPE>>(scaled, w, {y, ss_parts, parts, eps, rope}, m, n, k, tile_hint, stream, n);
+  }
+  NNIS_LAUNCH_CHECK("gemm_scaled");
+  return 0;
+}
 
 // y_dtype: NNIS_BF16 or NNIS_F32.  Picks the skinny kernel for M <= 64.  split_hint: 0, or the number of
 // waves (1, 2, 4, 8) that share a strip's K in the skinny kernel, overriding the choice made here.
@@ -333,26 +529,48 @@ extern "C" int nnis_gemm_bf16(const void* x, const void* w, void* y, int y_dtype
   const bf16_t* xp = (const bf16_t*)x;
   const bf16_t* wp = (const bf16_t*)w;
   if (m <= 64) {
-    // With few strips the waves of a block share a strip's K, so that each wave's
-    // share is one round of loads (4 steps of 64 for up to 32 tokens, 2 beyond);
-    // with thousands of strips there are waves enough to hide the latency.
-    const int strips = (n + 15) / 16;
-    const int chunks = (k + 63) / 64;
-    const int depth = m <= 32 ? 4 : 2;
-    int split = 1;
-    if (strips < 2048) {
-      while (split < 8 && chunks > split * depth) split *= 2;
-    }
-    if (split_hint == 1 || split_hint == 2 || split_hint == 4 || split_hint == 8) split = split_hint;  // for tuning runs
-    if (y_dtype == NNIS_F32) dispatch_skinny<float>(xp, wp, (float*)y, m, n, k, split, stream);
-    else dispatch_skinny<bf16_t>(xp, wp, (bf16_t*)y, m, n, k, split, stream);
+    const int split = skinny_split(m, n, k, split_hint);
+    if (y_dtype == NNIS_F32) dispatch_skinny<float*>(xp, wp, (float*)y, m, n, k, split, stream);
+    else dispatch_skinny<bf16_t*>(xp, wp, (bf16_t*)y, m, n, k, split, stream);
     NNIS_LAUNCH_CHECK("gemm_skinny");
   } else {
     NNIS_REQUIRE((m + 63) / 64 <= 65535, "gemm_bf16: %d rows exceed the grid limit", m);
-    const int tile_hint = split_hint >= 16 ? split_hint / 16 : 0;  // hints of 16, 32, 48 pick the tile: 128x128, 64x128, 64x64
-    if (y_dtype == NNIS_F32) dispatch_tiled<float>(xp, wp, (float*)y, m, n, k, tile_hint, stream);
-    else dispatch_tiled<bf16_t>(xp, wp, (bf16_t*)y, m, n, k, tile_hint, stream);
+    const int tile_hint = split_hint >= 16 ? split_hint / 16 : 0;  // hints of 16, 32, 48, 64 pick the tile: 128x128, 64x128, 64x64, 64x64 with K in steps of 128
+    if (y_dtype == NNIS_F32) dispatch_tiled<float*>(xp, wp, (float*)y, m, n, k, tile_hint, stream);
+    else dispatch_tiled<bf16_t*>(xp, wp, (bf16_t*)y, m, n, k, tile_hint, stream);
     NNIS_LAUNCH_CHECK("gemm_tiled");
+  }
+  return 0;
+}
+
+// The projection that ends a part of a pre-norm block: resid += x . w^T in 32-bit, in place, and the norm
+// that follows prepared -- scaled = bf16(resid * gain) and parts of each row's sum of squares in ss
+// [parts, m].  Returns the number of parts in *parts (ss must hold nnis_gemm_residual_parts(m, n) rows).
+extern "C" int nnis_gemm_residual_parts(int m, int n) {
+  if (m <= 64) return (n + 15) / 16;
+  return 2 * ((n + 63) / 64);  // the narrowest tile's wave columns; wider tiles use fewer
+}
+
+extern "C" int nnis_gemm_residual(const void* x, const void* w, float* resid, const void* gain, int gain_dtype, void* scaled,
+                                  float* ss, int m, int n, int k, int* parts, void* stream_ptr) {
+  NNIS_REQUIRE(m >= 0 && n > 0 && k > 0, "gemm_residual: bad sizes m=%d n=%d k=%d", m, n, k);
+  NNIS_REQUIRE(k % 8 == 0, "gemm_residual: K=%d is not a multiple of 8 (16-byte loads)", k);
+  NNIS_REQUIRE(nnis_dtype_ok(gain_dtype), "gemm_residual: unknown norm weight dtype %d", gain_dtype);
+  NNIS_REQUIRE(resid && gain && scaled && ss && parts, "gemm_residual: missing operand");
+  for (const void* p : {x, w, (const void*)resid, gain, (const void*)scaled})
+    NNIS_REQUIRE((uintptr_t)p % 16 == 0, "gemm_residual: operands must be 16-byte aligned");
+  *parts = 0;
+  if (m == 0) return 0;
+  hipStream_t stream = (hipStream_t)stream_ptr;
+  ResidualOut out = {resid, gain, gain_dtype, (bf16_t*)scaled, ss};
+  if (m <= 64) {
+    *parts = (n + 15) / 16;
+    dispatch_skinny<ResidualOut>((const bf16_t*)x, (const bf16_t*)w, out, m, n, k, skinny_split(m, n, k, 0), stream);
+    NNIS_LAUNCH_CHECK("gemm_residual");
+  } else {
+    NNIS_REQUIRE((m + 63) / 64 <= 65535, "gemm_residual: %d rows exceed the grid limit", m);
+    *parts = dispatch_tiled<ResidualOut>((const bf16_t*)x, (const bf16_t*)w, out, m, n, k, 0, stream);
+    NNIS_LAUNCH_CHECK("gemm_residual");
   }
   return 0;
 }

@@ -41,7 +41,7 @@ FLAGS = [
     "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
 ]
-HEADERS = ["common.h"]
+HEADERS = ["common.h", "epilogue.h"]
 CORE_SOURCES = ["elementwise.hip", "gemm.hip", "gemm_mfma.hip", "gemm_fused.hip", "sampling.hip"]
 ATTENTION_SOURCES = ["attention.hip"]
 PREBUILT_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 112, 128)

@@ -32,6 +32,10 @@ _CORE_SIGNATURES = {
     "nnis_gemm_bf16": [_VOID, _VOID, _VOID, _INT, _INT, _INT, _INT, _INT, _VOID],
     "nnis_gemm_fused": [_VOID, _VOID, _VOID, _VOID, _INT, _FLT, _VOID, _INT, _INT, _INT, _INT, _VOID, _VOID, _VOID, _INT,
                         _VOID, _VOID, _VOID, _VOID, _VOID, _INT, _INT, _INT, _INT, _INT, _VOID],
+    "nnis_gemm_residual_parts": [_INT, _INT],
+    "nnis_gemm_residual": [_VOID, _VOID, _VOID, _VOID, _INT, _VOID, _VOID, _INT, _INT, _INT, _VOID, _VOID],
+    "nnis_gemm_scaled": [_VOID, _VOID, _INT, _FLT, _VOID, _INT, _INT, _INT, _INT, _VOID, _VOID, _VOID, _INT, _VOID, _VOID,
+                         _VOID, _VOID, _VOID, _INT, _INT, _INT, _INT, _INT, _VOID],
     "nnis_sample": [_VOID, _VOID, _INT, _INT, _VOID, _VOID, _VOID, _VOID, _VOID, _VOID, _VOID],
 }
 _ATTN_SIGNATURES = {
@@ -296,24 +300,7 @@ def gemm_fused(x_in: torch.Tensor, delta: Optional[torch.Tensor], x_out: Optiona
         _dev(delta, "delta"), _dev(x_out, "x_out")
         if delta.shape != x_in.shape or delta.dtype != torch.bfloat16 or x_out.shape != x_in.shape or x_out.dtype != torch.float32:
             raise KernelError("gemm_fused: delta must be bfloat16 and x_out float32, both shaped like x")
-    expect = {EPILOGUE_STORE: (m, n), EPILOGUE_SILU: (m, n // 2)}.get(epilogue)
-    r = rope or {}
-    if epilogue == EPILOGUE_ROPE:
-        expect = (m, r["heads"] * r["head_dim"])
-        for name in ("cos", "sin", "tok_slot", "tok_pos"):
-            _dev(r[name], name)
-        if r["cos"].dtype != torch.float32 or r["cos"].shape != r["sin"].shape or r["cos"].shape[1] != r["head_dim"] // 2:
-            raise KernelError("gemm_fused: rotation tables must be float32 [positions, head_dim / 2]")
-        if r["tok_slot"].dtype != torch.int32 or r["tok_pos"].dtype != torch.int32 or min(r["tok_slot"].numel(), r["tok_pos"].numel()) < m:
-            raise KernelError("gemm_fused: tok_slot / tok_pos must be int32 with one entry per token")
-        if r.get("k_pages") is not None:
-            kp, vp, bt = r["k_pages"], r["v_pages"], r["block_table"]
-            _dev(kp, "k_pages"), _dev(vp, "v_pages"), _dev(bt, "block_table")
-            if (kp.dtype != torch.bfloat16 or vp.dtype != torch.bfloat16 or bt.dtype != torch.int32
-                    or not _pages_fit(kp, vp, r["kv_heads"], r["head_dim"])):
-                raise KernelError("gemm_fused: cache pages must be bfloat16 in the cache's layout, the block table int32")
-    if expect is None or tuple(y.shape) != expect:
-        raise KernelError(f"gemm_fused: y {tuple(y.shape)} does not fit epilogue {epilogue} (expected {expect})")
+    r = _check_epilogue("gemm_fused", m, n, y, epilogue, rope)
     lib = core()
     bt = r.get("block_table")
     _check(lib, lib.nnis_gemm_fused(
@@ -321,6 +308,86 @@ def gemm_fused(x_in: torch.Tensor, delta: Optional[torch.Tensor], x_out: Optiona
         float(eps), w.data_ptr(), m, n, k, int(epilogue), y.data_ptr(), _ptr(r.get("cos")), _ptr(r.get("sin")),
         r["cos"].shape[0] if r.get("cos") is not None else 0, _ptr(r.get("tok_slot")), _ptr(r.get("tok_pos")),
         _ptr(r.get("k_pages")), _ptr(r.get("v_pages")), _ptr(bt), bt.shape[1] if bt is not None else 0,
+        r.get("heads", 0), r.get("kv_heads", 0), r.get("head_dim", 0), int(split), _stream()))
+    return y
+
+
+def _check_epilogue(what: str, m: int, n: int, y: torch.Tensor, epilogue: int, rope: Optional[dict]) -> dict:
+    """Checks y and the rotating epilogue's arguments against the sizes; returns the arguments (or {})."""
+    expect = {EPILOGUE_STORE: (m, n), EPILOGUE_SILU: (m, n // 2)}.get(epilogue)
+    r = rope or {}
+    if epilogue == EPILOGUE_ROPE:
+        expect = (m, r["heads"] * r["head_dim"])
+        for name in ("cos", "sin", "tok_slot", "tok_pos"):
+            _dev(r[name], name)
+        if r["cos"].dtype != torch.float32 or r["cos"].shape != r["sin"].shape or r["cos"].shape[1] != r["head_dim"] // 2:
+            raise KernelError(f"{what}: rotation tables must be float32 [positions, head_dim / 2]")
+        if r["tok_slot"].dtype != torch.int32 or r["tok_pos"].dtype != torch.int32 or min(r["tok_slot"].numel(), r["tok_pos"].numel()) < m:
+            raise KernelError(f"{what}: tok_slot / tok_pos must be int32 with one entry per token")
+        if r.get("k_pages") is not None:
+            kp, vp, bt = r["k_pages"], r["v_pages"], r["block_table"]
+            _dev(kp, "k_pages"), _dev(vp, "v_pages"), _dev(bt, "block_table")
+            if (kp.dtype != torch.bfloat16 or vp.dtype != torch.bfloat16 or bt.dtype != torch.int32
+                    or not _pages_fit(kp, vp, r["kv_heads"], r["head_dim"])):
+                raise KernelError(f"{what}: cache pages must be bfloat16 in the cache's layout, the block table int32")
+    if expect is None or tuple(y.shape) != expect or y.dtype != torch.bfloat16 or not y.is_contiguous():
+        raise KernelError(f"{what}: y {tuple(y.shape)} {y.dtype} does not fit epilogue {epilogue} (expected bfloat16 {expect})")
+    return r
+
+
+def gemm_residual_parts(m: int, n: int) -> int:
+    """Rows of the ``ss`` scratch that ``gemm_residual`` may fill for these sizes."""
+    return core().nnis_gemm_residual_parts(int(m), int(n))
+
+
+def gemm_residual(x: torch.Tensor, w: torch.Tensor, resid: torch.Tensor, gain: torch.Tensor, scaled: torch.Tensor,
+                  ss: torch.Tensor) -> int:
+    """The projection that ends a part of a pre-norm block: ``resid`` (float32
+    [m, n]) takes x @ w^T in, in place, and the norm that follows is prepared:
+    ``scaled`` = bfloat16(resid * gain) and, in ``ss`` [parts, m], parts of
+    each row's sum of squares.  Returns how many parts were written; the
+    norm's 1 / sqrt(mean + eps) is taken by ``gemm_scaled``, which reads them."""
+    m, k = x.shape
+    n = w.shape[0]
+    for t, what in ((x, "x"), (w, "weight"), (resid, "resid"), (gain, "gain"), (scaled, "scaled"), (ss, "ss")):
+        _dev(t, what)
+        if not t.is_contiguous():
+            raise KernelError(f"gemm_residual: {what} must be contiguous")
+    if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or w.shape[1] != k:
+        raise KernelError("gemm_residual: x must be bfloat16 [m, k] and the weight bfloat16 [n, k]")
+    if resid.dtype != torch.float32 or tuple(resid.shape) != (m, n) or scaled.dtype != torch.bfloat16 or tuple(scaled.shape) != (m, n):
+        raise KernelError("gemm_residual: resid must be float32 [m, n] and scaled bfloat16 [m, n]")
+    if gain.numel() != n:
+        raise KernelError(f"gemm_residual: norm weight of {gain.numel()} for width {n}")
+    if ss.dtype != torch.float32 or ss.numel() < gemm_residual_parts(m, n) * m:
+        raise KernelError("gemm_residual: ss must be float32 with gemm_residual_parts(m, n) * m elements")
+    lib = core()
+    parts = ctypes.c_int(0)
+    _check(lib, lib.nnis_gemm_residual(x.data_ptr(), w.data_ptr(), resid.data_ptr(), gain.data_ptr(), _code(gain),
+                                       scaled.data_ptr(), ss.data_ptr(), m, n, k, ctypes.addressof(parts), _stream()))
+    return parts.value
+
+
+def gemm_scaled(scaled: torch.Tensor, ss: torch.Tensor, parts: int, eps: float, w: torch.Tensor, y: torch.Tensor,
+                epilogue: int = EPILOGUE_STORE, rope: Optional[dict] = None, split: int = 0) -> torch.Tensor:
+    """y = epilogue( (W . scaled) / sqrt(sum of the parts of ss / k + eps) ):
+    the second half of an RMSNorm whose first half ``gemm_residual`` took, with
+    the epilogues of ``gemm_fused``."""
+    m, k = scaled.shape
+    n = w.shape[0]
+    for t, what in ((scaled, "scaled"), (ss, "ss"), (w, "weight"), (y, "y")):
+        _dev(t, what)
+    if scaled.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or w.shape[1] != k or not scaled.is_contiguous():
+        raise KernelError("gemm_scaled: scaled must be bfloat16 [m, k] and the weight bfloat16 [n, k]")
+    if ss.dtype != torch.float32 or parts <= 0 or ss.numel() < parts * m:
+        raise KernelError("gemm_scaled: ss must be float32 [parts, m]")
+    r = _check_epilogue("gemm_scaled", m, n, y, epilogue, rope)
+    lib = core()
+    bt = r.get("block_table")
+    _check(lib, lib.nnis_gemm_scaled(
+        scaled.data_ptr(), ss.data_ptr(), int(parts), float(eps), w.data_ptr(), m, n, k, int(epilogue), y.data_ptr(),
+        _ptr(r.get("cos")), _ptr(r.get("sin")), r["cos"].shape[0] if r.get("cos") is not None else 0, _ptr(r.get("tok_slot")),
+        _ptr(r.get("tok_pos")), _ptr(r.get("k_pages")), _ptr(r.get("v_pages")), _ptr(bt), bt.shape[1] if bt is not None else 0,
         r.get("heads", 0), r.get("kv_heads", 0), r.get("head_dim", 0), int(split), _stream()))
     return y
 
@@ -440,18 +507,25 @@ def decode_max_waves(heads: int, kv_heads: int, head_dim: int) -> int:
 
 
 def decode_plan(batch: int, kv_heads: int, longest: int, max_waves: int = 4):
-    """(splits, waves) of a decode step's attention.  The kernel is bound by
-    memory latency (a wave has one block of 32 keys in flight beside the one it
-    works on), so the keys are spread over about a thousand waves, down to one
-    page of 64 keys a wave.  Four waves of a block merge in LDS; beyond that the keys are
-    cut into runs that a second kernel sums.  Powers of two.  Measured on the
-    SmolLM2-135M shape: batch 8 at 1.7k keys runs 1.11 ms a step with (4, 4)
-    against 1.41 with (1, 8) and 2.78 with (1, 1)."""
+    """(splits, waves) of a decode step's attention.  A block of 4 waves deals
+    a sequence's pages among its waves.  Cutting the keys into runs for more
+    blocks costs a second kernel that sums the runs (dearer the more runs), so
+    it pays only from about 16 pages on; then a wave gets 2 to 4 pages, in at
+    most 8 runs and about a thousand waves on the chip.  Powers of two.
+    Measured on 9 query / 3 key-value heads of 64 (microseconds a layer, runs
+    of 1/2/4/8/16): batch 1 at 1k keys 7.9/8.3/8.7/10.7, at 8k 30/20/15/14/17;
+    batch 8 at 2k 11.6/11.0/9.5/9.3/13.6; batch 32 at 4k 27/25/31/34/45."""
     pages = (longest + 63) // 64
-    parallel = max(1, min(pages, 1024 // max(1, batch * kv_heads)))
-    parallel = 1 << (parallel.bit_length() - 1)
-    waves = min(max_waves, parallel)
-    return parallel // waves, waves
+    waves = 1
+    while waves * 2 <= min(max_waves, pages):
+        waves *= 2
+    splits = 1
+    if pages > 16:
+        wanted = min(8, (pages + 7) // 8)
+        room = max(1, 1024 // max(1, batch * kv_heads * waves))
+        while splits * 2 <= room and splits < wanted:
+            splits *= 2
+    return splits, waves
 
 
 # One column tile a wave (and so up to 8 waves a block) for long sequences was measured slower than the full

@@ -78,8 +78,17 @@ class DecoderModel:
         for position in self.positions.values():
             x = position.embed(x, ctx, rt)
         stream = (x, None)
-        for index, entry in enumerate(self.spec.schedule):
-            stream = self.layers[entry.layer].forward(stream, ctx, cache.view(index), rt)
+        schedule = self.spec.schedule
+        for index, entry in enumerate(schedule):
+            layer = self.layers[entry.layer]
+            # a block may prepare the first norm of the block that comes next, if that block shows it one
+            following = None
+            if index + 1 < len(schedule) and getattr(layer, "entry_norm", None) is not None:
+                following = getattr(self.layers[schedule[index + 1].layer], "entry_norm", None)
+            if following is not None:
+                stream = layer.forward(stream, ctx, cache.view(index), rt, following=following)
+            else:
+                stream = layer.forward(stream, ctx, cache.view(index), rt)
         x, pending = stream
         if want_rows.shape[0] == 0:
             return rt.empty(0, self.spec.vocab_size, dtype=torch.float32)

@@ -56,6 +56,7 @@ class CausalSelfAttention(Mixer):
         return KVRequest(self.kv_heads, self.head_dim, self.window)
 
     takes_pending_norm = True
+    adds_to_residual = True
 
     def _project_rotate_store(self, x, ctx, view, rt):
         """Queries [tokens, heads * head_dim], rotated; keys and values of the
@@ -86,11 +87,13 @@ class CausalSelfAttention(Mixer):
         )
         return q
 
-    def forward(self, x, ctx, view, rt):
+    def forward(self, x, ctx, view, rt, into=None):
         q = self._project_rotate_store(x, ctx, view, rt)
         tokens = q.shape[0]
         attn = rt.empty(tokens, self.heads * self.head_dim)
         rt.ops.attention(q, attn, view, ctx, self.heads, self.kv_heads, self.head_dim, self.scale, self.window or 0)
+        if into is not None and into.can_take(attn, self.out.weight):
+            return into.take(attn, self.out.weight)  # the output projection adds to the stream itself
         return self.out(attn, rt)
 
 

@@ -6,12 +6,17 @@ The residual stream is kept in 32-bit as a pair (x, pending): ``pending`` is a
 part's output not yet added.  The sum is taken by the next norm in the same
 kernel that normalises, and a mixer or feed-forward that starts with a
 projection may take sum and norm into that projection's kernel
-(``PendingNorm``), so the stream is read and written once per part.
+(``PendingNorm``), so the stream is read and written once per part.  A part
+that ends with a projection (``adds_to_residual``) may go further and add its
+output to the stream in that projection's kernel, which then also prepares
+the norm that follows (``ResidualInto``); the block names that norm -- its own
+second one, or the first of the block that comes next (``following``).
 """
 
 from __future__ import annotations
 
 from .base import Block, build_part, register_part
+from .lazy import PendingNorm, ResidualInto
 
 
 class PreNormBlock(Block):
@@ -37,19 +42,40 @@ class PreNormBlock(Block):
     def cache_request(self):
         return self.mixer.cache_request()
 
-    def forward(self, stream, ctx, view, rt):
-        x, pending = stream
-        normed = self.norm1.defer(x, pending, rt)
-        if getattr(self.mixer, "takes_pending_norm", False):
-            mixed = self.mixer.forward(normed, ctx, view, rt)
+    @property
+    def entry_norm(self):
+        """The norm a stream meets first here: a block before this one may prepare it."""
+        return self.norm1
+
+    def _run(self, part, normed, args, then, rt):
+        """Runs a mixer or feed-forward on a pending norm; returns the pending
+        norm ``then`` of the stream with the part's output (or, without
+        ``then``, the stream and the output not yet added)."""
+        given = normed if getattr(part, "takes_pending_norm", False) else normed.materialize()
+        if then is not None and getattr(part, "adds_to_residual", False):
+            out = part.forward(given, *args, into=ResidualInto(normed, then, rt))
         else:
-            mixed = self.mixer.forward(normed.materialize(), ctx, view, rt)
-        normed = self.norm2.defer(normed.residual, mixed, rt)
-        if getattr(self.feed_forward, "takes_pending_norm", False):
-            out = self.feed_forward.forward(normed, ctx, rt)
+            out = part.forward(given, *args)
+        if isinstance(out, PendingNorm):
+            return out
+        if then is None:
+            return normed.residual, out
+        return then.defer(normed.residual, out, rt)
+
+    def forward(self, stream, ctx, view, rt, following=None):
+        """stream: (x, pending), or this block's first norm, pending, from the
+        block before.  following: the next block's first norm, if that block
+        takes it pending; then the return value is that pending norm, else the
+        pair (x, pending)."""
+        if isinstance(stream, PendingNorm):
+            if stream.norm is not self.norm1:
+                raise ValueError("the pending norm handed to a block is not the block's own first norm")
+            normed = stream
         else:
-            out = self.feed_forward.forward(normed.materialize(), ctx, rt)
-        return normed.residual, out
+            x, pending = stream
+            normed = self.norm1.defer(x, pending, rt)
+        normed = self._run(self.mixer, normed, (ctx, view, rt), self.norm2, rt)
+        return self._run(self.feed_forward, normed, (ctx, rt), following, rt)
 
 
 register_part("block", "pre_norm", PreNormBlock)

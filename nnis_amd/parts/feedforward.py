@@ -38,18 +38,21 @@ class GatedFeedForward(FeedForward):
         return self.gate_up.weight_bytes() + self.down.weight_bytes()
 
     takes_pending_norm = True
+    adds_to_residual = True
 
-    def forward(self, x, ctx, rt):
+    def forward(self, x, ctx, rt, into=None):
         from .lazy import PendingNorm
 
-        if isinstance(x, PendingNorm):
-            if x.can_fuse(self.gate_up.weight):
-                # residual sum, norm, both projections and the gating in one kernel
-                hidden = x.fused(self.gate_up.weight, rt.empty(x.rows, self.inner), rt.ops.EPILOGUE_SILU)
-                return self.down(hidden, rt)
-            x = x.materialize()
-        gate_up = self.gate_up(x, rt)
-        hidden = rt.ops.silu_mul(gate_up, rt.empty(x.shape[0], self.inner))
+        if isinstance(x, PendingNorm) and x.can_fuse(self.gate_up.weight):
+            # (residual sum,) norm, both projections and the gating in one kernel
+            hidden = x.fused(self.gate_up.weight, rt.empty(x.rows, self.inner), rt.ops.EPILOGUE_SILU)
+        else:
+            if isinstance(x, PendingNorm):
+                x = x.materialize()
+            gate_up = self.gate_up(x, rt)
+            hidden = rt.ops.silu_mul(gate_up, rt.empty(x.shape[0], self.inner))
+        if into is not None and into.can_take(hidden, self.down.weight):
+            return into.take(hidden, self.down.weight)  # the down projection adds to the stream itself
         return self.down(hidden, rt)
 
 

@@ -223,14 +223,50 @@ def test_prefill_attention_on_the_matrix_cores(heads, kv_heads, head_dim):
             assert (got[100, 0] - vs[2][17, 0]).abs().max().item() < 0.05
 
 
-@pytest.mark.parametrize("m", [1, 8, 16, 17, 40, 64])
+@pytest.mark.parametrize("m", [1, 8, 19, 64, 100, 300])
+@pytest.mark.parametrize("n, k", [(576, 576), (100, 72), (2048, 1536), (48, 8)])
+@pytest.mark.parametrize("gain_dtype", ["bfloat16", "float32"])
+def test_residual_projection_prepares_the_norm(m, n, k, gain_dtype):
+    """resid += x . w^T in place; scaled = bfloat16(resid * gain); the parts of
+    ss add up to each row's sum of squares."""
+    ops = _ops()
+    torch.manual_seed(m + n + k)
+    x = torch.randn(m, k).bfloat16()
+    w = (torch.randn(n, k) / math.sqrt(k)).bfloat16()
+    resid = torch.randn(m, n) * 2
+    gain = (1 + 0.3 * torch.randn(n)).to(DT[gain_dtype])
+    want = resid.double() + x.double() @ w.double().t()
+    resid_gpu = resid.cuda()
+    scaled = torch.full((m, n), 9.0, dtype=torch.bfloat16, device="cuda")
+    rows = ops.gemm_residual_parts(m, n)
+    ss = torch.full((rows + 1, m), 7.0, device="cuda")
+    parts = ops.gemm_residual(x.cuda(), w.cuda(), resid_gpu, gain.cuda(), scaled, ss)
+    assert 0 < parts <= rows
+    assert (ss[parts:] == 7.0).all()  # nothing beyond the parts it names
+    got = resid_gpu.cpu().double()
+    assert ((got - want).abs() <= 1e-5 * (1 + want.abs())).all(), (got - want).abs().max().item()
+    # scaled is the rounding of the 32-bit product of the new residual and the gain
+    exact = (resid_gpu.cpu() * gain.float()).bfloat16()
+    assert torch.equal(scaled.cpu(), exact)
+    total = ss[:parts].cpu().double().sum(dim=0)
+    assert ((total - got.pow(2).sum(dim=1)).abs() <= 1e-5 * got.pow(2).sum(dim=1)).all()
+
+
+@pytest.mark.parametrize("m", [1, 8, 16, 17, 40, 64, 65, 200, 300])
 @pytest.mark.parametrize("k", [64, 96, 576, 1096])
-@pytest.mark.parametrize("with_delta", [False, True])
+@pytest.mark.parametrize("with_delta", [False, True, "prepared"])
 @pytest.mark.parametrize("gain_dtype", ["bfloat16", "float32"])
 def test_fused_norm_projection(m, k, with_delta, gain_dtype):
     """Residual sum + RMSNorm + projection in one kernel, with each epilogue,
-    against the plain functions one after another."""
+    against the plain functions one after another.  "prepared": the sum and
+    the first half of the norm are taken by the projection before (here one by
+    the identity, so that it adds ``delta`` itself), the second half by the
+    kernel under test."""
     ops = _ops()
+    prepared = with_delta == "prepared"
+    with_delta = bool(with_delta)
+    if m > 64 and not prepared:
+        pytest.skip("the kernel that takes the sum and the norm itself is for up to 64 tokens")
     torch.manual_seed(m * 7 + k)
     eps = 2e-5
     x = torch.randn(m, k) * 2
@@ -239,7 +275,17 @@ def test_fused_norm_projection(m, k, with_delta, gain_dtype):
     summed = x + (delta.float() if with_delta else 0)
     normed = P.rms_norm(summed.double(), gain.double(), eps)
 
+    if prepared:
+        resid = x.cuda()
+        scaled = torch.empty(m, k, dtype=torch.bfloat16, device="cuda")
+        ss = torch.empty(ops.gemm_residual_parts(m, k), m, device="cuda")
+        parts = ops.gemm_residual(delta.cuda(), torch.eye(k).bfloat16().cuda(), resid, gain.cuda(), scaled, ss)
+        assert torch.equal(resid.cpu(), summed)
+
     def run(w, y, epilogue, rope=None):
+        if prepared:
+            ops.gemm_scaled(scaled, ss, parts, eps, w.cuda(), y, epilogue, rope)
+            return y.cpu().double()
         x_out = torch.full((m, k), 9.0, device="cuda") if with_delta else None
         ops.gemm_fused(x.cuda(), delta.cuda() if with_delta else None, x_out, gain.cuda(), eps, w.cuda(), y, epilogue, rope)
         if with_delta:
@@ -266,7 +312,7 @@ def test_fused_norm_projection(m, k, with_delta, gain_dtype):
     cos_np, sin_np = P.rope_tables(512, head_dim, 10000.0)
     slots = [(i * 5) % 7 - (1 if i % 9 == 4 else 0) * 100 for i in range(m)]  # some padding rows
     slots = [s if s >= 0 else -1 for s in slots]
-    positions = [(i * 37) % 300 for i in range(m)]
+    positions = [(i * 37) % 320 for i in range(m)]  # no two tokens at one position (37 and 320 share no factor)
     table = torch.arange(7 * 5, dtype=torch.int32).view(7, 5).flip(0).contiguous()
     k_pages, v_pages = _empty_pages(35, kv_heads, head_dim, torch.bfloat16, 7.0, 7.0, "cuda")
     rope = dict(cos=torch.from_numpy(cos_np).cuda(), sin=torch.from_numpy(sin_np).cuda(), tok_slot=_i32(slots),
@@ -288,6 +334,64 @@ def test_fused_norm_projection(m, k, with_delta, gain_dtype):
     written = sum(1 for _ in seen)
     assert int((k_plain != 7.0).any(dim=-1).sum()) <= written * kv_heads
     assert int((v_plain != 7.0).any(dim=-1).sum()) <= written * kv_heads
+
+
+@pytest.mark.parametrize("hint", [16, 32, 48, 64])
+@pytest.mark.parametrize("m", [65, 200])
+def test_scaled_projection_with_every_tile(hint, m):
+    """The tiled kernel's epilogues with each of its tile shapes (the hint picks
+    one): pairs of strips in a wave, one or two of them."""
+    ops = _ops()
+    torch.manual_seed(hint + m)
+    k, eps = 96, 1e-5
+    v = torch.randn(m, k) * 2
+    gain = (1 + 0.3 * torch.randn(k)).bfloat16()
+    normed = P.rms_norm(v.double(), gain.double(), eps)
+    resid = v.cuda()
+    scaled = torch.empty(m, k, dtype=torch.bfloat16, device="cuda")
+    ss = torch.empty(ops.gemm_residual_parts(m, k), m, device="cuda")
+    parts = ops.gemm_residual(torch.zeros(m, 8, dtype=torch.bfloat16, device="cuda"), torch.zeros(k, 8, dtype=torch.bfloat16, device="cuda"),
+                              resid, gain.cuda(), scaled, ss)
+
+    def close(got, want, what):
+        assert ((got - want).abs() <= 2e-2 * (1 + want.abs())).all(), (what, (got - want).abs().max().item())
+
+    n = 300
+    w = (torch.randn(n, k) / math.sqrt(k)).bfloat16()
+    y = torch.empty(m, n, dtype=torch.bfloat16, device="cuda")
+    close(ops.gemm_scaled(scaled, ss, parts, eps, w.cuda(), y, ops.EPILOGUE_STORE, None, hint).cpu().double(), normed @ w.double().t(), "store")
+    inner = 200
+    w = (torch.randn(2 * inner, k) / math.sqrt(k)).bfloat16()
+    both = normed @ w.double().t()
+    y = torch.empty(m, inner, dtype=torch.bfloat16, device="cuda")
+    close(ops.gemm_scaled(scaled, ss, parts, eps, w.cuda(), y, ops.EPILOGUE_SILU, None, hint).cpu().double(),
+          P.silu(both[:, :inner]) * both[:, inner:], "silu")
+    heads, kv_heads, head_dim = 5, 2, 64
+    w = (torch.randn((heads + 2 * kv_heads) * head_dim, k) / math.sqrt(k)).bfloat16()
+    qkv = (normed @ w.double().t()).view(m, heads + 2 * kv_heads, head_dim)
+    cos_np, sin_np = P.rope_tables(256, head_dim, 10000.0)
+    positions = [(i * 37) % 256 for i in range(m)]
+    slots = [0 if i % 11 else -1 for i in range(m)]
+    table = _i32([[3, 1, 0, 2]])
+    k_pages, v_pages = _empty_pages(4, kv_heads, head_dim, torch.bfloat16, 7.0, 7.0, "cuda")
+    rope = dict(cos=torch.from_numpy(cos_np).cuda(), sin=torch.from_numpy(sin_np).cuda(), tok_slot=_i32(slots),
+                tok_pos=_i32(positions), k_pages=k_pages, v_pages=v_pages, block_table=table, heads=heads,
+                kv_heads=kv_heads, head_dim=head_dim)
+    y = torch.empty(m, heads * head_dim, dtype=torch.bfloat16, device="cuda")
+    got_q = ops.gemm_scaled(scaled, ss, parts, eps, w.cuda(), y, ops.EPILOGUE_ROPE, rope, hint).cpu().double()
+    pos = torch.tensor(positions)
+    turned = P.rope_rotate_half(qkv[:, :heads + kv_heads], torch.from_numpy(cos_np)[pos].double(), torch.from_numpy(sin_np)[pos].double())
+    close(got_q.view(m, heads, head_dim), turned[:, :heads], "queries")
+    k_plain, v_plain = _read_pages(k_pages, v_pages, head_dim)
+    written = 0
+    for t in range(m):
+        if slots[t] < 0:
+            continue
+        written += 1
+        page, inside = table[0, positions[t] // 64].item(), positions[t] % 64
+        close(k_plain[page, :, inside, :].double(), turned[t, heads:], "keys")
+        close(v_plain[page, :, inside, :].double(), qkv[t, heads + kv_heads:], "values")
+    assert int((k_plain != 7.0).any(dim=-1).sum()) <= written * kv_heads  # padding rows wrote nothing
 
 
 def _k_index(head_dim):
