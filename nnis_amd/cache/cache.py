@@ -187,6 +187,29 @@ class SequenceCache:
         for group in self.kv_groups:
             group.flush()
 
+    def grow_by_one(self, slots: Sequence[int]) -> List[int]:
+        """One more token for each of the slots (a decode step): returns their
+        lengths before.  Only a sequence that starts a new page takes the long
+        way; all or nothing as ``grow``."""
+        lengths = self.lengths
+        try:
+            before = [lengths[slot] for slot in slots]
+        except KeyError as error:
+            raise InvalidInput(f"cache slot {error.args[0]} is not held") from None
+        crossing = {slot: 1 for slot, length in zip(slots, before) if length % PAGE_TOKENS == 0}
+        if before and max(before) >= self.max_positions:
+            self.check_room({slot: 1 for slot in slots})  # raises, naming the slot
+        if crossing:
+            self.check_room(crossing)
+            for slot in crossing:
+                for group in self.kv_groups:
+                    group.grow(slot, lengths[slot] + 1)
+            for group in self.kv_groups:
+                group.flush()
+        for slot, length in zip(slots, before):
+            lengths[slot] = length + 1
+        return before
+
     def bytes_per_token(self) -> int:
         return sum(group.bytes_per_token() for group in self.kv_groups)
 

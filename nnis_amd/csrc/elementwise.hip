@@ -451,19 +451,9 @@ __device__ __forceinline__ bool better(float v, int i, float best_v, int best_i)
   return v > best_v || (v == best_v && i < best_i);
 }
 
-__global__ void argmax_kernel(const float* __restrict__ logits, int* __restrict__ out, int vocab) {
-  __shared__ float s_val[16];
-  __shared__ int s_idx[16];
-  const float* row = logits + (size_t)blockIdx.x * vocab;
-  float best_v = -INFINITY;
-  int best_i = 0x7fffffff;
-  for (int c = threadIdx.x; c < vocab; c += blockDim.x) {
-    const float v = row[c];
-    if (better(v, c, best_v, best_i)) {
-      best_v = v;
-      best_i = c;
-    }
-  }
+constexpr int kArgmaxChunk = 4096;  // columns a block of the first pass takes: 16 a thread, all asked for at once
+
+__device__ __forceinline__ void wave_best(float& best_v, int& best_i) {
 #pragma unroll
   for (int offset = kWave / 2; offset > 0; offset >>= 1) {
     const float ov = __shfl_xor(best_v, offset, kWave);
@@ -473,6 +463,48 @@ __global__ void argmax_kernel(const float* __restrict__ logits, int* __restrict_
       best_i = oi;
     }
   }
+}
+
+// first pass: block (chunk, row) leaves the best of its chunk of the row in part_v / part_i [rows, chunks]
+__global__ __launch_bounds__(256) void argmax_chunk_kernel(const float* __restrict__ logits, float* __restrict__ part_v,
+                                                           int* __restrict__ part_i, int vocab, int chunks) {
+  __shared__ float s_val[4];
+  __shared__ int s_idx[4];
+  const int chunk = blockIdx.x, row_index = blockIdx.y;
+  const float* row = logits + (size_t)row_index * vocab;
+  const int c0 = chunk * kArgmaxChunk;
+  float v[16];
+  if (vocab % 4 == 0) {  // rows are 16-byte aligned: four loads of four a thread
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int c = c0 + (j * 256 + threadIdx.x) * 4;
+      f32x4_t four = {-INFINITY, -INFINITY, -INFINITY, -INFINITY};
+      if (c + 4 <= vocab) four = *(const f32x4_t*)(row + c);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[4 * j + e] = four[e];
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int c = c0 + (j * 256 + threadIdx.x) * 4 + e;
+        v[4 * j + e] = c < vocab ? row[c] : -INFINITY;
+      }
+  }
+  float best_v = -INFINITY;
+  int best_i = 0x7fffffff;
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int c = c0 + (j * 256 + threadIdx.x) * 4 + e;
+      if (c < vocab && better(v[4 * j + e], c, best_v, best_i)) {
+        best_v = v[4 * j + e];
+        best_i = c;
+      }
+    }
+  wave_best(best_v, best_i);
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
   if (lane == 0) {
     s_val[wave] = best_v;
@@ -480,22 +512,53 @@ __global__ void argmax_kernel(const float* __restrict__ logits, int* __restrict_
   }
   __syncthreads();
   if (threadIdx.x == 0) {
-    const int waves = (blockDim.x + kWave - 1) / kWave;
-    for (int w = 1; w < waves; ++w) {
+    for (int w = 1; w < 4; ++w) {
       if (better(s_val[w], s_idx[w], best_v, best_i)) {
         best_v = s_val[w];
         best_i = s_idx[w];
       }
     }
-    out[blockIdx.x] = best_i == 0x7fffffff ? 0 : best_i;
+    part_v[(size_t)row_index * chunks + chunk] = best_v;
+    part_i[(size_t)row_index * chunks + chunk] = best_i;
   }
 }
 
-extern "C" int nnis_argmax(const float* logits, int* out, int rows, int vocab, void* stream) {
+// second pass: a wave per row over the chunks' bests
+__global__ __launch_bounds__(64) void argmax_rows_kernel(const float* __restrict__ part_v, const int* __restrict__ part_i,
+                                                         int* __restrict__ out, int chunks) {
+  const int row_index = blockIdx.x;
+  float best_v = -INFINITY;
+  int best_i = 0x7fffffff;
+  for (int c = threadIdx.x; c < chunks; c += kWave) {
+    const float v = part_v[(size_t)row_index * chunks + c];
+    const int i = part_i[(size_t)row_index * chunks + c];
+    if (better(v, i, best_v, best_i)) {
+      best_v = v;
+      best_i = i;
+    }
+  }
+  wave_best(best_v, best_i);
+  if (threadIdx.x == 0) out[row_index] = best_i == 0x7fffffff ? 0 : best_i;
+}
+
+// scratch: at least nnis_argmax_scratch(rows, vocab) 4-byte words, 16-byte aligned
+extern "C" int nnis_argmax_scratch(int rows, int vocab) {
+  const int chunks = (vocab + kArgmaxChunk - 1) / kArgmaxChunk;
+  return 2 * rows * chunks;
+}
+
+extern "C" int nnis_argmax(const float* logits, int* out, int rows, int vocab, void* scratch, void* stream) {
   NNIS_REQUIRE(rows >= 0 && vocab > 0, "argmax: bad sizes rows=%d vocab=%d", rows, vocab);
   if (rows == 0) return 0;
-  const int threads = vocab >= 8192 ? 1024 : (vocab >= 1024 ? 256 : 64);
-  hipLaunchKernelGGL(argmax_kernel, dim3(rows), dim3(threads), 0, (hipStream_t)stream, logits, out, vocab);
+  NNIS_REQUIRE(scratch != nullptr, "argmax: needs scratch memory");
+  NNIS_REQUIRE(rows <= 65535, "argmax: %d rows exceed the grid limit", rows);
+  const int chunks = (vocab + kArgmaxChunk - 1) / kArgmaxChunk;
+  float* part_v = (float*)scratch;
+  int* part_i = (int*)(part_v + (size_t)rows * chunks);
+  hipLaunchKernelGGL(argmax_chunk_kernel, dim3(chunks, rows), dim3(256), 0, (hipStream_t)stream, logits, part_v, part_i, vocab,
+                     chunks);
+  NNIS_LAUNCH_CHECK("argmax");
+  hipLaunchKernelGGL(argmax_rows_kernel, dim3(rows), dim3(64), 0, (hipStream_t)stream, part_v, part_i, out, chunks);
   NNIS_LAUNCH_CHECK("argmax");
   return 0;
 }

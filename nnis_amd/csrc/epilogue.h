@@ -12,18 +12,25 @@ enum : int { EPI_STORE = 0, EPI_SILU = 1, EPI_ROPE = 2 };
 typedef __attribute__((ext_vector_type(4))) __bf16 epi_bf16x4;
 typedef __attribute__((ext_vector_type(4))) float epi_f32x4;
 
-// SiLU(gate) * up as /root/reference/crates/nnis-model/src/fused_swiglu.rs:14-28: gate / (1 + exp(-gate)) * up.
+// SiLU(gate) * up as /root/reference/crates/nnis-model/src/fused_swiglu.rs:14-28: gate / (1 + exp(-gate)) * up,
+// with the hardware's base-2 exponential and reciprocal (each within an ulp of 32-bit; the result is
+// rounded to bfloat16).  The 32-bit path of the model has a kernel of its own with the library's exp.
+__device__ __forceinline__ float silu_times(float gate, float up) {
+  const float e = __builtin_amdgcn_exp2f(gate * -1.4426950408889634f);
+  return gate * __builtin_amdgcn_rcpf(1.0f + e) * up;
+}
+
 // column: the first of the lane's four channels; inner: channels of the feed-forward
 __device__ __forceinline__ void epilogue_silu(bf16_t* y, int token, int inner, int column, const float (&gate)[4],
                                               const float (&up)[4]) {
   if (column + 4 <= inner && inner % 4 == 0) {
     epi_bf16x4 packed;
 #pragma unroll
-    for (int e = 0; e < 4; ++e) packed[e] = (__bf16)(gate[e] / (1.0f + expf(-gate[e])) * up[e]);
+    for (int e = 0; e < 4; ++e) packed[e] = (__bf16)silu_times(gate[e], up[e]);
     *(epi_bf16x4*)(y + (size_t)token * inner + column) = packed;
   } else {
     for (int e = 0; e < 4; ++e)
-      if (column + e < inner) y[(size_t)token * inner + column + e] = (bf16_t)(gate[e] / (1.0f + expf(-gate[e])) * up[e]);
+      if (column + e < inner) y[(size_t)token * inner + column + e] = (bf16_t)silu_times(gate[e], up[e]);
   }
 }
 

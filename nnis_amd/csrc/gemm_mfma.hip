@@ -81,35 +81,54 @@ struct ResidualOut {
   float* ss;         // [parts, m]; a part is 16 columns (skinny kernel) or a wave's columns (tiled kernel)
 };
 
-// four consecutive columns of a token: the lane's accumulator acc
-__device__ __forceinline__ float residual_take(const ResidualOut& o, size_t index, int column, f32x4 acc, int valid, bool vector_ok) {
+// four consecutive columns of a token: what the stream and the gain hold there, asked for early
+struct ResidualHeld {
+  f32x4 v, g;
+};
+
+__device__ __forceinline__ ResidualHeld residual_ask(const ResidualOut& o, size_t index, int column, int valid, bool vector_ok) {
   typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
-  float sq = 0.0f;
+  ResidualHeld h;
+  h.v = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
+  h.g = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
   if (valid == 4 && vector_ok) {
-    f32x4 v = *(const f32x4*)(o.resid + index);
-    f32x4 g;
+    h.v = *(const f32x4*)(o.resid + index);
     if (o.gain_dtype == NNIS_F32) {
-      g = *(const f32x4*)((const float*)o.gain + column);
+      h.g = *(const f32x4*)((const float*)o.gain + column);
     } else {
       const bf16x4 packed = *(const bf16x4*)((const bf16_t*)o.gain + column);
 #pragma unroll
-      for (int e = 0; e < 4; ++e) g[e] = (float)packed[e];
+      for (int e = 0; e < 4; ++e) h.g[e] = (float)packed[e];
     }
-    bf16x4 scaled;
+  } else {
+    for (int e = 0; e < valid; ++e) {
+      h.v[e] = o.resid[index + e];
+      h.g[e] = load_as_f32(o.gain, o.gain_dtype, column + e);
+    }
+  }
+  return h;
+}
+
+// ... and the lane's accumulator acc taken in; returns the lane's part of the row's sum of squares
+__device__ __forceinline__ float residual_take(const ResidualOut& o, const ResidualHeld& h, size_t index, f32x4 acc, int valid,
+                                               bool vector_ok) {
+  typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+  float sq = 0.0f;
+  f32x4 v = h.v;
+  bf16x4 scaled;
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      v[e] += acc[e];
-      sq = fmaf(v[e], v[e], sq);
-      scaled[e] = (__bf16)(v[e] * g[e]);
-    }
+  for (int e = 0; e < 4; ++e) {
+    v[e] += acc[e];
+    if (e < valid) sq = fmaf(v[e], v[e], sq);
+    scaled[e] = (__bf16)(v[e] * h.g[e]);
+  }
+  if (valid == 4 && vector_ok) {
     *(f32x4*)(o.resid + index) = v;
     *(bf16x4*)(o.scaled + index) = scaled;
   } else {
     for (int e = 0; e < valid; ++e) {
-      const float v = o.resid[index + e] + acc[e];
-      sq = fmaf(v, v, sq);
-      o.resid[index + e] = v;
-      o.scaled[index + e] = (bf16_t)(v * load_as_f32(o.gain, o.gain_dtype, column + e));
+      o.resid[index + e] = v[e];
+      o.scaled[index + e] = scaled[e];
     }
   }
   return sq;
@@ -167,6 +186,22 @@ __global__ __launch_bounds__(KSPLIT > 4 ? 64 * KSPLIT : 256) void gemm_skinny_ke
 #pragma unroll
   for (int t = 0; t < MT; ++t) acc[t] = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
 
+  // lane holds D[weight row 4g + e][token r]: four consecutive outputs of one token
+  const int n0 = strip * 16 + g * 4;
+  const int valid = n - n0 >= 4 ? 4 : (n - n0 > 0 ? n - n0 : 0);
+  const bool vector_ok = (n % 4) == 0;
+  constexpr bool kResidual = std::is_same<OutT, ResidualOut>::value;
+  ResidualHeld held[kResidual ? MT : 1];
+  if constexpr (kResidual) {
+    if (active && part == 0) {  // the wave that ends the strip asks for the stream before its weights
+#pragma unroll
+      for (int t = 0; t < MT; ++t) {
+        const int token = t * 16 + r;
+        held[t] = residual_ask(y, (size_t)(token < m ? token : 0) * n + n0, n0, (token < m) ? valid : 0, vector_ok);
+      }
+    }
+  }
+
   if (active) {
     int w_row = strip * 16 + r;
     w_row = w_row < n ? w_row : n - 1;  // rows beyond N read a valid row and are not stored
@@ -221,16 +256,12 @@ __global__ __launch_bounds__(KSPLIT > 4 ? 64 * KSPLIT : 256) void gemm_skinny_ke
   }
   if (!active) return;
 
-  // lane holds D[weight row 4g + e][token r]: four consecutive outputs of one token
-  const int n0 = strip * 16 + g * 4;
-  const int valid = n - n0 >= 4 ? 4 : (n - n0 > 0 ? n - n0 : 0);
-  const bool vector_ok = (n % 4) == 0;
 #pragma unroll
   for (int t = 0; t < MT; ++t) {
     const int token = t * 16 + r;
-    if constexpr (std::is_same<OutT, ResidualOut>::value) {
+    if constexpr (kResidual) {
       float sq = 0.0f;
-      if (token < m && valid > 0) sq = residual_take(y, (size_t)token * n + n0, n0, acc[t], valid, vector_ok);
+      if (token < m && valid > 0) sq = residual_take(y, held[t], (size_t)token * n + n0, acc[t], valid, vector_ok);
       sq += __shfl_xor(sq, 16, kWave);
       sq += __shfl_xor(sq, 32, kWave);
       if (g == 0 && token < m) y.ss[(size_t)strip * m + token] = sq;
@@ -323,6 +354,23 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
         tok_page[i] = (slot >= 0 && y.rope.k_pages) ? y.rope.block_table[(size_t)slot * y.rope.max_pages + tok_pos[i] / kPageTokens] : -1;
       }
     }
+  }
+
+  // a residual epilogue asks for the stream and the gain before the product (small tiles: registers)
+  constexpr bool kResidual = std::is_same<OutT, ResidualOut>::value;
+  constexpr bool kAskEarly = kResidual && TM * TN <= 8;
+  ResidualHeld held[kAskEarly ? TM : 1][kAskEarly ? TN : 1];
+  if constexpr (kAskEarly) {
+    const bool vector_ok = (n % 4) == 0;
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const int token = row0 + wave_m * WM + i * 16 + r;
+        const int n0 = col0 + wave_n * WN + j * 16 + g * 4;
+        const int valid = (token < m) ? (n - n0 >= 4 ? 4 : (n - n0 > 0 ? n - n0 : 0)) : 0;
+        held[i][j] = residual_ask(y, (size_t)(token < m ? token : 0) * n + (valid > 0 ? n0 : 0), valid > 0 ? n0 : 0, valid, vector_ok);
+      }
   }
 
   bf16x8 a_stage[PF][A_CHUNKS], b_stage[PF][B_CHUNKS];
@@ -418,11 +466,13 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
       const int n0 = col0 + wave_n * WN + j * 16 + g * 4;
       const int valid = n - n0 >= 4 ? 4 : (n - n0 > 0 ? n - n0 : 0);
       if (token >= m || valid <= 0) continue;
-      if constexpr (std::is_same<OutT, ResidualOut>::value) sq += residual_take(y, (size_t)token * n + n0, n0, acc[i][j], valid, vector_ok);
-      else if constexpr (EPI == EPI_STORE) store4(y.y, (size_t)token * n + n0, acc[i][j] * scale, valid, vector_ok);
+      if constexpr (kResidual) {
+        if constexpr (kAskEarly) sq += residual_take(y, held[i][j], (size_t)token * n + n0, acc[i][j], valid, vector_ok);
+        else sq += residual_take(y, residual_ask(y, (size_t)token * n + n0, n0, valid, vector_ok), (size_t)token * n + n0, acc[i][j], valid, vector_ok);
+      } else if constexpr (EPI == EPI_STORE) store4(y.y, (size_t)token * n + n0, acc[i][j] * scale, valid, vector_ok);
       else store4(y, (size_t)token * n + n0, acc[i][j], valid, vector_ok);
     }
-    if constexpr (std::is_same<OutT, ResidualOut>::value) {
+    if constexpr (kResidual) {
       // a part of the row's sum of squares: this wave's columns
       sq += __shfl_xor(sq, 16, kWave);
       sq += __shfl_xor(sq, 32, kWave);

@@ -109,6 +109,8 @@ class Engine:
         """As ``step``, but the rows may view a buffer that the next step
         overwrites: for callers that read them at once (the generation loop)."""
         self._borrowed = False
+        if self.use_graphs and entries and all(len(e.tokens) == 1 for e in entries):
+            return self._decode_step(entries)
         growth = self._validate(entries)
         pos0 = [self.cache.length(e.slot) for e in entries]
         counts = [len(e.tokens) for e in entries]
@@ -129,9 +131,6 @@ class Engine:
             row += n
             seq_start[index + 1] = row
         self.cache.grow(growth)
-
-        if self.use_graphs and all(n == 1 for n in counts):
-            return self._graph_step(entries, pos0)
 
         # the staging buffer is reused: wait until the previous step's copy has left it
         torch.cuda.current_stream().synchronize() if self._staging is not None else None
@@ -157,16 +156,31 @@ class Engine:
         )
         return self.model.forward(dev[0], ctx, self.cache, dev[6], self.rt)
 
-    def _graph_step(self, entries: Sequence[StepEntry], pos0: List[int]) -> torch.Tensor:
-        """A step of single tokens, replayed from a captured graph.  The rows
+    def _decode_step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        """A step of single tokens, replayed from a captured graph: the same
+        checks as any step, without the arrays a prompt needs.  The rows
         returned view the graph's output buffer: read them before the next step."""
         from .graph import DecodeGraphs
 
+        slots = [e.slot for e in entries]
+        ids = [int(e.tokens[0]) for e in entries]
+        if len(set(slots)) != len(slots):
+            twice = next(s for s in slots if slots.count(s) > 1)
+            raise InvalidInput(f"slot {twice} appears twice in one step")
+        if min(ids) < 0 or max(ids) >= self.vocab_size:
+            bad = next(t for t in ids if not 0 <= t < self.vocab_size)
+            raise InvalidInput(f"token id {bad} is out of range for vocabulary {self.vocab_size}")
+        for entry in entries:
+            if entry.want is not None:
+                for place in entry.want:
+                    if int(place) != 0:
+                        raise InvalidInput(f"slot {entry.slot}: wanted place {place} is not among its 1 tokens")
+        pos0 = self.cache.grow_by_one(slots)
         if self._graphs is None:
             self._graphs = DecodeGraphs(self)
-        plan = self.model.decode_plan(len(entries), max(p + 1 for p in pos0), self.rt)
+        plan = self.model.decode_plan(len(entries), max(pos0) + 1, self.rt)
         graph = self._graphs.get(len(entries), plan)
-        logits = graph.run([int(e.tokens[0]) for e in entries], [e.slot for e in entries], pos0)
+        logits = graph.run(ids, slots, pos0)
         wanted = [i for i, e in enumerate(entries) if e.want is None or len(e.want) > 0]
         if len(wanted) == len(entries):
             self._borrowed = True

@@ -27,7 +27,8 @@ _CORE_SIGNATURES = {
     "nnis_rope_kv_write": [_VOID, _INT, _VOID, _INT, _VOID, _VOID, _INT, _INT, _VOID, _VOID, _VOID, _VOID, _INT,
                            _VOID, _INT, _INT, _INT, _INT, _INT, _VOID],
     "nnis_silu_mul": [_VOID, _INT, _VOID, _INT, _INT, _INT, _VOID],
-    "nnis_argmax": [_VOID, _VOID, _INT, _INT, _VOID],
+    "nnis_argmax": [_VOID, _VOID, _INT, _INT, _VOID, _VOID],
+    "nnis_argmax_scratch": [_INT, _INT],
     "nnis_gemm_ordered": [_VOID, _INT, _VOID, _INT, _VOID, _INT, _INT, _INT, _INT, _VOID],
     "nnis_gemm_bf16": [_VOID, _VOID, _VOID, _INT, _INT, _INT, _INT, _INT, _VOID],
     "nnis_gemm_fused": [_VOID, _VOID, _VOID, _VOID, _INT, _FLT, _VOID, _INT, _INT, _INT, _INT, _VOID, _VOID, _VOID, _INT,
@@ -216,8 +217,11 @@ def argmax(logits: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     rows, vocab = logits.shape
     if logits.dtype != torch.float32 or out.dtype != torch.int32 or out.numel() < rows:
         raise KernelError("argmax: logits must be float32 [rows, vocab] and out int32 [rows]")
+    if not logits.is_contiguous():
+        raise KernelError("argmax: logits must be contiguous")
     lib = core()
-    _check(lib, lib.nnis_argmax(logits.data_ptr(), out.data_ptr(), rows, vocab, _stream()))
+    scratch = torch.empty(max(1, lib.nnis_argmax_scratch(rows, vocab)), dtype=torch.float32, device=logits.device)
+    _check(lib, lib.nnis_argmax(logits.data_ptr(), out.data_ptr(), rows, vocab, scratch.data_ptr(), _stream()))
     return out
 
 

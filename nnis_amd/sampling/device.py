@@ -27,6 +27,16 @@ class DeviceSelector:
             cache.add_state_region(RNG_REGION, (), torch.int64)
         self.rng = cache.state_regions[RNG_REGION]
         self._weights = None
+        self._picked = None       # int32 on the device, reused from step to step
+        self._picked_host = None  # its pinned twin: the copy back needs no staging
+
+    def _to_host(self, picked: torch.Tensor, rows: int) -> List[int]:
+        if self._picked_host is None or self._picked_host.numel() < rows:
+            self._picked_host = torch.empty(max(rows, 64), dtype=torch.int32, pin_memory=True)
+        host = self._picked_host[:rows]
+        host.copy_(picked[:rows], non_blocking=True)
+        torch.cuda.current_stream().synchronize()
+        return host.tolist()
 
     def start(self, slot: int, params: Optional[SamplingParams]) -> None:
         """Called when a sequence starts: seeds its generator."""
@@ -39,7 +49,9 @@ class DeviceSelector:
         """One token per row of ``logits`` (float32 [rows, vocab] on the device)."""
         rows = logits.shape[0]
         ops = self.rt.ops
-        picked = torch.empty(rows, dtype=torch.int32, device=self.rt.device)
+        if self._picked is None or self._picked.numel() < rows:
+            self._picked = torch.empty(max(rows, 64), dtype=torch.int32, device=self.rt.device)
+        picked = self._picked[:rows]
         ops.argmax(logits, picked)
         if any(p is not None for p in params):
             row_slot = np.asarray([s if p is not None else -1 for s, p in zip(slots, params)], dtype=np.int32)
@@ -66,4 +78,4 @@ class DeviceSelector:
                         raise InvalidInput(f"sampling refused row {row}: a logit is not finite")
                     out.append(sampled_host[row])
             return out
-        return picked.cpu().tolist()
+        return self._to_host(picked, rows)

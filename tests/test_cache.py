@@ -147,3 +147,33 @@ def test_a_page_holds_every_key_and_value_once(head_dim):
     assert k_offset(5, 8) - k_offset(4, 8) == 8
     # lane (r, g) of a value load: channel 16 t + r, tokens 32 h + 8 g ..; consecutive lanes r, then g
     assert v_offset(1, 0) - v_offset(0, 0) == 8 and v_offset(0, 8) - v_offset(15, 0) == 8
+
+
+def test_one_more_token_each_is_all_or_nothing():
+    cache = _cache(max_tokens=192)  # 3 pages, 3 slots
+    a, b = cache.acquire(), cache.acquire()
+    cache.grow({a: 64, b: 63})
+    free = cache.kv_groups[0].table.pool.free
+    assert cache.grow_by_one([a, b]) == [64, 63]  # a starts its second page, b fills its first
+    assert cache.length(a) == 65 and cache.length(b) == 64
+    assert cache.kv_groups[0].table.pool.free == free - 1
+    assert cache.kv_groups[0].block_table[a, :2].tolist() == cache.kv_groups[0].table.rows[a]
+    # b needs a page now and none is left: nothing changes, a included
+    with pytest.raises(CacheFull):
+        cache.grow_by_one([a, b])
+    assert cache.length(a) == 65 and cache.length(b) == 64 and cache.kv_groups[0].table.pool.free == 0
+    with pytest.raises(InvalidInput, match="not held"):
+        cache.grow_by_one([a, 7])
+    assert cache.length(a) == 65
+    cache.release(b)
+    c = cache.acquire()
+    for _ in range(64):
+        cache.grow_by_one([c])  # the page that b gave back
+    assert cache.length(c) == 64 and cache.kv_groups[0].table.pool.free == 0
+    lone = SequenceCache([(0, KVRequest(1, 16))], {}, max_tokens=640, max_positions=70, dtype=torch.float32, device="cpu")
+    s = lone.acquire()
+    lone.grow({s: 69})
+    assert lone.grow_by_one([s]) == [69]
+    with pytest.raises(CacheFull, match="positions end at 70"):
+        lone.grow_by_one([s])
+    assert lone.length(s) == 70

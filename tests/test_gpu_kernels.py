@@ -575,12 +575,16 @@ def test_argmax(vocab):
         logits[2] = 0.5  # all equal: index 0
         logits[3, 3] = float("nan")
         logits[3, 20] = 30.0
+    if vocab > 9000:
+        logits[4, 8999] = logits[4, 100] = 12.0  # a tie between two blocks' shares of the row
     out = torch.empty(5, dtype=torch.int32, device="cuda")
     ops.argmax(logits.cuda(), out)
     want = [int(np.nanargmax(row)) for row in logits.numpy()]
     assert out.cpu().tolist() == want
     if vocab >= 63:
         assert want[:3] == [7, vocab - 1, 0]
+    if vocab > 9000:
+        assert want[4] == 100
 
 
 def test_refusals():
