@@ -272,15 +272,19 @@ __global__ __launch_bounds__(KSPLIT > 4 ? 64 * KSPLIT : 256) void gemm_skinny_ke
 }
 
 // -----------------------------------------------------------------------------
-// tiled: BM x BN output tile per block of 4 waves (2 x 2), K in steps of BK (64 or 128)
+// tiled: BM x BN output tile per block of 4 waves (2 x 2), K in steps of BK (64; steps of 128 and tiles of
+// 32 rows were measured no faster on products from 2048 x 576 x 576 to 2048 x 6144 x 2048)
 // -----------------------------------------------------------------------------
 // chunk c of row `row` of a staged tile (CHUNKS chunks of 16 bytes a row) lives at chunk c ^ (row % CHUNKS)
 template <int CHUNKS>
 __device__ __forceinline__ int swizzled(int row, int chunk) { return row * CHUNKS + (chunk ^ (row & (CHUNKS - 1))); }
 
+#ifndef NNIS_TILE_GROUP_ROWS
+#define NNIS_TILE_GROUP_ROWS 512
+#endif
 template <int BM, int BN, int BK, typename OutT>
 __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
-                                                         OutT y, int m, int n, int k) {
+                                                         OutT y, int m, int n, int k, int col_blocks) {
   constexpr int WM = BM / 2, WN = BN / 2;  // a wave's part of the tile
   constexpr int TM = WM / 16, TN = WN / 16;
   constexpr int CH = BK / 8;  // 16-byte chunks per staged row
@@ -296,7 +300,24 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
   const int wave = tid / kWave, lane = tid % kWave;
   const int wave_m = wave / 2, wave_n = wave % 2;
   const int r = lane % 16, g = lane / 16;
-  const int row0 = blockIdx.y * BM, col0 = blockIdx.x * BN;
+  // Blocks go to the chip's 8 dies in turn (block i to die i % 8), and each die has an L2 of its own: the
+  // tiles are dealt so that a die's blocks cover a band of consecutive rows of X with all their column
+  // blocks, and each die reads its band once instead of every die reading all of X.
+  int col_block, row_block;
+  {
+    const int total = gridDim.x, die = blockIdx.x % 8, nth = blockIdx.x / 8;
+    const int each = total / 8, more = total % 8;  // the first `more` dies have one block more
+    const int tile = die * each + (die < more ? die : more) + nth;
+    // within the order of the tiles, kGroup row blocks go through the column blocks together, rows fastest:
+    // a column block of W serves them all while it is near
+    constexpr int kGroup = NNIS_TILE_GROUP_ROWS / BM;
+    const int row_blocks = total / col_blocks;
+    const int group = tile / (kGroup * col_blocks), within = tile % (kGroup * col_blocks);
+    const int rows_here = min(kGroup, row_blocks - group * kGroup);
+    row_block = group * kGroup + within % rows_here;
+    col_block = within / rows_here;
+  }
+  const int row0 = row_block * BM, col0 = col_block * BN;
 
   f32x4 acc[TM][TN];
 #pragma unroll
@@ -324,7 +345,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
     const int index = tid + c * 256;
     int row;
     if constexpr (kPaired) {
-      row = paired_weight_row<EPI, BN>(y.rope, blockIdx.x, index / CH, n);
+      row = paired_weight_row<EPI, BN>(y.rope, col_block, index / CH, n);
       row = row >= 0 ? row : 0;  // rows beyond the end read a valid row and are not stored
     } else {
       row = col0 + index / CH;
@@ -433,7 +454,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
       const float scale = row_scale[wave_m * WM + i * 16 + r];
 #pragma unroll
       for (int u = 0; u < TN / 2; ++u) {
-        const int first = paired_weight_row<EPI, BN>(y.rope, blockIdx.x, wave_n * WN + 32 * u, n);  // the unit's first lower row
+        const int first = paired_weight_row<EPI, BN>(y.rope, col_block, wave_n * WN + 32 * u, n);  // the unit's first lower row
         if (first < 0) continue;
         float lo[4], hi[4];
 #pragma unroll
@@ -476,7 +497,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
       // a part of the row's sum of squares: this wave's columns
       sq += __shfl_xor(sq, 16, kWave);
       sq += __shfl_xor(sq, 32, kWave);
-      if (g == 0 && token < m) y.ss[(size_t)(blockIdx.x * 2 + wave_n) * m + token] = sq;
+      if (g == 0 && token < m) y.ss[(size_t)(col_block * 2 + wave_n) * m + token] = sq;
     }
   }
   }
@@ -511,8 +532,9 @@ void dispatch_skinny(const bf16_t* x, const bf16_t* w, OutT y, int m, int n, int
 // `columns`: the weight rows the grid covers (n, or the rows of all pair units)
 template <int BM, int BN, int BK, typename OutT>
 void launch_tiled(const bf16_t* x, const bf16_t* w, OutT y, int m, int n, int k, int columns, hipStream_t stream) {
-  hipLaunchKernelGGL((gemm_tiled_kernel<BM, BN, BK, OutT>), dim3((columns + BN - 1) / BN, (m + BM - 1) / BM), dim3(256), 0,
-                     stream, x, w, y, m, n, k);
+  const int col_blocks = (columns + BN - 1) / BN, row_blocks = (m + BM - 1) / BM;
+  hipLaunchKernelGGL((gemm_tiled_kernel<BM, BN, BK, OutT>), dim3((unsigned)col_blocks * row_blocks), dim3(256), 0, stream, x, w,
+                     y, m, n, k, col_blocks);
 }
 
 // returns the number of wave columns (parts of a row that a residual epilogue sums by itself)
@@ -524,11 +546,10 @@ int dispatch_tiled(const bf16_t* x, const bf16_t* w, OutT y, int m, int n, int k
   const long long blocks_128 = (long long)((m + 127) / 128) * ((columns + 127) / 128);
   const long long blocks_64_128 = (long long)((m + 63) / 64) * ((columns + 127) / 128);
   int tile = blocks_128 >= 384 ? 1 : (blocks_64_128 >= 256 ? 2 : 3);
-  if (tile_hint >= 1 && tile_hint <= 4) tile = tile_hint;  // for tuning runs
+  if (tile_hint >= 1 && tile_hint <= 3) tile = tile_hint;  // for tuning runs
   if (tile == 1) launch_tiled<128, 128, 64, OutT>(x, w, y, m, n, k, columns, stream);
   else if (tile == 2) launch_tiled<64, 128, 64, OutT>(x, w, y, m, n, k, columns, stream);
-  else if (tile == 3) launch_tiled<64, 64, 64, OutT>(x, w, y, m, n, k, columns, stream);
-  else launch_tiled<64, 64, 128, OutT>(x, w, y, m, n, k, columns, stream);
+  else launch_tiled<64, 64, 64, OutT>(x, w, y, m, n, k, columns, stream);
   const int width = tile <= 2 ? 128 : 64;
   return 2 * ((columns + width - 1) / width);
 }
@@ -585,7 +606,7 @@ extern "C" int nnis_gemm_bf16(const void* x, const void* w, void* y, int y_dtype
     NNIS_LAUNCH_CHECK("gemm_skinny");
   } else {
     NNIS_REQUIRE((m + 63) / 64 <= 65535, "gemm_bf16: %d rows exceed the grid limit", m);
-    const int tile_hint = split_hint >= 16 ? split_hint / 16 : 0;  // hints of 16, 32, 48, 64 pick the tile: 128x128, 64x128, 64x64, 64x64 with K in steps of 128
+    const int tile_hint = split_hint >= 16 ? split_hint / 16 : 0;  // hints of 16, 32, 48 pick the tile: 128x128, 64x128, 64x64
     if (y_dtype == NNIS_F32) dispatch_tiled<float*>(xp, wp, (float*)y, m, n, k, tile_hint, stream);
     else dispatch_tiled<bf16_t*>(xp, wp, (bf16_t*)y, m, n, k, tile_hint, stream);
     NNIS_LAUNCH_CHECK("gemm_tiled");
