@@ -194,7 +194,7 @@ __device__ __forceinline__ f32x4 score_tile(const QFrag& keys, const QFrag& quer
 // Softmax state of C column tiles and their outputs
 template <int C>
 struct AttnState {
-  float m[C];       // running maximum (base-2 scaled score) of this lane's column, equal over lane groups
+  float m[C];       // reference of the softmax (a base-2 scaled score near the running maximum) of this lane's column, equal over lane groups
   float l[C];       // this lane's part of the running sum
   f32x4 o[C][kTilesD];
 };
@@ -241,37 +241,51 @@ __device__ __forceinline__ void attend_block(AttnState<C>& st, const QFrag (&q)[
     f32x4 s[2];
     float block_max = -INFINITY;
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
-      s[t] = score_tile(f.keys[t], q[c]);
+    for (int t = 0; t < 2; ++t) s[t] = score_tile(f.keys[t], q[c]);
+    // most blocks lie wholly inside what every lane's column reads: then no key needs a look at its index
+    if (!__all(key0 >= lo[c] && key0 + 31 <= hi[c])) {
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const int key = key0 + 8 * g + 4 * t + e;
-        s[t][e] = (key >= lo[c] && key <= hi[c]) ? s[t][e] * scale_log2 : -INFINITY;
-        block_max = fmaxf(block_max, s[t][e]);
-      }
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int key = key0 + 8 * g + 4 * t + e;
+          s[t][e] = (key >= lo[c] && key <= hi[c]) ? s[t][e] : -INFINITY;
+        }
     }
-    block_max = fmaxf(block_max, __shfl_xor(block_max, 16, kWave));
-    block_max = fmaxf(block_max, __shfl_xor(block_max, 32, kWave));
-    const float m_new = fmaxf(st.m[c], block_max);
-    const float m_safe = m_new == -INFINITY ? 0.0f : m_new;  // a column that has seen no key yet
-    const float alpha = __builtin_amdgcn_exp2f(st.m[c] - m_safe);
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) block_max = fmaxf(block_max, s[t][e]);
+    block_max *= scale_log2;  // the scale is positive: the largest score stays the largest
+    // The column's reference of the softmax (st.m, equal in its four lane groups) moves only when a score
+    // rises more than kLazyRise above it -- always for the first keys, whose reference is -inf.  Until then
+    // the sums are sums of 2^(score - reference) with terms up to 2^kLazyRise: the result is the same up
+    // to rounding, and the block needs no maximum over the lane groups and no scaling of its outputs.
+    if (__any(block_max > st.m[c] + kLazyRise)) {
+      float moved = fmaxf(st.m[c], block_max);
+      moved = fmaxf(moved, __shfl_xor(moved, 16, kWave));
+      moved = fmaxf(moved, __shfl_xor(moved, 32, kWave));
+      const float shrink = st.m[c] == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(st.m[c] - moved);
+      st.l[c] *= shrink;
+#pragma unroll
+      for (int t = 0; t < kTilesD; ++t) st.o[c][t] = st.o[c][t] * shrink;
+      st.m[c] = moved;
+    }
+    const float base = st.m[c] == -INFINITY ? 0.0f : st.m[c];  // a column that has seen no key yet
     bf16x8 p;
     float sum = 0.0f;
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        const float w = __builtin_amdgcn_exp2f(s[t][e] - m_safe);
+        const float w = __builtin_amdgcn_exp2f(fmaf(s[t][e], scale_log2, -base));  // -inf for a masked key: 0
         sum += w;
         p[4 * t + e] = (__bf16)w;
       }
-    st.l[c] = st.l[c] * alpha + sum;
-    st.m[c] = m_new;
+    st.l[c] += sum;
 #pragma unroll
-    for (int t = 0; t < kTilesD; ++t) {
-      st.o[c][t] = st.o[c][t] * alpha;
+    for (int t = 0; t < kTilesD; ++t)
       st.o[c][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.values[t], p, st.o[c][t], 0, 0, 0);
-    }
   }
 }
 
@@ -320,47 +334,49 @@ __device__ __forceinline__ const bf16_t* v_page_ptr(const MfmaArgs& a, int page,
   return a.v_pages + ((size_t)page * a.kv_heads + kv_head) * nnis_v_page_elems(HD);
 }
 
-// Waves of a block that dealt a run of key blocks among themselves: waves 1.. leave
-// their states in LDS, wave 0 folds them into its own.  Returns false for the
-// waves that are done.  `merge` holds [waves - 1][C][kTilesD * 4 + 2][64] floats.
+// Waves of a block (a power of two) that dealt a run of key blocks among themselves fold their states
+// into wave 0's, in halving rounds: the upper half of the waves still in play leave their states in LDS,
+// the lower half take one each.  Returns false for the waves that are done.  `merge` holds
+// [waves / 2][C][kTilesD * 4 + 2][64] floats.
 template <int C>
 __device__ __forceinline__ bool merge_waves(AttnState<C>& st, float* merge, int wave, int waves, int lane) {
   constexpr int kValues = kTilesD * 4 + 2;
-  if (waves == 1) return true;
-  if (wave > 0) {
-    float* mine = merge + (size_t)(wave - 1) * C * kValues * kWave;
+  for (int half = waves >> 1; half >= 1; half >>= 1) {
+    if (wave >= half && wave < 2 * half) {
+      float* mine = merge + (size_t)(wave - half) * C * kValues * kWave;
 #pragma unroll
-    for (int c = 0; c < C; ++c) {
-      float* col = mine + (size_t)c * kValues * kWave + lane;
+      for (int c = 0; c < C; ++c) {
+        float* col = mine + (size_t)c * kValues * kWave + lane;
 #pragma unroll
-      for (int t = 0; t < kTilesD; ++t)
+        for (int t = 0; t < kTilesD; ++t)
 #pragma unroll
-        for (int e = 0; e < 4; ++e) col[(4 * t + e) * kWave] = st.o[c][t][e];
-      col[(kTilesD * 4) * kWave] = st.m[c];
-      col[(kTilesD * 4 + 1) * kWave] = st.l[c];
+          for (int e = 0; e < 4; ++e) col[(4 * t + e) * kWave] = st.o[c][t][e];
+        col[(kTilesD * 4) * kWave] = st.m[c];
+        col[(kTilesD * 4 + 1) * kWave] = st.l[c];
+      }
     }
-  }
-  __syncthreads();
-  if (wave > 0) return false;
-  for (int other = 0; other < waves - 1; ++other) {
-    const float* theirs = merge + (size_t)other * C * kValues * kWave;
+    __syncthreads();
+    if (wave < half) {
+      const float* theirs = merge + (size_t)wave * C * kValues * kWave;
 #pragma unroll
-    for (int c = 0; c < C; ++c) {
-      const float* col = theirs + (size_t)c * kValues * kWave + lane;
-      const float m_other = col[(kTilesD * 4) * kWave];
-      const float m_new = fmaxf(st.m[c], m_other);
-      const float m_safe = m_new == -INFINITY ? 0.0f : m_new;
-      const float mine_w = __builtin_amdgcn_exp2f(st.m[c] - m_safe);
-      const float their_w = __builtin_amdgcn_exp2f(m_other - m_safe);
-      st.l[c] = st.l[c] * mine_w + col[(kTilesD * 4 + 1) * kWave] * their_w;
-      st.m[c] = m_new;
+      for (int c = 0; c < C; ++c) {
+        const float* col = theirs + (size_t)c * kValues * kWave + lane;
+        const float m_other = col[(kTilesD * 4) * kWave];
+        const float m_new = fmaxf(st.m[c], m_other);
+        const float m_safe = m_new == -INFINITY ? 0.0f : m_new;
+        const float mine_w = __builtin_amdgcn_exp2f(st.m[c] - m_safe);
+        const float their_w = __builtin_amdgcn_exp2f(m_other - m_safe);
+        st.l[c] = st.l[c] * mine_w + col[(kTilesD * 4 + 1) * kWave] * their_w;
+        st.m[c] = m_new;
 #pragma unroll
-      for (int t = 0; t < kTilesD; ++t)
+        for (int t = 0; t < kTilesD; ++t)
 #pragma unroll
-        for (int e = 0; e < 4; ++e) st.o[c][t][e] = st.o[c][t][e] * mine_w + col[(4 * t + e) * kWave] * their_w;
+          for (int e = 0; e < 4; ++e) st.o[c][t][e] = st.o[c][t][e] * mine_w + col[(4 * t + e) * kWave] * their_w;
+      }
     }
+    if (half > 1) __syncthreads();  // the next round writes where this one read
   }
-  return true;
+  return wave == 0;
 }
 
 // Runs the pages first, first + stride, ... (`mine` of them) of a sequence through the
@@ -533,7 +549,7 @@ __device__ __forceinline__ void finish_decode(AttnState<C>& st, const bool (&liv
 // more than one split every block leaves its state in `partial` for the combine kernel.
 template <int C>
 __global__ __launch_bounds__(64 * kBlockWaves) void attention_decode_kernel(MfmaArgs a, int waves) {
-  extern __shared__ float merge[];  // [waves - 1][C][kTilesD * 4 + 2][64]
+  extern __shared__ float merge[];  // [waves / 2][C][kTilesD * 4 + 2][64]
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave, r = lane % 16, g = lane / 16;
   const int token = blockIdx.x, kv_head = blockIdx.y, split = blockIdx.z;
   const int slot = a.tok_slot[token];
@@ -599,7 +615,7 @@ __device__ __forceinline__ bf16x4 low4(bf16x8 v) { return __builtin_shufflevecto
 __device__ __forceinline__ bf16x4 high4(bf16x8 v) { return __builtin_shufflevector(v, v, 4, 5, 6, 7); }
 
 __global__ __launch_bounds__(64 * kKeysWaves) void attention_decode_keys_kernel(MfmaArgs a, int waves) {
-  extern __shared__ float merge[];  // [waves - 1][kTilesD * 4 + 2][64]
+  extern __shared__ float merge[];  // [waves / 2][kTilesD * 4 + 2][64]
   constexpr int kStageRow = kPageTokens + 8;  // bfloat16 per head: a page's probabilities, rows apart in the banks
   __shared__ __attribute__((aligned(16))) bf16_t stage[kKeysWaves][4][kStageRow];
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave, r = lane % 16, g = lane / 16;
@@ -799,6 +815,7 @@ int fill_common(MfmaArgs& a, const void* q, void* out, const void* k_pages, cons
   NNIS_REQUIRE(heads > 0 && kv_heads > 0 && heads % kv_heads == 0, "attention: %d heads do not divide into %d kv heads",
                heads, kv_heads);
   NNIS_REQUIRE(window >= 0 && max_pages > 0, "attention: bad window %d or block table width %d", window, max_pages);
+  NNIS_REQUIRE(scale > 0.0f, "attention: the scale of the scores must be positive");
   NNIS_REQUIRE(((uintptr_t)q % 16 == 0) && ((uintptr_t)out % 16 == 0) && ((uintptr_t)k_pages % 16 == 0) &&
                    ((uintptr_t)v_pages % 16 == 0),
                "attention: operands must be 16-byte aligned");
@@ -834,9 +851,9 @@ extern "C" int nnis_attention_prefill_max_waves(int heads, int kv_heads, int col
   int qt, gh;
   prefill_shape(heads, kv_heads, columns, &qt, &gh);
   const size_t per_wave = (size_t)qt * gh * (kTilesD * 4 + 2) * kWave * sizeof(float);
-  const int waves = 1 + (int)(65536 / per_wave);
-  const int fit = waves >= 8 ? 8 : (waves >= 4 ? 4 : (waves >= 2 ? 2 : 1));
-  return fit < kBlockWaves ? fit : kBlockWaves;
+  int waves = 1;  // a power of two; half of them leave a state in LDS at a time
+  while (waves * 2 <= kBlockWaves && waves * per_wave <= 65536) waves *= 2;
+  return waves;
 }
 
 extern "C" int nnis_attention_prefill_bf16(const void* q, void* out, const void* k_pages, const void* v_pages,
@@ -855,9 +872,9 @@ extern "C" int nnis_attention_prefill_bf16(const void* q, void* out, const void*
   const dim3 grid(tiles, kv_heads * chunks);
   NNIS_REQUIRE(grid.y <= 65535, "attention: %d head chunks exceed the grid limit", grid.y);
   const size_t per_wave = (size_t)qt * gh * (kTilesD * 4 + 2) * kWave * sizeof(float);
-  NNIS_REQUIRE(waves >= 1 && waves <= kBlockWaves && (waves - 1) * per_wave <= 65536,
-               "attention: %d waves a block do not fit this head size (LDS)", waves);
-  const size_t lds = (waves - 1) * per_wave;
+  NNIS_REQUIRE(waves >= 1 && waves <= kBlockWaves && (waves & (waves - 1)) == 0 && (waves / 2) * per_wave <= 65536,
+               "attention: %d waves a block: a power of two that fits this head size (LDS) is needed", waves);
+  const size_t lds = (waves / 2) * per_wave;
   const dim3 block(kWave * waves);
   hipStream_t s = (hipStream_t)stream;
   bool launched = true;
@@ -891,11 +908,11 @@ extern "C" int nnis_attention_prefill_bf16(const void* q, void* out, const void*
 extern "C" int nnis_attention_decode_max_waves(int heads, int kv_heads) {
   const int group = heads / (kv_heads > 0 ? kv_heads : 1);
   const int tiles = (group + 15) / 16;
-  const int per_wave = tiles * (kTilesD * 4 + 2) * kWave * 4;  // bytes of LDS a wave beyond the first needs
-  const int waves = 1 + 65536 / per_wave;
-  const int fit = waves >= 8 ? 8 : (waves >= 4 ? 4 : (waves >= 2 ? 2 : 1));
+  const int per_wave = tiles * (kTilesD * 4 + 2) * kWave * 4;  // bytes of LDS a wave's state takes in the merge
   const int most = (group <= 4 && HD <= kKeysMaxHD && kKeysWaves < kBlockWaves) ? kKeysWaves : kBlockWaves;
-  return fit < most ? fit : most;
+  int waves = 1;
+  while (waves * 2 <= most && waves * per_wave <= 65536) waves *= 2;
+  return waves;
 }
 
 // With splits > 1 the call needs scratch memory: `partial`, float32 of at least tokens * heads * splits *
@@ -912,8 +929,8 @@ extern "C" int nnis_attention_decode_bf16(const void* q, void* out, const void* 
   NNIS_REQUIRE(splits == 1 || partial != nullptr, "attention: splits need scratch memory");
   NNIS_REQUIRE((uintptr_t)partial % 16 == 0, "attention: scratch memory must be 16-byte aligned");
   NNIS_REQUIRE(kv_heads <= 65535, "attention: %d kv heads exceed the grid limit", kv_heads);
-  NNIS_REQUIRE(waves >= 1 && waves <= nnis_attention_decode_max_waves(heads, kv_heads),
-               "attention: %d waves a block; this head size and group take at most %d", waves,
+  NNIS_REQUIRE(waves >= 1 && waves <= nnis_attention_decode_max_waves(heads, kv_heads) && (waves & (waves - 1)) == 0,
+               "attention: %d waves a block; this head size and group take a power of two up to %d", waves,
                nnis_attention_decode_max_waves(heads, kv_heads));
   if (tokens <= 0) return 0;
   const int group = heads / kv_heads;
@@ -927,7 +944,7 @@ extern "C" int nnis_attention_decode_bf16(const void* q, void* out, const void* 
   const dim3 grid(tokens, kv_heads, splits);
   hipStream_t s = (hipStream_t)stream;
   const int tiles = (group + 15) / 16;
-  const size_t lds = (size_t)(waves - 1) * tiles * (kTilesD * 4 + 2) * kWave * sizeof(float);
+  const size_t lds = (size_t)(waves / 2) * tiles * (kTilesD * 4 + 2) * kWave * sizeof(float);
 #if NNIS_HEAD_DIM <= 128
   {
     if (kind == 2 || (kind == 0 && keys_fit)) {
