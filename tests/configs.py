@@ -34,3 +34,21 @@ TINY_C = llama(
 
 # name -> (config, weight seed)
 TINY_CONFIGS = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2)}
+
+# The layer sizes of the models the library is measured on, with two layers and a
+# small vocabulary so that the plain implementation stays quick: grouped heads 3:1
+# with a width that is no power of two; one key/value head per query head; groups of 8.
+SHAPE_CONFIGS = {
+    "smollm2-135m": (llama(
+        num_hidden_layers=2, hidden_size=576, num_attention_heads=9, num_key_value_heads=3, intermediate_size=1536,
+        vocab_size=3001, rope_theta=100000.0, rms_norm_eps=1e-5, tie_word_embeddings=True,
+        max_position_embeddings=2048, torch_dtype="bfloat16"), 11),
+    "smollm2-1.7b": (llama(
+        num_hidden_layers=2, hidden_size=2048, num_attention_heads=32, num_key_value_heads=32, intermediate_size=8192,
+        vocab_size=3001, rope_theta=130000.0, rms_norm_eps=1e-5, tie_word_embeddings=True,
+        max_position_embeddings=2048, torch_dtype="bfloat16"), 12),
+    "tinyllama-1.1b": (llama(
+        num_hidden_layers=2, hidden_size=2048, num_attention_heads=32, num_key_value_heads=4, intermediate_size=5632,
+        vocab_size=3001, rope_theta=10000.0, rms_norm_eps=1e-5, tie_word_embeddings=False,
+        max_position_embeddings=2048, torch_dtype="bfloat16"), 13),
+}

@@ -10,7 +10,7 @@ import torch
 
 import plain_llama as P
 import replay
-from configs import TINY_CONFIGS
+from configs import SHAPE_CONFIGS, TINY_CONFIGS
 
 pytestmark = pytest.mark.gpu
 
@@ -68,3 +68,55 @@ def test_schedules_agree_with_the_plain_model(model_dirs, tmp_path, name, dtype)
     between = max(float(np.abs(rows[("w" + n, p)] - rows[(tag + n, p)]).max())
                   for tag in "tb" for n, t in requests.items() for p in range(len(t)))
     assert between <= (1e-5 if dtype == "float32" else 2e-2), between
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("shape", sorted(SHAPE_CONFIGS))
+def test_measured_shapes_agree_with_the_plain_model(tmp_path, shape, dtype):
+    """The same three schedules at the layer sizes the library is measured on
+    (two layers of each): wide rows, one key/value head per query head, groups
+    of 8, a prompt of several pages.  32-bit: against the plain model, as for
+    the tiny ones.  bfloat16: at these widths rounding alone moves a logit by
+    more than the tiny models' bound, so the yardstick is the plain model run
+    with its activations rounded to bfloat16 where the engine keeps them so:
+    the engine may be off the 32-bit plain logits by at most 1.5 times what
+    that twin is off in root mean square, and twice in the worst logit.  A
+    fault (a wrong key, a mask off by one, a stale slot) moves logits by their
+    own size, tens of times more."""
+    import nnis_amd
+
+    config, seed = SHAPE_CONFIGS[shape]
+    folder = tmp_path / "model"
+    folder.mkdir()
+    nnis_amd.write_random_model(str(folder), config, seed)
+    vocab = config["vocab_size"]
+    rng = np.random.default_rng(seed)
+    requests = {f"r{i}": rng.integers(0, vocab, size=n).tolist() for i, n in enumerate([1, 37, 65, 130, 300])}
+    plain = P.PlainLlama(str(folder), torch.float32)
+    plain_logits = {n: plain.logits(t) for n, t in requests.items()}
+    schedules = (("w", "whole", replay.whole(requests)), ("t", "last 32 one by one", replay.tail_one_by_one(requests)),
+                 ("b", "unequal batches", replay.unequal_batches(requests, batch=3, decode=32)))
+    steps = []
+    for tag, _, schedule in schedules:
+        for step in schedule:
+            steps.append({"entries": [dict(e, id=tag + e["id"]) for e in step["entries"]], "end": [tag + n for n in step.get("end", [])]})
+    out = tmp_path / "out"
+    out.mkdir()
+    rows = replay.run_trace(str(folder), dtype, steps, str(out), max_tokens=12 * 64, vocab=vocab)
+    total = sum(len(t) for t in requests.values())
+    assert len(rows) == 3 * total
+    if dtype == "bfloat16":
+        twin = {n: plain.logits(t, P.bf16_round) for n, t in requests.items()}
+        twin_error = torch.cat([(twin[n] - plain_logits[n]).flatten() for n in requests]).double()
+        twin_rms, twin_worst = float(twin_error.pow(2).mean().sqrt()), float(twin_error.abs().max())
+        assert 1e-4 < twin_rms < 2e-2  # the yardstick itself is rounding, not nothing and not a fault
+    for tag, what, _ in schedules:
+        part = {(n[1:], p): row for (n, p), row in rows.items() if n[0] == tag}
+        assert len(part) == total
+        if dtype == "float32":
+            _compare(part, plain_logits, 2e-5, 2e-5, f"{shape} {dtype} {what}")
+            continue
+        error = np.concatenate([(row - plain_logits[n][p].numpy()).ravel() for (n, p), row in part.items()]).astype(np.float64)
+        rms, worst = float(np.sqrt(np.mean(error ** 2))), float(np.abs(error).max())
+        assert rms <= 1.5 * twin_rms, (shape, what, rms, twin_rms)
+        assert worst <= 2.0 * twin_worst, (shape, what, worst, twin_worst)
