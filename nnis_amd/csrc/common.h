@@ -110,3 +110,13 @@ __device__ __forceinline__ float block_sum(float v, float* scratch) {
   for (int w = 0; w < waves; ++w) total += scratch[w];
   return total;
 }
+
+// Blocks go to the chip's 8 dies in turn (block i to die i % 8), each die with an L2 of its own.  A kernel
+// for few tokens whose blocks are (unit of weight rows) x (tile of 16 * MT tokens) deals them so that all
+// token tiles of a unit run on one die, one after the other: the unit's weight rows come from memory once.
+// Launch ((units + 7) / 8) * 8 * tiles blocks; a block whose unit is beyond the last leaves.
+__device__ __forceinline__ void nnis_deal_tiles(int block, int tiles, int& unit_block, int& tile) {
+  const int die = block % 8, nth = block / 8;
+  unit_block = (nth / tiles) * 8 + die;
+  tile = nth % tiles;
+}

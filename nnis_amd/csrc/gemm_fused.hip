@@ -30,6 +30,8 @@ typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
+constexpr size_t kRereadWeightBytes = 8u << 20;
+
 struct FusedArgs {
   // prepared by the projection before: the operand and parts of each row's sum of squares
   const bf16_t* scaled;  // [m, k]
@@ -73,7 +75,7 @@ __device__ __forceinline__ void load_gain8(const void* base, int dtype, int inde
 }
 
 template <int MT, int KSPLIT, int EPI, bool PREP>
-__global__ __launch_bounds__(KSPLIT > 4 ? 64 * KSPLIT : 256) void gemm_fused_kernel(FusedArgs a) {
+__global__ __launch_bounds__(KSPLIT > 4 ? 64 * KSPLIT : 256) void gemm_fused_kernel(FusedArgs a, int tiles) {
   constexpr bool PAIR = EPI != EPI_STORE;
   constexpr int NACC = PAIR ? 2 : 1;
   constexpr int kWaves = KSPLIT > 4 ? KSPLIT : 4;
@@ -84,7 +86,10 @@ __global__ __launch_bounds__(KSPLIT > 4 ? 64 * KSPLIT : 256) void gemm_fused_ker
   __shared__ float part_ss[KSPLIT > 1 ? kWaves : 1][MT][kWave];
 
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
-  const int unit = blockIdx.x * kUnits + wave / KSPLIT;
+  int unit_block, tile;
+  nnis_deal_tiles(blockIdx.x, tiles, unit_block, tile);
+  const int unit = unit_block * kUnits + wave / KSPLIT;
+  const int token0 = tile * 16 * MT;  // this block's tokens: token0 + (0 .. 16 * MT - 1)
   const int part = wave % KSPLIT;
   const int r = lane % 16, g = lane / 16;
   const int k = a.k, m = a.m, n = a.n;
@@ -119,7 +124,7 @@ __global__ __launch_bounds__(KSPLIT > 4 ? 64 * KSPLIT : 256) void gemm_fused_ker
   if (EPI == EPI_ROPE && ends_unit) {
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
-      int token = t * 16 + r;
+      int token = token0 + t * 16 + r;
       token = token < m ? token : m - 1;
       tok_slot[t] = a.rope.tok_slot[token];
       tok_pos[t] = a.rope.tok_pos[token];
@@ -144,7 +149,7 @@ __global__ __launch_bounds__(KSPLIT > 4 ? 64 * KSPLIT : 256) void gemm_fused_ker
       // lane group g takes every fourth part; the groups are added with the sums of squares below
 #pragma unroll
       for (int t = 0; t < MT; ++t) {
-        const int token = t * 16 + r;
+        const int token = token0 + t * 16 + r;
 #pragma unroll
         for (int i = 0; i < kPartRegs; ++i) {
           const int p = g + 4 * i;
@@ -171,7 +176,7 @@ __global__ __launch_bounds__(KSPLIT > 4 ? 64 * KSPLIT : 256) void gemm_fused_ker
     size_t x_row[MT];
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
-      int token = t * 16 + r;
+      int token = token0 + t * 16 + r;
       token = token < m ? token : m - 1;
       x_row[t] = (size_t)token * k;
     }
@@ -273,7 +278,7 @@ __global__ __launch_bounds__(KSPLIT > 4 ? 64 * KSPLIT : 256) void gemm_fused_ker
               if (a.delta) {
 #pragma unroll
                 for (int e = 0; e < 8; ++e) v[e] += (float)dl[d][half][t][e];
-                if (writes_x && t * 16 + r < m) {
+                if (writes_x && token0 + t * 16 + r < m) {
                   *(f32x4*)(a.x_out + x_row[t] + kk) = (f32x4){v[0], v[1], v[2], v[3]};
                   *(f32x4*)(a.x_out + x_row[t] + kk + 4) = (f32x4){v[4], v[5], v[6], v[7]};
                 }
@@ -296,7 +301,7 @@ __global__ __launch_bounds__(KSPLIT > 4 ? 64 * KSPLIT : 256) void gemm_fused_ker
     for (int t = 0; t < MT; ++t) {
 #pragma unroll
       for (int i = 0; i < kPartRegs; ++i) ss[t] += ss_held[t][i];
-      const int token = t * 16 + r;
+      const int token = token0 + t * 16 + r;
       if (token < m)
         for (int p = g + 4 * kPartRegs; p < a.parts; p += 4) ss[t] += a.ss_parts[(size_t)p * m + token];  // wide rows
     }
@@ -337,7 +342,7 @@ __global__ __launch_bounds__(KSPLIT > 4 ? 64 * KSPLIT : 256) void gemm_fused_ker
   const float inv_k = 1.0f / (float)k;
 #pragma unroll
   for (int t = 0; t < MT; ++t) {
-    const int token = t * 16 + r;
+    const int token = token0 + t * 16 + r;
     if (token >= m) continue;
     const float scale = 1.0f / sqrtf(ss[t] * inv_k + a.eps);
     if (EPI == EPI_STORE) {
@@ -365,9 +370,11 @@ template <int MT, int KSPLIT, int EPI>
 void launch_fused(const FusedArgs& a, int units, hipStream_t stream) {
   constexpr int kWaves = KSPLIT > 4 ? KSPLIT : 4;
   constexpr int kUnits = kWaves / KSPLIT;
-  const dim3 grid((units + kUnits - 1) / kUnits), block(64 * kWaves);
-  if (a.scaled) hipLaunchKernelGGL((gemm_fused_kernel<MT, KSPLIT, EPI, true>), grid, block, 0, stream, a);
-  else hipLaunchKernelGGL((gemm_fused_kernel<MT, KSPLIT, EPI, false>), grid, block, 0, stream, a);
+  const int unit_blocks = (units + kUnits - 1) / kUnits;
+  const int tiles = (a.m + 16 * MT - 1) / (16 * MT);
+  const dim3 grid(tiles == 1 ? unit_blocks : (unit_blocks + 7) / 8 * 8 * tiles), block(64 * kWaves);
+  if (a.scaled) hipLaunchKernelGGL((gemm_fused_kernel<MT, KSPLIT, EPI, true>), grid, block, 0, stream, a, tiles);
+  else hipLaunchKernelGGL((gemm_fused_kernel<MT, KSPLIT, EPI, false>), grid, block, 0, stream, a, tiles);
 }
 
 template <int MT, int EPI>
@@ -378,9 +385,13 @@ void dispatch_fused_split(const FusedArgs& a, int units, int split, hipStream_t 
   else launch_fused<MT, 1, EPI>(a, units, stream);
 }
 
+// Weights that the dies' L2 keep (a few MB) are cheaper to read again than a wave is to load with the work of
+// several token tiles: then a block takes one tile of 16 tokens and the grid the rest.  Large weights are
+// read once, by waves that take all tiles (up to 4).
 template <int EPI>
 void dispatch_fused(const FusedArgs& a, int units, int split, hipStream_t stream) {
-  const int tiles = (a.m + 15) / 16;
+  int tiles = (a.m + 15) / 16;
+  if ((size_t)a.n * a.k * sizeof(bf16_t) <= kRereadWeightBytes) tiles = 1;
   if (tiles == 1) dispatch_fused_split<1, EPI>(a, units, split, stream);
   else if (tiles == 2) dispatch_fused_split<2, EPI>(a, units, split, stream);
   else if (tiles == 3) dispatch_fused_split<3, EPI>(a, units, split, stream);
@@ -416,7 +427,8 @@ int run_fused(FusedArgs& a, int epilogue, int table_positions, int split_hint, h
   }
   // few units: their waves share K so that each wave's share is one round of loads
   const int chunks = (k + 63) / 64;
-  const int depth = a.scaled ? (a.m <= 32 ? 4 : 2) : 2;
+  const int per_wave = (size_t)n * k * sizeof(bf16_t) <= kRereadWeightBytes ? 1 : (a.m + 15) / 16;  // token tiles a wave takes
+  const int depth = a.scaled ? (per_wave <= 2 ? 4 : 2) : (per_wave == 1 ? 2 : 1);  // the kernel's steps in flight
   int split = 1;
   if (units < 2048) {
     while (split < 8 && chunks > split * depth) split *= 2;

@@ -170,13 +170,16 @@ __device__ __forceinline__ int paired_weight_row(const RopeTarget& rope, int blo
 template <int MT, int KSPLIT, typename OutT>
 __global__ __launch_bounds__(KSPLIT > 4 ? 64 * KSPLIT : 256) void gemm_skinny_kernel(const bf16_t* __restrict__ x,
                                                                                    const bf16_t* __restrict__ w,
-                                                                                   OutT y, int m, int n, int k) {
+                                                                                   OutT y, int m, int n, int k, int tiles) {
   constexpr int kWaves = KSPLIT > 4 ? KSPLIT : 4;
   constexpr int kStrips = kWaves / KSPLIT;  // strips of 16 weight rows per block
   constexpr int DEPTH = MT <= 2 ? 4 : 2;
   __shared__ float partial[KSPLIT > 1 ? kWaves : 1][MT][kWave][4];
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
-  const int strip = blockIdx.x * kStrips + wave / KSPLIT;
+  int strip_block, tile;
+  nnis_deal_tiles(blockIdx.x, tiles, strip_block, tile);
+  const int strip = strip_block * kStrips + wave / KSPLIT;
+  const int token0 = tile * 16 * MT;  // this block's tokens: token0 + (0 .. 16 * MT - 1)
   const int part = wave % KSPLIT;
   const int r = lane % 16, g = lane / 16;
   const int strips = (n + 15) / 16;
@@ -196,7 +199,7 @@ __global__ __launch_bounds__(KSPLIT > 4 ? 64 * KSPLIT : 256) void gemm_skinny_ke
     if (active && part == 0) {  // the wave that ends the strip asks for the stream before its weights
 #pragma unroll
       for (int t = 0; t < MT; ++t) {
-        const int token = t * 16 + r;
+        const int token = token0 + t * 16 + r;
         held[t] = residual_ask(y, (size_t)(token < m ? token : 0) * n + n0, n0, (token < m) ? valid : 0, vector_ok);
       }
     }
@@ -209,7 +212,7 @@ __global__ __launch_bounds__(KSPLIT > 4 ? 64 * KSPLIT : 256) void gemm_skinny_ke
     const bf16_t* x_ptr[MT];
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
-      int token = t * 16 + r;
+      int token = token0 + t * 16 + r;
       token = token < m ? token : m - 1;
       x_ptr[t] = x + (size_t)token * k;
     }
@@ -258,7 +261,7 @@ __global__ __launch_bounds__(KSPLIT > 4 ? 64 * KSPLIT : 256) void gemm_skinny_ke
 
 #pragma unroll
   for (int t = 0; t < MT; ++t) {
-    const int token = t * 16 + r;
+    const int token = token0 + t * 16 + r;
     if constexpr (kResidual) {
       float sq = 0.0f;
       if (token < m && valid > 0) sq = residual_take(y, held[t], (size_t)token * n + n0, acc[t], valid, vector_ok);
@@ -508,8 +511,10 @@ void launch_skinny(const bf16_t* x, const bf16_t* w, OutT y, int m, int n, int k
   const int strips = (n + 15) / 16;
   const int waves = KSPLIT > 4 ? KSPLIT : 4;
   const int per_block = waves / KSPLIT;
-  hipLaunchKernelGGL((gemm_skinny_kernel<MT, KSPLIT, OutT>), dim3((strips + per_block - 1) / per_block),
-                     dim3(64 * waves), 0, stream, x, w, y, m, n, k);
+  const int strip_blocks = (strips + per_block - 1) / per_block;
+  const int tiles = (m + 16 * MT - 1) / (16 * MT);
+  hipLaunchKernelGGL((gemm_skinny_kernel<MT, KSPLIT, OutT>), dim3(tiles == 1 ? strip_blocks : (strip_blocks + 7) / 8 * 8 * tiles),
+                     dim3(64 * waves), 0, stream, x, w, y, m, n, k, tiles);
 }
 
 template <int MT, typename OutT>
@@ -520,9 +525,16 @@ void dispatch_skinny_split(const bf16_t* x, const bf16_t* w, OutT y, int m, int 
   else launch_skinny<MT, 1, OutT>(x, w, y, m, n, k, stream);
 }
 
+// token tiles a wave of the skinny kernel takes: all of them (up to 4) when the weights are large and
+// should be read once; one, with the other tiles in blocks of their own on the same die, when the dies' L2
+// keep the weights (a few MB) and a wave's work is what the kernel's time hangs on
+int skinny_tiles_per_wave(int m, int n, int k) {
+  return (size_t)n * k * sizeof(bf16_t) <= (8u << 20) ? 1 : (m + 15) / 16;
+}
+
 template <typename OutT>
 void dispatch_skinny(const bf16_t* x, const bf16_t* w, OutT y, int m, int n, int k, int split, hipStream_t stream) {
-  const int tiles = (m + 15) / 16;
+  const int tiles = skinny_tiles_per_wave(m, n, k);
   if (tiles == 1) dispatch_skinny_split<1, OutT>(x, w, y, m, n, k, split, stream);
   else if (tiles == 2) dispatch_skinny_split<2, OutT>(x, w, y, m, n, k, split, stream);
   else if (tiles == 3) dispatch_skinny_split<3, OutT>(x, w, y, m, n, k, split, stream);
@@ -560,7 +572,7 @@ int dispatch_tiled(const bf16_t* x, const bf16_t* w, OutT y, int m, int n, int k
 int skinny_split(int m, int n, int k, int split_hint) {
   const int strips = (n + 15) / 16;
   const int chunks = (k + 63) / 64;
-  const int depth = m <= 32 ? 4 : 2;
+  const int depth = skinny_tiles_per_wave(m, n, k) <= 2 ? 4 : 2;
   int split = 1;
   if (strips < 2048) {
     while (split < 8 && chunks > split * depth) split *= 2;
