@@ -81,6 +81,9 @@ __device__ __forceinline__ void epilogue_rope(const RopeTarget& a, int token, in
   }
 }
 
-// the tiled kernel on an operand that a residual epilogue prepared (gemm_mfma.hip); m > 64
+// which of the two families of kernels a product of these sizes takes (gemm_mfma.hip)
+bool nnis_gemm_takes_few_tokens(int m, int n, int k);
+
+// the tiled kernel on an operand that a residual epilogue prepared (gemm_mfma.hip)
 int nnis_gemm_scaled_tiled(const bf16_t* scaled, const float* ss_parts, int parts, float eps, const bf16_t* w, int m, int n,
                            int k, int epilogue, bf16_t* y, const RopeTarget& rope, int tile_hint, hipStream_t stream);

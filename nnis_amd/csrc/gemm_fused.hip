@@ -30,7 +30,7 @@ typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
-constexpr size_t kRereadWeightBytes = 8u << 20;
+constexpr size_t kRereadWeightBytes = 8u << 20;  // as in gemm_mfma.hip
 
 struct FusedArgs {
   // prepared by the projection before: the operand and parts of each row's sum of squares
@@ -420,8 +420,8 @@ int run_fused(FusedArgs& a, int epilogue, int table_positions, int split_hint, h
   } else {
     return nnis_fail("gemm_fused: unknown epilogue %d", epilogue);
   }
-  if (a.m > 64) {
-    NNIS_REQUIRE(a.scaled != nullptr, "gemm_fused: takes 1 to 64 tokens, got %d", a.m);
+  if (!nnis_gemm_takes_few_tokens(a.m, n, k)) {
+    NNIS_REQUIRE(a.scaled != nullptr, "gemm_fused: %d tokens are too many for a weight of %d x %d", a.m, n, k);
     const int tile_hint = split_hint >= 16 ? split_hint / 16 : 0;
     return nnis_gemm_scaled_tiled(a.scaled, a.ss_parts, a.parts, a.eps, a.w, a.m, n, k, epilogue, a.y, a.rope, tile_hint, stream);
   }
@@ -451,7 +451,7 @@ extern "C" int nnis_gemm_fused(const float* x_in, const void* delta, float* x_ou
                                const float* sin_table, int table_positions, const int* tok_slot, const int* tok_pos,
                                void* k_pages, void* v_pages, const int* block_table, int max_pages, int heads, int kv_heads,
                                int head_dim, int split_hint, void* stream_ptr) {
-  NNIS_REQUIRE(m > 0 && m <= 64, "gemm_fused: takes 1 to 64 tokens, got %d", m);
+  NNIS_REQUIRE(m > 0 && nnis_gemm_takes_few_tokens(m, n, k), "gemm_fused: %d tokens are too many for a weight of %d x %d", m, n, k);
   NNIS_REQUIRE(n > 0 && k > 0 && k % 8 == 0, "gemm_fused: bad sizes n=%d k=%d (K must be a multiple of 8)", n, k);
   NNIS_REQUIRE(nnis_dtype_ok(norm_w_dtype), "gemm_fused: unknown norm weight dtype %d", norm_w_dtype);
   NNIS_REQUIRE(eps > 0.0f, "gemm_fused: eps must be positive");

@@ -23,6 +23,10 @@
 
 #include <type_traits>
 
+#ifndef NNIS_FEW_TOKENS
+#define NNIS_FEW_TOKENS 256
+#endif
+
 namespace {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
@@ -67,6 +71,10 @@ __device__ __forceinline__ void store4(bf16_t* y, size_t index, f32x4 v, int val
 // issues the loads of DEPTH steps of 64 k (weights and activations) before the
 // first multiply, so its whole share of K is usually one round trip.
 // -----------------------------------------------------------------------------
+// Weights up to this size stay in the dies' L2 over a kernel: reading them again costs little
+constexpr size_t kRereadWeightBytes = 8u << 20;
+constexpr int kFewTokens = NNIS_FEW_TOKENS;
+
 // What a projection that ends a part of a pre-norm block does with its result instead of storing it
 // (OutT = ResidualOut): the residual stream takes it in, and the norm that follows is prepared.
 //   v = resid + y (32-bit, in place);  scaled = bf16(v * gain);  ss[part][token] = sum over the part's
@@ -529,7 +537,7 @@ void dispatch_skinny_split(const bf16_t* x, const bf16_t* w, OutT y, int m, int 
 // should be read once; one, with the other tiles in blocks of their own on the same die, when the dies' L2
 // keep the weights (a few MB) and a wave's work is what the kernel's time hangs on
 int skinny_tiles_per_wave(int m, int n, int k) {
-  return (size_t)n * k * sizeof(bf16_t) <= (8u << 20) ? 1 : (m + 15) / 16;
+  return (size_t)n * k * sizeof(bf16_t) <= kRereadWeightBytes ? 1 : (m + 15) / 16;
 }
 
 template <typename OutT>
@@ -549,21 +557,31 @@ void launch_tiled(const bf16_t* x, const bf16_t* w, OutT y, int m, int n, int k,
                      y, m, n, k, col_blocks);
 }
 
-// returns the number of wave columns (parts of a row that a residual epilogue sums by itself)
-template <typename OutT>
-int dispatch_tiled(const bf16_t* x, const bf16_t* w, OutT y, int m, int n, int k, int tile_hint, hipStream_t stream,
-                   int columns = 0) {
-  if (columns <= 0) columns = n;
-  // the largest tile that still gives every compute unit a block or two
+// 1: 128x128, 2: 64x128, 3: 64x64 -- the largest tile that still gives every compute unit a block or two
+int pick_tile(int m, int columns, int tile_hint) {
   const long long blocks_128 = (long long)((m + 127) / 128) * ((columns + 127) / 128);
   const long long blocks_64_128 = (long long)((m + 63) / 64) * ((columns + 127) / 128);
   int tile = blocks_128 >= 384 ? 1 : (blocks_64_128 >= 256 ? 2 : 3);
   if (tile_hint >= 1 && tile_hint <= 3) tile = tile_hint;  // for tuning runs
+  return tile;
+}
+
+// wave columns of the tiled kernel for these sizes: the parts of a row that a residual epilogue sums by itself
+int tiled_parts(int m, int columns, int tile_hint) {
+  const int width = pick_tile(m, columns, tile_hint) <= 2 ? 128 : 64;
+  return 2 * ((columns + width - 1) / width);
+}
+
+// returns the number of wave columns
+template <typename OutT>
+int dispatch_tiled(const bf16_t* x, const bf16_t* w, OutT y, int m, int n, int k, int tile_hint, hipStream_t stream,
+                   int columns = 0) {
+  if (columns <= 0) columns = n;
+  const int tile = pick_tile(m, columns, tile_hint);
   if (tile == 1) launch_tiled<128, 128, 64, OutT>(x, w, y, m, n, k, columns, stream);
   else if (tile == 2) launch_tiled<64, 128, 64, OutT>(x, w, y, m, n, k, columns, stream);
   else launch_tiled<64, 64, 64, OutT>(x, w, y, m, n, k, columns, stream);
-  const int width = tile <= 2 ? 128 : 64;
-  return 2 * ((columns + width - 1) / width);
+  return tiled_parts(m, columns, tile_hint);
 }
 
 // With few strips the waves of a block share a strip's K, so that each wave's
@@ -582,6 +600,18 @@ int skinny_split(int m, int n, int k, int split_hint) {
 }
 
 }  // namespace
+
+// The kernel for few tokens (a wave owns 16 weight rows, no LDS for operands) against the tiled one: up to
+// 64 tokens always.  Beyond, up to kFewTokens, when the weights are small enough to be read once per tile of
+// 16 tokens and its blocks (strips x token tiles) are few enough; measured on products of 32 to 384 tokens
+// with weights of 576 x 576 to 3072 x 576 and 576 x 1536, in microseconds:
+//   few tokens: 3 + 0.004 * strips * tiles * K / 576      tiled: 2 + 0.011 * K
+bool nnis_gemm_takes_few_tokens(int m, int n, int k) {
+  if (m <= 64) return true;
+  if (m > kFewTokens || (size_t)n * k * sizeof(bf16_t) > kRereadWeightBytes) return false;
+  const double strips = (n + 15) / 16, tiles = (m + 15) / 16;
+  return 3.0 + 0.004 * strips * tiles * k / 576.0 <= 2.0 + 0.011 * k;
+}
 
 int nnis_gemm_scaled_tiled(const bf16_t* scaled, const float* ss_parts, int parts, float eps, const bf16_t* w, int m, int n,
                            int k, int epilogue, bf16_t* y, const RopeTarget& rope, int tile_hint, hipStream_t stream) {
@@ -611,7 +641,7 @@ extern "C" int nnis_gemm_bf16(const void* x, const void* w, void* y, int y_dtype
   hipStream_t stream = (hipStream_t)stream_ptr;
   const bf16_t* xp = (const bf16_t*)x;
   const bf16_t* wp = (const bf16_t*)w;
-  if (m <= 64) {
+  if (nnis_gemm_takes_few_tokens(m, n, k)) {
     const int split = skinny_split(m, n, k, split_hint);
     if (y_dtype == NNIS_F32) dispatch_skinny<float*>(xp, wp, (float*)y, m, n, k, split, stream);
     else dispatch_skinny<bf16_t*>(xp, wp, (bf16_t*)y, m, n, k, split, stream);
@@ -628,14 +658,15 @@ extern "C" int nnis_gemm_bf16(const void* x, const void* w, void* y, int y_dtype
 
 // The projection that ends a part of a pre-norm block: resid += x . w^T in 32-bit, in place, and the norm
 // that follows prepared -- scaled = bf16(resid * gain) and parts of each row's sum of squares in ss
-// [parts, m].  Returns the number of parts in *parts (ss must hold nnis_gemm_residual_parts(m, n) rows).
+// [parts, m].  Returns the number of parts in *parts; ss has ss_rows rows of m floats, of which
+// nnis_gemm_residual_parts(m, n) are always enough.
 extern "C" int nnis_gemm_residual_parts(int m, int n) {
-  if (m <= 64) return (n + 15) / 16;
-  return 2 * ((n + 63) / 64);  // the narrowest tile's wave columns; wider tiles use fewer
+  (void)m;
+  return (n + 15) / 16;  // the kernel for few tokens: a part per strip of 16 columns; the tiled one uses fewer
 }
 
 extern "C" int nnis_gemm_residual(const void* x, const void* w, float* resid, const void* gain, int gain_dtype, void* scaled,
-                                  float* ss, int m, int n, int k, int* parts, void* stream_ptr) {
+                                  float* ss, int ss_rows, int m, int n, int k, int* parts, void* stream_ptr) {
   NNIS_REQUIRE(m >= 0 && n > 0 && k > 0, "gemm_residual: bad sizes m=%d n=%d k=%d", m, n, k);
   NNIS_REQUIRE(k % 8 == 0, "gemm_residual: K=%d is not a multiple of 8 (16-byte loads)", k);
   NNIS_REQUIRE(nnis_dtype_ok(gain_dtype), "gemm_residual: unknown norm weight dtype %d", gain_dtype);
@@ -646,7 +677,10 @@ extern "C" int nnis_gemm_residual(const void* x, const void* w, float* resid, co
   if (m == 0) return 0;
   hipStream_t stream = (hipStream_t)stream_ptr;
   ResidualOut out = {resid, gain, gain_dtype, (bf16_t*)scaled, ss};
-  if (m <= 64) {
+  const bool few = nnis_gemm_takes_few_tokens(m, n, k);
+  const int writes = few ? (n + 15) / 16 : tiled_parts(m, n, 0);
+  NNIS_REQUIRE(writes <= ss_rows, "gemm_residual: ss has %d rows of %d tokens, %d are needed", ss_rows, m, writes);
+  if (few) {
     *parts = (n + 15) / 16;
     dispatch_skinny<ResidualOut>((const bf16_t*)x, (const bf16_t*)w, out, m, n, k, skinny_split(m, n, k, 0), stream);
     NNIS_LAUNCH_CHECK("gemm_residual");

@@ -34,7 +34,7 @@ _CORE_SIGNATURES = {
     "nnis_gemm_fused": [_VOID, _VOID, _VOID, _VOID, _INT, _FLT, _VOID, _INT, _INT, _INT, _INT, _VOID, _VOID, _VOID, _INT,
                         _VOID, _VOID, _VOID, _VOID, _VOID, _INT, _INT, _INT, _INT, _INT, _VOID],
     "nnis_gemm_residual_parts": [_INT, _INT],
-    "nnis_gemm_residual": [_VOID, _VOID, _VOID, _VOID, _INT, _VOID, _VOID, _INT, _INT, _INT, _VOID, _VOID],
+    "nnis_gemm_residual": [_VOID, _VOID, _VOID, _VOID, _INT, _VOID, _VOID, _INT, _INT, _INT, _INT, _VOID, _VOID],
     "nnis_gemm_scaled": [_VOID, _VOID, _INT, _FLT, _VOID, _INT, _INT, _INT, _INT, _VOID, _VOID, _VOID, _INT, _VOID, _VOID,
                          _VOID, _VOID, _VOID, _INT, _INT, _INT, _INT, _INT, _VOID],
     "nnis_sample": [_VOID, _VOID, _INT, _INT, _VOID, _VOID, _VOID, _VOID, _VOID, _VOID, _VOID],
@@ -363,12 +363,13 @@ def gemm_residual(x: torch.Tensor, w: torch.Tensor, resid: torch.Tensor, gain: t
         raise KernelError("gemm_residual: resid must be float32 [m, n] and scaled bfloat16 [m, n]")
     if gain.numel() != n:
         raise KernelError(f"gemm_residual: norm weight of {gain.numel()} for width {n}")
-    if ss.dtype != torch.float32 or ss.numel() < gemm_residual_parts(m, n) * m:
-        raise KernelError("gemm_residual: ss must be float32 with gemm_residual_parts(m, n) * m elements")
+    if ss.dtype != torch.float32 or ss.numel() < m:
+        raise KernelError("gemm_residual: ss must be float32 [rows, m] (gemm_residual_parts(m, n) rows are always enough)")
     lib = core()
     parts = ctypes.c_int(0)
     _check(lib, lib.nnis_gemm_residual(x.data_ptr(), w.data_ptr(), resid.data_ptr(), gain.data_ptr(), _code(gain),
-                                       scaled.data_ptr(), ss.data_ptr(), m, n, k, ctypes.addressof(parts), _stream()))
+                                       scaled.data_ptr(), ss.data_ptr(), ss.numel() // m, m, n, k, ctypes.addressof(parts),
+                                       _stream()))
     return parts.value
 
 

@@ -223,8 +223,8 @@ def test_prefill_attention_on_the_matrix_cores(heads, kv_heads, head_dim):
             assert (got[100, 0] - vs[2][17, 0]).abs().max().item() < 0.05
 
 
-@pytest.mark.parametrize("m", [1, 8, 19, 64, 100, 300])
-@pytest.mark.parametrize("n, k", [(576, 576), (100, 72), (2048, 1536), (48, 8)])
+@pytest.mark.parametrize("m", [1, 8, 19, 64, 67, 100, 300])
+@pytest.mark.parametrize("n, k", [(576, 576), (100, 72), (2048, 1536), (48, 8), (64, 176), (3072, 576)])
 @pytest.mark.parametrize("gain_dtype", ["bfloat16", "float32"])
 def test_residual_projection_prepares_the_norm(m, n, k, gain_dtype):
     """resid += x . w^T in place; scaled = bfloat16(resid * gain); the parts of
@@ -590,6 +590,9 @@ def test_argmax(vocab):
 def test_refusals():
     ops = _ops()
     f = lambda *shape, dtype=torch.float32: torch.zeros(*shape, dtype=dtype, device="cuda")  # noqa: E731
+    with pytest.raises(KernelError, match="ss has 1 rows"):  # scratch too small for the parts it would write
+        ops.gemm_residual(f(70, 176, dtype=torch.bfloat16), f(64, 176, dtype=torch.bfloat16), f(70, 64),
+                          f(64, dtype=torch.bfloat16), f(70, 64, dtype=torch.bfloat16), f(1, 70))
     with pytest.raises(KernelError):
         ops.gemm_ordered(f(3, 8), f(5, 9), f(3, 5))
     with pytest.raises(KernelError, match="GPU"):
