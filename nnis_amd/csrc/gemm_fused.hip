@@ -420,7 +420,7 @@ int run_fused(FusedArgs& a, int epilogue, int table_positions, int split_hint, h
   } else {
     return nnis_fail("gemm_fused: unknown epilogue %d", epilogue);
   }
-  if (!nnis_gemm_takes_few_tokens(a.m, n, k)) {
+  if (!nnis_gemm_takes_few_tokens(a.m, n, k) || (split_hint >= 16 && a.scaled != nullptr)) {  // a tile hint asks for the tiled kernel
     NNIS_REQUIRE(a.scaled != nullptr, "gemm_fused: %d tokens are too many for a weight of %d x %d", a.m, n, k);
     const int tile_hint = split_hint >= 16 ? split_hint / 16 : 0;
     return nnis_gemm_scaled_tiled(a.scaled, a.ss_parts, a.parts, a.eps, a.w, a.m, n, k, epilogue, a.y, a.rope, tile_hint, stream);

@@ -11,7 +11,7 @@
 //    memory straight into operand registers; a wave owns a strip of 16 weight
 //    rows; X (small, shared by all waves) comes through the caches.  Waves of
 //    a block may split K and add their parts through LDS.
-//  * gemm_tiled_kernel: any M (prefill).  128x128 or 64x128 or 64x64 output
+//  * gemm_tiled_kernel: any M (prefill).  64x128 or 64x64 output
 //    tiles, K staged through LDS in steps of 64 with an XOR swizzle of the
 //    16-byte chunks so that operand reads are free of bank conflicts, global
 //    loads of the next step in flight while the current one is multiplied.
@@ -303,7 +303,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
   // Global loads run PF steps ahead of the multiply, in registers; the step after
   // the current one lies in the other LDS buffer.  With few blocks on a compute
   // unit nothing else hides the latency of a load, so short products need depth.
-  constexpr int PF = (BM * BN * BK >= 128 * 128 * 64) ? 3 : 4;
+  constexpr int PF = 3;
   __shared__ bf16x8 a_tile[2][BM * CH];
   __shared__ bf16x8 b_tile[2][BN * CH];
 
@@ -405,50 +405,60 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
       }
   }
 
+  // Registers hold the loads of the next PF steps, slot (step % PF).  The loop body is PF steps in one
+  // straight line that every round runs in full -- a load or an LDS write behind a branch makes the
+  // compiler wait for every load in flight at the next use of any, and the steps loaded ahead would be
+  // waited for at once.  So the steps are rounded up to whole rounds; a step beyond the end of K is loaded
+  // all the same (from the last whole chunk of the row, a valid address), turned into zeros on its way into
+  // LDS and multiplied as zeros.  With PF = 3 the products of this library (K = 576, 1536, 2048, 5632, 8192)
+  // run at most two such steps.
   bf16x8 a_stage[PF][A_CHUNKS], b_stage[PF][B_CHUNKS];
   const int steps = (k + BK - 1) / BK;
+  const int last_chunk = k - 8 - chunk_k;  // offset of the row's last whole chunk from this thread's first
 
 #define NNIS_FETCH(slot, step)                                                                   \
   do {                                                                                           \
     const int k0 = (step) * BK;                                                                  \
-    const bool in = k0 + chunk_k + 8 <= k;                                                       \
-    _Pragma("unroll") for (int c = 0; c < A_CHUNKS; ++c) a_stage[slot][c] = in ? load_chunk(a_src[c] + k0) : zero_chunk(); \
-    _Pragma("unroll") for (int c = 0; c < B_CHUNKS; ++c) b_stage[slot][c] = in ? load_chunk(b_src[c] + k0) : zero_chunk(); \
+    const int from = k0 <= last_chunk ? k0 : last_chunk;                                         \
+    _Pragma("unroll") for (int c = 0; c < A_CHUNKS; ++c) a_stage[slot][c] = load_chunk(a_src[c] + from); \
+    _Pragma("unroll") for (int c = 0; c < B_CHUNKS; ++c) b_stage[slot][c] = load_chunk(b_src[c] + from); \
   } while (0)
-#define NNIS_STAGE(slot, buffer)                                                                 \
+#define NNIS_STAGE(slot, step, buffer)                                                           \
   do {                                                                                           \
-    _Pragma("unroll") for (int c = 0; c < A_CHUNKS; ++c) a_tile[buffer][a_dst[c]] = a_stage[slot][c]; \
-    _Pragma("unroll") for (int c = 0; c < B_CHUNKS; ++c) b_tile[buffer][b_dst[c]] = b_stage[slot][c]; \
+    const bool in = (step) * BK <= last_chunk;                                                   \
+    _Pragma("unroll") for (int c = 0; c < A_CHUNKS; ++c) a_tile[buffer][a_dst[c]] = in ? a_stage[slot][c] : zero_chunk(); \
+    _Pragma("unroll") for (int c = 0; c < B_CHUNKS; ++c) b_tile[buffer][b_dst[c]] = in ? b_stage[slot][c] : zero_chunk(); \
   } while (0)
 
 #pragma unroll
-  for (int s = 0; s < PF; ++s)
-    if (s < steps) NNIS_FETCH(s, s);
-  NNIS_STAGE(0, 0);
+  for (int s = 0; s < PF; ++s) NNIS_FETCH(s, s);
+  NNIS_STAGE(0, 0, 0);
   __syncthreads();
   for (int base = 0; base < steps; base += PF) {
 #pragma unroll
     for (int j = 0; j < PF; ++j) {
       const int step = base + j;
-      if (step < steps) {  // uniform over the block
-        const int buffer = step & 1;
-        // slot j went to LDS a step ago: refill it with the step PF ahead
-        if (step + PF < steps) NNIS_FETCH(j, step + PF);
+      const int buffer = step & 1;
+      // slot j went to LDS a step ago: the step PF ahead takes its place
+      NNIS_FETCH(j, step + PF);
 #pragma unroll
-        for (int half = 0; half < BK / 32; ++half) {  // an instruction takes 32 k
-          bf16x8 a_frag[TM], b_frag[TN];
+      for (int half = 0; half < BK / 32; ++half) {  // an instruction takes 32 k
+        bf16x8 a_frag[TM], b_frag[TN];
 #pragma unroll
-          for (int i = 0; i < TM; ++i) a_frag[i] = a_tile[buffer][swizzled<CH>(wave_m * WM + i * 16 + r, half * 4 + g)];
+        for (int i = 0; i < TM; ++i) a_frag[i] = a_tile[buffer][swizzled<CH>(wave_m * WM + i * 16 + r, half * 4 + g)];
 #pragma unroll
-          for (int jj = 0; jj < TN; ++jj) b_frag[jj] = b_tile[buffer][swizzled<CH>(wave_n * WN + jj * 16 + r, half * 4 + g)];
+        for (int jj = 0; jj < TN; ++jj) b_frag[jj] = b_tile[buffer][swizzled<CH>(wave_n * WN + jj * 16 + r, half * 4 + g)];
 #pragma unroll
-          for (int i = 0; i < TM; ++i)
+        for (int i = 0; i < TM; ++i)
 #pragma unroll
-            for (int jj = 0; jj < TN; ++jj) acc[i][jj] = mfma(b_frag[jj], a_frag[i], acc[i][jj]);
-        }
-        if (step + 1 < steps) NNIS_STAGE((j + 1) % PF, buffer ^ 1);
-        __syncthreads();
+          for (int jj = 0; jj < TN; ++jj) acc[i][jj] = mfma(b_frag[jj], a_frag[i], acc[i][jj]);
       }
+      NNIS_STAGE((j + 1) % PF, step + 1, buffer ^ 1);
+      __syncthreads();
+      // Nothing of a later step moves up into this one: its slot's zero-or-data choice would wait for
+      // loads that have steps of time left.  (The smaller tile only: a wave of the larger one gains more
+      // from the next step's LDS reads among this step's matrix instructions.)
+      if constexpr (TM * TN <= 4) __builtin_amdgcn_sched_barrier(0);
     }
   }
 #undef NNIS_FETCH
@@ -557,18 +567,18 @@ void launch_tiled(const bf16_t* x, const bf16_t* w, OutT y, int m, int n, int k,
                      y, m, n, k, col_blocks);
 }
 
-// 1: 128x128, 2: 64x128, 3: 64x64 -- the largest tile that still gives every compute unit a block or two
+// 2: 64x128, 3: 64x64 -- the larger tile when it still gives every compute unit a block.  (A tile of
+// 128x128 was measured slower than 64x128 on every product from 2048 x 576 x 576 to 2048 x 6144 x 2048.)
 int pick_tile(int m, int columns, int tile_hint) {
-  const long long blocks_128 = (long long)((m + 127) / 128) * ((columns + 127) / 128);
   const long long blocks_64_128 = (long long)((m + 63) / 64) * ((columns + 127) / 128);
-  int tile = blocks_128 >= 384 ? 1 : (blocks_64_128 >= 256 ? 2 : 3);
-  if (tile_hint >= 1 && tile_hint <= 3) tile = tile_hint;  // for tuning runs
+  int tile = blocks_64_128 >= 256 ? 2 : 3;
+  if (tile_hint == 2 || tile_hint == 3) tile = tile_hint;  // for tuning runs
   return tile;
 }
 
 // wave columns of the tiled kernel for these sizes: the parts of a row that a residual epilogue sums by itself
 int tiled_parts(int m, int columns, int tile_hint) {
-  const int width = pick_tile(m, columns, tile_hint) <= 2 ? 128 : 64;
+  const int width = pick_tile(m, columns, tile_hint) == 2 ? 128 : 64;
   return 2 * ((columns + width - 1) / width);
 }
 
@@ -578,8 +588,7 @@ int dispatch_tiled(const bf16_t* x, const bf16_t* w, OutT y, int m, int n, int k
                    int columns = 0) {
   if (columns <= 0) columns = n;
   const int tile = pick_tile(m, columns, tile_hint);
-  if (tile == 1) launch_tiled<128, 128, 64, OutT>(x, w, y, m, n, k, columns, stream);
-  else if (tile == 2) launch_tiled<64, 128, 64, OutT>(x, w, y, m, n, k, columns, stream);
+  if (tile == 2) launch_tiled<64, 128, 64, OutT>(x, w, y, m, n, k, columns, stream);
   else launch_tiled<64, 64, 64, OutT>(x, w, y, m, n, k, columns, stream);
   return tiled_parts(m, columns, tile_hint);
 }
@@ -641,14 +650,14 @@ extern "C" int nnis_gemm_bf16(const void* x, const void* w, void* y, int y_dtype
   hipStream_t stream = (hipStream_t)stream_ptr;
   const bf16_t* xp = (const bf16_t*)x;
   const bf16_t* wp = (const bf16_t*)w;
-  if (nnis_gemm_takes_few_tokens(m, n, k)) {
+  if (nnis_gemm_takes_few_tokens(m, n, k) && split_hint < 16) {  // a tile hint asks for the tiled kernel
     const int split = skinny_split(m, n, k, split_hint);
     if (y_dtype == NNIS_F32) dispatch_skinny<float*>(xp, wp, (float*)y, m, n, k, split, stream);
     else dispatch_skinny<bf16_t*>(xp, wp, (bf16_t*)y, m, n, k, split, stream);
     NNIS_LAUNCH_CHECK("gemm_skinny");
   } else {
     NNIS_REQUIRE((m + 63) / 64 <= 65535, "gemm_bf16: %d rows exceed the grid limit", m);
-    const int tile_hint = split_hint >= 16 ? split_hint / 16 : 0;  // hints of 16, 32, 48 pick the tile: 128x128, 64x128, 64x64
+    const int tile_hint = split_hint >= 16 ? split_hint / 16 : 0;  // hints of 32 and 48 pick the tile: 64x128, 64x64
     if (y_dtype == NNIS_F32) dispatch_tiled<float*>(xp, wp, (float*)y, m, n, k, tile_hint, stream);
     else dispatch_tiled<bf16_t*>(xp, wp, (bf16_t*)y, m, n, k, tile_hint, stream);
     NNIS_LAUNCH_CHECK("gemm_tiled");

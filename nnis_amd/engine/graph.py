@@ -14,6 +14,8 @@ Nothing is memset inside the captured region (buffers come from
 
 from __future__ import annotations
 
+import gc
+import weakref
 from typing import Dict, List, Sequence, Tuple
 
 import numpy as np
@@ -33,7 +35,9 @@ def bucket(batch: int) -> int:
 
 class DecodeGraph:
     def __init__(self, engine, padded: int, plan: Tuple[int, int]):
-        self.engine = engine
+        # not a strong reference: engine -> graphs -> engine would keep both alive until the cycle
+        # collector runs, and that may be in the middle of another engine's capture
+        self.engine = engine if isinstance(engine, weakref.ProxyTypes) else weakref.proxy(engine)
         self.padded = padded
         splits, waves = plan
         device = engine.rt.device
@@ -64,8 +68,17 @@ class DecodeGraph:
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
         self.graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(self.graph):
-            self.logits = self._forward()
+        # A graph that the cycle collector destroys while another is being captured aborts the process:
+        # collect now, and keep the collector off until the capture ends.
+        gc.collect()
+        collecting = gc.isenabled()
+        gc.disable()
+        try:
+            with torch.cuda.graph(self.graph):
+                self.logits = self._forward()
+        finally:
+            if collecting:
+                gc.enable()
 
     def run(self, ids: Sequence[int], slots: Sequence[int], positions: Sequence[int]) -> torch.Tensor:
         count = len(ids)
@@ -87,7 +100,7 @@ class DecodeGraphs:
     """The graphs of one engine, made on first use."""
 
     def __init__(self, engine):
-        self.engine = engine
+        self.engine = weakref.proxy(engine)
         self.graphs: Dict[Tuple[int, Tuple[int, int]], DecodeGraph] = {}
 
     def get(self, batch: int, plan: Tuple[int, int]) -> DecodeGraph:

@@ -41,7 +41,7 @@ FLAGS = [
     "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
 ]
-HEADERS = ["common.h", "epilogue.h"]
+HEADERS = {"core": ["common.h", "epilogue.h"], "attention": ["common.h"]}  # what a module's sources include
 CORE_SOURCES = ["elementwise.hip", "gemm.hip", "gemm_mfma.hip", "gemm_fused.hip", "sampling.hip"]
 ATTENTION_SOURCES = ["attention.hip"]
 PREBUILT_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 112, 128)
@@ -66,7 +66,8 @@ def module_recipe(module: str) -> Tuple[List[str], Dict[str, str]]:
 
 def _module_hash(sources: List[str], defines: Dict[str, str]) -> str:
     digest = hashlib.sha256()
-    for name in HEADERS + sources:
+    headers = HEADERS["attention" if sources == ATTENTION_SOURCES else "core"]
+    for name in headers + sources:
         with open(os.path.join(CSRC, name), "rb") as handle:
             digest.update(name.encode())
             digest.update(handle.read())

@@ -336,7 +336,7 @@ def test_fused_norm_projection(m, k, with_delta, gain_dtype):
     assert int((v_plain != 7.0).any(dim=-1).sum()) <= written * kv_heads
 
 
-@pytest.mark.parametrize("hint", [16, 32, 48])
+@pytest.mark.parametrize("hint", [32, 48])
 @pytest.mark.parametrize("m", [65, 200])
 def test_scaled_projection_with_every_tile(hint, m):
     """The tiled kernel's epilogues with each of its tile shapes (the hint picks
