@@ -13,6 +13,8 @@
 //                V [page][kv_head][head_dim][token in page]
 #include "common.h"
 
+#include <algorithm>
+
 #ifndef NNIS_HEAD_DIM
 #error "compile with -DNNIS_HEAD_DIM=<head size>"
 #endif
@@ -425,79 +427,104 @@ __device__ __forceinline__ void attend_run(AttnState<C>& st, const QFrag (&q)[C]
 }
 
 // ---- prefill: a wave = (query tile, kv head, chunk of GH query heads); C = QT * GH column tiles --------
+// An item is a (tile, kv head, chunk of heads); the tiles come longest first, and item i = tile i / per_tile.
+// A tile's work grows with its place in its sequence, and a chip with fewer items than twice its compute
+// units runs them all at once: its time is the most loaded unit's.  So the grid is folded: block b < singles
+// has item b alone, block b >= singles has item b and then item items - 1 - (b - singles), a heavy and a
+// light one.
 template <int QT, int GH>
-__global__ __launch_bounds__(64 * kBlockWaves) void attention_prefill_kernel(MfmaArgs a, int waves) {
+__global__ __launch_bounds__(64 * kBlockWaves) void attention_prefill_kernel(MfmaArgs a, int waves, int items, int singles,
+                                                                            int per_tile) {
   extern __shared__ float merge[];
   constexpr int C = QT * GH;
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave, r = lane % 16, g = lane / 16;
-  const int tile = blockIdx.x;
   const int group = a.heads / a.kv_heads;
   const int chunks = (group + GH - 1) / GH;
-  const int kv_head = blockIdx.y / chunks;
-  const int head0 = kv_head * group + (blockIdx.y % chunks) * GH;
-  const int seq = a.tile_seq[tile];
-  const int row0 = a.tile_row0[tile];
-  const int slot = a.seq_slot[seq];
-  const int start = a.seq_start[seq];
-  const int rows = a.seq_start[seq + 1] - start;
-  const int pos0 = a.seq_pos0[seq];
-  const int* pages = a.block_table + (size_t)slot * a.max_pages;
+  // both items' places in the step, asked for together: each is a chain of dependent loads
+  const int count = (int)blockIdx.x < singles ? 1 : 2;
+  int item_of[2], seq_of[2], row0_of[2], slot_of[2], start_of[2], rows_of[2], pos0_of[2];
+#pragma unroll
+  for (int which = 0; which < 2; ++which) {
+    item_of[which] = which == 0 ? (int)blockIdx.x : items - 1 - ((int)blockIdx.x - singles);
+    const int tile = (which < count ? item_of[which] : item_of[0]) / per_tile;
+    seq_of[which] = __builtin_amdgcn_readfirstlane(a.tile_seq[tile]);
+    row0_of[which] = __builtin_amdgcn_readfirstlane(a.tile_row0[tile]);
+  }
+#pragma unroll
+  for (int which = 0; which < 2; ++which) {
+    slot_of[which] = __builtin_amdgcn_readfirstlane(a.seq_slot[seq_of[which]]);
+    start_of[which] = __builtin_amdgcn_readfirstlane(a.seq_start[seq_of[which]]);
+    rows_of[which] = __builtin_amdgcn_readfirstlane(a.seq_start[seq_of[which] + 1]) - start_of[which];
+    pos0_of[which] = __builtin_amdgcn_readfirstlane(a.seq_pos0[seq_of[which]]);
+  }
+  auto run_item = [&](int which) __attribute__((always_inline)) {
+    const int part = item_of[which] % per_tile;
+    const int kv_head = part / chunks;
+    const int head0 = kv_head * group + (part % chunks) * GH;
+    const int row0 = row0_of[which], start = start_of[which], rows = rows_of[which], pos0 = pos0_of[which];
+    const int* pages = a.block_table + (size_t)slot_of[which] * a.max_pages;
 
-  QFrag q[C];
-  int lo[C], hi[C];
-  bool live[C];
-  int last = -1;
+    QFrag q[C];
+    int lo[C], hi[C];
+    bool live[C];
+    int last = -1;
 #pragma unroll
-  for (int qt = 0; qt < QT; ++qt)
+    for (int qt = 0; qt < QT; ++qt)
 #pragma unroll
-    for (int gh = 0; gh < GH; ++gh) {
-      const int c = qt * GH + gh;
-      const int row = row0 + 16 * qt + r;
-      const int head = head0 + gh;
-      live[c] = row < rows && head < kv_head * group + group;
-      const int safe_row = row < rows ? row : rows - 1;
-      const int safe_head = head < a.heads ? head : a.heads - 1;
-      q[c] = load_row_operand(a.q + ((size_t)(start + safe_row) * a.heads + safe_head) * HD, g);
-      hi[c] = live[c] ? pos0 + row : -1;
-      lo[c] = (a.window > 0 && hi[c] + 1 > a.window) ? hi[c] + 1 - a.window : 0;
-      last = hi[c] > last ? hi[c] : last;
-    }
-  // the wave runs to the farthest key any of its columns reads, from the nearest
-  int first = 0x7fffffff;
-#pragma unroll
-  for (int c = 0; c < C; ++c) first = (live[c] && lo[c] < first) ? lo[c] : first;
-#pragma unroll
-  for (int offset = kWave / 2; offset > 0; offset >>= 1) {
-    last = max(last, __shfl_xor(last, offset, kWave));
-    first = min(first, __shfl_xor(first, offset, kWave));
-  }
-  AttnState<C> st;
-  init_state(st);
-  if (last >= 0) {
-    const int first_page = first / kPageTokens, page_count = last / kPageTokens + 1 - first_page;
-    const int mine = page_count > wave ? (page_count - wave + waves - 1) / waves : 0;  // pages of this wave
-    attend_run<C, (HD > 64 ? 2 : (C <= 2 ? 4 : (C == 3 ? 3 : 2)))>(st, q, a, pages, kv_head, first_page + wave, waves, mine, last, lo, hi, lane);
-  }
-  if (!merge_waves<C>(st, merge, wave, waves, lane)) return;
-#pragma unroll
-  for (int qt = 0; qt < QT; ++qt)
-#pragma unroll
-    for (int gh = 0; gh < GH; ++gh) {
-      const int c = qt * GH + gh;
-      float total = st.l[c];
-      total += __shfl_xor(total, 16, kWave);
-      total += __shfl_xor(total, 32, kWave);
-      if (!live[c]) continue;
-      const float inv = 1.0f / total;
-      bf16_t* dst = a.out + ((size_t)(start + row0 + 16 * qt + r) * a.heads + head0 + gh) * HD;
-#pragma unroll
-      for (int t = 0; t < kTilesD; ++t) {
-        bf16x4 packed;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) packed[e] = (__bf16)(st.o[c][t][e] * inv);
-        *(bf16x4*)(dst + 16 * t + 4 * g) = packed;
+      for (int gh = 0; gh < GH; ++gh) {
+        const int c = qt * GH + gh;
+        const int row = row0 + 16 * qt + r;
+        const int head = head0 + gh;
+        live[c] = row < rows && head < kv_head * group + group;
+        const int safe_row = row < rows ? row : rows - 1;
+        const int safe_head = head < a.heads ? head : a.heads - 1;
+        q[c] = load_row_operand(a.q + ((size_t)(start + safe_row) * a.heads + safe_head) * HD, g);
+        hi[c] = live[c] ? pos0 + row : -1;
+        lo[c] = (a.window > 0 && hi[c] + 1 > a.window) ? hi[c] + 1 - a.window : 0;
+        last = hi[c] > last ? hi[c] : last;
       }
+    // the wave runs to the farthest key any of its columns reads, from the nearest
+    int first = 0x7fffffff;
+#pragma unroll
+    for (int c = 0; c < C; ++c) first = (live[c] && lo[c] < first) ? lo[c] : first;
+#pragma unroll
+    for (int offset = kWave / 2; offset > 0; offset >>= 1) {
+      last = max(last, __shfl_xor(last, offset, kWave));
+      first = min(first, __shfl_xor(first, offset, kWave));
     }
+    AttnState<C> st;
+    init_state(st);
+    if (last >= 0) {
+      const int first_page = first / kPageTokens, page_count = last / kPageTokens + 1 - first_page;
+      const int mine = page_count > wave ? (page_count - wave + waves - 1) / waves : 0;  // pages of this wave
+      attend_run<C, (HD > 64 ? 2 : (C <= 2 ? 4 : (C == 3 ? 3 : 2)))>(st, q, a, pages, kv_head, first_page + wave, waves, mine, last, lo, hi, lane);
+    }
+    if (!merge_waves<C>(st, merge, wave, waves, lane)) return;
+#pragma unroll
+    for (int qt = 0; qt < QT; ++qt)
+#pragma unroll
+      for (int gh = 0; gh < GH; ++gh) {
+        const int c = qt * GH + gh;
+        float total = st.l[c];
+        total += __shfl_xor(total, 16, kWave);
+        total += __shfl_xor(total, 32, kWave);
+        if (!live[c]) continue;
+        const float inv = 1.0f / total;
+        bf16_t* dst = a.out + ((size_t)(start + row0 + 16 * qt + r) * a.heads + head0 + gh) * HD;
+#pragma unroll
+        for (int t = 0; t < kTilesD; ++t) {
+          bf16x4 packed;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) packed[e] = (__bf16)(st.o[c][t][e] * inv);
+          *(bf16x4*)(dst + 16 * t + 4 * g) = packed;
+        }
+      }
+  };
+  run_item(0);
+  if (count > 1) {
+    __syncthreads();  // the first item's merge has been read
+    run_item(1);
+  }
 }
 
 // The end of a decode block: the waves' states merge in LDS; the wave that is left writes the output
@@ -828,6 +855,18 @@ int fill_common(MfmaArgs& a, const void* q, void* out, const void* k_pages, cons
 }
 }  // namespace
 
+// compute units of the device in use (the library serves one device a process)
+static int compute_units() {
+  static const int units = [] {
+    int device = 0, n = 0;
+    if (hipGetDevice(&device) != hipSuccess ||
+        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || n <= 0)
+      n = 256;
+    return n;
+  }();
+  return units;
+}
+
 // rows of 16*QT queries per tile, as the host must cut them
 // `columns`: the most column tiles a wave carries, 1 .. kMaxColumns (0: as many as the head size allows).
 // Fewer columns mean more, lighter blocks and more waves to deal a tile's keys to.
@@ -869,20 +908,29 @@ extern "C" int nnis_attention_prefill_bf16(const void* q, void* out, const void*
   int qt, gh;
   prefill_shape(heads, kv_heads, columns, &qt, &gh);
   const int chunks = (group + gh - 1) / gh;
-  const dim3 grid(tiles, kv_heads * chunks);
-  NNIS_REQUIRE(grid.y <= 65535, "attention: %d head chunks exceed the grid limit", grid.y);
+  const int per_tile = kv_heads * chunks;
+  NNIS_REQUIRE((long long)tiles * per_tile <= 0x7fffffff, "attention: %d tiles x %d head chunks exceed the grid limit", tiles, per_tile);
+  const int items = tiles * per_tile;
+  // blocks: one per item while each compute unit gets at most one; beyond that two items a block, until
+  // every block has two
+  const int units = compute_units();
+  const int blocks = std::max((items + 1) / 2, std::min(items, units));
+  const int singles = 2 * blocks - items;
+  const dim3 grid(blocks);
   const size_t per_wave = (size_t)qt * gh * (kTilesD * 4 + 2) * kWave * sizeof(float);
   NNIS_REQUIRE(waves >= 1 && waves <= kBlockWaves && (waves & (waves - 1)) == 0 && (waves / 2) * per_wave <= 65536,
                "attention: %d waves a block: a power of two that fits this head size (LDS) is needed", waves);
   const size_t lds = (waves / 2) * per_wave;
   const dim3 block(kWave * waves);
   hipStream_t s = (hipStream_t)stream;
+#define NNIS_PREFILL(QT_, GH_) \
+  hipLaunchKernelGGL((attention_prefill_kernel<QT_, GH_>), grid, block, lds, s, a, waves, items, singles, per_tile)
   bool launched = true;
   if constexpr (kMaxColumns >= 4) {
-    if (qt == 4 && gh == 1) hipLaunchKernelGGL((attention_prefill_kernel<4, 1>), grid, block, lds, s, a, waves);
-    else if (qt == 2 && gh == 2) hipLaunchKernelGGL((attention_prefill_kernel<2, 2>), grid, block, lds, s, a, waves);
-    else if (qt == 1 && gh == 3) hipLaunchKernelGGL((attention_prefill_kernel<1, 3>), grid, block, lds, s, a, waves);
-    else if (qt == 1 && gh == 4) hipLaunchKernelGGL((attention_prefill_kernel<1, 4>), grid, block, lds, s, a, waves);
+    if (qt == 4 && gh == 1) NNIS_PREFILL(4, 1);
+    else if (qt == 2 && gh == 2) NNIS_PREFILL(2, 2);
+    else if (qt == 1 && gh == 3) NNIS_PREFILL(1, 3);
+    else if (qt == 1 && gh == 4) NNIS_PREFILL(1, 4);
     else launched = false;
   } else {
     launched = false;
@@ -890,17 +938,18 @@ extern "C" int nnis_attention_prefill_bf16(const void* q, void* out, const void*
   if (!launched) {
     launched = true;
     if constexpr (kMaxColumns >= 2) {
-      if (qt == 2 && gh == 1) hipLaunchKernelGGL((attention_prefill_kernel<2, 1>), grid, block, lds, s, a, waves);
-      else if (qt == 1 && gh == 2) hipLaunchKernelGGL((attention_prefill_kernel<1, 2>), grid, block, lds, s, a, waves);
+      if (qt == 2 && gh == 1) NNIS_PREFILL(2, 1);
+      else if (qt == 1 && gh == 2) NNIS_PREFILL(1, 2);
       else launched = false;
     } else {
       launched = false;
     }
   }
   if (!launched) {
-    if (qt == 1 && gh == 1) hipLaunchKernelGGL((attention_prefill_kernel<1, 1>), grid, block, lds, s, a, waves);
+    if (qt == 1 && gh == 1) NNIS_PREFILL(1, 1);
     else return nnis_fail("attention: no kernel for %d query tiles x %d heads", qt, gh);
   }
+#undef NNIS_PREFILL
   NNIS_LAUNCH_CHECK("attention_prefill");
   return 0;
 }

@@ -89,13 +89,14 @@ struct ResidualOut {
   float* ss;         // [parts, m]; a part is 16 columns (skinny kernel) or a wave's columns (tiled kernel)
 };
 
-// four consecutive columns of a token: what the stream and the gain hold there, asked for early
+// four consecutive columns of a token: what the stream and the gain hold there, asked for early.  A gain in
+// bfloat16 stays as it was loaded (two words in g) until it is taken: arithmetic on it here would make the
+// kernel wait for the load before its main loop.
 struct ResidualHeld {
   f32x4 v, g;
 };
 
 __device__ __forceinline__ ResidualHeld residual_ask(const ResidualOut& o, size_t index, int column, int valid, bool vector_ok) {
-  typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
   ResidualHeld h;
   h.v = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
   h.g = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
@@ -104,9 +105,9 @@ __device__ __forceinline__ ResidualHeld residual_ask(const ResidualOut& o, size_
     if (o.gain_dtype == NNIS_F32) {
       h.g = *(const f32x4*)((const float*)o.gain + column);
     } else {
-      const bf16x4 packed = *(const bf16x4*)((const bf16_t*)o.gain + column);
-#pragma unroll
-      for (int e = 0; e < 4; ++e) h.g[e] = (float)packed[e];
+      const float2 packed = *(const float2*)((const bf16_t*)o.gain + column);
+      h.g[0] = packed.x;
+      h.g[1] = packed.y;
     }
   } else {
     for (int e = 0; e < valid; ++e) {
@@ -122,13 +123,20 @@ __device__ __forceinline__ float residual_take(const ResidualOut& o, const Resid
                                                bool vector_ok) {
   typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
   float sq = 0.0f;
-  f32x4 v = h.v;
+  f32x4 v = h.v, gain = h.g;
+  if (valid == 4 && vector_ok && o.gain_dtype != NNIS_F32) {  // four bfloat16 in two words: a float's upper half each
+    const unsigned lo = __float_as_uint(h.g[0]), hi = __float_as_uint(h.g[1]);
+    gain[0] = __uint_as_float(lo << 16);
+    gain[1] = __uint_as_float(lo & 0xffff0000u);
+    gain[2] = __uint_as_float(hi << 16);
+    gain[3] = __uint_as_float(hi & 0xffff0000u);
+  }
   bf16x4 scaled;
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
     v[e] += acc[e];
     if (e < valid) sq = fmaf(v[e], v[e], sq);
-    scaled[e] = (__bf16)(v[e] * h.g[e]);
+    scaled[e] = (__bf16)(v[e] * gain[e]);
   }
   if (valid == 4 && vector_ok) {
     *(f32x4*)(o.resid + index) = v;
@@ -283,29 +291,41 @@ __global__ __launch_bounds__(KSPLIT > 4 ? 64 * KSPLIT : 256) void gemm_skinny_ke
 }
 
 // -----------------------------------------------------------------------------
-// tiled: BM x BN output tile per block of 4 waves (2 x 2), K in steps of BK (64; steps of 128 and tiles of
-// 32 rows were measured no faster on products from 2048 x 576 x 576 to 2048 x 6144 x 2048)
+// tiled: BM x BN output tile per block of 4 waves (2 x 2), K in steps of BK = 64.  The operands go from
+// memory straight into LDS (no registers between), a ring of kStages stages deep.  Measured on products from
+// 2048 x 576 x 576 to 2048 x 6144 x 2048, in place of loads through registers: 10 to 17% less time; steps of
+// 32 k, and frags of the next step read before the barrier, were slower; tiles of 128 x 256 and 256 x 256
+// with 8 waves gain only where they still make 500 blocks and more.
 // -----------------------------------------------------------------------------
 // chunk c of row `row` of a staged tile (CHUNKS chunks of 16 bytes a row) lives at chunk c ^ (row % CHUNKS)
 template <int CHUNKS>
 __device__ __forceinline__ int swizzled(int row, int chunk) { return row * CHUNKS + (chunk ^ (row & (CHUNKS - 1))); }
 
+typedef __attribute__((address_space(1))) const void* global_ptr_t;
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+// The loads into LDS are not the compiler's to wait for: the kernel counts them itself.
+template <int N>
+__device__ __forceinline__ void wait_loads_but() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
+
+extern __shared__ __align__(16) char tile_lds[];  // kStages stages of BM + BN rows of BK
+
 #ifndef NNIS_TILE_GROUP_ROWS
 #define NNIS_TILE_GROUP_ROWS 512
 #endif
+constexpr int kTileStages = 3;
 template <int BM, int BN, int BK, typename OutT>
 __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                                                          OutT y, int m, int n, int k, int col_blocks) {
   constexpr int WM = BM / 2, WN = BN / 2;  // a wave's part of the tile
   constexpr int TM = WM / 16, TN = WN / 16;
   constexpr int CH = BK / 8;  // 16-byte chunks per staged row
-  constexpr int A_CHUNKS = BM * CH / 256, B_CHUNKS = BN * CH / 256;  // chunks a thread stages per step
-  // Global loads run PF steps ahead of the multiply, in registers; the step after
-  // the current one lies in the other LDS buffer.  With few blocks on a compute
-  // unit nothing else hides the latency of a load, so short products need depth.
-  constexpr int PF = 3;
-  __shared__ bf16x8 a_tile[2][BM * CH];
-  __shared__ bf16x8 b_tile[2][BN * CH];
+  static_assert(CH == 8, "a load instruction of a wave fills 8 rows of 8 chunks");
+  // One load instruction of a wave moves 64 x 16 bytes into 1 KB of LDS that is contiguous: 8 rows of a
+  // stage, lane l to row l / 8, place l % 8.  The swizzle is made on the way in by the choice of the source:
+  // place p of row r holds chunk p ^ (r % 8).
+  constexpr int A_LOADS = BM / 32, B_LOADS = BN / 32;  // a wave's load instructions per step (4 waves x 8 rows each)
+  constexpr int LOADS = A_LOADS + B_LOADS;
+  constexpr int A_BYTES = BM * BK * 2, STAGE_BYTES = (BM + BN) * BK * 2;
 
   const int tid = threadIdx.x;
   const int wave = tid / kWave, lane = tid % kWave;
@@ -336,46 +356,78 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
 #pragma unroll
     for (int j = 0; j < TN; ++j) acc[i][j] = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
 
-  // what this thread stages: rows and chunk of each of its 16-byte pieces
-  const bf16_t* a_src[A_CHUNKS];
-  const bf16_t* b_src[B_CHUNKS];
-  int a_dst[A_CHUNKS], b_dst[B_CHUNKS];
-  const int chunk_k = (tid % CH) * 8;
+  // what this lane loads: its chunk (the same for every load: rows 8 apart) of rows 8 (4 o + wave) + lane / 8
+  const bf16_t* a_src[A_LOADS];
+  const bf16_t* b_src[B_LOADS];
+  const int chunk_k = ((lane % 8) ^ (lane / 8)) * 8;
 #pragma unroll
-  for (int c = 0; c < A_CHUNKS; ++c) {
-    const int index = tid + c * 256;  // row = index / CH, chunk = index % CH
-    int row = row0 + index / CH;
+  for (int o = 0; o < A_LOADS; ++o) {
+    int row = row0 + (o * 4 + wave) * 8 + lane / 8;
     row = row < m ? row : m - 1;
-    a_src[c] = x + (size_t)row * k + chunk_k;
-    a_dst[c] = swizzled<CH>(index / CH, index % CH);
+    a_src[o] = x + (size_t)row * k + chunk_k;
   }
   constexpr int EPI = scaled_epilogue<OutT>::value;  // -1: the product is stored or added as it is
   constexpr bool kPaired = EPI == EPI_SILU || EPI == EPI_ROPE;
 #pragma unroll
-  for (int c = 0; c < B_CHUNKS; ++c) {
-    const int index = tid + c * 256;
+  for (int o = 0; o < B_LOADS; ++o) {
+    const int tile_row = (o * 4 + wave) * 8 + lane / 8;
     int row;
     if constexpr (kPaired) {
-      row = paired_weight_row<EPI, BN>(y.rope, col_block, index / CH, n);
+      row = paired_weight_row<EPI, BN>(y.rope, col_block, tile_row, n);
       row = row >= 0 ? row : 0;  // rows beyond the end read a valid row and are not stored
     } else {
-      row = col0 + index / CH;
+      row = col0 + tile_row;
       row = row < n ? row : n - 1;
     }
-    b_src[c] = w + (size_t)row * k + chunk_k;
-    b_dst[c] = swizzled<CH>(index / CH, index % CH);
+    b_src[o] = w + (size_t)row * k + chunk_k;
   }
-  // a prepared operand: the rows' scales, for the epilogue; and what the rotation needs of each token
-  __shared__ float row_scale[EPI >= 0 ? BM : 1];
+  // Step s lies in stage s % kTileStages.  A step first asks for the step kTileStages - 1 ahead, into the
+  // stage that was read a step ago (every wave is past the barrier that ended that step, and what it read
+  // there its matrix instructions have taken); then multiplies its own stage; then waits until all but the
+  // newest kTileStages - 2 steps' loads of this wave have arrived (loads arrive in the order they were
+  // asked for), and for the other waves' at the barrier.  A step beyond the end of K is asked for all the
+  // same, so that the count holds: from the row's last whole chunk, a valid address, and nobody reads it.
+  // In the last step of a K that is no multiple of BK the same holds for the chunks beyond K; the lanes
+  // that hold them as the first operand make them zeros.
+  const int steps = (k + BK - 1) / BK;
+  int last_chunk = k - 8 - chunk_k;  // offset of the row's last whole chunk from this lane's first
+  last_chunk = last_chunk > -chunk_k ? last_chunk : -chunk_k;
+  auto ask = [&](int step, int stage) {
+    char* base = tile_lds + stage * STAGE_BYTES + wave * 1024;
+    const int k0 = step * BK;
+    const int from = k0 <= last_chunk ? k0 : last_chunk;
+#pragma unroll
+    for (int o = 0; o < A_LOADS; ++o)
+      __builtin_amdgcn_global_load_lds((global_ptr_t)(a_src[o] + from), (lds_ptr_t)(base + o * 4096), 16, 0, 0);
+#pragma unroll
+    for (int o = 0; o < B_LOADS; ++o)
+      __builtin_amdgcn_global_load_lds((global_ptr_t)(b_src[o] + from), (lds_ptr_t)(base + A_BYTES + o * 4096), 16, 0, 0);
+  };
+  const bool ragged = (k % BK) != 0;
+
+#pragma unroll
+  for (int s = 0; s < kTileStages - 1; ++s) ask(s, s);
+
+  // Behind the first steps' loads, so that one wait covers both: a prepared operand's row scales, for the
+  // epilogue, and what the rotation needs of each token
+  __shared__ float row_scale[EPI >= 0 ? 4 : 1][EPI >= 0 ? BM : 1];  // each wave's share of a row's sum of squares
   int tok_pos[TM], tok_page[TM];
   if constexpr (EPI >= 0) {
-    if (tid < BM) {
-      const int token = row0 + tid;
-      float total = 0.0f;
-      if (token < m)
-        for (int p = 0; p < y.parts; ++p) total += y.ss_parts[(size_t)p * m + token];
-      row_scale[tid] = 1.0f / sqrtf(total / (float)k + y.eps);
+    // lane = row, wave w takes the parts w, w + 4, ..: eight loads at a time, none waiting for another
+    static_assert(BM == 64, "a lane per row of the tile");
+    const int token = row0 + lane < m ? row0 + lane : m - 1;
+    float total = 0.0f;
+    for (int p0 = wave; p0 < y.parts; p0 += 32) {
+      float part[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        const int p = p0 + 4 * u;
+        part[u] = y.ss_parts[(size_t)(p < y.parts ? p : y.parts - 1) * m + token];
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u) total += p0 + 4 * u < y.parts ? part[u] : 0.0f;
     }
+    row_scale[wave][lane] = total;
     if constexpr (EPI == EPI_ROPE) {
 #pragma unroll
       for (int i = 0; i < TM; ++i) {
@@ -405,65 +457,48 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
       }
   }
 
-  // Registers hold the loads of the next PF steps, slot (step % PF).  The loop body is PF steps in one
-  // straight line that every round runs in full -- a load or an LDS write behind a branch makes the
-  // compiler wait for every load in flight at the next use of any, and the steps loaded ahead would be
-  // waited for at once.  So the steps are rounded up to whole rounds; a step beyond the end of K is loaded
-  // all the same (from the last whole chunk of the row, a valid address), turned into zeros on its way into
-  // LDS and multiplied as zeros.  With PF = 3 the products of this library (K = 576, 1536, 2048, 5632, 8192)
-  // run at most two such steps.
-  bf16x8 a_stage[PF][A_CHUNKS], b_stage[PF][B_CHUNKS];
-  const int steps = (k + BK - 1) / BK;
-  const int last_chunk = k - 8 - chunk_k;  // offset of the row's last whole chunk from this thread's first
-
-#define NNIS_FETCH(slot, step)                                                                   \
-  do {                                                                                           \
-    const int k0 = (step) * BK;                                                                  \
-    const int from = k0 <= last_chunk ? k0 : last_chunk;                                         \
-    _Pragma("unroll") for (int c = 0; c < A_CHUNKS; ++c) a_stage[slot][c] = load_chunk(a_src[c] + from); \
-    _Pragma("unroll") for (int c = 0; c < B_CHUNKS; ++c) b_stage[slot][c] = load_chunk(b_src[c] + from); \
-  } while (0)
-#define NNIS_STAGE(slot, step, buffer)                                                           \
-  do {                                                                                           \
-    const bool in = (step) * BK <= last_chunk;                                                   \
-    _Pragma("unroll") for (int c = 0; c < A_CHUNKS; ++c) a_tile[buffer][a_dst[c]] = in ? a_stage[slot][c] : zero_chunk(); \
-    _Pragma("unroll") for (int c = 0; c < B_CHUNKS; ++c) b_tile[buffer][b_dst[c]] = in ? b_stage[slot][c] : zero_chunk(); \
-  } while (0)
-
+  wait_loads_but<(kTileStages - 2) * LOADS>();
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+  int stage = 0;
+  for (int step = 0; step < steps; ++step) {
+    ask(step + kTileStages - 1, stage == 0 ? kTileStages - 1 : stage - 1);
+    const bf16x8* a_tile = (const bf16x8*)(tile_lds + stage * STAGE_BYTES);
+    const bf16x8* b_tile = (const bf16x8*)(tile_lds + stage * STAGE_BYTES + A_BYTES);
 #pragma unroll
-  for (int s = 0; s < PF; ++s) NNIS_FETCH(s, s);
-  NNIS_STAGE(0, 0, 0);
-  __syncthreads();
-  for (int base = 0; base < steps; base += PF) {
+    for (int half = 0; half < BK / 32; ++half) {  // an instruction takes 32 k
+      bf16x8 a_frag[TM], b_frag[TN];
 #pragma unroll
-    for (int j = 0; j < PF; ++j) {
-      const int step = base + j;
-      const int buffer = step & 1;
-      // slot j went to LDS a step ago: the step PF ahead takes its place
-      NNIS_FETCH(j, step + PF);
+      for (int i = 0; i < TM; ++i) a_frag[i] = a_tile[swizzled<CH>(wave_m * WM + i * 16 + r, half * 4 + g)];
 #pragma unroll
-      for (int half = 0; half < BK / 32; ++half) {  // an instruction takes 32 k
-        bf16x8 a_frag[TM], b_frag[TN];
+      for (int jj = 0; jj < TN; ++jj) b_frag[jj] = b_tile[swizzled<CH>(wave_n * WN + jj * 16 + r, half * 4 + g)];
+      if (ragged && step == steps - 1 && step * BK + (half * 4 + g) * 8 + 8 > k) {
 #pragma unroll
-        for (int i = 0; i < TM; ++i) a_frag[i] = a_tile[buffer][swizzled<CH>(wave_m * WM + i * 16 + r, half * 4 + g)];
-#pragma unroll
-        for (int jj = 0; jj < TN; ++jj) b_frag[jj] = b_tile[buffer][swizzled<CH>(wave_n * WN + jj * 16 + r, half * 4 + g)];
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-          for (int jj = 0; jj < TN; ++jj) acc[i][jj] = mfma(b_frag[jj], a_frag[i], acc[i][jj]);
+        for (int i = 0; i < TM; ++i) a_frag[i] = zero_chunk();
       }
-      NNIS_STAGE((j + 1) % PF, step + 1, buffer ^ 1);
-      __syncthreads();
-      // Nothing of a later step moves up into this one: its slot's zero-or-data choice would wait for
-      // loads that have steps of time left.  (The smaller tile only: a wave of the larger one gains more
-      // from the next step's LDS reads among this step's matrix instructions.)
-      if constexpr (TM * TN <= 4) __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int jj = 0; jj < TN; ++jj) acc[i][jj] = mfma(b_frag[jj], a_frag[i], acc[i][jj]);
     }
+    // what this wave read of its stage has arrived too: the stage is the next step's to fill
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    wait_loads_but<(kTileStages - 2) * LOADS>();
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    stage = stage + 1 == kTileStages ? 0 : stage + 1;
   }
-#undef NNIS_FETCH
-#undef NNIS_STAGE
+  wait_loads_but<0>();  // the steps asked for beyond the end: nothing of this block is in flight when it ends
 
+  // a prepared operand's norm: 1 / sqrt(mean of squares + eps) of a tile row
+  auto scale_of = [&](int row) -> float {
+    if constexpr (EPI >= 0) {
+      const float total = (row_scale[0][row] + row_scale[1][row]) + (row_scale[2][row] + row_scale[3][row]);
+      return 1.0f / sqrtf(total / (float)k + y.eps);
+    } else {
+      return 1.0f;
+    }
+  };
   // first operand = weight rows: lane holds D[n = 4g + e][token = r]
   const bool vector_ok = (n % 4) == 0;
   if constexpr (kPaired) {
@@ -472,7 +507,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
     for (int i = 0; i < TM; ++i) {
       const int token = row0 + wave_m * WM + i * 16 + r;
       if (token >= m) continue;
-      const float scale = row_scale[wave_m * WM + i * 16 + r];
+      const float scale = scale_of(wave_m * WM + i * 16 + r);
 #pragma unroll
       for (int u = 0; u < TN / 2; ++u) {
         const int first = paired_weight_row<EPI, BN>(y.rope, col_block, wave_n * WN + 32 * u, n);  // the unit's first lower row
@@ -502,7 +537,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
     const int token = row0 + wave_m * WM + i * 16 + r;
     float sq = 0.0f;
     float scale = 1.0f;
-    if constexpr (EPI == EPI_STORE) scale = row_scale[wave_m * WM + i * 16 + r];
+    if constexpr (EPI == EPI_STORE) scale = scale_of(wave_m * WM + i * 16 + r);
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
       const int n0 = col0 + wave_n * WN + j * 16 + g * 4;
@@ -563,8 +598,13 @@ void dispatch_skinny(const bf16_t* x, const bf16_t* w, OutT y, int m, int n, int
 template <int BM, int BN, int BK, typename OutT>
 void launch_tiled(const bf16_t* x, const bf16_t* w, OutT y, int m, int n, int k, int columns, hipStream_t stream) {
   const int col_blocks = (columns + BN - 1) / BN, row_blocks = (m + BM - 1) / BM;
-  hipLaunchKernelGGL((gemm_tiled_kernel<BM, BN, BK, OutT>), dim3((unsigned)col_blocks * row_blocks), dim3(256), 0, stream, x, w,
-                     y, m, n, k, col_blocks);
+  constexpr int lds_bytes = kTileStages * (BM + BN) * BK * 2;
+  // beyond 64 KB a kernel has to be told once; a refusal shows as the launch's failure
+  static const hipError_t allowed = hipFuncSetAttribute((const void*)gemm_tiled_kernel<BM, BN, BK, OutT>,
+                                                        hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+  (void)allowed;
+  hipLaunchKernelGGL((gemm_tiled_kernel<BM, BN, BK, OutT>), dim3((unsigned)col_blocks * row_blocks), dim3(256), lds_bytes,
+                     stream, x, w, y, m, n, k, col_blocks);
 }
 
 // 2: 64x128, 3: 64x64 -- the larger tile when it still gives every compute unit a block.  (A tile of
