@@ -654,12 +654,12 @@ int skinny_split(int m, int n, int k, int split_hint) {
 // 64 tokens always.  Beyond, up to kFewTokens, when the weights are small enough to be read once per tile of
 // 16 tokens and its blocks (strips x token tiles) are few enough; measured on products of 32 to 384 tokens
 // with weights of 576 x 576 to 3072 x 576 and 576 x 1536, in microseconds:
-//   few tokens: 3 + 0.004 * strips * tiles * K / 576      tiled: 2 + 0.011 * K
+//   few tokens: 3 + 0.004 * strips * tiles * K / 576      tiled: 2.6 + 0.0057 * K
 bool nnis_gemm_takes_few_tokens(int m, int n, int k) {
   if (m <= 64) return true;
   if (m > kFewTokens || (size_t)n * k * sizeof(bf16_t) > kRereadWeightBytes) return false;
   const double strips = (n + 15) / 16, tiles = (m + 15) / 16;
-  return 3.0 + 0.004 * strips * tiles * k / 576.0 <= 2.0 + 0.011 * k;
+  return 3.0 + 0.004 * strips * tiles * k / 576.0 <= 2.6 + 0.0057 * k;
 }
 
 int nnis_gemm_scaled_tiled(const bf16_t* scaled, const float* ss_parts, int parts, float eps, const bf16_t* w, int m, int n,

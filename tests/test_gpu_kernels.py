@@ -223,6 +223,66 @@ def test_prefill_attention_on_the_matrix_cores(heads, kv_heads, head_dim):
             assert (got[100, 0] - vs[2][17, 0]).abs().max().item() < 0.05
 
 
+@pytest.mark.parametrize("heads, kv_heads, head_dim, lengths", [(9, 3, 64, (1500, 700, 90)), (8, 8, 16, (1300, 1000, 100))])
+def test_prefill_attention_with_more_items_than_compute_units(heads, kv_heads, head_dim, lengths):
+    """Steps of so many tiles that a block takes two of them, a long one and
+    then a short one.  The second sequence goes on from position 100.  One
+    loud key far back for a row of the shortest tiles and one for a row of
+    the longest."""
+    ops = _ops()
+    torch.manual_seed(heads + head_dim)
+    sequences = [(1, 0, lengths[0]), (2, 100, lengths[1]), (0, 0, lengths[2])]  # (slot, first new position, new tokens)
+    total = {slot: pos0 + n for slot, pos0, n in sequences}
+    ks = [torch.randn(total[s], kv_heads, head_dim).bfloat16().float() for s in range(3)]
+    vs = [torch.randn(total[s], kv_heads, head_dim).bfloat16().float() for s in range(3)]
+    scale = 1.0 / math.sqrt(head_dim)
+    queries = {slot: torch.zeros(total[slot], heads, head_dim) for slot in total}
+    for slot, pos0, n in sequences:
+        queries[slot][pos0:] = torch.randn(n, heads, head_dim).bfloat16().float()
+    loud = [(0, 40, 3), (1, lengths[0] - 2, 70)]  # (slot, position of the row, position of the key), head 0
+    for slot, row, key in loud:
+        loud_q = queries[slot][row, 0]
+        ks[slot][key, 0] = (loud_q * (14.0 / scale / loud_q.pow(2).sum())).bfloat16().float()
+    pages = sum((n + 63) // 64 for n in total.values())
+    k_pages, v_pages, table = _paged(ks, vs, torch.bfloat16, kv_heads, head_dim, pages=pages, max_pages=max(total.values()) // 64 + 1)
+    q = torch.cat([queries[slot][pos0:] for slot, pos0, _ in sequences]).bfloat16().reshape(sum(lengths), -1).cuda()
+    want = torch.cat([P.causal_attention(queries[slot], ks[slot], vs[slot], scale)[pos0:] for slot, pos0, _ in sequences])
+    starts = [0, lengths[0], lengths[0] + lengths[1], sum(lengths)]
+    tile = ops.prefill_tile_rows(heads, kv_heads, head_dim)
+    items = sorted(((pos0 + min(row0 + tile, n), seq, row0) for seq, (_, pos0, n) in enumerate(sequences)
+                    for row0 in range(0, n, tile)), reverse=True)  # longest first, as the engine hands them over
+    group_chunks = kv_heads * -(-(heads // kv_heads) // max(1, min(heads // kv_heads, 4)))
+    assert len(items) * group_chunks > 256 + 32  # more than the compute units of the chip: the grid folds
+    for waves in (8, 2):
+        waves = min(waves, ops.prefill_max_waves(heads, kv_heads, head_dim))
+        out = torch.full((sum(lengths), heads * head_dim), 3.0, dtype=torch.bfloat16, device="cuda")
+        ops.attention_prefill_bf16(q, out, k_pages, v_pages, table, _i32([s for _, s, _ in items]), _i32([r for _, _, r in items]),
+                                   _i32([s for s, _, _ in sequences]), _i32(starts), _i32([p for _, p, _ in sequences]),
+                                   heads, kv_heads, head_dim, scale, 0, waves)
+        got = out.cpu().float().view(sum(lengths), heads, head_dim)
+        error = (got - want).abs().amax(dim=(1, 2))
+        assert error.max().item() <= 2e-2, (waves, int(error.argmax()), error.max().item())
+        for slot, row, key in loud:
+            seq = [s for s, _, _ in sequences].index(slot)
+            packed = starts[seq] + row - sequences[seq][1]
+            assert (got[packed, 0] - vs[slot][key, 0]).abs().max().item() < 0.05
+
+
+@pytest.mark.parametrize("hint", [32, 48])
+def test_gemm_tiled_over_many_blocks(hint):
+    """Both tiles of the tiled kernel over a grid of hundreds of blocks in
+    bands and groups, with a ragged edge in every dimension; whole-number
+    operands, so a block that took another's rows or columns shows."""
+    ops = _ops()
+    torch.manual_seed(hint)
+    m, n, k = 2300, 1100, 584
+    x = torch.randint(-3, 4, (m, k)).to(torch.bfloat16)
+    w = torch.randint(-3, 4, (n, k)).to(torch.bfloat16)
+    y = torch.full((m, n), 7.0, dtype=torch.float32, device="cuda")
+    ops.gemm_bf16(x.cuda(), w.cuda(), y, hint)
+    assert torch.equal(y.cpu().double(), x.double() @ w.double().t())
+
+
 @pytest.mark.parametrize("m", [1, 8, 19, 64, 67, 100, 300])
 @pytest.mark.parametrize("n, k", [(576, 576), (100, 72), (2048, 1536), (48, 8), (64, 176), (3072, 576)])
 @pytest.mark.parametrize("gain_dtype", ["bfloat16", "float32"])
