@@ -9,8 +9,8 @@
 // maximum; output = sum of weights * values / sum of weights.  All of it in
 // 32-bit, whatever the storage type.
 //
-// Page layouts:  K [page][kv_head][token in page][head_dim]
-//                V [page][kv_head][head_dim][token in page]
+// Pages: [page][kv_head][64 tokens of one head], keys and values each in the in-page order of common.h
+// (keys in chunks of 8 channels, values in tiles of 16 channels with 8 tokens of a channel together).
 #include "common.h"
 
 #include <algorithm>

@@ -86,4 +86,5 @@ bool nnis_gemm_takes_few_tokens(int m, int n, int k);
 
 // the tiled kernel on an operand that a residual epilogue prepared (gemm_mfma.hip)
 int nnis_gemm_scaled_tiled(const bf16_t* scaled, const float* ss_parts, int parts, float eps, const bf16_t* w, int m, int n,
-                           int k, int epilogue, bf16_t* y, const RopeTarget& rope, int tile_hint, hipStream_t stream);
+                           int k, int epilogue, bf16_t* y, const RopeTarget& rope, int tile_hint, float* workspace,
+                           size_t workspace_bytes, hipStream_t stream);

@@ -7,14 +7,15 @@
 // operands agree.  Its result D[i][j] (i: row of the first operand, j: row of
 // the second) lies with lane l as D[4 * (l / 16) + e][l % 16], e = 0..3.
 //
-//  * gemm_skinny_kernel: M <= 64 (decode).  The weight is streamed once from
-//    memory straight into operand registers; a wave owns a strip of 16 weight
-//    rows; X (small, shared by all waves) comes through the caches.  Waves of
-//    a block may split K and add their parts through LDS.
-//  * gemm_tiled_kernel: any M (prefill).  64x128 or 64x64 output
-//    tiles, K staged through LDS in steps of 64 with an XOR swizzle of the
-//    16-byte chunks so that operand reads are free of bank conflicts, global
-//    loads of the next step in flight while the current one is multiplied.
+//  * gemm_skinny_kernel: few tokens (decode; nnis_gemm_takes_few_tokens says
+//    how many).  The weight is streamed from memory straight into operand
+//    registers; a wave owns a strip of 16 weight rows; X (small, shared by all
+//    waves) comes through the caches.  Waves of a block may split K and add
+//    their parts through LDS.
+//  * gemm_tiled_kernel: any M (prefill).  64x128 or 64x64 output tiles, K in
+//    steps of 64 that go from memory straight into LDS, a ring of stages
+//    deep, with an XOR swizzle of the 16-byte chunks so that operand reads
+//    are free of bank conflicts.
 //
 // Both need K % 8 == 0 and 16-byte aligned operands (the host checks) and take
 // any M and N.
@@ -292,7 +293,7 @@ __global__ __launch_bounds__(KSPLIT > 4 ? 64 * KSPLIT : 256) void gemm_skinny_ke
 
 // -----------------------------------------------------------------------------
 // tiled: BM x BN output tile per block of 4 waves (2 x 2), K in steps of BK = 64.  The operands go from
-// memory straight into LDS (no registers between), a ring of kStages stages deep.  Measured on products from
+// memory straight into LDS (no registers between), a ring of NS stages deep.  Measured on products from
 // 2048 x 576 x 576 to 2048 x 6144 x 2048, in place of loads through registers: 10 to 17% less time; steps of
 // 32 k, and frags of the next step read before the barrier, were slower; tiles of 128 x 256 and 256 x 256
 // with 8 waves gain only where they still make 500 blocks and more.
@@ -307,15 +308,17 @@ typedef __attribute__((address_space(3))) void* lds_ptr_t;
 template <int N>
 __device__ __forceinline__ void wait_loads_but() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory"); }
 
-extern __shared__ __align__(16) char tile_lds[];  // kStages stages of BM + BN rows of BK
+extern __shared__ __align__(16) char tile_lds[];  // NS stages of BM + BN rows of BK
 
 #ifndef NNIS_TILE_GROUP_ROWS
 #define NNIS_TILE_GROUP_ROWS 512
 #endif
-constexpr int kTileStages = 3;
-template <int BM, int BN, int BK, typename OutT>
+// NS stages: 3 where a compute unit runs several blocks; 6 where the grid leaves it one block at most, and
+// the loads in flight are all that hides the memory's latency (64 tokens x 11264 x 2048: 20.9 us with 3, 19.7 with 6)
+template <int BM, int BN, int BK, int NS, typename OutT>
 __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
-                                                         OutT y, int m, int n, int k, int col_blocks) {
+                                                         OutT y, int m, int n, int k, int col_blocks, int ksplit,
+                                                         float* __restrict__ partial) {
   constexpr int WM = BM / 2, WN = BN / 2;  // a wave's part of the tile
   constexpr int TM = WM / 16, TN = WN / 16;
   constexpr int CH = BK / 8;  // 16-byte chunks per staged row
@@ -334,15 +337,19 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
   // Blocks go to the chip's 8 dies in turn (block i to die i % 8), and each die has an L2 of its own: the
   // tiles are dealt so that a die's blocks cover a band of consecutive rows of X with all their column
   // blocks, and each die reads its band once instead of every die reading all of X.
-  int col_block, row_block;
+  // With ksplit > 1 the grid holds every tile ksplit times, part p of K for each (tiles of a part together).
+  int col_block, row_block, part;
   {
     const int total = gridDim.x, die = blockIdx.x % 8, nth = blockIdx.x / 8;
     const int each = total / 8, more = total % 8;  // the first `more` dies have one block more
-    const int tile = die * each + (die < more ? die : more) + nth;
+    const int item = die * each + (die < more ? die : more) + nth;
+    const int tiles = total / ksplit;
+    part = item / tiles;
+    const int tile = item % tiles;
     // within the order of the tiles, kGroup row blocks go through the column blocks together, rows fastest:
     // a column block of W serves them all while it is near
     constexpr int kGroup = NNIS_TILE_GROUP_ROWS / BM;
-    const int row_blocks = total / col_blocks;
+    const int row_blocks = tiles / col_blocks;
     const int group = tile / (kGroup * col_blocks), within = tile % (kGroup * col_blocks);
     const int rows_here = min(kGroup, row_blocks - group * kGroup);
     row_block = group * kGroup + within % rows_here;
@@ -381,15 +388,18 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
     }
     b_src[o] = w + (size_t)row * k + chunk_k;
   }
-  // Step s lies in stage s % kTileStages.  A step first asks for the step kTileStages - 1 ahead, into the
+  // Step s lies in stage s % NS.  A step first asks for the step NS - 1 ahead, into the
   // stage that was read a step ago (every wave is past the barrier that ended that step, and what it read
   // there its matrix instructions have taken); then multiplies its own stage; then waits until all but the
-  // newest kTileStages - 2 steps' loads of this wave have arrived (loads arrive in the order they were
+  // newest NS - 2 steps' loads of this wave have arrived (loads arrive in the order they were
   // asked for), and for the other waves' at the barrier.  A step beyond the end of K is asked for all the
   // same, so that the count holds: from the row's last whole chunk, a valid address, and nobody reads it.
   // In the last step of a K that is no multiple of BK the same holds for the chunks beyond K; the lanes
   // that hold them as the first operand make them zeros.
   const int steps = (k + BK - 1) / BK;
+  const int steps_a_part = (steps + ksplit - 1) / ksplit;
+  const int step0 = part * steps_a_part;  // this block multiplies steps step0 .. step1 - 1 (none, for a part beyond the end)
+  const int step1 = step0 + steps_a_part < steps ? step0 + steps_a_part : steps;
   int last_chunk = k - 8 - chunk_k;  // offset of the row's last whole chunk from this lane's first
   last_chunk = last_chunk > -chunk_k ? last_chunk : -chunk_k;
   auto ask = [&](int step, int stage) {
@@ -406,13 +416,13 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
   const bool ragged = (k % BK) != 0;
 
 #pragma unroll
-  for (int s = 0; s < kTileStages - 1; ++s) ask(s, s);
+  for (int s = 0; s < NS - 1; ++s) ask(step0 + s, s);
 
   // Behind the first steps' loads, so that one wait covers both: a prepared operand's row scales, for the
   // epilogue, and what the rotation needs of each token
   __shared__ float row_scale[EPI >= 0 ? 4 : 1][EPI >= 0 ? BM : 1];  // each wave's share of a row's sum of squares
   int tok_pos[TM], tok_page[TM];
-  if constexpr (EPI >= 0) {
+  if constexpr (EPI >= 0) if (ksplit == 1) {  // (with K in parts the reduce kernel does this)
     // lane = row, wave w takes the parts w, w + 4, ..: eight loads at a time, none waiting for another
     static_assert(BM == 64, "a lane per row of the tile");
     const int token = row0 + lane < m ? row0 + lane : m - 1;
@@ -444,7 +454,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
   constexpr bool kResidual = std::is_same<OutT, ResidualOut>::value;
   constexpr bool kAskEarly = kResidual && TM * TN <= 8;
   ResidualHeld held[kAskEarly ? TM : 1][kAskEarly ? TN : 1];
-  if constexpr (kAskEarly) {
+  if constexpr (kAskEarly) if (ksplit == 1) {
     const bool vector_ok = (n % 4) == 0;
 #pragma unroll
     for (int i = 0; i < TM; ++i)
@@ -457,12 +467,12 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
       }
   }
 
-  wait_loads_but<(kTileStages - 2) * LOADS>();
+  wait_loads_but<(NS - 2) * LOADS>();
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
   int stage = 0;
-  for (int step = 0; step < steps; ++step) {
-    ask(step + kTileStages - 1, stage == 0 ? kTileStages - 1 : stage - 1);
+  for (int step = step0; step < step1; ++step) {
+    ask(step + NS - 1, stage == 0 ? NS - 1 : stage - 1);
     const bf16x8* a_tile = (const bf16x8*)(tile_lds + stage * STAGE_BYTES);
     const bf16x8* b_tile = (const bf16x8*)(tile_lds + stage * STAGE_BYTES + A_BYTES);
 #pragma unroll
@@ -483,13 +493,27 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
     }
     // what this wave read of its stage has arrived too: the stage is the next step's to fill
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    wait_loads_but<(kTileStages - 2) * LOADS>();
+    wait_loads_but<(NS - 2) * LOADS>();
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
-    stage = stage + 1 == kTileStages ? 0 : stage + 1;
+    stage = stage + 1 == NS ? 0 : stage + 1;
   }
   wait_loads_but<0>();  // the steps asked for beyond the end: nothing of this block is in flight when it ends
 
+  // A part of K: the sums go to `partial` [part][token][grid column] as they are; gemm_reduce_kernel adds the
+  // parts and does what would follow here.
+  if (ksplit > 1) {
+    const size_t width = (size_t)col_blocks * BN;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      const int token = row0 + wave_m * WM + i * 16 + r;
+      if (token >= m) continue;
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        *(f32x4*)(partial + ((size_t)part * m + token) * width + col0 + wave_n * WN + j * 16 + g * 4) = acc[i][j];
+    }
+    return;
+  }
   // a prepared operand's norm: 1 / sqrt(mean of squares + eps) of a tile row
   auto scale_of = [&](int row) -> float {
     if constexpr (EPI >= 0) {
@@ -559,6 +583,114 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
   }
 }
 
+// The parts of K that gemm_tiled_kernel left in `partial` [ksplit][m][width], added in the order of the parts,
+// and the product's epilogue: stored, or taken into the residual stream with the next norm prepared (a part of
+// a row's sum of squares per 64 columns).  A thread has 4 columns of a token, a block 16 tokens x 64 columns.
+template <typename OutT>
+__global__ __launch_bounds__(256) void gemm_reduce_kernel(const float* __restrict__ partial, OutT y, int m, int n, int width,
+                                                          int ksplit) {
+  constexpr bool kResidual = std::is_same<OutT, ResidualOut>::value;
+  const int token = blockIdx.y * 16 + threadIdx.x / 16;
+  const int n0 = blockIdx.x * 64 + (threadIdx.x % 16) * 4;
+  const int valid = token < m ? (n - n0 >= 4 ? 4 : (n - n0 > 0 ? n - n0 : 0)) : 0;
+  const bool vector_ok = (n % 4) == 0;
+  const size_t index = (size_t)(valid > 0 ? token : 0) * n + (valid > 0 ? n0 : 0);
+  ResidualHeld held;
+  if constexpr (kResidual) held = residual_ask(y, index, valid > 0 ? n0 : 0, valid, vector_ok);
+  f32x4 part[8];
+#pragma unroll
+  for (int p = 0; p < 8; ++p) {
+    part[p] = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
+    if (p < ksplit && valid > 0) part[p] = *(const f32x4*)(partial + ((size_t)p * m + token) * width + n0);
+  }
+  f32x4 sum = part[0];
+#pragma unroll
+  for (int p = 1; p < 8; ++p) sum += part[p];
+  if constexpr (kResidual) {
+    float sq = valid > 0 ? residual_take(y, held, index, sum, valid, vector_ok) : 0.0f;
+#pragma unroll
+    for (int offset = 1; offset < 16; offset <<= 1) sq += __shfl_xor(sq, offset, kWave);
+    if (threadIdx.x % 16 == 0 && token < m) y.ss[(size_t)blockIdx.x * m + token] = sq;
+  } else {
+    if (valid > 0) store4(y, index, sum, valid, vector_ok);
+  }
+}
+
+// The same for a prepared operand (ScaledOut): a thread has the four lower and the four upper sums of a pair
+// unit (32 grid columns: 16 lower, then 16 upper rows; for EPI_STORE simply 2 x 4 columns 16 apart) of one
+// token, a block 16 tokens x 4 units.  The 16 lanes of a token add the parts of its sum of squares.
+template <int EPI>
+__global__ __launch_bounds__(256) void gemm_reduce_scaled_kernel(const float* __restrict__ partial, ScaledOut<EPI> y, int m, int n,
+                                                                 int k, int width, int ksplit) {
+  const int token = blockIdx.y * 16 + threadIdx.x / 16;
+  const int sub = threadIdx.x % 16;
+  const int unit = blockIdx.x * 4 + sub / 4, quad = sub % 4;
+  const int safe_token = token < m ? token : m - 1;
+  float squares = 0.0f;
+  for (int p0 = sub; p0 < y.parts; p0 += 64) {
+    float part[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int p = p0 + 16 * u;
+      part[u] = y.ss_parts[(size_t)(p < y.parts ? p : y.parts - 1) * m + safe_token];
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) squares += p0 + 16 * u < y.parts ? part[u] : 0.0f;
+  }
+  int pos = 0, page = -1;
+  if constexpr (EPI == EPI_ROPE) {
+    const int slot = y.rope.tok_slot[safe_token];
+    pos = y.rope.tok_pos[safe_token];
+    if (slot >= 0 && y.rope.k_pages) page = y.rope.block_table[(size_t)slot * y.rope.max_pages + pos / kPageTokens];
+  }
+  const int column = unit * 32 + quad * 4;  // the lower four; the upper four are 16 on
+  const bool inside = token < m && column + 16 < width;
+  f32x4 lo_part[8], hi_part[8];
+#pragma unroll
+  for (int p = 0; p < 8; ++p) {
+    lo_part[p] = hi_part[p] = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
+    if (p < ksplit && inside) {
+      const float* from = partial + ((size_t)p * m + token) * width + column;
+      lo_part[p] = *(const f32x4*)from;
+      hi_part[p] = *(const f32x4*)(from + 16);
+    }
+  }
+#pragma unroll
+  for (int offset = 1; offset < 16; offset <<= 1) squares += __shfl_xor(squares, offset, kWave);
+  const float scale = 1.0f / sqrtf(squares / (float)k + y.eps);
+  f32x4 lo_sum = lo_part[0], hi_sum = hi_part[0];
+#pragma unroll
+  for (int p = 1; p < 8; ++p) {
+    lo_sum += lo_part[p];
+    hi_sum += hi_part[p];
+  }
+  if (!inside) return;
+  float lo[4], hi[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    lo[e] = lo_sum[e] * scale;
+    hi[e] = hi_sum[e] * scale;
+  }
+  if constexpr (EPI == EPI_STORE) {
+    const bool vector_ok = (n % 4) == 0;
+    const int rest_lo = n - column, rest_hi = n - column - 16;
+    if (rest_lo > 0) store4(y.y, (size_t)token * n + column, (f32x4){lo[0], lo[1], lo[2], lo[3]}, rest_lo >= 4 ? 4 : rest_lo, vector_ok);
+    if (rest_hi > 0) store4(y.y, (size_t)token * n + column + 16, (f32x4){hi[0], hi[1], hi[2], hi[3]}, rest_hi >= 4 ? 4 : rest_hi, vector_ok);
+  } else if constexpr (EPI == EPI_SILU) {
+    if (unit * 16 < n / 2) epilogue_silu(y.y, token, n / 2, unit * 16 + quad * 4, lo, hi);
+  } else {
+    const int hd = y.rope.head_dim, per_head = hd / 32;
+    if (unit >= (y.rope.heads + 2 * y.rope.kv_heads) * per_head) return;
+    const int head = unit / per_head, f0 = (unit % per_head) * 16 + quad * 4;
+    epi_f32x4 c = {1.0f, 1.0f, 1.0f, 1.0f}, sn = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (head < y.rope.heads + y.rope.kv_heads) {
+      c = *(const epi_f32x4*)(y.rope.cos_table + (size_t)pos * (hd / 2) + f0);
+      sn = *(const epi_f32x4*)(y.rope.sin_table + (size_t)pos * (hd / 2) + f0);
+    }
+    epilogue_rope(y.rope, token, pos, head >= y.rope.heads ? page : -1, head, f0, lo, hi, c, sn);
+  }
+}
+
 template <int MT, int KSPLIT, typename OutT>
 void launch_skinny(const bf16_t* x, const bf16_t* w, OutT y, int m, int n, int k, hipStream_t stream) {
   const int strips = (n + 15) / 16;
@@ -594,17 +726,63 @@ void dispatch_skinny(const bf16_t* x, const bf16_t* w, OutT y, int m, int n, int
   else dispatch_skinny_split<4, OutT>(x, w, y, m, n, k, split, stream);
 }
 
-// `columns`: the weight rows the grid covers (n, or the rows of all pair units)
-template <int BM, int BN, int BK, typename OutT>
-void launch_tiled(const bf16_t* x, const bf16_t* w, OutT y, int m, int n, int k, int columns, hipStream_t stream) {
-  const int col_blocks = (columns + BN - 1) / BN, row_blocks = (m + BM - 1) / BM;
-  constexpr int lds_bytes = kTileStages * (BM + BN) * BK * 2;
+#ifndef NNIS_DEEP_RING_BLOCKS
+#define NNIS_DEEP_RING_BLOCKS 256
+#endif
+constexpr int kDeepRingBlocks = NNIS_DEEP_RING_BLOCKS;  // grids up to this many blocks take the ring of 6 stages
+
+// Scratch for the parts of a K that is cut among blocks (the caller's; nothing is allocated here)
+struct Workspace {
+  float* floats;
+  size_t bytes;
+};
+
+// Parts of K for a tiled product of `tiles` tiles: a power of two up to 8, as long as the chip still has
+// compute units without a block, a part keeps at least 4 steps of 64, and the parts fit the workspace.
+int tiled_ksplit(int tiles, int m, int width, int k, size_t workspace_bytes) {
+  const int steps = (k + 63) / 64;
+  int ksplit = 1;
+  while (ksplit < 8 && tiles * ksplit * 2 <= 256 && steps / (ksplit * 2) >= 4) ksplit *= 2;
+  while (ksplit > 1 && (size_t)ksplit * m * width * sizeof(float) > workspace_bytes) ksplit /= 2;
+  return ksplit;
+}
+
+// `columns`: the weight rows the grid covers (n, or the rows of all pair units).  Returns the parts of a
+// row's sum of squares that a residual epilogue wrote.
+template <int BM, int BN, int BK, int NS, typename OutT>
+int launch_tiled_staged(const bf16_t* x, const bf16_t* w, OutT y, int m, int n, int k, int col_blocks, int row_blocks, int ksplit,
+                        Workspace ws, hipStream_t stream) {
+  constexpr int lds_bytes = NS * (BM + BN) * BK * 2;
   // beyond 64 KB a kernel has to be told once; a refusal shows as the launch's failure
-  static const hipError_t allowed = hipFuncSetAttribute((const void*)gemm_tiled_kernel<BM, BN, BK, OutT>,
+  static const hipError_t allowed = hipFuncSetAttribute((const void*)gemm_tiled_kernel<BM, BN, BK, NS, OutT>,
                                                         hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
   (void)allowed;
-  hipLaunchKernelGGL((gemm_tiled_kernel<BM, BN, BK, OutT>), dim3((unsigned)col_blocks * row_blocks), dim3(256), lds_bytes,
-                     stream, x, w, y, m, n, k, col_blocks);
+  hipLaunchKernelGGL((gemm_tiled_kernel<BM, BN, BK, NS, OutT>), dim3((unsigned)col_blocks * row_blocks * ksplit), dim3(256),
+                     lds_bytes, stream, x, w, y, m, n, k, col_blocks, ksplit, ws.floats);
+  if (ksplit > 1) {
+    constexpr int EPI = scaled_epilogue<OutT>::value;
+    if constexpr (EPI >= 0) {
+      hipLaunchKernelGGL((gemm_reduce_scaled_kernel<EPI>), dim3((col_blocks * BN + 127) / 128, (m + 15) / 16), dim3(256), 0, stream,
+                         ws.floats, y, m, n, k, col_blocks * BN, ksplit);
+    } else {
+      hipLaunchKernelGGL((gemm_reduce_kernel<OutT>), dim3((n + 63) / 64, (m + 15) / 16), dim3(256), 0, stream, ws.floats, y, m, n,
+                         col_blocks * BN, ksplit);
+    }
+    return (n + 63) / 64;
+  }
+  return 2 * col_blocks;  // a part per wave column
+}
+
+// `columns`: the weight rows the grid covers (n, or the rows of all pair units).  Returns the parts of a
+// row's sum of squares that a residual epilogue wrote.
+template <int BM, int BN, int BK, typename OutT>
+int launch_tiled(const bf16_t* x, const bf16_t* w, OutT y, int m, int n, int k, int columns, Workspace ws, hipStream_t stream) {
+  const int col_blocks = (columns + BN - 1) / BN, row_blocks = (m + BM - 1) / BM;
+  const int ksplit = ws.floats ? tiled_ksplit(col_blocks * row_blocks, m, col_blocks * BN, k, ws.bytes) : 1;
+  const int steps_a_part = ((k + BK - 1) / BK + ksplit - 1) / ksplit;
+  if (col_blocks * row_blocks * ksplit <= kDeepRingBlocks && steps_a_part >= 6)
+    return launch_tiled_staged<BM, BN, BK, 6, OutT>(x, w, y, m, n, k, col_blocks, row_blocks, ksplit, ws, stream);
+  return launch_tiled_staged<BM, BN, BK, 3, OutT>(x, w, y, m, n, k, col_blocks, row_blocks, ksplit, ws, stream);
 }
 
 // 2: 64x128, 3: 64x64 -- the larger tile when it still gives every compute unit a block.  (A tile of
@@ -616,21 +794,20 @@ int pick_tile(int m, int columns, int tile_hint) {
   return tile;
 }
 
-// wave columns of the tiled kernel for these sizes: the parts of a row that a residual epilogue sums by itself
+// the most parts of a row's sum of squares that a residual epilogue of the tiled kernel writes for these sizes
 int tiled_parts(int m, int columns, int tile_hint) {
   const int width = pick_tile(m, columns, tile_hint) == 2 ? 128 : 64;
-  return 2 * ((columns + width - 1) / width);
+  return 2 * ((columns + width - 1) / width);  // with K in parts: one per 64 columns, which is no more
 }
 
-// returns the number of wave columns
+// returns the parts of a row's sum of squares written (a residual epilogue)
 template <typename OutT>
-int dispatch_tiled(const bf16_t* x, const bf16_t* w, OutT y, int m, int n, int k, int tile_hint, hipStream_t stream,
+int dispatch_tiled(const bf16_t* x, const bf16_t* w, OutT y, int m, int n, int k, int tile_hint, Workspace ws, hipStream_t stream,
                    int columns = 0) {
   if (columns <= 0) columns = n;
   const int tile = pick_tile(m, columns, tile_hint);
-  if (tile == 2) launch_tiled<64, 128, 64, OutT>(x, w, y, m, n, k, columns, stream);
-  else launch_tiled<64, 64, 64, OutT>(x, w, y, m, n, k, columns, stream);
-  return tiled_parts(m, columns, tile_hint);
+  if (tile == 2) return launch_tiled<64, 128, 64, OutT>(x, w, y, m, n, k, columns, ws, stream);
+  return launch_tiled<64, 64, 64, OutT>(x, w, y, m, n, k, columns, ws, stream);
 }
 
 // With few strips the waves of a block share a strip's K, so that each wave's
@@ -650,28 +827,49 @@ int skinny_split(int m, int n, int k, int split_hint) {
 
 }  // namespace
 
-// The kernel for few tokens (a wave owns 16 weight rows, no LDS for operands) against the tiled one: up to
-// 64 tokens always.  Beyond, up to kFewTokens, when the weights are small enough to be read once per tile of
-// 16 tokens and its blocks (strips x token tiles) are few enough; measured on products of 32 to 384 tokens
-// with weights of 576 x 576 to 3072 x 576 and 576 x 1536, in microseconds:
-//   few tokens: 3 + 0.004 * strips * tiles * K / 576      tiled: 2.6 + 0.0057 * K
+// The kernel for few tokens (a wave owns 16 weight rows, no LDS for operands) against the tiled one.
+//  * Up to 16 tokens: always.
+//  * Up to 64 tokens: unless the weights are large and wide.  A wave of the kernel for few tokens reads all
+//    the tokens' activations beside its 16 weight rows -- with 64 tokens four times the bytes of the weights --
+//    while a tile shares them among its waves through LDS; the tiled kernel needs enough column blocks to
+//    fill the chip, though.  Measured with 64 tokens and K = 2048, microseconds: 11264 rows 34 against 18
+//    tiled, 16384 rows 45 against 19, but 2560 rows 12.5 against 14.8.
+//  * Beyond, up to kFewTokens: when the weights are small enough to be read once per tile of 16 tokens and
+//    its blocks (strips x token tiles) are few enough; measured on products of 32 to 384 tokens with weights
+//    of 576 x 576 to 3072 x 576 and 576 x 1536, in microseconds:
+//      few tokens: 3 + 0.004 * strips * tiles * K / 576      tiled: 2.6 + 0.0057 * K
 bool nnis_gemm_takes_few_tokens(int m, int n, int k) {
-  if (m <= 64) return true;
-  if (m > kFewTokens || (size_t)n * k * sizeof(bf16_t) > kRereadWeightBytes) return false;
+  if (m <= 16) return true;
+  const bool large = (size_t)n * k * sizeof(bf16_t) > kRereadWeightBytes;
+  if (m <= 64) return !(large && (n + 63) / 64 >= 128);
+  if (m > kFewTokens || large) return false;
   const double strips = (n + 15) / 16, tiles = (m + 15) / 16;
   return 3.0 + 0.004 * strips * tiles * k / 576.0 <= 2.6 + 0.0057 * k;
 }
 
+// The same for a product whose tiled kernel may cut K into parts (it stores, or adds to the stream): large
+// weights with few columns still fill the chip then.  Measured with 64 tokens, microseconds: 2048 x 5632
+// 28 for few tokens against 15 in 8 parts, 2048 x 8192 39 against 18.
+static bool takes_few_tokens_with_parts(int m, int n, int k, bool workspace) {
+  if (m <= 16 || m > 64 || !workspace) return nnis_gemm_takes_few_tokens(m, n, k);
+  const bool large = (size_t)n * k * sizeof(bf16_t) > kRereadWeightBytes;
+  int parts = 1;
+  while (parts < 8 && ((k + 63) / 64) / (parts * 2) >= 4) parts *= 2;
+  return !(large && (n + 63) / 64 * parts >= 128);
+}
+
 int nnis_gemm_scaled_tiled(const bf16_t* scaled, const float* ss_parts, int parts, float eps, const bf16_t* w, int m, int n,
-                           int k, int epilogue, bf16_t* y, const RopeTarget& rope, int tile_hint, hipStream_t stream) {
+                           int k, int epilogue, bf16_t* y, const RopeTarget& rope, int tile_hint, float* workspace,
+                           size_t workspace_bytes, hipStream_t stream) {
+  const Workspace ws = {workspace, workspace ? workspace_bytes : 0};
   NNIS_REQUIRE((m + 63) / 64 <= 65535, "gemm_scaled: %d rows exceed the grid limit", m);
   if (epilogue == EPI_STORE) {
-    dispatch_tiled<ScaledOut<EPI_STORE>>(scaled, w, {y, ss_parts, parts, eps, rope}, m, n, k, tile_hint, stream);
+    dispatch_tiled<ScaledOut<EPI_STORE>>(scaled, w, {y, ss_parts, parts, eps, rope}, m, n, k, tile_hint, ws, stream);
   } else if (epilogue == EPI_SILU) {
-    dispatch_tiled<ScaledOut<EPI_SILU>>(scaled, w, {y, ss_parts, parts, eps, rope}, m, n, k, tile_hint, stream,
+    dispatch_tiled<ScaledOut<EPI_SILU>>(scaled, w, {y, ss_parts, parts, eps, rope}, m, n, k, tile_hint, ws, stream,
                                         32 * ((n / 2 + 15) / 16));
   } else {
-    dispatch_tiled<ScaledOut<EPI_ROPE>>(scaled, w, {y, ss_parts, parts, eps, rope}, m, n, k, tile_hint, stream, n);
+    dispatch_tiled<ScaledOut<EPI_ROPE>>(scaled, w, {y, ss_parts, parts, eps, rope}, m, n, k, tile_hint, ws, stream, n);
   }
   NNIS_LAUNCH_CHECK("gemm_scaled");
   return 0;
@@ -680,7 +878,7 @@ int nnis_gemm_scaled_tiled(const bf16_t* scaled, const float* ss_parts, int part
 // y_dtype: NNIS_BF16 or NNIS_F32.  Picks the skinny kernel for M <= 64.  split_hint: 0, or the number of
 // waves (1, 2, 4, 8) that share a strip's K in the skinny kernel, overriding the choice made here.
 extern "C" int nnis_gemm_bf16(const void* x, const void* w, void* y, int y_dtype, int m, int n, int k, int split_hint,
-                              void* stream_ptr) {
+                              float* workspace, size_t workspace_bytes, void* stream_ptr) {
   NNIS_REQUIRE(nnis_dtype_ok(y_dtype), "gemm_bf16: unknown output dtype %d", y_dtype);
   NNIS_REQUIRE(m >= 0 && n > 0 && k > 0, "gemm_bf16: bad sizes m=%d n=%d k=%d", m, n, k);
   NNIS_REQUIRE(k % 8 == 0, "gemm_bf16: K=%d is not a multiple of 8 (16-byte loads); use the ordered kernel", k);
@@ -690,7 +888,9 @@ extern "C" int nnis_gemm_bf16(const void* x, const void* w, void* y, int y_dtype
   hipStream_t stream = (hipStream_t)stream_ptr;
   const bf16_t* xp = (const bf16_t*)x;
   const bf16_t* wp = (const bf16_t*)w;
-  if (nnis_gemm_takes_few_tokens(m, n, k) && split_hint < 16) {  // a tile hint asks for the tiled kernel
+  NNIS_REQUIRE((uintptr_t)workspace % 16 == 0, "gemm_bf16: the workspace must be 16-byte aligned");
+  const Workspace ws = {workspace, workspace ? workspace_bytes : 0};
+  if (takes_few_tokens_with_parts(m, n, k, workspace != nullptr) && split_hint < 16) {  // a tile hint asks for the tiled kernel
     const int split = skinny_split(m, n, k, split_hint);
     if (y_dtype == NNIS_F32) dispatch_skinny<float*>(xp, wp, (float*)y, m, n, k, split, stream);
     else dispatch_skinny<bf16_t*>(xp, wp, (bf16_t*)y, m, n, k, split, stream);
@@ -698,8 +898,8 @@ extern "C" int nnis_gemm_bf16(const void* x, const void* w, void* y, int y_dtype
   } else {
     NNIS_REQUIRE((m + 63) / 64 <= 65535, "gemm_bf16: %d rows exceed the grid limit", m);
     const int tile_hint = split_hint >= 16 ? split_hint / 16 : 0;  // hints of 32 and 48 pick the tile: 64x128, 64x64
-    if (y_dtype == NNIS_F32) dispatch_tiled<float*>(xp, wp, (float*)y, m, n, k, tile_hint, stream);
-    else dispatch_tiled<bf16_t*>(xp, wp, (bf16_t*)y, m, n, k, tile_hint, stream);
+    if (y_dtype == NNIS_F32) dispatch_tiled<float*>(xp, wp, (float*)y, m, n, k, tile_hint, ws, stream);
+    else dispatch_tiled<bf16_t*>(xp, wp, (bf16_t*)y, m, n, k, tile_hint, ws, stream);
     NNIS_LAUNCH_CHECK("gemm_tiled");
   }
   return 0;
@@ -715,7 +915,8 @@ extern "C" int nnis_gemm_residual_parts(int m, int n) {
 }
 
 extern "C" int nnis_gemm_residual(const void* x, const void* w, float* resid, const void* gain, int gain_dtype, void* scaled,
-                                  float* ss, int ss_rows, int m, int n, int k, int* parts, void* stream_ptr) {
+                                  float* ss, int ss_rows, int m, int n, int k, int* parts, float* workspace,
+                                  size_t workspace_bytes, void* stream_ptr) {
   NNIS_REQUIRE(m >= 0 && n > 0 && k > 0, "gemm_residual: bad sizes m=%d n=%d k=%d", m, n, k);
   NNIS_REQUIRE(k % 8 == 0, "gemm_residual: K=%d is not a multiple of 8 (16-byte loads)", k);
   NNIS_REQUIRE(nnis_dtype_ok(gain_dtype), "gemm_residual: unknown norm weight dtype %d", gain_dtype);
@@ -726,7 +927,8 @@ extern "C" int nnis_gemm_residual(const void* x, const void* w, float* resid, co
   if (m == 0) return 0;
   hipStream_t stream = (hipStream_t)stream_ptr;
   ResidualOut out = {resid, gain, gain_dtype, (bf16_t*)scaled, ss};
-  const bool few = nnis_gemm_takes_few_tokens(m, n, k);
+  NNIS_REQUIRE((uintptr_t)workspace % 16 == 0, "gemm_residual: the workspace must be 16-byte aligned");
+  const bool few = takes_few_tokens_with_parts(m, n, k, workspace != nullptr);
   const int writes = few ? (n + 15) / 16 : tiled_parts(m, n, 0);
   NNIS_REQUIRE(writes <= ss_rows, "gemm_residual: ss has %d rows of %d tokens, %d are needed", ss_rows, m, writes);
   if (few) {
@@ -735,7 +937,8 @@ extern "C" int nnis_gemm_residual(const void* x, const void* w, float* resid, co
     NNIS_LAUNCH_CHECK("gemm_residual");
   } else {
     NNIS_REQUIRE((m + 63) / 64 <= 65535, "gemm_residual: %d rows exceed the grid limit", m);
-    *parts = dispatch_tiled<ResidualOut>((const bf16_t*)x, (const bf16_t*)w, out, m, n, k, 0, stream);
+    *parts = dispatch_tiled<ResidualOut>((const bf16_t*)x, (const bf16_t*)w, out, m, n, k, 0, {workspace, workspace ? workspace_bytes : 0},
+                                         stream);
     NNIS_LAUNCH_CHECK("gemm_residual");
   }
   return 0;

@@ -19,6 +19,7 @@ PAGE_TOKENS = 64
 _VOID = ctypes.c_void_p
 _INT = ctypes.c_int
 _FLT = ctypes.c_float
+_SIZE = ctypes.c_size_t
 _U64 = ctypes.c_uint64
 
 _CORE_SIGNATURES = {
@@ -30,13 +31,13 @@ _CORE_SIGNATURES = {
     "nnis_argmax": [_VOID, _VOID, _INT, _INT, _VOID, _VOID],
     "nnis_argmax_scratch": [_INT, _INT],
     "nnis_gemm_ordered": [_VOID, _INT, _VOID, _INT, _VOID, _INT, _INT, _INT, _INT, _VOID],
-    "nnis_gemm_bf16": [_VOID, _VOID, _VOID, _INT, _INT, _INT, _INT, _INT, _VOID],
+    "nnis_gemm_bf16": [_VOID, _VOID, _VOID, _INT, _INT, _INT, _INT, _INT, _VOID, _SIZE, _VOID],
     "nnis_gemm_fused": [_VOID, _VOID, _VOID, _VOID, _INT, _FLT, _VOID, _INT, _INT, _INT, _INT, _VOID, _VOID, _VOID, _INT,
                         _VOID, _VOID, _VOID, _VOID, _VOID, _INT, _INT, _INT, _INT, _INT, _VOID],
     "nnis_gemm_residual_parts": [_INT, _INT],
-    "nnis_gemm_residual": [_VOID, _VOID, _VOID, _VOID, _INT, _VOID, _VOID, _INT, _INT, _INT, _INT, _VOID, _VOID],
+    "nnis_gemm_residual": [_VOID, _VOID, _VOID, _VOID, _INT, _VOID, _VOID, _INT, _INT, _INT, _INT, _VOID, _VOID, _SIZE, _VOID],
     "nnis_gemm_scaled": [_VOID, _VOID, _INT, _FLT, _VOID, _INT, _INT, _INT, _INT, _VOID, _VOID, _VOID, _INT, _VOID, _VOID,
-                         _VOID, _VOID, _VOID, _INT, _INT, _INT, _INT, _INT, _VOID],
+                         _VOID, _VOID, _VOID, _INT, _INT, _INT, _INT, _INT, _VOID, _SIZE, _VOID],
     "nnis_sample": [_VOID, _VOID, _INT, _INT, _VOID, _VOID, _VOID, _VOID, _VOID, _VOID, _VOID],
 }
 _ATTN_SIGNATURES = {
@@ -275,6 +276,21 @@ def attention_rows(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_
 # dispatch by operand types
 # ---------------------------------------------------------------------------
 
+# Where the tiled product cuts K among blocks (few tiles, a long K) the parts meet in this scratch: 256 blocks
+# of 64 x 64 sums at most.  Kept per device; calls on one device share it, so they follow one another on one
+# stream.  It is made outside a graph capture only: a capture that finds none goes without the cut.
+GEMM_WORKSPACE_BYTES = 4 << 20
+_gemm_workspaces = {}
+
+
+def _gemm_workspace(device) -> Optional[torch.Tensor]:
+    key = (device.type, device.index)
+    held = _gemm_workspaces.get(key)
+    if held is None and not torch.cuda.is_current_stream_capturing():
+        held = _gemm_workspaces[key] = torch.empty(GEMM_WORKSPACE_BYTES // 4, dtype=torch.float32, device=device)
+    return held
+
+
 def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, split: int = 0) -> torch.Tensor:
     """out[M, N] = x[M, K] @ w[N, K]^T on the matrix cores: bfloat16 operands,
     32-bit accumulation, bfloat16 or float32 output.  K must be a multiple of 8."""
@@ -286,7 +302,9 @@ def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, split: int = 
     if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
         raise KernelError(f"gemm_bf16 takes bfloat16 operands, got {x.dtype} and {w.dtype}")
     lib = core()
-    _check(lib, lib.nnis_gemm_bf16(x.data_ptr(), w.data_ptr(), out.data_ptr(), _code(out), m, n, k, int(split), _stream()))
+    work = _gemm_workspace(x.device)
+    _check(lib, lib.nnis_gemm_bf16(x.data_ptr(), w.data_ptr(), out.data_ptr(), _code(out), m, n, k, int(split), _ptr(work),
+                                   GEMM_WORKSPACE_BYTES if work is not None else 0, _stream()))
     return out
 
 
@@ -376,9 +394,10 @@ def gemm_residual(x: torch.Tensor, w: torch.Tensor, resid: torch.Tensor, gain: t
         raise KernelError("gemm_residual: ss must be float32 [rows, m] (gemm_residual_parts(m, n) rows are always enough)")
     lib = core()
     parts = ctypes.c_int(0)
+    work = _gemm_workspace(x.device)
     _check(lib, lib.nnis_gemm_residual(x.data_ptr(), w.data_ptr(), resid.data_ptr(), gain.data_ptr(), _code(gain),
                                        scaled.data_ptr(), ss.data_ptr(), ss.numel() // m, m, n, k, ctypes.addressof(parts),
-                                       _stream()))
+                                       _ptr(work), GEMM_WORKSPACE_BYTES if work is not None else 0, _stream()))
     return parts.value
 
 
@@ -397,12 +416,14 @@ def gemm_scaled(scaled: torch.Tensor, ss: torch.Tensor, parts: int, eps: float, 
         raise KernelError("gemm_scaled: ss must be float32 [parts, m]")
     r = _check_epilogue("gemm_scaled", m, n, y, epilogue, rope)
     lib = core()
+    work = _gemm_workspace(scaled.device)
     bt = r.get("block_table")
     _check(lib, lib.nnis_gemm_scaled(
         scaled.data_ptr(), ss.data_ptr(), int(parts), float(eps), w.data_ptr(), m, n, k, int(epilogue), y.data_ptr(),
         _ptr(r.get("cos")), _ptr(r.get("sin")), r["cos"].shape[0] if r.get("cos") is not None else 0, _ptr(r.get("tok_slot")),
         _ptr(r.get("tok_pos")), _ptr(r.get("k_pages")), _ptr(r.get("v_pages")), _ptr(bt), bt.shape[1] if bt is not None else 0,
-        r.get("heads", 0), r.get("kv_heads", 0), r.get("head_dim", 0), int(split), _stream()))
+        r.get("heads", 0), r.get("kv_heads", 0), r.get("head_dim", 0), int(split), _ptr(work),
+        GEMM_WORKSPACE_BYTES if work is not None else 0, _stream()))
     return y
 
 

@@ -83,7 +83,8 @@ def test_gemm_ordered(m, n, k, x_dtype, w_dtype, y_dtype):
 
 
 @pytest.mark.parametrize("m", [1, 8, 16, 17, 40, 64, 65, 130, 300])
-@pytest.mark.parametrize("n, k", [(576, 576), (960, 576), (1000, 96), (70, 176), (3072, 64), (64, 1536), (17, 8), (200, 1096)])
+@pytest.mark.parametrize("n, k", [(576, 576), (960, 576), (1000, 96), (70, 176), (3072, 64), (64, 1536), (17, 8), (200, 1096),
+                                  (2050, 2312)])  # the last: large weights, few columns -- K is cut among blocks beyond 16 tokens
 @pytest.mark.parametrize("y_dtype", ["bfloat16", "float32"])
 def test_gemm_bf16_on_the_matrix_cores(m, n, k, y_dtype):
     """Skinny (M <= 64) and tiled kernels at sizes with tails in every
@@ -284,7 +285,7 @@ def test_gemm_tiled_over_many_blocks(hint):
 
 
 @pytest.mark.parametrize("m", [1, 8, 19, 64, 67, 100, 300])
-@pytest.mark.parametrize("n, k", [(576, 576), (100, 72), (2048, 1536), (48, 8), (64, 176), (3072, 576)])
+@pytest.mark.parametrize("n, k", [(576, 576), (100, 72), (2048, 1536), (48, 8), (64, 176), (3072, 576), (2080, 2304)])
 @pytest.mark.parametrize("gain_dtype", ["bfloat16", "float32"])
 def test_residual_projection_prepares_the_norm(m, n, k, gain_dtype):
     """resid += x . w^T in place; scaled = bfloat16(resid * gain); the parts of
