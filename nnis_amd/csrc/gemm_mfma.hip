@@ -313,9 +313,12 @@ extern __shared__ __align__(16) char tile_lds[];  // NS stages of BM + BN rows o
 #ifndef NNIS_TILE_GROUP_ROWS
 #define NNIS_TILE_GROUP_ROWS 512
 #endif
-// NS stages: 3 where a compute unit runs several blocks; 6 where the grid leaves it one block at most, and
-// the loads in flight are all that hides the memory's latency (64 tokens x 11264 x 2048: 20.9 us with 3, 19.7 with 6)
-template <int BM, int BN, int BK, int NS, typename OutT>
+// NS stages: 3 where a compute unit runs several blocks; 6 where the grid leaves it one block at most and K is
+// long, so that the loads in flight are all that hides the memory's latency (64 tokens x 11264 x 2048: 20.9 us
+// with 3, 19.7 with 6; a K of 9 steps in 256 blocks took 13.4 us with 6 against 11.7)
+// SPLIT: K is cut into ksplit parts, a block leaves its part's sums in `partial` and gemm_reduce_kernel does the
+// rest (a variant of its own, so that the other has no branch around the loads that prepare its epilogue).
+template <int BM, int BN, int BK, int NS, bool SPLIT, typename OutT>
 __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                                                          OutT y, int m, int n, int k, int col_blocks, int ksplit,
                                                          float* __restrict__ partial) {
@@ -422,7 +425,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
   // epilogue, and what the rotation needs of each token
   __shared__ float row_scale[EPI >= 0 ? 4 : 1][EPI >= 0 ? BM : 1];  // each wave's share of a row's sum of squares
   int tok_pos[TM], tok_page[TM];
-  if constexpr (EPI >= 0) if (ksplit == 1) {  // (with K in parts the reduce kernel does this)
+  if constexpr (EPI >= 0 && !SPLIT) {  // (with K in parts the reduce kernel does this)
     // lane = row, wave w takes the parts w, w + 4, ..: eight loads at a time, none waiting for another
     static_assert(BM == 64, "a lane per row of the tile");
     const int token = row0 + lane < m ? row0 + lane : m - 1;
@@ -454,7 +457,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
   constexpr bool kResidual = std::is_same<OutT, ResidualOut>::value;
   constexpr bool kAskEarly = kResidual && TM * TN <= 8;
   ResidualHeld held[kAskEarly ? TM : 1][kAskEarly ? TN : 1];
-  if constexpr (kAskEarly) if (ksplit == 1) {
+  if constexpr (kAskEarly && !SPLIT) {
     const bool vector_ok = (n % 4) == 0;
 #pragma unroll
     for (int i = 0; i < TM; ++i)
@@ -502,7 +505,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
 
   // A part of K: the sums go to `partial` [part][token][grid column] as they are; gemm_reduce_kernel adds the
   // parts and does what would follow here.
-  if (ksplit > 1) {
+  if constexpr (SPLIT) {
     const size_t width = (size_t)col_blocks * BN;
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
@@ -513,7 +516,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
         *(f32x4*)(partial + ((size_t)part * m + token) * width + col0 + wave_n * WN + j * 16 + g * 4) = acc[i][j];
     }
     return;
-  }
+  } else {
   // a prepared operand's norm: 1 / sqrt(mean of squares + eps) of a tile row
   auto scale_of = [&](int row) -> float {
     if constexpr (EPI >= 0) {
@@ -581,6 +584,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
     }
   }
   }
+  }  // !SPLIT
 }
 
 // The parts of K that gemm_tiled_kernel left in `partial` [ksplit][m][width], added in the order of the parts,
@@ -747,19 +751,23 @@ int tiled_ksplit(int tiles, int m, int width, int k, size_t workspace_bytes) {
   return ksplit;
 }
 
-// `columns`: the weight rows the grid covers (n, or the rows of all pair units).  Returns the parts of a
-// row's sum of squares that a residual epilogue wrote.
+template <int BM, int BN, int BK, int NS, bool SPLIT, typename OutT>
+void launch_tiled_kernel(const bf16_t* x, const bf16_t* w, OutT y, int m, int n, int k, int col_blocks, int row_blocks, int ksplit,
+                         Workspace ws, hipStream_t stream) {
+  constexpr int lds_bytes = NS * (BM + BN) * BK * 2;
+  // beyond 64 KB a kernel has to be told once; a refusal shows as the launch's failure
+  static const hipError_t allowed = hipFuncSetAttribute((const void*)gemm_tiled_kernel<BM, BN, BK, NS, SPLIT, OutT>,
+                                                        hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+  (void)allowed;
+  hipLaunchKernelGGL((gemm_tiled_kernel<BM, BN, BK, NS, SPLIT, OutT>), dim3((unsigned)col_blocks * row_blocks * ksplit), dim3(256),
+                     lds_bytes, stream, x, w, y, m, n, k, col_blocks, ksplit, ws.floats);
+}
+
 template <int BM, int BN, int BK, int NS, typename OutT>
 int launch_tiled_staged(const bf16_t* x, const bf16_t* w, OutT y, int m, int n, int k, int col_blocks, int row_blocks, int ksplit,
                         Workspace ws, hipStream_t stream) {
-  constexpr int lds_bytes = NS * (BM + BN) * BK * 2;
-  // beyond 64 KB a kernel has to be told once; a refusal shows as the launch's failure
-  static const hipError_t allowed = hipFuncSetAttribute((const void*)gemm_tiled_kernel<BM, BN, BK, NS, OutT>,
-                                                        hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-  (void)allowed;
-  hipLaunchKernelGGL((gemm_tiled_kernel<BM, BN, BK, NS, OutT>), dim3((unsigned)col_blocks * row_blocks * ksplit), dim3(256),
-                     lds_bytes, stream, x, w, y, m, n, k, col_blocks, ksplit, ws.floats);
   if (ksplit > 1) {
+    launch_tiled_kernel<BM, BN, BK, NS, true, OutT>(x, w, y, m, n, k, col_blocks, row_blocks, ksplit, ws, stream);
     constexpr int EPI = scaled_epilogue<OutT>::value;
     if constexpr (EPI >= 0) {
       hipLaunchKernelGGL((gemm_reduce_scaled_kernel<EPI>), dim3((col_blocks * BN + 127) / 128, (m + 15) / 16), dim3(256), 0, stream,
@@ -770,6 +778,7 @@ int launch_tiled_staged(const bf16_t* x, const bf16_t* w, OutT y, int m, int n, 
     }
     return (n + 63) / 64;
   }
+  launch_tiled_kernel<BM, BN, BK, NS, false, OutT>(x, w, y, m, n, k, col_blocks, row_blocks, 1, ws, stream);
   return 2 * col_blocks;  // a part per wave column
 }
 
@@ -780,7 +789,7 @@ int launch_tiled(const bf16_t* x, const bf16_t* w, OutT y, int m, int n, int k, 
   const int col_blocks = (columns + BN - 1) / BN, row_blocks = (m + BM - 1) / BM;
   const int ksplit = ws.floats ? tiled_ksplit(col_blocks * row_blocks, m, col_blocks * BN, k, ws.bytes) : 1;
   const int steps_a_part = ((k + BK - 1) / BK + ksplit - 1) / ksplit;
-  if (col_blocks * row_blocks * ksplit <= kDeepRingBlocks && steps_a_part >= 6)
+  if (col_blocks * row_blocks * ksplit <= kDeepRingBlocks && steps_a_part >= 16)
     return launch_tiled_staged<BM, BN, BK, 6, OutT>(x, w, y, m, n, k, col_blocks, row_blocks, ksplit, ws, stream);
   return launch_tiled_staged<BM, BN, BK, 3, OutT>(x, w, y, m, n, k, col_blocks, row_blocks, ksplit, ws, stream);
 }
