@@ -601,15 +601,18 @@ __global__ __launch_bounds__(256) void gemm_reduce_kernel(const float* __restric
   const size_t index = (size_t)(valid > 0 ? token : 0) * n + (valid > 0 ? n0 : 0);
   ResidualHeld held;
   if constexpr (kResidual) held = residual_ask(y, index, valid > 0 ? n0 : 0, valid, vector_ok);
+  // every load is asked for before any is used: none stands behind a branch (a part beyond the last reads
+  // the last again and counts as zero)
   f32x4 part[8];
+  const float* from = partial + (size_t)(valid > 0 ? token : 0) * width + (valid > 0 ? n0 : 0);
 #pragma unroll
-  for (int p = 0; p < 8; ++p) {
-    part[p] = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
-    if (p < ksplit && valid > 0) part[p] = *(const f32x4*)(partial + ((size_t)p * m + token) * width + n0);
-  }
+  for (int p = 0; p < 8; ++p) part[p] = *(const f32x4*)(from + (size_t)(p < ksplit ? p : ksplit - 1) * m * width);
   f32x4 sum = part[0];
 #pragma unroll
-  for (int p = 1; p < 8; ++p) sum += part[p];
+  for (int p = 1; p < 8; ++p) {
+    const float keep = p < ksplit ? 1.0f : 0.0f;
+    sum += part[p] * keep;
+  }
   if constexpr (kResidual) {
     float sq = valid > 0 ? residual_take(y, held, index, sum, valid, vector_ok) : 0.0f;
 #pragma unroll
@@ -649,15 +652,15 @@ __global__ __launch_bounds__(256) void gemm_reduce_scaled_kernel(const float* __
   }
   const int column = unit * 32 + quad * 4;  // the lower four; the upper four are 16 on
   const bool inside = token < m && column + 16 < width;
+  // every load is asked for before any is used: none stands behind a branch (a part beyond the last reads
+  // the last again and counts as zero)
   f32x4 lo_part[8], hi_part[8];
+  const float* from = partial + (size_t)safe_token * width + (inside ? column : 0);
 #pragma unroll
   for (int p = 0; p < 8; ++p) {
-    lo_part[p] = hi_part[p] = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
-    if (p < ksplit && inside) {
-      const float* from = partial + ((size_t)p * m + token) * width + column;
-      lo_part[p] = *(const f32x4*)from;
-      hi_part[p] = *(const f32x4*)(from + 16);
-    }
+    const float* at = from + (size_t)(p < ksplit ? p : ksplit - 1) * m * width;
+    lo_part[p] = *(const f32x4*)at;
+    hi_part[p] = *(const f32x4*)(at + 16);
   }
 #pragma unroll
   for (int offset = 1; offset < 16; offset <<= 1) squares += __shfl_xor(squares, offset, kWave);
@@ -665,8 +668,9 @@ __global__ __launch_bounds__(256) void gemm_reduce_scaled_kernel(const float* __
   f32x4 lo_sum = lo_part[0], hi_sum = hi_part[0];
 #pragma unroll
   for (int p = 1; p < 8; ++p) {
-    lo_sum += lo_part[p];
-    hi_sum += hi_part[p];
+    const float keep = p < ksplit ? 1.0f : 0.0f;
+    lo_sum += lo_part[p] * keep;
+    hi_sum += hi_part[p] * keep;
   }
   if (!inside) return;
   float lo[4], hi[4];
