@@ -18,6 +18,12 @@
 #ifndef NNIS_HEAD_DIM
 #error "compile with -DNNIS_HEAD_DIM=<head size>"
 #endif
+#ifndef NNIS_PREFILL_RING_NARROW
+#define NNIS_PREFILL_RING_NARROW 3
+#endif
+#ifndef NNIS_PREFILL_RING_WIDE
+#define NNIS_PREFILL_RING_WIDE 2
+#endif
 
 thread_local char g_nnis_error[512] = {0};
 extern "C" const char* nnis_last_error() { return g_nnis_error; }
@@ -384,8 +390,13 @@ __device__ __forceinline__ bool merge_waves(AttnState<C>& st, float* merge, int 
 // Runs the pages first, first + stride, ... (`mine` of them) of a sequence through the
 // softmax state, each as two blocks of 32 keys one after the other (so both halves of a
 // value line are used while it is near).  RING blocks' operands are in flight at a time:
-// a block's place is asked for again as soon as it has been worked on, so a wave with
-// up to RING blocks waits for memory once.  Blocks that start beyond `last_key` are left out.
+// a block's place is asked for again as soon as it has been worked on.  A load behind a
+// branch makes the compiler take it for not issued when it counts what may still be in
+// flight at a use, and every block then waits for all the loads asked for after its own.  So
+// a run of at least two rounds goes through a loop of whole rounds whose every block has a
+// successor RING on, RING blocks in one straight line with nothing behind a branch; what is
+// left of it, and a short run, take the loop that looks at every block.  Blocks that start
+// beyond `last_key` are left out.
 template <int C, int RING>
 __device__ __forceinline__ void attend_run(AttnState<C>& st, const QFrag (&q)[C], const MfmaArgs& a, const int* pages,
                                            int kv_head, int first, int stride, int mine, int last_key,
@@ -411,20 +422,40 @@ __device__ __forceinline__ void attend_run(AttnState<C>& st, const QFrag (&q)[C]
     const int page = run.page(n & 63);
     load_block(into, k_base + page * k_page_stride, v_base + page * v_page_stride, b & 1, r, g);
   };
+  auto work = [&](const BlockFrags& f, int b) {
+    attend_block<C>(st, q, f, (first + (b >> 1) * stride) * kPageTokens + (b & 1) * 32, lo, hi, a.scale_log2, g);
+  };
+  int b0 = 0;
+  if (blocks >= 2 * RING) {
 #pragma unroll
-  for (int i = 0; i < RING; ++i)
-    if (i < blocks) ask(ring[i], i);
-  for (int b0 = 0; b0 < blocks; b0 += RING) {
+    for (int i = 0; i < RING; ++i) ask(ring[i], i);
+    for (; b0 + 2 * RING <= blocks; b0 += RING) {
+#pragma unroll
+      for (int i = 0; i < RING; ++i) {
+        work(ring[i], b0 + i);
+        ask(ring[i], b0 + i + RING);
+      }
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < RING; ++i)
+      if (i < blocks) ask(ring[i], i);
+  }
+  for (; b0 < blocks; b0 += RING) {
 #pragma unroll
     for (int i = 0; i < RING; ++i) {
       const int b = b0 + i;
       if (b < blocks) {
-        attend_block<C>(st, q, ring[i], (first + (b >> 1) * stride) * kPageTokens + (b & 1) * 32, lo, hi, a.scale_log2, g);
+        work(ring[i], b);
         if (b + RING < blocks) ask(ring[i], b + RING);
       }
     }
   }
 }
+
+// key blocks a prefilling wave has in flight: as many as its registers hold beside C columns' states
+template <int C>
+constexpr int kPrefillRing = HD > 64 ? 2 : (C <= 2 ? NNIS_PREFILL_RING_NARROW : NNIS_PREFILL_RING_WIDE);
 
 // ---- prefill: a wave = (query tile, kv head, chunk of GH query heads); C = QT * GH column tiles --------
 // An item is a (tile, kv head, chunk of heads); the tiles come longest first, and item i = tile i / per_tile.
@@ -497,7 +528,7 @@ __global__ __launch_bounds__(64 * kBlockWaves) void attention_prefill_kernel(Mfm
     if (last >= 0) {
       const int first_page = first / kPageTokens, page_count = last / kPageTokens + 1 - first_page;
       const int mine = page_count > wave ? (page_count - wave + waves - 1) / waves : 0;  // pages of this wave
-      attend_run<C, (HD > 64 ? 2 : (C <= 2 ? 4 : (C == 3 ? 3 : 2)))>(st, q, a, pages, kv_head, first_page + wave, waves, mine, last, lo, hi, lane);
+      attend_run<C, kPrefillRing<C>>(st, q, a, pages, kv_head, first_page + wave, waves, mine, last, lo, hi, lane);
     }
     if (!merge_waves<C>(st, merge, wave, waves, lane)) return;
 #pragma unroll
@@ -695,69 +726,87 @@ __global__ __launch_bounds__(64 * kKeysWaves) void attention_decode_keys_kernel(
       load_keys_page(into, k_base + page * k_page_stride, v_base + page * v_page_stride, lane);
     };
     bf16_t* mine_stage = &stage[wave][0][0];
+    // page n of this wave's run, whose operands are in f, through the softmax state
+    auto work = [&](const KeysPage& f, int n) {
+      const int key0 = (first + n * stride) * kPageTokens;
+      // scores of this lane's head for keys key0 + 4 blk + (0..3): two chains of products, added
+      f32x4 s0 = {0.0f, 0.0f, 0.0f, 0.0f}, s1 = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-    for (int i = 0; i < kKeysRing; ++i)
-      if (i < mine) ask(ring[i], i);
-    for (int n0 = 0; n0 < mine; n0 += kKeysRing) {
+      for (int c = 0; c < HD / 8; ++c) {
+        s0 = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(low4(f.k[c]), low4(q[c]), s0, 0, 0, 0);
+        s1 = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(high4(f.k[c]), high4(q[c]), s1, 0, 0, 0);
+      }
+      f32x4 s = s0 + s1;
+      const bool inside = key0 >= first_key && key0 + kPageTokens - 1 <= pos;  // every key of the page is read
+      float top = -INFINITY;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int key = key0 + 4 * blk + e;
+        s[e] = (inside || (key >= first_key && key <= pos)) ? s[e] * a.scale_log2 : -INFINITY;
+        top = fmaxf(top, s[e]);
+      }
+      if (__any(top > reference + kLazyRise)) {  // also the first page, whose reference is -inf
+        float moved = fmaxf(reference, top);
+#pragma unroll
+        for (int offset = 4; offset < kWave; offset <<= 1) moved = fmaxf(moved, __shfl_xor(moved, offset, kWave));
+        // the lanes 16 g + r with r < 4 hold head r in both layouts: the outputs are scaled by the same factor
+        const float shrink = reference == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(reference - moved);
+        sum *= shrink;
+#pragma unroll
+        for (int t = 0; t < kTilesD; ++t) st.o[0][t] = st.o[0][t] * shrink;
+        reference = moved;
+      }
+      const float base = reference == -INFINITY ? 0.0f : reference;
+      bf16x4 p;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float w = __builtin_amdgcn_exp2f(s[e] - base);
+        sum += w;
+        p[e] = (__bf16)w;
+      }
+      // through LDS into the columns operand: column = head, 8 consecutive keys a lane
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();  // the reads of the page before are done
+      *(bf16x4*)(mine_stage + j * kStageRow + 4 * blk) = p;
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        bf16x8 columns = *(const bf16x8*)(mine_stage + (r < 4 ? r : 0) * kStageRow + 32 * h + 8 * g);
+        if (r >= 4) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) columns[e] = (__bf16)0.0f;
+        }
+#pragma unroll
+        for (int t = 0; t < kTilesD; ++t)
+          st.o[0][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.v[h][t], columns, st.o[0][t], 0, 0, 0);
+      }
+    };
+    // A run of at least two rounds: whole rounds whose every page has a successor kKeysRing on, in one straight
+    // line with no load behind a branch (see attend_run); the rest, and a short run, page by page.
+    int n0 = 0;
+    if (mine >= 2 * kKeysRing) {
+#pragma unroll
+      for (int i = 0; i < kKeysRing; ++i) ask(ring[i], i);
+      for (; n0 + 2 * kKeysRing <= mine; n0 += kKeysRing) {
+#pragma unroll
+        for (int i = 0; i < kKeysRing; ++i) {
+          work(ring[i], n0 + i);
+          ask(ring[i], n0 + i + kKeysRing);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < kKeysRing; ++i)
+        if (i < mine) ask(ring[i], i);
+    }
+    for (; n0 < mine; n0 += kKeysRing) {
 #pragma unroll
       for (int i = 0; i < kKeysRing; ++i) {
         const int n = n0 + i;
         if (n >= mine) continue;
-        const KeysPage& f = ring[i];
-        const int key0 = (first + n * stride) * kPageTokens;
-        // scores of this lane's head for keys key0 + 4 blk + (0..3): two chains of products, added
-        f32x4 s0 = {0.0f, 0.0f, 0.0f, 0.0f}, s1 = {0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-        for (int c = 0; c < HD / 8; ++c) {
-          s0 = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(low4(f.k[c]), low4(q[c]), s0, 0, 0, 0);
-          s1 = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(high4(f.k[c]), high4(q[c]), s1, 0, 0, 0);
-        }
-        f32x4 s = s0 + s1;
-        const bool inside = key0 >= first_key && key0 + kPageTokens - 1 <= pos;  // every key of the page is read
-        float top = -INFINITY;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int key = key0 + 4 * blk + e;
-          s[e] = (inside || (key >= first_key && key <= pos)) ? s[e] * a.scale_log2 : -INFINITY;
-          top = fmaxf(top, s[e]);
-        }
-        if (__any(top > reference + kLazyRise)) {  // also the first page, whose reference is -inf
-          float moved = fmaxf(reference, top);
-#pragma unroll
-          for (int offset = 4; offset < kWave; offset <<= 1) moved = fmaxf(moved, __shfl_xor(moved, offset, kWave));
-          // the lanes 16 g + r with r < 4 hold head r in both layouts: the outputs are scaled by the same factor
-          const float shrink = reference == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(reference - moved);
-          sum *= shrink;
-#pragma unroll
-          for (int t = 0; t < kTilesD; ++t) st.o[0][t] = st.o[0][t] * shrink;
-          reference = moved;
-        }
-        const float base = reference == -INFINITY ? 0.0f : reference;
-        bf16x4 p;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const float w = __builtin_amdgcn_exp2f(s[e] - base);
-          sum += w;
-          p[e] = (__bf16)w;
-        }
-        // through LDS into the columns operand: column = head, 8 consecutive keys a lane
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();  // the reads of the page before are done
-        *(bf16x4*)(mine_stage + j * kStageRow + 4 * blk) = p;
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-#pragma unroll
-        for (int h = 0; h < 2; ++h) {
-          bf16x8 columns = *(const bf16x8*)(mine_stage + (r < 4 ? r : 0) * kStageRow + 32 * h + 8 * g);
-          if (r >= 4) {
-#pragma unroll
-            for (int e = 0; e < 8; ++e) columns[e] = (__bf16)0.0f;
-          }
-#pragma unroll
-          for (int t = 0; t < kTilesD; ++t)
-            st.o[0][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.v[h][t], columns, st.o[0][t], 0, 0, 0);
-        }
+        work(ring[i], n);
         if (n + kKeysRing < mine) ask(ring[i], n + kKeysRing);
       }
     }
