@@ -7,7 +7,9 @@ key/value heads of 64, inner 1536, vocabulary 49152, tied head) with random
 weights, a batch of 8 sequences whose prompts are uniform in [128, 2048]
 tokens, in a cache sized for 8192 tokens per sequence.  A step is one decode
 step of the whole batch through the generation path: token ids in, the model,
-greedy selection on the device, token ids out.  ``value`` is decoded tokens per
+greedy selection on the device, token ids out to the host (which reads a
+step's tokens while the next step, fed from the device, is under way, as the
+generation loop does for greedy batches).  ``value`` is decoded tokens per
 second.  The prefill figure is one step over a 2,048-token prompt.  Peaks used
 for the fractions are the published MI355X ones: HBM 8 TB/s; dense matrix
 rate 2.5 PFLOP/s for bfloat16, 157.3 TFLOP/s for 32-bit.
@@ -100,18 +102,37 @@ def main() -> int:
             slots = [engine.start_sequence() for _ in range(batch)]
             prompts = [rng.integers(0, SHAPE["vocab"], size=n).tolist() for n in lengths]
             logits = engine.step([StepEntry(s, p, None) for s, p in zip(slots, prompts)])
-            tokens = selector.select(logits, slots, [None] * batch)
+            greedy = [None] * batch
+            if engine.use_graphs:
+                # as the generation loop runs greedy batches: a step ahead of the host, which reads a
+                # step's tokens while the next step, fed from the device, is under way
+                pending = selector.select_start(logits, slots, greedy)
 
-            def one_step(tokens):
-                logits = engine.step_view([StepEntry(s, [t], None) for s, t in zip(slots, tokens)])
-                return selector.select(logits, slots, [None] * batch)
+                def one_step(pending):
+                    following = selector.select_start(engine.step_from_device(slots, pending.device), slots, greedy)
+                    pending.result()
+                    return following
+
+                def finish(pending):
+                    pending.result()
+            else:
+                pending = selector.select(logits, slots, greedy)
+
+                def one_step(tokens):
+                    logits = engine.step_view([StepEntry(s, [t], None) for s, t in zip(slots, tokens)])
+                    return selector.select(logits, slots, greedy)
+
+                def finish(tokens):
+                    pass
 
             for _ in range(warmup):
-                tokens = one_step(tokens)
+                pending = one_step(pending)
+            finish(pending)
             sync()
             start = time.perf_counter()
             for _ in range(steps):
-                tokens = one_step(tokens)
+                pending = one_step(pending)
+            finish(pending)
             sync()
             seconds = time.perf_counter() - start
             context_tokens = sum(engine.length(s) for s in slots) - batch * steps / 2.0  # mean over the timed steps

@@ -113,6 +113,27 @@ def generate(engine, requests: Sequence[GenerationRequest], selector=None, max_b
         raise CacheFull("the cache has no free slot")
 
     step = getattr(engine, "step_view", engine.step)  # the logits are read at once: no copy needed
+    # An engine that takes a step's ids from the device, with a selector that leaves them there, runs a step
+    # ahead of the host (below); any other pair runs step by step.
+    ahead = getattr(engine, "use_graphs", False) and hasattr(engine, "step_from_device") and hasattr(selector, "select_start")
+
+    def take(index: int, token: int, slot_of) -> bool:
+        """Books one emitted token; returns whether the sequence goes on."""
+        result = results[index]
+        result.tokens.append(token)
+        callback = requests[index].on_token
+        keep_going = True if callback is None else callback(index, token) is not False
+        if token in stops[index]:
+            result.finish_reason = "stop"
+        elif len(result.tokens) >= requests[index].max_new_tokens:
+            result.finish_reason = "length"
+        elif not keep_going:
+            result.finish_reason = "callback"
+        if result.finish_reason:
+            engine.end_sequence(slot_of.pop(index))  # the slot is free for the next batch at once
+            return False
+        return True
+
     for batch in plan_batches(needs, engine.free_pages(), limit):
         live = list(batch)
         slot_of = {}
@@ -123,27 +144,56 @@ def generate(engine, requests: Sequence[GenerationRequest], selector=None, max_b
             feed = {index: list(requests[index].prompt) for index in live}
             while live:
                 logits = step([StepEntry(slot_of[i], feed[i], None) for i in live])
+                pending = None
+                if ahead:
+                    pending = selector.select_start(logits, [slot_of[i] for i in live], [requests[i].sampling for i in live])
+                if pending is not None:
+                    _run_ahead(engine, selector, requests, results, slot_of, live, pending, take)
+                    live = []
+                    break
                 tokens = selector.select(logits, [slot_of[i] for i in live], [requests[i].sampling for i in live])
                 still = []
                 for index, token in zip(live, tokens):
-                    token = int(token)
-                    result = results[index]
-                    result.tokens.append(token)
-                    callback = requests[index].on_token
-                    keep_going = True if callback is None else callback(index, token) is not False
-                    if token in stops[index]:
-                        result.finish_reason = "stop"
-                    elif len(result.tokens) >= requests[index].max_new_tokens:
-                        result.finish_reason = "length"
-                    elif not keep_going:
-                        result.finish_reason = "callback"
-                    if result.finish_reason:
-                        engine.end_sequence(slot_of.pop(index))  # the slot is free for the next batch at once
-                    else:
-                        feed[index] = [token]
+                    if take(index, int(token), slot_of):
+                        feed[index] = [int(token)]
                         still.append(index)
                 live = still
         finally:
             for slot in slot_of.values():  # only on an error: give everything back
                 engine.end_sequence(slot)
     return results
+
+
+def _run_ahead(engine, selector, requests, results, slot_of, rows, pending, take) -> None:
+    """The decode steps of a batch of greedy sequences, a step ahead of the
+    host.  ``pending``: the selection of the tokens that come next, asked for
+    but not read; its row j belongs to request ``rows[j]``.  Before the host
+    reads them, the step that feeds them back is put on the stream, with their
+    ids taken from the device, for every sequence that cannot end with that
+    token by its length (``max_new_tokens``).  A sequence that the token then
+    ends (a stop token, a callback) has run one step for nothing: that step's
+    row is dropped, the sequence's slot is given back as always, and nothing it
+    computed is read (the rows of a step do not depend on one another).  The
+    tokens, their order and the reasons for ending are those of the loop that
+    runs step by step."""
+    import torch
+
+    while rows:
+        # who goes on whatever the token is: those whose count stays below their limit with it
+        onward = [j for j, index in enumerate(rows)
+                  if index in slot_of and len(results[index].tokens) + 1 < requests[index].max_new_tokens]
+        following = None
+        if onward:
+            ids = pending.device
+            if len(onward) != len(rows):
+                ids = ids.index_select(0, torch.tensor(onward, dtype=torch.long, device=ids.device)).contiguous()
+            logits = engine.step_from_device([slot_of[rows[j]] for j in onward], ids)
+            following = selector.select_start(logits, [slot_of[rows[j]] for j in onward], [None] * len(onward))
+        tokens = pending.result()
+        for j, index in enumerate(rows):
+            if index in slot_of:  # (else ended by an earlier token: this row ran for nothing)
+                take(index, int(tokens[j]), slot_of)
+        if following is None:
+            return
+        rows = [rows[j] for j in onward]  # the rows of `following`; those that ended are skipped when it is read
+        pending = following

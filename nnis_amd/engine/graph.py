@@ -80,11 +80,13 @@ class DecodeGraph:
             if collecting:
                 gc.enable()
 
-    def run(self, ids: Sequence[int], slots: Sequence[int], positions: Sequence[int]) -> torch.Tensor:
-        count = len(ids)
+    def run(self, ids, slots: Sequence[int], positions: Sequence[int], ids_device: torch.Tensor = None) -> torch.Tensor:
+        """``ids``: the step's token ids, or None when they are on the device
+        already: then row j's id is ``ids_device[j]`` (int32)."""
+        count = len(slots)
         self.copied.synchronize()  # the previous copy has left the pinned buffer
         host = self.host.numpy()
-        host[0, :count] = ids
+        host[0, :count] = ids if ids is not None else -1
         host[1, :count] = slots
         host[2, :count] = positions
         host[0, count:] = -1
@@ -92,6 +94,8 @@ class DecodeGraph:
         host[2, count:] = 0
         self.meta.copy_(self.host, non_blocking=True)
         self.copied.record()
+        if ids is None:
+            self.meta[0, :count].copy_(ids_device[:count], non_blocking=True)
         self.graph.replay()
         return self.logits
 

@@ -156,18 +156,32 @@ class Engine:
         )
         return self.model.forward(dev[0], ctx, self.cache, dev[6], self.rt)
 
-    def _decode_step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+    def step_from_device(self, slots: Sequence[int], ids_device: torch.Tensor) -> torch.Tensor:
+        """A step of one token per sequence whose ids are on the device already
+        (int32, row j for ``slots[j]``; what a selection kernel wrote, so in
+        range by construction): the host has not read them yet, and the step is
+        on its way before it does.  Logits at every row, as ``step_view``
+        returns them.  Only where decode steps are replayed from graphs
+        (``use_graphs``)."""
+        if not self.use_graphs:
+            raise InvalidInput("steps from device ids need an engine that replays decode steps from graphs")
+        if ids_device.dtype != torch.int32 or ids_device.dim() != 1 or ids_device.numel() < len(slots) or not slots:
+            raise InvalidInput("step_from_device: one int32 id per slot is needed")
+        self._borrowed = False
+        return self._decode_step([StepEntry(s, (), None) for s in slots], ids_device)
+
+    def _decode_step(self, entries: Sequence[StepEntry], ids_device: Optional[torch.Tensor] = None) -> torch.Tensor:
         """A step of single tokens, replayed from a captured graph: the same
         checks as any step, without the arrays a prompt needs.  The rows
         returned view the graph's output buffer: read them before the next step."""
         from .graph import DecodeGraphs
 
         slots = [e.slot for e in entries]
-        ids = [int(e.tokens[0]) for e in entries]
+        ids = [int(e.tokens[0]) for e in entries] if ids_device is None else None
         if len(set(slots)) != len(slots):
             twice = next(s for s in slots if slots.count(s) > 1)
             raise InvalidInput(f"slot {twice} appears twice in one step")
-        if min(ids) < 0 or max(ids) >= self.vocab_size:
+        if ids is not None and (min(ids) < 0 or max(ids) >= self.vocab_size):
             bad = next(t for t in ids if not 0 <= t < self.vocab_size)
             raise InvalidInput(f"token id {bad} is out of range for vocabulary {self.vocab_size}")
         for entry in entries:
@@ -180,7 +194,7 @@ class Engine:
             self._graphs = DecodeGraphs(self)
         plan = self.model.decode_plan(len(entries), max(pos0) + 1, self.rt)
         graph = self._graphs.get(len(entries), plan)
-        logits = graph.run(ids, slots, pos0)
+        logits = graph.run(ids, slots, pos0, ids_device)
         wanted = [i for i, e in enumerate(entries) if e.want is None or len(e.want) > 0]
         if len(wanted) == len(entries):
             self._borrowed = True

@@ -17,6 +17,20 @@ from .params import SamplingParams
 RNG_REGION = "sampler.rng"
 
 
+class PendingTokens:
+    """Tokens that a selection kernel has been asked for: on the device at
+    once (in stream order), on the host when ``result`` returns."""
+
+    def __init__(self, device: torch.Tensor, host: torch.Tensor, event):
+        self.device = device
+        self._host = host
+        self._event = event
+
+    def result(self) -> List[int]:
+        self._event.synchronize()
+        return self._host.tolist()
+
+
 class DeviceSelector:
     def __init__(self, engine):
         self.engine = engine
@@ -29,6 +43,8 @@ class DeviceSelector:
         self._weights = None
         self._picked = None       # int32 on the device, reused from step to step
         self._picked_host = None  # its pinned twin: the copy back needs no staging
+        self._pairs = [None, None]  # (device, pinned host, event) of select_start, used in turn
+        self._turn = 0
 
     def _to_host(self, picked: torch.Tensor, rows: int) -> List[int]:
         if self._picked_host is None or self._picked_host.numel() < rows:
@@ -37,6 +53,29 @@ class DeviceSelector:
         host.copy_(picked[:rows], non_blocking=True)
         torch.cuda.current_stream().synchronize()
         return host.tolist()
+
+    def select_start(self, logits: torch.Tensor, slots: Sequence[int], params: Sequence[Optional[SamplingParams]]):
+        """Greedy rows only: the selection is put on the stream and the copy of
+        the tokens to the host behind it; nothing waits.  Returns a
+        ``PendingTokens`` -- the tokens on the device (for a step that starts
+        before the host has read them) and ``result()``, which waits for the
+        copy -- or None when a row samples (then ``select`` is the way).  Two
+        results may be outstanding at a time: the third call reuses the first's
+        buffers."""
+        if any(p is not None for p in params):
+            return None
+        rows = logits.shape[0]
+        self._turn ^= 1
+        pair = self._pairs[self._turn]
+        if pair is None or pair[0].numel() < rows:
+            size = max(rows, 64)
+            pair = self._pairs[self._turn] = (torch.empty(size, dtype=torch.int32, device=self.rt.device),
+                                              torch.empty(size, dtype=torch.int32, pin_memory=True), torch.cuda.Event())
+        device, host, event = pair
+        self.rt.ops.argmax(logits, device[:rows])
+        host[:rows].copy_(device[:rows], non_blocking=True)
+        event.record()
+        return PendingTokens(device[:rows], host[:rows], event)
 
     def start(self, slot: int, params: Optional[SamplingParams]) -> None:
         """Called when a sequence starts: seeds its generator."""

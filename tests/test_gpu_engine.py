@@ -121,6 +121,58 @@ def test_greedy_generation_through_the_entry_point(model_dirs, name):
             assert row[token].item() >= row.max().item() - 3e-2
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_running_a_step_ahead_changes_nothing(model_dirs, dtype):
+    """Greedy batches run a step ahead of the host (the next step takes its
+    ids from the device before the host has read them).  Tokens, their order
+    in the callbacks and the reasons for ending are those of the loop that runs
+    step by step: with stop tokens that are met on the way, limits of 1 and 2
+    tokens, a callback that ends a sequence, more requests than a batch takes,
+    and every slot given back."""
+    from nnis_amd.engine.generate import GenerationRequest, generate
+    from nnis_amd.sampling.device import DeviceSelector
+
+    engine = _engine(model_dirs, "A", dtype, max_tokens=8 * 64)
+    assert engine.use_graphs
+    config, seed = TINY_CONFIGS["A"]
+    rng = np.random.default_rng(7)
+    prompts = [rng.integers(0, config["vocab_size"], size=n).tolist() for n in (5, 11, 17, 1, 30, 2, 9)]
+    limits = [9, 1, 2, 12, 7, 9, 5]
+
+    class StepByStep:  # a selector without select_start: the loop waits for every token
+        def __init__(self, inner):
+            self.start, self.select = inner.start, inner.select
+
+    def run(selector, stops, stop_after):
+        seen = []
+
+        def watch(index, token):
+            seen.append((index, token))
+            return not (index == 3 and sum(1 for i, _ in seen if i == 3) >= stop_after)
+
+        requests = [GenerationRequest(p, max_new_tokens=n, stop_token_ids=stops[i], on_token=watch)
+                    for i, (p, n) in enumerate(zip(prompts, limits))]
+        free = engine.free_slots()
+        out = generate(engine, requests, selector=selector, max_batch=3)
+        assert engine.free_slots() == free and engine.free_pages() == 8
+        return [(r.tokens, r.finish_reason) for r in out], seen
+
+    no_stops = [[] for _ in prompts]
+    plain_run, _ = run(StepByStep(DeviceSelector(engine)), no_stops, 99)
+    # stop tokens that the sequences do meet: the 4th token of request 0, the 2nd of request 4, the last of 5
+    stops = [[] for _ in prompts]
+    stops[0], stops[4], stops[5] = [plain_run[0][0][3]], [plain_run[4][0][1]], [plain_run[5][0][-1]]
+    want, want_seen = run(StepByStep(DeviceSelector(engine)), stops, 4)
+    got, got_seen = run(DeviceSelector(engine), stops, 4)
+    assert got == want
+    assert sorted(got_seen) == sorted(want_seen)
+    for index in range(len(prompts)):  # each request's tokens reach the callback in their order
+        assert [t for i, t in got_seen if i == index] == got[index][0]
+    reasons = [reason for _, reason in got]
+    assert reasons[0] == "stop" and reasons[1] == "length" and reasons[3] == "callback" and len(got[3][0]) == 4
+    assert len(got[0][0]) <= 4 and len(got[4][0]) <= 2
+
+
 def test_command_line(model_dirs):
     plain = P.PlainLlama(model_dirs["B"])
     prompt = [3, 141, 59, 26, 535]
