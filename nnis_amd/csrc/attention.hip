@@ -1016,11 +1016,13 @@ extern "C" int nnis_attention_decode_max_waves(int heads, int kv_heads) {
 // With splits > 1 the call needs scratch memory: `partial`, float32 of at least tokens * heads * splits *
 // (head_dim + 4), contents of no matter.  Two calls that run at the same time must not share it.
 // kind: 0 picks the kernel (keys on lanes for groups of up to 4 heads, else heads in columns); 1 and 2 ask
-// for columns or keys on lanes and fail where that kernel does not take the sizes.
+// for columns or keys on lanes and fail where that kernel does not take the sizes.  combine: 0 leaves the
+// runs in `partial` ([tokens, heads, splits, head_dim + 4]: outputs, reference, sum) and writes no output: the
+// projection that follows, or nnis_attention_combine, adds them up.
 extern "C" int nnis_attention_decode_bf16(const void* q, void* out, const void* k_pages, const void* v_pages,
                                           const int* block_table, int max_pages, const int* tok_slot, const int* tok_pos,
                                           int tokens, int heads, int kv_heads, int head_dim, int window, float scale,
-                                          int splits, int waves, float* partial, int kind, void* stream) {
+                                          int splits, int waves, float* partial, int kind, int combine, void* stream) {
   MfmaArgs a;
   if (fill_common(a, q, out, k_pages, v_pages, block_table, max_pages, heads, kv_heads, head_dim, window, scale)) return 1;
   NNIS_REQUIRE(splits >= 1 && splits <= 65535, "attention: bad number of splits %d", splits);
@@ -1048,7 +1050,7 @@ extern "C" int nnis_attention_decode_bf16(const void* q, void* out, const void* 
     if (kind == 2 || (kind == 0 && keys_fit)) {
       hipLaunchKernelGGL(attention_decode_keys_kernel, grid, dim3(kWave * waves), lds, s, a, waves);
       NNIS_LAUNCH_CHECK("attention_decode");
-      if (splits > 1) {
+      if (splits > 1 && combine) {
         hipLaunchKernelGGL(attention_combine_kernel, dim3(tokens, heads), dim3(HD < 64 ? 64 : (HD > 256 ? 256 : HD)), 0, s,
                            partial, (bf16_t*)out, tok_slot, heads, splits);
         NNIS_LAUNCH_CHECK("attention_combine");
@@ -1061,11 +1063,24 @@ extern "C" int nnis_attention_decode_bf16(const void* q, void* out, const void* 
   else if (tiles == 2) hipLaunchKernelGGL((attention_decode_kernel<(kMaxColumns >= 2 ? 2 : 1)>), grid, dim3(kWave * waves), lds, s, a, waves);
   else hipLaunchKernelGGL((attention_decode_kernel<kMaxColumns>), grid, dim3(kWave * waves), lds, s, a, waves);  // 3 or 4 tiles
   NNIS_LAUNCH_CHECK("attention_decode");
-  if (splits > 1) {
+  if (splits > 1 && combine) {
     hipLaunchKernelGGL(attention_combine_kernel, dim3(tokens, heads), dim3(HD < 64 ? 64 : (HD > 256 ? 256 : HD)), 0, s, partial,
                        (bf16_t*)out, tok_slot, heads, splits);
     NNIS_LAUNCH_CHECK("attention_combine");
   }
+  return 0;
+}
+
+// The sum over the key runs that a call with combine = 0 left in `partial`, for a consumer that does not
+// take the runs as they are.
+extern "C" int nnis_attention_combine(const float* partial, void* out, const int* tok_slot, int tokens, int heads, int head_dim,
+                                      int splits, void* stream) {
+  NNIS_REQUIRE(head_dim == HD, "attention: this module is compiled for head_dim %d, got %d", HD, head_dim);
+  NNIS_REQUIRE(partial && out && tok_slot && splits >= 1 && heads > 0, "attention_combine: missing operand");
+  if (tokens <= 0) return 0;
+  hipLaunchKernelGGL(attention_combine_kernel, dim3(tokens, heads), dim3(HD < 64 ? 64 : (HD > 256 ? 256 : HD)), 0,
+                     (hipStream_t)stream, partial, (bf16_t*)out, tok_slot, heads, splits);
+  NNIS_LAUNCH_CHECK("attention_combine");
   return 0;
 }
 #else
@@ -1076,8 +1091,11 @@ extern "C" int nnis_attention_prefill_bf16(const void*, void*, const void*, cons
   return nnis_fail("attention: the matrix-core kernels need a head size in steps of 16; this module has %d", NNIS_HEAD_DIM);
 }
 extern "C" int nnis_attention_decode_max_waves(int, int) { return 1; }
+extern "C" int nnis_attention_combine(const float*, void*, const int*, int, int, int, int, void*) {
+  return nnis_fail("attention: the matrix-core kernels need a head size in steps of 16; this module has %d", NNIS_HEAD_DIM);
+}
 extern "C" int nnis_attention_decode_bf16(const void*, void*, const void*, const void*, const int*, int, const int*, const int*,
-                                          int, int, int, int, int, float, int, int, float*, int, void*) {
+                                          int, int, int, int, int, float, int, int, float*, int, int, void*) {
   return nnis_fail("attention: the matrix-core kernels need a head size in steps of 16; this module has %d", NNIS_HEAD_DIM);
 }
 #endif

@@ -184,10 +184,82 @@ __device__ __forceinline__ int paired_weight_row(const RopeTarget& rope, int blo
   return (unit / per_head) * rope.head_dim + (unit % per_head) * 16 + rr + (upper ? rope.head_dim / 2 : 0);
 }
 
-template <int MT, int KSPLIT, typename OutT>
+// The activations as the decode attention leaves them when it cuts a sequence's keys into runs: per (token,
+// head, run) head_dim outputs, the run's softmax reference (a power of two's exponent) and its sum, in rows of
+// head_dim + 4 floats.  x[token][head * head_dim + d] = sum_s O_s[d] 2^(m_s - M) / sum_s l_s 2^(m_s - M), M the
+// largest m_s: what attention_combine_kernel computes, term by term in the same order.
+struct RunsIn {
+  const float* partial;  // [tokens, heads, runs, head_dim + 4]
+  const int* tok_slot;   // [tokens]; a negative slot is a padding row: its activations count as zeros
+  int runs, heads, head_dim;
+};
+constexpr int kMostRuns = 8;
+
+extern __shared__ __align__(16) char skinny_lds[];  // RUNS: the block's activations, [16 * MT][k + 8] bfloat16
+
+// The block's threads make the activations of `tokens` tokens from token0 on, [tokens][k] in rows of x_row
+// elements at x_tile, from up to MOST runs.  A thread's loads of two items (4 channels of a token each) are
+// asked for together, before any is used; a run beyond the last reads the last again and counts for nothing.
+template <int MOST>
+__device__ __forceinline__ void make_activations(const RunsIn& runs, bf16_t* x_tile, int x_row, int token0, int tokens, int k) {
+  typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+  typedef __attribute__((ext_vector_type(2))) float f32x2;
+  const int groups = k / 4, row_floats = runs.head_dim + 4;
+  const int items = tokens > 0 ? tokens * groups : 0;
+  constexpr int kTogether = 2;
+  for (int first = threadIdx.x; first < items; first += kTogether * blockDim.x) {
+    f32x2 state[kTogether][MOST];  // a run's reference and sum
+    f32x4 out[kTogether][MOST];
+    bool live[kTogether];
+#pragma unroll
+    for (int i = 0; i < kTogether; ++i) {
+      int item = first + i * blockDim.x;
+      item = item < items ? item : items - 1;  // (the last again: stored twice, the same)
+      const int local = item / groups, channel = (item % groups) * 4;
+      const int token = token0 + local;
+      live[i] = runs.tok_slot[token] >= 0;
+      const int head = channel / runs.head_dim, d = channel % runs.head_dim;
+      const float* base = runs.partial + ((size_t)token * runs.heads + head) * runs.runs * row_floats;
+#pragma unroll
+      for (int s = 0; s < MOST; ++s) {
+        const float* p = base + (size_t)(s < runs.runs ? s : runs.runs - 1) * row_floats;
+        state[i][s] = *(const f32x2*)(p + runs.head_dim);
+        out[i][s] = *(const f32x4*)(p + d);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < kTogether; ++i) {
+      int item = first + i * blockDim.x;
+      item = item < items ? item : items - 1;
+      const int local = item / groups, channel = (item % groups) * 4;
+      float top = -INFINITY;
+#pragma unroll
+      for (int s = 0; s < MOST; ++s) top = s < runs.runs ? fmaxf(top, state[i][s][0]) : top;
+      f32x4 num = {0.0f, 0.0f, 0.0f, 0.0f};
+      float den = 0.0f;
+#pragma unroll
+      for (int s = 0; s < MOST; ++s) {
+        if (s < runs.runs) {
+          const float weight = state[i][s][0] == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(state[i][s][0] - top);
+          num += out[i][s] * weight;
+          den += state[i][s][1] * weight;
+        }
+      }
+      bf16x4 made;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) made[e] = live[i] ? (__bf16)(num[e] / den) : (__bf16)0.0f;  // a padding row: zeros
+      *(bf16x4*)(x_tile + (size_t)local * x_row + channel) = made;
+    }
+  }
+}
+
+// RUNS: x is not read but made, by the block for its 16 * MT tokens, from `runs` into LDS (every block makes
+// the same few KB again: cheaper than a kernel of its own between the attention and this projection).
+template <int MT, int KSPLIT, bool RUNS, typename OutT>
 __global__ __launch_bounds__(KSPLIT > 4 ? 64 * KSPLIT : 256) void gemm_skinny_kernel(const bf16_t* __restrict__ x,
                                                                                    const bf16_t* __restrict__ w,
-                                                                                   OutT y, int m, int n, int k, int tiles) {
+                                                                                   OutT y, int m, int n, int k, int tiles,
+                                                                                   RunsIn runs) {
   constexpr int kWaves = KSPLIT > 4 ? KSPLIT : 4;
   constexpr int kStrips = kWaves / KSPLIT;  // strips of 16 weight rows per block
   constexpr int DEPTH = MT <= 2 ? 4 : 2;
@@ -197,6 +269,7 @@ __global__ __launch_bounds__(KSPLIT > 4 ? 64 * KSPLIT : 256) void gemm_skinny_ke
   nnis_deal_tiles(blockIdx.x, tiles, strip_block, tile);
   const int strip = strip_block * kStrips + wave / KSPLIT;
   const int token0 = tile * 16 * MT;  // this block's tokens: token0 + (0 .. 16 * MT - 1)
+  const int x_row = k + 8;  // elements of a row of the activations in LDS: 16 rows apart fall into different banks
   const int part = wave % KSPLIT;
   const int r = lane % 16, g = lane / 16;
   const int strips = (n + 15) / 16;
@@ -222,39 +295,69 @@ __global__ __launch_bounds__(KSPLIT > 4 ? 64 * KSPLIT : 256) void gemm_skinny_ke
     }
   }
 
-  if (active) {
-    int w_row = strip * 16 + r;
-    w_row = w_row < n ? w_row : n - 1;  // rows beyond N read a valid row and are not stored
-    const bf16_t* w_ptr = w + (size_t)w_row * k;
-    const bf16_t* x_ptr[MT];
+  int w_row = strip * 16 + r;
+  w_row = w_row < n ? w_row : n - 1;  // rows beyond N read a valid row and are not stored
+  const bf16_t* w_ptr = w + (size_t)(active ? w_row : 0) * k;
+  const int chunks = (k + 63) / 64;
+  // a round: DEPTH steps of 64 k of this wave (base, base + KSPLIT, ..): their weights ...
+  auto ask_weights = [&](int base, bf16x8 (&wa)[DEPTH], bf16x8 (&wb)[DEPTH]) {
 #pragma unroll
-    for (int t = 0; t < MT; ++t) {
-      int token = token0 + t * 16 + r;
-      token = token < m ? token : m - 1;
-      x_ptr[t] = x + (size_t)token * k;
+    for (int d = 0; d < DEPTH; ++d) {
+      const int ka = (base + d * KSPLIT) * 64 + g * 16, kb = ka + 8;
+      wa[d] = ka + 8 <= k ? load_chunk(w_ptr + ka) : zero_chunk();  // zeros also for steps beyond the last
+      wb[d] = kb + 8 <= k ? load_chunk(w_ptr + kb) : zero_chunk();
     }
-    const int chunks = (k + 63) / 64;
-    for (int base = part; base < chunks; base += KSPLIT * DEPTH) {
-      bf16x8 wa[DEPTH], wb[DEPTH], xa[DEPTH][MT], xb[DEPTH][MT];
+  };
+  const bf16_t* x_ptr[MT];
 #pragma unroll
-      for (int d = 0; d < DEPTH; ++d) {
-        const int ka = (base + d * KSPLIT) * 64 + g * 16, kb = ka + 8;
-        const bool in_a = ka + 8 <= k, in_b = kb + 8 <= k;  // false also for steps beyond the last
-        wa[d] = in_a ? load_chunk(w_ptr + ka) : zero_chunk();
-        wb[d] = in_b ? load_chunk(w_ptr + kb) : zero_chunk();
+  for (int t = 0; t < MT; ++t) {
+    int token = token0 + t * 16 + r;
+    token = token < m ? token : m - 1;
+    x_ptr[t] = x + (size_t)token * k;
+  }
+  auto load_x = [&](int t, int kk) -> bf16x8 {
+    if constexpr (RUNS) return *(const bf16x8*)(skinny_lds + ((size_t)(t * 16 + r) * x_row + kk) * sizeof(bf16_t));
+    else return load_chunk(x_ptr[t] + kk);
+  };
+  // ... and their activations and products
+  auto multiply = [&](int base, const bf16x8 (&wa)[DEPTH], const bf16x8 (&wb)[DEPTH]) {
+    bf16x8 xa[DEPTH][MT], xb[DEPTH][MT];
 #pragma unroll
-        for (int t = 0; t < MT; ++t) {
-          xa[d][t] = in_a ? load_chunk(x_ptr[t] + ka) : zero_chunk();
-          xb[d][t] = in_b ? load_chunk(x_ptr[t] + kb) : zero_chunk();
-        }
+    for (int d = 0; d < DEPTH; ++d) {
+      const int ka = (base + d * KSPLIT) * 64 + g * 16, kb = ka + 8;
+#pragma unroll
+      for (int t = 0; t < MT; ++t) {
+        xa[d][t] = ka + 8 <= k ? load_x(t, ka) : zero_chunk();
+        xb[d][t] = kb + 8 <= k ? load_x(t, kb) : zero_chunk();
       }
+    }
 #pragma unroll
-      for (int d = 0; d < DEPTH; ++d)
+    for (int d = 0; d < DEPTH; ++d)
 #pragma unroll
-        for (int t = 0; t < MT; ++t) {
-          acc[t] = mfma(wa[d], xa[d][t], acc[t]);
-          acc[t] = mfma(wb[d], xb[d][t], acc[t]);
-        }
+      for (int t = 0; t < MT; ++t) {
+        acc[t] = mfma(wa[d], xa[d][t], acc[t]);
+        acc[t] = mfma(wb[d], xb[d][t], acc[t]);
+      }
+  };
+  int base = part;
+  if constexpr (RUNS) {
+    // the first round's weights are asked for before the block makes its activations: the two latencies overlap
+    bf16x8 wa[DEPTH], wb[DEPTH];
+    if (active && base < chunks) ask_weights(base, wa, wb);
+    const int tokens_here = min(16 * MT, m - token0);  // rows beyond them are never multiplied into a stored result
+    if (runs.runs <= 4) make_activations<4>(runs, (bf16_t*)skinny_lds, x_row, token0, tokens_here, k);
+    else make_activations<kMostRuns>(runs, (bf16_t*)skinny_lds, x_row, token0, tokens_here, k);
+    __syncthreads();
+    if (active && base < chunks) {
+      multiply(base, wa, wb);
+      base += KSPLIT * DEPTH;
+    }
+  }
+  if (active) {
+    for (; base < chunks; base += KSPLIT * DEPTH) {
+      bf16x8 wa[DEPTH], wb[DEPTH];
+      ask_weights(base, wa, wb);
+      multiply(base, wa, wb);
     }
   }
 
@@ -699,23 +802,35 @@ __global__ __launch_bounds__(256) void gemm_reduce_scaled_kernel(const float* __
   }
 }
 
+// bytes of LDS the kernel's RUNS variant needs for the activations of 16 * MT tokens
+size_t skinny_runs_lds(int token_tiles, int k) { return (size_t)16 * token_tiles * (k + 8) * sizeof(bf16_t); }
+
+// runs: null, or where the activations come from instead of x (the variant of the kernel that makes them)
 template <int MT, int KSPLIT, typename OutT>
-void launch_skinny(const bf16_t* x, const bf16_t* w, OutT y, int m, int n, int k, hipStream_t stream) {
+void launch_skinny(const bf16_t* x, const bf16_t* w, OutT y, int m, int n, int k, const RunsIn* runs, hipStream_t stream) {
   const int strips = (n + 15) / 16;
   const int waves = KSPLIT > 4 ? KSPLIT : 4;
   const int per_block = waves / KSPLIT;
   const int strip_blocks = (strips + per_block - 1) / per_block;
   const int tiles = (m + 16 * MT - 1) / (16 * MT);
-  hipLaunchKernelGGL((gemm_skinny_kernel<MT, KSPLIT, OutT>), dim3(tiles == 1 ? strip_blocks : (strip_blocks + 7) / 8 * 8 * tiles),
-                     dim3(64 * waves), 0, stream, x, w, y, m, n, k, tiles);
+  const dim3 grid(tiles == 1 ? strip_blocks : (strip_blocks + 7) / 8 * 8 * tiles), block(64 * waves);
+  if constexpr (std::is_same<OutT, ResidualOut>::value) {
+    if (runs) {
+      hipLaunchKernelGGL((gemm_skinny_kernel<MT, KSPLIT, true, OutT>), grid, block, skinny_runs_lds(MT, k), stream, x, w, y, m, n, k,
+                         tiles, *runs);
+      return;
+    }
+  }
+  hipLaunchKernelGGL((gemm_skinny_kernel<MT, KSPLIT, false, OutT>), grid, block, 0, stream, x, w, y, m, n, k, tiles, RunsIn{});
 }
 
 template <int MT, typename OutT>
-void dispatch_skinny_split(const bf16_t* x, const bf16_t* w, OutT y, int m, int n, int k, int split, hipStream_t stream) {
-  if (split == 8) launch_skinny<MT, 8, OutT>(x, w, y, m, n, k, stream);
-  else if (split == 4) launch_skinny<MT, 4, OutT>(x, w, y, m, n, k, stream);
-  else if (split == 2) launch_skinny<MT, 2, OutT>(x, w, y, m, n, k, stream);
-  else launch_skinny<MT, 1, OutT>(x, w, y, m, n, k, stream);
+void dispatch_skinny_split(const bf16_t* x, const bf16_t* w, OutT y, int m, int n, int k, int split, const RunsIn* runs,
+                           hipStream_t stream) {
+  if (split == 8) launch_skinny<MT, 8, OutT>(x, w, y, m, n, k, runs, stream);
+  else if (split == 4) launch_skinny<MT, 4, OutT>(x, w, y, m, n, k, runs, stream);
+  else if (split == 2) launch_skinny<MT, 2, OutT>(x, w, y, m, n, k, runs, stream);
+  else launch_skinny<MT, 1, OutT>(x, w, y, m, n, k, runs, stream);
 }
 
 // token tiles a wave of the skinny kernel takes: all of them (up to 4) when the weights are large and
@@ -726,12 +841,13 @@ int skinny_tiles_per_wave(int m, int n, int k) {
 }
 
 template <typename OutT>
-void dispatch_skinny(const bf16_t* x, const bf16_t* w, OutT y, int m, int n, int k, int split, hipStream_t stream) {
+void dispatch_skinny(const bf16_t* x, const bf16_t* w, OutT y, int m, int n, int k, int split, hipStream_t stream,
+                     const RunsIn* runs = nullptr) {
   const int tiles = skinny_tiles_per_wave(m, n, k);
-  if (tiles == 1) dispatch_skinny_split<1, OutT>(x, w, y, m, n, k, split, stream);
-  else if (tiles == 2) dispatch_skinny_split<2, OutT>(x, w, y, m, n, k, split, stream);
-  else if (tiles == 3) dispatch_skinny_split<3, OutT>(x, w, y, m, n, k, split, stream);
-  else dispatch_skinny_split<4, OutT>(x, w, y, m, n, k, split, stream);
+  if (tiles == 1) dispatch_skinny_split<1, OutT>(x, w, y, m, n, k, split, runs, stream);
+  else if (tiles == 2) dispatch_skinny_split<2, OutT>(x, w, y, m, n, k, split, runs, stream);
+  else if (tiles == 3) dispatch_skinny_split<3, OutT>(x, w, y, m, n, k, split, runs, stream);
+  else dispatch_skinny_split<4, OutT>(x, w, y, m, n, k, split, runs, stream);
 }
 
 #ifndef NNIS_DEEP_RING_BLOCKS
@@ -954,5 +1070,38 @@ extern "C" int nnis_gemm_residual(const void* x, const void* w, float* resid, co
                                          stream);
     NNIS_LAUNCH_CHECK("gemm_residual");
   }
+  return 0;
+}
+
+// Whether nnis_gemm_residual_runs takes these sizes: few tokens (the kernel whose blocks each make their
+// tokens' activations in LDS), 2 to 8 runs, activations of a block within 64 KB.
+extern "C" int nnis_gemm_residual_runs_fits(int m, int n, int heads, int head_dim, int runs) {
+  if (m <= 0 || m > 64 || n <= 0 || heads <= 0 || head_dim <= 0 || head_dim % 4 != 0) return 0;
+  const long long k = (long long)heads * head_dim;
+  if (k % 8 != 0 || k > (1 << 20)) return 0;
+  if (runs < 2 || runs > kMostRuns) return 0;
+  if (!nnis_gemm_takes_few_tokens(m, n, (int)k)) return 0;
+  return skinny_runs_lds(skinny_tiles_per_wave(m, n, (int)k), (int)k) <= 65536 ? 1 : 0;
+}
+
+// nnis_gemm_residual on activations that the decode attention left as runs of keys (`partial`: [m, heads,
+// runs, head_dim + 4] float32, see RunsIn): the sum over the runs is made inside the projection instead of by
+// a kernel between the two.  tok_slot [m]: rows with a negative slot count as zeros.
+extern "C" int nnis_gemm_residual_runs(const float* partial, int runs, int heads, int head_dim, const int* tok_slot, const void* w,
+                                       float* resid, const void* gain, int gain_dtype, void* scaled, float* ss, int ss_rows,
+                                       int m, int n, int* parts, void* stream_ptr) {
+  NNIS_REQUIRE(nnis_gemm_residual_runs_fits(m, n, heads, head_dim, runs),
+               "gemm_residual_runs: %d tokens x %d rows on %d heads of %d in %d runs are not taken", m, n, heads, head_dim, runs);
+  NNIS_REQUIRE(nnis_dtype_ok(gain_dtype), "gemm_residual_runs: unknown norm weight dtype %d", gain_dtype);
+  NNIS_REQUIRE(partial && tok_slot && w && resid && gain && scaled && ss && parts, "gemm_residual_runs: missing operand");
+  for (const void* p : {(const void*)partial, w, (const void*)resid, gain, (const void*)scaled})
+    NNIS_REQUIRE((uintptr_t)p % 16 == 0, "gemm_residual_runs: operands must be 16-byte aligned");
+  const int k = heads * head_dim;
+  *parts = (n + 15) / 16;
+  NNIS_REQUIRE(*parts <= ss_rows, "gemm_residual_runs: ss has %d rows of %d tokens, %d are needed", ss_rows, m, *parts);
+  const RunsIn in = {partial, tok_slot, runs, heads, head_dim};
+  ResidualOut out = {resid, gain, gain_dtype, (bf16_t*)scaled, ss};
+  dispatch_skinny<ResidualOut>(nullptr, (const bf16_t*)w, out, m, n, k, skinny_split(m, n, k, 0), (hipStream_t)stream_ptr, &in);
+  NNIS_LAUNCH_CHECK("gemm_residual_runs");
   return 0;
 }

@@ -6,6 +6,7 @@ runs hand-written device code; none has a host or library stand-in.
 from __future__ import annotations
 
 import ctypes
+import os
 from typing import Optional
 
 import torch
@@ -38,6 +39,9 @@ _CORE_SIGNATURES = {
     "nnis_gemm_residual": [_VOID, _VOID, _VOID, _VOID, _INT, _VOID, _VOID, _INT, _INT, _INT, _INT, _VOID, _VOID, _SIZE, _VOID],
     "nnis_gemm_scaled": [_VOID, _VOID, _INT, _FLT, _VOID, _INT, _INT, _INT, _INT, _VOID, _VOID, _VOID, _INT, _VOID, _VOID,
                          _VOID, _VOID, _VOID, _INT, _INT, _INT, _INT, _INT, _VOID, _SIZE, _VOID],
+    "nnis_gemm_residual_runs_fits": [_INT, _INT, _INT, _INT, _INT],
+    "nnis_gemm_residual_runs": [_VOID, _INT, _INT, _INT, _VOID, _VOID, _VOID, _VOID, _INT, _VOID, _VOID, _INT, _INT, _INT, _VOID,
+                                _VOID],
     "nnis_sample": [_VOID, _VOID, _INT, _INT, _VOID, _VOID, _VOID, _VOID, _VOID, _VOID, _VOID],
 }
 _ATTN_SIGNATURES = {
@@ -48,7 +52,8 @@ _ATTN_SIGNATURES = {
                                     _INT, _INT, _INT, _FLT, _INT, _INT, _VOID],
     "nnis_attention_prefill_max_waves": [_INT, _INT, _INT],
     "nnis_attention_decode_bf16": [_VOID, _VOID, _VOID, _VOID, _VOID, _INT, _VOID, _VOID, _INT, _INT, _INT, _INT, _INT, _FLT,
-                                   _INT, _INT, _VOID, _INT, _VOID],
+                                   _INT, _INT, _VOID, _INT, _INT, _VOID],
+    "nnis_attention_combine": [_VOID, _VOID, _VOID, _INT, _INT, _INT, _INT, _VOID],
     "nnis_attention_decode_max_waves": [_INT, _INT],
 }
 
@@ -377,10 +382,14 @@ def gemm_residual(x: torch.Tensor, w: torch.Tensor, resid: torch.Tensor, gain: t
     [m, n]) takes x @ w^T in, in place, and the norm that follows is prepared:
     ``scaled`` = bfloat16(resid * gain) and, in ``ss`` [parts, m], parts of
     each row's sum of squares.  Returns how many parts were written; the
-    norm's 1 / sqrt(mean + eps) is taken by ``gemm_scaled``, which reads them."""
+    norm's 1 / sqrt(mean + eps) is taken by ``gemm_scaled``, which reads them.
+    ``x`` may be the ``KeyRuns`` of a decode attention (where ``fits``): the
+    kernel then adds the runs up itself on its way."""
     m, k = x.shape
     n = w.shape[0]
-    for t, what in ((x, "x"), (w, "weight"), (resid, "resid"), (gain, "gain"), (scaled, "scaled"), (ss, "ss")):
+    runs = x if isinstance(x, KeyRuns) else None
+    for t, what in ((x if runs is None else x.partial, "x"), (w, "weight"), (resid, "resid"), (gain, "gain"), (scaled, "scaled"),
+                    (ss, "ss")):
         _dev(t, what)
         if not t.is_contiguous():
             raise KernelError(f"gemm_residual: {what} must be contiguous")
@@ -394,6 +403,13 @@ def gemm_residual(x: torch.Tensor, w: torch.Tensor, resid: torch.Tensor, gain: t
         raise KernelError("gemm_residual: ss must be float32 [rows, m] (gemm_residual_parts(m, n) rows are always enough)")
     lib = core()
     parts = ctypes.c_int(0)
+    if runs is not None:
+        if not runs.fits(n):
+            raise KernelError("gemm_residual: these key runs are not taken; add them up first (KeyRuns.combine)")
+        _check(lib, lib.nnis_gemm_residual_runs(runs.partial.data_ptr(), runs.runs, runs.heads, runs.head_dim, runs.tok_slot.data_ptr(),
+                                                w.data_ptr(), resid.data_ptr(), gain.data_ptr(), _code(gain), scaled.data_ptr(),
+                                                ss.data_ptr(), ss.numel() // m, m, n, ctypes.addressof(parts), _stream()))
+        return parts.value
     work = _gemm_workspace(x.device)
     _check(lib, lib.nnis_gemm_residual(x.data_ptr(), w.data_ptr(), resid.data_ptr(), gain.data_ptr(), _code(gain),
                                        scaled.data_ptr(), ss.data_ptr(), ss.numel() // m, m, n, k, ctypes.addressof(parts),
@@ -490,12 +506,15 @@ def attention_prefill_bf16(q, out, k_pages, v_pages, block_table, tile_seq, tile
 
 
 def attention_decode_bf16(q, out, k_pages, v_pages, block_table, tok_slot, tok_pos, heads, kv_heads, head_dim, scale,
-                          window=0, splits=1, partial=None, waves=1, kernel="auto"):
+                          window=0, splits=1, partial=None, waves=1, kernel="auto", keep_runs=False):
     """One query token per sequence over its cached keys.  The keys are cut
     into ``splits`` runs, each a block of ``waves`` waves that deal its pages
     among themselves and merge in LDS; the runs are summed by a second kernel.
     ``partial``: float32 scratch of tokens * heads * splits * (head_dim + 4)
-    when splits > 1 (``decode_scratch`` keeps one per device).  ``kernel``:
+    when splits > 1 (``decode_scratch`` keeps one per device).  ``keep_runs``
+    (with splits > 1): the second kernel is left out and a ``KeyRuns`` is
+    returned in place of ``out`` -- the projection that follows adds the runs
+    up itself (``gemm_residual``), or ``KeyRuns.combine()`` does.  ``kernel``:
     "keys" (keys on lanes; groups of up to 4 heads of up to 128 channels),
     "columns" (heads in the columns of a tile; any group the head size
     carries) or "auto", which takes "keys" where it fits."""
@@ -514,8 +533,41 @@ def attention_decode_bf16(q, out, k_pages, v_pages, block_table, tok_slot, tok_p
                                                block_table.data_ptr(), block_table.shape[1], tok_slot.data_ptr(),
                                                tok_pos.data_ptr(), tokens, heads, kv_heads, head_dim, int(window),
                                                float(scale), int(splits), int(waves), _ptr(partial) if splits > 1 else None,
-                                               _DECODE_KERNELS[kernel], _stream()))
+                                               _DECODE_KERNELS[kernel], 0 if (keep_runs and splits > 1) else 1, _stream()))
+    if keep_runs and splits > 1:
+        return KeyRuns(partial, int(splits), tokens, heads, head_dim, tok_slot, out)
     return out
+
+
+# Up to this many tokens a decode step leaves its runs of keys to the output projection; beyond, every block of
+# the projection making the same activations again costs more than the kernel between the two.
+KEY_RUNS_MOST_TOKENS = int(os.environ.get("NNIS_KEY_RUNS_TOKENS", "4"))
+
+
+class KeyRuns:
+    """What the decode attention leaves when it cuts the keys into runs and is
+    told not to add them up: per (token, head, run) the run's outputs, its
+    softmax reference and its sum, in ``partial`` (the device's decode scratch:
+    valid until the next decode attention on this device).  A stand-in for the
+    attention's output [tokens, heads * head_dim] in bfloat16."""
+
+    dtype = torch.bfloat16
+
+    def __init__(self, partial, runs, tokens, heads, head_dim, tok_slot, out):
+        self.partial, self.runs, self.tokens, self.heads, self.head_dim = partial, runs, tokens, heads, head_dim
+        self.tok_slot, self.out = tok_slot, out
+        self.shape = (tokens, heads * head_dim)
+
+    def fits(self, rows_out: int) -> bool:
+        """Whether ``gemm_residual`` takes these runs for a weight of ``rows_out`` rows."""
+        return bool(core().nnis_gemm_residual_runs_fits(self.tokens, int(rows_out), self.heads, self.head_dim, self.runs))
+
+    def combine(self) -> torch.Tensor:
+        """The attention's output, added up by the kernel of its own."""
+        lib = attention_module(self.head_dim)
+        _check(lib, lib.nnis_attention_combine(self.partial.data_ptr(), self.out.data_ptr(), self.tok_slot.data_ptr(), self.tokens,
+                                               self.heads, self.head_dim, self.runs, _stream()))
+        return self.out
 
 
 _DECODE_KERNELS = {"auto": 0, "columns": 1, "keys": 2}
@@ -584,10 +636,12 @@ def _prefill_tiles(ctx, rows: int, device):
 
 
 def attention(q: torch.Tensor, out: torch.Tensor, view, ctx, heads: int, kv_heads: int, head_dim: int, scale: float,
-              window: int = 0) -> torch.Tensor:
+              window: int = 0, keep_runs: bool = False):
     """Attention of the step's tokens over the cache ``view``: bfloat16 with a
     head size in steps of 16 runs on the matrix cores (one kernel for single
-    tokens, one for runs of tokens); anything else takes the 32-bit kernel."""
+    tokens, one for runs of tokens); anything else takes the 32-bit kernel.
+    ``keep_runs``: a decode step whose keys are cut into runs may return them
+    as ``KeyRuns`` instead of the output (see ``attention_decode_bf16``)."""
     fast = (q.dtype == torch.bfloat16 and view.k_pages.dtype == torch.bfloat16 and head_dim % 16 == 0)
     if fast and ctx.decode and heads // kv_heads <= 16 * (4 if head_dim <= 64 else (2 if head_dim <= 128 else 1)):
         if ctx.splits:
@@ -599,7 +653,8 @@ def attention(q: torch.Tensor, out: torch.Tensor, view, ctx, heads: int, kv_head
         if splits > 1:
             partial = decode_scratch(q.device, q.shape[0] * heads * splits * (head_dim + 4))
         return attention_decode_bf16(q, out, view.k_pages, view.v_pages, view.block_table, ctx.tok_slot, ctx.tok_pos, heads,
-                                     kv_heads, head_dim, scale, window, splits, partial, waves)
+                                     kv_heads, head_dim, scale, window, splits, partial, waves,
+                                     keep_runs=keep_runs and q.shape[0] <= KEY_RUNS_MOST_TOKENS)
     if fast and not ctx.decode:
         # A tile's keys are a chain of dependent loads: the longest tile sets the kernel's time.  The waves of
         # a block deal the keys among themselves (their merge lives in LDS).

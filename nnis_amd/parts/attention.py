@@ -91,7 +91,11 @@ class CausalSelfAttention(Mixer):
         q = self._project_rotate_store(x, ctx, view, rt)
         tokens = q.shape[0]
         attn = rt.empty(tokens, self.heads * self.head_dim)
-        rt.ops.attention(q, attn, view, ctx, self.heads, self.kv_heads, self.head_dim, self.scale, self.window or 0)
+        # a decode step over long sequences leaves its runs of keys to the output projection, if that takes them
+        attn = rt.ops.attention(q, attn, view, ctx, self.heads, self.kv_heads, self.head_dim, self.scale, self.window or 0,
+                                keep_runs=into is not None)
+        if isinstance(attn, rt.ops.KeyRuns) and not (into.can_take(attn, self.out.weight) and attn.fits(self.out.weight.shape[0])):
+            attn = attn.combine()
         if into is not None and into.can_take(attn, self.out.weight):
             return into.take(attn, self.out.weight)  # the output projection adds to the stream itself
         return self.out(attn, rt)

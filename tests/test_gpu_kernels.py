@@ -224,6 +224,53 @@ def test_prefill_attention_on_the_matrix_cores(heads, kv_heads, head_dim):
             assert (got[100, 0] - vs[2][17, 0]).abs().max().item() < 0.05
 
 
+@pytest.mark.parametrize("heads, kv_heads, head_dim, splits, rows_out", [(9, 3, 64, 4, 576), (4, 2, 16, 8, 70), (8, 2, 128, 2, 1024),
+                                                                         (5, 5, 80, 3, 200)])
+def test_residual_projection_adds_up_key_runs(heads, kv_heads, head_dim, splits, rows_out):
+    """A decode attention that leaves its runs of keys, and the projection that
+    adds them up on its way: the stream, the prepared norm and its sums are
+    those of the path with the kernel of its own between the two, bit for bit
+    (a padding row's aside: nobody reads it)."""
+    ops = _ops()
+    torch.manual_seed(heads + head_dim + splits)
+    lengths = [700, 1, 65, 33]
+    ks = [torch.randn(n, kv_heads, head_dim).bfloat16().float() for n in lengths]
+    vs = [torch.randn(n, kv_heads, head_dim).bfloat16().float() for n in lengths]
+    k_pages, v_pages, table = _paged(ks, vs, torch.bfloat16, kv_heads, head_dim)
+    slots, positions = [0, 1, -1, 2, 3], [699, 0, 9, 64, 31]
+    live = [i for i, s in enumerate(slots) if s >= 0]
+    m, k = len(slots), heads * head_dim
+    q = torch.randn(m, k).bfloat16().cuda()
+    out = torch.zeros(m, k, dtype=torch.bfloat16, device="cuda")
+    partial = torch.full((m * heads * splits * (head_dim + 4),), float("nan"), dtype=torch.float32, device="cuda")
+    waves = min(2, ops.decode_max_waves(heads, kv_heads, head_dim))
+    runs = ops.attention_decode_bf16(q, out, k_pages, v_pages, table, _i32(slots), _i32(positions), heads, kv_heads, head_dim,
+                                     1.0 / math.sqrt(head_dim), 0, splits, partial, waves, keep_runs=True)
+    assert isinstance(runs, ops.KeyRuns) and runs.shape == (m, k) and runs.fits(rows_out)
+    w = (torch.randn(rows_out, k) / math.sqrt(k)).bfloat16().cuda()
+    gain = (1 + 0.3 * torch.randn(rows_out)).bfloat16().cuda()
+    resid = torch.randn(m, rows_out).cuda()
+
+    def project(x):
+        mine = resid.clone()
+        scaled = torch.zeros(m, rows_out, dtype=torch.bfloat16, device="cuda")
+        ss = torch.zeros(ops.gemm_residual_parts(m, rows_out), m, device="cuda")
+        parts = ops.gemm_residual(x, w, mine, gain, scaled, ss)
+        return mine[live].cpu(), scaled[live].cpu(), ss[:parts][:, live].cpu()
+
+    fused = project(runs)
+    added = runs.combine()
+    assert added.data_ptr() == out.data_ptr()
+    want = _plain_rows([(slots[i], positions[i], q[i].float().cpu().view(heads, head_dim)) for i in live], ks, vs, 1.0 / math.sqrt(head_dim))
+    assert (added[live].cpu().float().view(len(live), heads, head_dim) - want).abs().max().item() <= 2e-2
+    apart = project(added)
+    for got, expected in zip(fused, apart):
+        assert torch.equal(got, expected)
+    # runs that the projection does not take: too many of them, or too many tokens
+    assert not ops.KeyRuns(partial, 9, m, heads, head_dim, _i32(slots), out).fits(rows_out)
+    assert not ops.KeyRuns(partial, splits, 65, heads, head_dim, _i32(slots), out).fits(rows_out)
+
+
 @pytest.mark.parametrize("heads, kv_heads, head_dim, lengths", [(9, 3, 64, (1500, 700, 90)), (8, 8, 16, (1300, 1000, 100))])
 def test_prefill_attention_with_more_items_than_compute_units(heads, kv_heads, head_dim, lengths):
     """Steps of so many tiles that a block takes two of them, a long one and
