@@ -416,7 +416,9 @@ extern __shared__ __align__(16) char tile_lds[];  // NS stages of BM + BN rows o
 #ifndef NNIS_TILE_GROUP_ROWS
 #define NNIS_TILE_GROUP_ROWS 512
 #endif
-// NS stages: 3 where a compute unit runs several blocks; 6 where the grid leaves it one block at most and K is
+// NS stages: 2 for the 64 x 128 tile where the grid gives a compute unit three blocks and more (48 KB of LDS a
+// block instead of 72: three fit, and 2048 x 3072 x 576 takes 15.3 us instead of 17.5, 2048 x 6144 x 2048 68.5
+// instead of 75); 3 where a compute unit runs fewer; 6 where the grid leaves it one block at most and K is
 // long, so that the loads in flight are all that hides the memory's latency (64 tokens x 11264 x 2048: 20.9 us
 // with 3, 19.7 with 6; a K of 9 steps in 256 blocks took 13.4 us with 6 against 11.7)
 // SPLIT: K is cut into ksplit parts, a block leaves its part's sums in `partial` and gemm_reduce_kernel does the
@@ -854,6 +856,10 @@ void dispatch_skinny(const bf16_t* x, const bf16_t* w, OutT y, int m, int n, int
 #define NNIS_DEEP_RING_BLOCKS 256
 #endif
 constexpr int kDeepRingBlocks = NNIS_DEEP_RING_BLOCKS;  // grids up to this many blocks take the ring of 6 stages
+#ifndef NNIS_SHALLOW_RING_BLOCKS
+#define NNIS_SHALLOW_RING_BLOCKS 640
+#endif
+constexpr int kShallowRingBlocks = NNIS_SHALLOW_RING_BLOCKS;  // grids of 64 x 128 tiles from this many blocks on: 2 stages
 
 // Scratch for the parts of a K that is cut among blocks (the caller's; nothing is allocated here)
 struct Workspace {
@@ -909,8 +915,11 @@ int launch_tiled(const bf16_t* x, const bf16_t* w, OutT y, int m, int n, int k, 
   const int col_blocks = (columns + BN - 1) / BN, row_blocks = (m + BM - 1) / BM;
   const int ksplit = ws.floats ? tiled_ksplit(col_blocks * row_blocks, m, col_blocks * BN, k, ws.bytes) : 1;
   const int steps_a_part = ((k + BK - 1) / BK + ksplit - 1) / ksplit;
-  if (col_blocks * row_blocks * ksplit <= kDeepRingBlocks && steps_a_part >= 16)
+  const int blocks = col_blocks * row_blocks * ksplit;
+  if (blocks <= kDeepRingBlocks && steps_a_part >= 16)
     return launch_tiled_staged<BM, BN, BK, 6, OutT>(x, w, y, m, n, k, col_blocks, row_blocks, ksplit, ws, stream);
+  if (BN == 128 && ksplit == 1 && blocks >= kShallowRingBlocks)
+    return launch_tiled_staged<BM, BN, BK, 2, OutT>(x, w, y, m, n, k, col_blocks, row_blocks, 1, ws, stream);
   return launch_tiled_staged<BM, BN, BK, 3, OutT>(x, w, y, m, n, k, col_blocks, row_blocks, ksplit, ws, stream);
 }
 
