@@ -387,6 +387,54 @@ __device__ __forceinline__ bool merge_waves(AttnState<C>& st, float* merge, int 
   return wave == 0;
 }
 
+// The same for a group of `size` waves of the block, of any size, this wave its member `index`: in each round the
+// upper half of the members still in play (rounded down) hand their states to the lower ones through `slots`
+// (room for size / 2 states).  Every wave of the block runs `rounds` rounds, so that groups of different sizes
+// meet at the same barriers; a group that is done early only waits.  Returns true for the member that is left.
+template <int C>
+__device__ __forceinline__ bool merge_group(AttnState<C>& st, float* slots, int index, int size, int rounds, int lane) {
+  constexpr int kValues = kTilesD * 4 + 2;
+  int n = size;
+  for (int round = 0; round < rounds; ++round) {
+    const int keep = (n + 1) / 2;  // members [keep, n) hand over to members [0, n - keep)
+    if (index >= keep && index < n) {
+      float* mine = slots + (size_t)(index - keep) * C * kValues * kWave;
+#pragma unroll
+      for (int c = 0; c < C; ++c) {
+        float* col = mine + (size_t)c * kValues * kWave + lane;
+#pragma unroll
+        for (int t = 0; t < kTilesD; ++t)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) col[(4 * t + e) * kWave] = st.o[c][t][e];
+        col[(kTilesD * 4) * kWave] = st.m[c];
+        col[(kTilesD * 4 + 1) * kWave] = st.l[c];
+      }
+    }
+    __syncthreads();
+    if (index < n - keep) {
+      const float* theirs = slots + (size_t)index * C * kValues * kWave;
+#pragma unroll
+      for (int c = 0; c < C; ++c) {
+        const float* col = theirs + (size_t)c * kValues * kWave + lane;
+        const float m_other = col[(kTilesD * 4) * kWave];
+        const float m_new = fmaxf(st.m[c], m_other);
+        const float m_safe = m_new == -INFINITY ? 0.0f : m_new;
+        const float mine_w = __builtin_amdgcn_exp2f(st.m[c] - m_safe);
+        const float their_w = __builtin_amdgcn_exp2f(m_other - m_safe);
+        st.l[c] = st.l[c] * mine_w + col[(kTilesD * 4 + 1) * kWave] * their_w;
+        st.m[c] = m_new;
+#pragma unroll
+        for (int t = 0; t < kTilesD; ++t)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) st.o[c][t][e] = st.o[c][t][e] * mine_w + col[(4 * t + e) * kWave] * their_w;
+      }
+    }
+    if (round + 1 < rounds) __syncthreads();  // the next round writes where this one read
+    n = keep;
+  }
+  return index == 0;
+}
+
 // Runs the pages first, first + stride, ... (`mine` of them) of a sequence through the
 // softmax state, each as two blocks of 32 keys one after the other (so both halves of a
 // value line are used while it is near).  RING blocks' operands are in flight at a time:
@@ -461,8 +509,10 @@ constexpr int kPrefillRing = HD > 64 ? 2 : (C <= 2 ? NNIS_PREFILL_RING_NARROW : 
 // An item is a (tile, kv head, chunk of heads); the tiles come longest first, and item i = tile i / per_tile.
 // A tile's work grows with its place in its sequence, and a chip with fewer items than twice its compute
 // units runs them all at once: its time is the most loaded unit's.  So the grid is folded: block b < singles
-// has item b alone, block b >= singles has item b and then item items - 1 - (b - singles), a heavy and a
-// light one.
+// has item b alone, block b >= singles has item b and item items - 1 - (b - singles), a heavy and a light
+// one, side by side: the block's waves are dealt to the two in proportion to their pages (an item's time is
+// mostly the chain of loads before its first key and the merge after its last, which the two now spend
+// together; one after the other a 2,048-token prefill of 9/3 heads took 22 us a layer here, side by side 18).
 template <int QT, int GH>
 __global__ __launch_bounds__(64 * kBlockWaves) void attention_prefill_kernel(MfmaArgs a, int waves, int items, int singles,
                                                                             int per_tile) {
@@ -488,7 +538,8 @@ __global__ __launch_bounds__(64 * kBlockWaves) void attention_prefill_kernel(Mfm
     rows_of[which] = __builtin_amdgcn_readfirstlane(a.seq_start[seq_of[which] + 1]) - start_of[which];
     pos0_of[which] = __builtin_amdgcn_readfirstlane(a.seq_pos0[seq_of[which]]);
   }
-  auto run_item = [&](int which) __attribute__((always_inline)) {
+  // which: the item; this wave is member `index` of the `size` waves that take it; slots: their room for the merge
+  auto run_item = [&](int which, int index, int size, float* slots, int rounds) __attribute__((always_inline)) {
     const int part = item_of[which] % per_tile;
     const int kv_head = part / chunks;
     const int head0 = kv_head * group + (part % chunks) * GH;
@@ -527,10 +578,10 @@ __global__ __launch_bounds__(64 * kBlockWaves) void attention_prefill_kernel(Mfm
     init_state(st);
     if (last >= 0) {
       const int first_page = first / kPageTokens, page_count = last / kPageTokens + 1 - first_page;
-      const int mine = page_count > wave ? (page_count - wave + waves - 1) / waves : 0;  // pages of this wave
-      attend_run<C, kPrefillRing<C>>(st, q, a, pages, kv_head, first_page + wave, waves, mine, last, lo, hi, lane);
+      const int mine = page_count > index ? (page_count - index + size - 1) / size : 0;  // pages of this wave
+      attend_run<C, kPrefillRing<C>>(st, q, a, pages, kv_head, first_page + index, size, mine, last, lo, hi, lane);
     }
-    if (!merge_waves<C>(st, merge, wave, waves, lane)) return;
+    if (!merge_group<C>(st, slots, index, size, rounds, lane)) return;
 #pragma unroll
     for (int qt = 0; qt < QT; ++qt)
 #pragma unroll
@@ -551,10 +602,30 @@ __global__ __launch_bounds__(64 * kBlockWaves) void attention_prefill_kernel(Mfm
         }
       }
   };
-  run_item(0);
-  if (count > 1) {
-    __syncthreads();  // the first item's merge has been read
-    run_item(1);
+  int rounds = 0;
+  while ((1 << rounds) < waves) ++rounds;
+  if (count == 1) {
+    run_item(0, wave, waves, merge, rounds);
+  } else if (waves == 1) {
+    run_item(0, 0, 1, merge, 0);
+    run_item(1, 0, 1, merge, 0);
+  } else {
+    // pages of the two (up to the last row's position; a window's lower end does not matter for the shares)
+    int pages_of[2];
+#pragma unroll
+    for (int which = 0; which < 2; ++which) {
+      const int rows_here = min(row0_of[which] + 16 * QT, rows_of[which]);
+      pages_of[which] = (pos0_of[which] + rows_here - 1) / kPageTokens + 1;
+    }
+    // even shares (their merges then need waves / 2 states of room together), at least 2 waves each; of 2 waves, 1 each
+    int first_share = 1;
+    if (waves >= 4) {
+      first_share = 2 * ((waves * pages_of[0] + pages_of[0] + pages_of[1]) / (2 * (pages_of[0] + pages_of[1])));
+      first_share = first_share < 2 ? 2 : (first_share > waves - 2 ? waves - 2 : first_share);
+    }
+    constexpr int kValues = kTilesD * 4 + 2;
+    if (wave < first_share) run_item(0, wave, first_share, merge, rounds);
+    else run_item(1, wave - first_share, waves - first_share, merge + (size_t)(first_share / 2) * C * kValues * kWave, rounds);
   }
 }
 
