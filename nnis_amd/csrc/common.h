@@ -31,6 +31,26 @@ __host__ __device__ constexpr size_t nnis_v_offset(int channel, int token) {
   return ((((size_t)(channel / 16) * 2 + token / 32) * 4 + (token % 32) / 8) * 16 + channel % 16) * 8 + token % 8;
 }
 
+// The weights of the matrix-core products are kept packed (nnis_pack_weight): rows in strips of 16, K in
+// chunks of 64, both padded with zeros, and a strip's chunk (2 KB) in the order in which a wave's two
+// 16-byte loads take it as the first operand of v_mfma_f32_16x16x32_bf16:
+//   [strip][chunk][half][lane = 16 * (k % 64 / 16) + row % 16][8 elements],  half = k % 16 / 8
+// so that a load instruction of a wave reads 1 KB of consecutive memory whatever K is (rows of the
+// checkpoint's order are K * 2 bytes apart: 16 pieces of 64 bytes an instruction, measured at 55 to 80% of the
+// packed order's bandwidth on weights of 8 to 200 MB).
+// A strip is an odd number of chunks long (one chunk of padding where K gives an even number, never read), so
+// that the strips' first chunks, which a kernel's waves all ask for at once, do not lie a power of two apart
+// and meet in the same memory channels.
+constexpr int kPackedChunkElems = 1024;  // a strip's chunk
+constexpr int kPackedHalfElems = 512;
+__host__ __device__ constexpr int nnis_packed_chunks(int k) { return (k + 63) / 64; }
+__host__ __device__ constexpr size_t nnis_packed_strip_elems(int k) { return (size_t)(nnis_packed_chunks(k) | 1) * kPackedChunkElems; }
+__host__ __device__ constexpr size_t nnis_packed_elems(int n, int k) { return (size_t)((n + 15) / 16) * nnis_packed_strip_elems(k); }
+// where the lane that multiplies `row` with k group g (k % 64 / 16) finds its 8 elements of chunk 0, half 0
+__host__ __device__ constexpr size_t nnis_packed_lane(int row, int g, int k) {
+  return (size_t)(row >> 4) * nnis_packed_strip_elems(k) + (size_t)(g * 16 + (row & 15)) * 8;
+}
+
 extern thread_local char g_nnis_error[512];
 
 static inline int nnis_fail(const char* fmt, ...) {

@@ -44,7 +44,8 @@ struct FusedArgs {
   const void* norm_w;   // [k]
   int norm_w_dtype;
   float eps;
-  const bf16_t* w;  // [n, k]
+  const bf16_t* w;  // [n, k], packed (nnis_pack_weight)
+  int stream_weights;  // large weights, read once: loaded past the caches' keeping (as in gemm_mfma.hip)
   int m, n, k;
   bf16_t* y;  // store: [m, n]; silu: [m, n / 2]; rope: queries [m, heads * head_dim] (= rope.q_out)
   RopeTarget rope;
@@ -55,6 +56,12 @@ __device__ __forceinline__ bf16x8 zero8() {
 #pragma unroll
   for (int i = 0; i < 8; ++i) z[i] = (__bf16)0.0f;
   return z;
+}
+
+constexpr size_t kStreamWeightBytes = 16u << 20;  // as in gemm_mfma.hip
+
+__device__ __forceinline__ bf16x8 load_weight(const bf16_t* p, int stream) {
+  return stream ? __builtin_nontemporal_load((const bf16x8*)p) : *(const bf16x8*)p;
 }
 
 // eight consecutive floats of the norm weight, whatever its storage type
@@ -171,8 +178,9 @@ __global__ __launch_bounds__(KSPLIT > 4 ? 64 * KSPLIT : 256) void gemm_fused_ker
     int wr0 = row0 + r, wr1 = row1 + r;
     wr0 = wr0 < row_limit ? wr0 : row_limit - 1;
     wr1 = wr1 < n ? wr1 : n - 1;
-    const bf16_t* w0 = a.w + (size_t)wr0 * k;
-    const bf16_t* w1 = a.w + (size_t)wr1 * k;
+    const int chunks = nnis_packed_chunks(k);
+    const bf16_t* w0 = a.w + nnis_packed_lane(wr0, g, k);  // packed weights: chunk c at + c * 1024, the second half at + 512
+    const bf16_t* w1 = a.w + nnis_packed_lane(wr1, g, k);
     size_t x_row[MT];
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
@@ -182,7 +190,6 @@ __global__ __launch_bounds__(KSPLIT > 4 ? 64 * KSPLIT : 256) void gemm_fused_ker
     }
     const bool writes_x = !PREP && a.delta != nullptr && unit == 0;  // the first unit's waves cover every k once
     const bool gain_f32 = a.norm_w_dtype == NNIS_F32;
-    const int chunks = (k + 63) / 64;
     if constexpr (PREP) {
       for (int base = part; base < chunks; base += KSPLIT * DEPTH) {
         bf16x8 wa[DEPTH][2], wb[DEPTH][2], xs[DEPTH][2][MT];
@@ -190,10 +197,12 @@ __global__ __launch_bounds__(KSPLIT > 4 ? 64 * KSPLIT : 256) void gemm_fused_ker
         for (int d = 0; d < DEPTH; ++d)
 #pragma unroll
           for (int half = 0; half < 2; ++half) {
-            const int kk = (base + d * KSPLIT) * 64 + g * 16 + half * 8;
+            const int c = base + d * KSPLIT;
+            const int kk = c * 64 + g * 16 + half * 8;
             const bool in = kk + 8 <= k;
-            wa[d][half] = in ? *(const bf16x8*)(w0 + kk) : zero8();
-            wb[d][half] = (PAIR && in) ? *(const bf16x8*)(w1 + kk) : zero8();
+            const size_t at = (size_t)c * kPackedChunkElems + half * kPackedHalfElems;
+            wa[d][half] = in ? load_weight(w0 + at, a.stream_weights) : zero8();
+            wb[d][half] = (PAIR && in) ? load_weight(w1 + at, a.stream_weights) : zero8();
 #pragma unroll
             for (int t = 0; t < MT; ++t) xs[d][half][t] = in ? *(const bf16x8*)(a.scaled + x_row[t] + kk) : zero8();
           }
@@ -222,10 +231,12 @@ __global__ __launch_bounds__(KSPLIT > 4 ? 64 * KSPLIT : 256) void gemm_fused_ker
       for (int d = 0; d < DEPTH; ++d)
 #pragma unroll
         for (int half = 0; half < 2; ++half) {
-          const int kk = (base + d * KSPLIT) * 64 + g * 16 + half * 8;
+          const int c = base + d * KSPLIT;
+          const int kk = c * 64 + g * 16 + half * 8;
           const bool in = kk + 8 <= k;
-          wa[d][half] = in ? *(const bf16x8*)(w0 + kk) : zero8();
-          wb[d][half] = (PAIR && in) ? *(const bf16x8*)(w1 + kk) : zero8();
+          const size_t at = (size_t)c * kPackedChunkElems + half * kPackedHalfElems;
+          wa[d][half] = in ? load_weight(w0 + at, a.stream_weights) : zero8();
+          wb[d][half] = (PAIR && in) ? load_weight(w1 + at, a.stream_weights) : zero8();
           if (in) {
             if (gain_f32) {
               gr[d][half][0] = *(const f32x4*)((const float*)a.norm_w + kk);
@@ -402,6 +413,7 @@ void dispatch_fused(const FusedArgs& a, int units, int split, hipStream_t stream
 int run_fused(FusedArgs& a, int epilogue, int table_positions, int split_hint, float* workspace, size_t workspace_bytes,
               hipStream_t stream) {
   const int n = a.n, k = a.k;
+  a.stream_weights = (size_t)n * k * sizeof(bf16_t) > kStreamWeightBytes;
   int units;
   if (epilogue == EPI_STORE) {
     units = (n + 15) / 16;

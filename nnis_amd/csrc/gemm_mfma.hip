@@ -34,6 +34,11 @@ typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
 __device__ __forceinline__ bf16x8 load_chunk(const bf16_t* p) { return *(const bf16x8*)p; }
+// Weights that a kernel reads once and that are too large to be found in a cache by the next step: loaded past
+// the caches' keeping.  Measured with 1 token, microseconds, plain against streamed: 25 MB 7.5 / 7.0, 67 MB 14.4 /
+// 13.6, 201 MB 39.9 / 36.5; but 8.4 MB 3.9 / 4.4 and 1.8 MB 3.2 / 3.6, hence the limit.
+constexpr size_t kStreamWeightBytes = 16u << 20;
+__device__ __forceinline__ bf16x8 load_stream(const bf16_t* p) { return __builtin_nontemporal_load((const bf16x8*)p); }
 
 __device__ __forceinline__ bf16x8 zero_chunk() {
   bf16x8 z;
@@ -259,7 +264,7 @@ template <int MT, int KSPLIT, bool RUNS, typename OutT>
 __global__ __launch_bounds__(KSPLIT > 4 ? 64 * KSPLIT : 256) void gemm_skinny_kernel(const bf16_t* __restrict__ x,
                                                                                    const bf16_t* __restrict__ w,
                                                                                    OutT y, int m, int n, int k, int tiles,
-                                                                                   RunsIn runs) {
+                                                                                   int stream_weights, RunsIn runs) {
   constexpr int kWaves = KSPLIT > 4 ? KSPLIT : 4;
   constexpr int kStrips = kWaves / KSPLIT;  // strips of 16 weight rows per block
   constexpr int DEPTH = MT <= 2 ? 4 : 2;
@@ -295,17 +300,25 @@ __global__ __launch_bounds__(KSPLIT > 4 ? 64 * KSPLIT : 256) void gemm_skinny_ke
     }
   }
 
-  int w_row = strip * 16 + r;
-  w_row = w_row < n ? w_row : n - 1;  // rows beyond N read a valid row and are not stored
-  const bf16_t* w_ptr = w + (size_t)(active ? w_row : 0) * k;
-  const int chunks = (k + 63) / 64;
+  const int chunks = nnis_packed_chunks(k);
+  // packed weights: the strip's padding rows and the last chunk's padding are zeros that are there to read
+  const bf16_t* w_ptr = w + nnis_packed_lane(active ? strip * 16 + r : 0, g, k);
   // a round: DEPTH steps of 64 k of this wave (base, base + KSPLIT, ..): their weights ...
   auto ask_weights = [&](int base, bf16x8 (&wa)[DEPTH], bf16x8 (&wb)[DEPTH]) {
+    if (stream_weights) {
 #pragma unroll
-    for (int d = 0; d < DEPTH; ++d) {
-      const int ka = (base + d * KSPLIT) * 64 + g * 16, kb = ka + 8;
-      wa[d] = ka + 8 <= k ? load_chunk(w_ptr + ka) : zero_chunk();  // zeros also for steps beyond the last
-      wb[d] = kb + 8 <= k ? load_chunk(w_ptr + kb) : zero_chunk();
+      for (int d = 0; d < DEPTH; ++d) {
+        const int c = base + d * KSPLIT;
+        wa[d] = c < chunks ? load_stream(w_ptr + (size_t)c * kPackedChunkElems) : zero_chunk();  // zeros for steps beyond the last
+        wb[d] = c < chunks ? load_stream(w_ptr + (size_t)c * kPackedChunkElems + kPackedHalfElems) : zero_chunk();
+      }
+    } else {
+#pragma unroll
+      for (int d = 0; d < DEPTH; ++d) {
+        const int c = base + d * KSPLIT;
+        wa[d] = c < chunks ? load_chunk(w_ptr + (size_t)c * kPackedChunkElems) : zero_chunk();
+        wb[d] = c < chunks ? load_chunk(w_ptr + (size_t)c * kPackedChunkElems + kPackedHalfElems) : zero_chunk();
+      }
     }
   };
   const bf16_t* x_ptr[MT];
@@ -431,9 +444,9 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
   constexpr int TM = WM / 16, TN = WN / 16;
   constexpr int CH = BK / 8;  // 16-byte chunks per staged row
   static_assert(CH == 8, "a load instruction of a wave fills 8 rows of 8 chunks");
-  // One load instruction of a wave moves 64 x 16 bytes into 1 KB of LDS that is contiguous: 8 rows of a
-  // stage, lane l to row l / 8, place l % 8.  The swizzle is made on the way in by the choice of the source:
-  // place p of row r holds chunk p ^ (r % 8).
+  // One load instruction of a wave moves 64 x 16 bytes into 1 KB of LDS that is contiguous.  Of the activations
+  // that is 8 rows of a stage, lane l to row l / 8, place l % 8; the swizzle is made on the way in by the
+  // choice of the source: place p of row r holds chunk p ^ (r % 8).
   constexpr int A_LOADS = BM / 32, B_LOADS = BN / 32;  // a wave's load instructions per step (4 waves x 8 rows each)
   constexpr int LOADS = A_LOADS + B_LOADS;
   constexpr int A_BYTES = BM * BK * 2, STAGE_BYTES = (BM + BN) * BK * 2;
@@ -483,9 +496,13 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
   }
   constexpr int EPI = scaled_epilogue<OutT>::value;  // -1: the product is stored or added as it is
   constexpr bool kPaired = EPI == EPI_SILU || EPI == EPI_ROPE;
+  // The weights are packed in the order the matrix instruction takes them: a load instruction copies one half of
+  // a strip's chunk (1 KB, lane l's 16 bytes to place l) and the stage holds [strip of the tile][half][lane].
+  const int chunks = nnis_packed_chunks(k);
 #pragma unroll
   for (int o = 0; o < B_LOADS; ++o) {
-    const int tile_row = (o * 4 + wave) * 8 + lane / 8;
+    const int piece = o * 4 + wave;  // (strip of the tile, half)
+    const int tile_row = (piece / 2) * 16 + r;
     int row;
     if constexpr (kPaired) {
       row = paired_weight_row<EPI, BN>(y.rope, col_block, tile_row, n);
@@ -494,7 +511,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
       row = col0 + tile_row;
       row = row < n ? row : n - 1;
     }
-    b_src[o] = w + (size_t)row * k + chunk_k;
+    b_src[o] = w + nnis_packed_lane(row, g, k) + (piece % 2) * kPackedHalfElems;
   }
   // Step s lies in stage s % NS.  A step first asks for the step NS - 1 ahead, into the
   // stage that was read a step ago (every wave is past the barrier that ended that step, and what it read
@@ -517,9 +534,10 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
 #pragma unroll
     for (int o = 0; o < A_LOADS; ++o)
       __builtin_amdgcn_global_load_lds((global_ptr_t)(a_src[o] + from), (lds_ptr_t)(base + o * 4096), 16, 0, 0);
+    const size_t from_chunk = (size_t)(step < chunks ? step : chunks - 1) * kPackedChunkElems;
 #pragma unroll
     for (int o = 0; o < B_LOADS; ++o)
-      __builtin_amdgcn_global_load_lds((global_ptr_t)(b_src[o] + from), (lds_ptr_t)(base + A_BYTES + o * 4096), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((global_ptr_t)(b_src[o] + from_chunk), (lds_ptr_t)(base + A_BYTES + o * 4096), 16, 0, 0);
   };
   const bool ragged = (k % BK) != 0;
 
@@ -587,10 +605,10 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
     for (int half = 0; half < BK / 32; ++half) {  // an instruction takes 32 k
       bf16x8 a_frag[TM], b_frag[TN];
 #pragma unroll
-      for (int i = 0; i < TM; ++i) a_frag[i] = a_tile[swizzled<CH>(wave_m * WM + i * 16 + r, half * 4 + g)];
+      for (int i = 0; i < TM; ++i) a_frag[i] = a_tile[swizzled<CH>(wave_m * WM + i * 16 + r, g * 2 + half)];  // k as the weights are packed
 #pragma unroll
-      for (int jj = 0; jj < TN; ++jj) b_frag[jj] = b_tile[swizzled<CH>(wave_n * WN + jj * 16 + r, half * 4 + g)];
-      if (ragged && step == steps - 1 && step * BK + (half * 4 + g) * 8 + 8 > k) {
+      for (int jj = 0; jj < TN; ++jj) b_frag[jj] = b_tile[((wave_n * TN + jj) * 2 + half) * kWave + lane];
+      if (ragged && step == steps - 1 && step * BK + (g * 2 + half) * 8 + 8 > k) {
 #pragma unroll
         for (int i = 0; i < TM; ++i) a_frag[i] = zero_chunk();
       }
@@ -816,14 +834,16 @@ void launch_skinny(const bf16_t* x, const bf16_t* w, OutT y, int m, int n, int k
   const int strip_blocks = (strips + per_block - 1) / per_block;
   const int tiles = (m + 16 * MT - 1) / (16 * MT);
   const dim3 grid(tiles == 1 ? strip_blocks : (strip_blocks + 7) / 8 * 8 * tiles), block(64 * waves);
+  const int stream_weights = (size_t)n * k * sizeof(bf16_t) > kStreamWeightBytes;
   if constexpr (std::is_same<OutT, ResidualOut>::value) {
     if (runs) {
       hipLaunchKernelGGL((gemm_skinny_kernel<MT, KSPLIT, true, OutT>), grid, block, skinny_runs_lds(MT, k), stream, x, w, y, m, n, k,
-                         tiles, *runs);
+                         tiles, stream_weights, *runs);
       return;
     }
   }
-  hipLaunchKernelGGL((gemm_skinny_kernel<MT, KSPLIT, false, OutT>), grid, block, 0, stream, x, w, y, m, n, k, tiles, RunsIn{});
+  hipLaunchKernelGGL((gemm_skinny_kernel<MT, KSPLIT, false, OutT>), grid, block, 0, stream, x, w, y, m, n, k, tiles, stream_weights,
+                     RunsIn{});
 }
 
 template <int MT, typename OutT>
@@ -1112,5 +1132,36 @@ extern "C" int nnis_gemm_residual_runs(const float* partial, int runs, int heads
   ResidualOut out = {resid, gain, gain_dtype, (bf16_t*)scaled, ss};
   dispatch_skinny<ResidualOut>(nullptr, (const bf16_t*)w, out, m, n, k, skinny_split(m, n, k, 0), (hipStream_t)stream_ptr, &in);
   NNIS_LAUNCH_CHECK("gemm_residual_runs");
+  return 0;
+}
+
+// The packed order of a weight [n, k] in the checkpoint's order (common.h has the layout): a thread moves
+// the 16 bytes of one lane's load, or writes the padding's zeros.
+__global__ __launch_bounds__(256) void pack_weight_kernel(const bf16_t* __restrict__ w, bf16_t* __restrict__ packed, int n, int k,
+                                                          size_t pieces) {
+  const size_t piece = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (piece >= pieces) return;
+  const int stride = nnis_packed_strip_elems(k) / kPackedChunkElems;  // chunks from strip to strip
+  const int lane = piece % 64, half = (piece / 64) % 2;
+  const size_t block = piece / 128;
+  const int chunk = block % stride;
+  const int strip = block / stride;
+  const int row = strip * 16 + lane % 16, kk = chunk * 64 + (lane / 16) * 16 + half * 8;
+  typedef __attribute__((ext_vector_type(4))) unsigned bits128;
+  bits128 v = {0u, 0u, 0u, 0u};
+  if (row < n && kk + 8 <= k) v = *(const bits128*)(w + (size_t)row * k + kk);  // (a padding chunk's kk is beyond k)
+  *(bits128*)(packed + piece * 8) = v;
+}
+
+// packed [(n + 15) / 16 strips][nnis_packed_strip_elems(k)] = the weight w [n, k] (bfloat16, K a multiple of 8) in the order the
+// matrix-core products read
+extern "C" int nnis_pack_weight(const void* w, void* packed, int n, int k, void* stream_ptr) {
+  NNIS_REQUIRE(n > 0 && k > 0 && k % 8 == 0, "pack_weight: bad sizes n=%d k=%d (K must be a multiple of 8)", n, k);
+  NNIS_REQUIRE(w && packed && (uintptr_t)w % 16 == 0 && (uintptr_t)packed % 16 == 0, "pack_weight: operands must be 16-byte aligned");
+  const size_t pieces = nnis_packed_elems(n, k) / 8;
+  NNIS_REQUIRE((pieces + 255) / 256 <= 0x7fffffffull, "pack_weight: %d x %d is more than a grid takes", n, k);
+  hipLaunchKernelGGL(pack_weight_kernel, dim3((unsigned)((pieces + 255) / 256)), dim3(256), 0, (hipStream_t)stream_ptr, (const bf16_t*)w,
+                     (bf16_t*)packed, n, k, pieces);
+  NNIS_LAUNCH_CHECK("pack_weight");
   return 0;
 }

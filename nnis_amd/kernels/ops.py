@@ -42,6 +42,7 @@ _CORE_SIGNATURES = {
     "nnis_gemm_residual_runs_fits": [_INT, _INT, _INT, _INT, _INT],
     "nnis_gemm_residual_runs": [_VOID, _INT, _INT, _INT, _VOID, _VOID, _VOID, _VOID, _INT, _VOID, _VOID, _INT, _INT, _INT, _VOID,
                                 _VOID],
+    "nnis_pack_weight": [_VOID, _VOID, _INT, _INT, _VOID],
     "nnis_sample": [_VOID, _VOID, _INT, _INT, _VOID, _VOID, _VOID, _VOID, _VOID, _VOID, _VOID],
 }
 _ATTN_SIGNATURES = {
@@ -281,6 +282,62 @@ def attention_rows(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_
 # dispatch by operand types
 # ---------------------------------------------------------------------------
 
+class PackedWeight:
+    """A bfloat16 weight [n, k] in the order the matrix-core products read it
+    (``pack_weight``): strips of 16 rows, chunks of 64 k, both padded with
+    zeros (and a strip to an odd number of chunks), a strip's chunk laid out
+    as a wave's loads take it.  ``data`` is the
+    flat packed storage; ``shape`` and ``dtype`` are the weight's own."""
+
+    dtype = torch.bfloat16
+    is_cuda = True
+
+    def __init__(self, data: torch.Tensor, n: int, k: int):
+        self.data = data
+        self.shape = (int(n), int(k))
+
+    @property
+    def device(self):
+        return self.data.device
+
+    def data_ptr(self) -> int:
+        return self.data.data_ptr()
+
+    def is_contiguous(self) -> bool:
+        return True
+
+    def storage_bytes(self) -> int:
+        return self.data.numel() * self.data.element_size()
+
+
+def packed_weight_elems(n: int, k: int) -> int:
+    """Strips of 16 rows, each an odd number of chunks of 64 k (1024 elements) long."""
+    return ((n + 15) // 16) * (((k + 63) // 64) | 1) * 1024
+
+
+def packs(weight: torch.Tensor) -> bool:
+    """Whether a weight is one that ``pack_weight`` takes."""
+    return weight.is_cuda and weight.dim() == 2 and weight.dtype == torch.bfloat16 and weight.shape[1] % 8 == 0
+
+
+def pack_weight(w: torch.Tensor) -> PackedWeight:
+    """The packed copy of a bfloat16 weight [n, k] (K a multiple of 8) that
+    ``gemm_bf16``, ``gemm_fused``, ``gemm_residual`` and ``gemm_scaled`` take."""
+    _dev(w, "weight")
+    if not packs(w):
+        raise KernelError(f"pack_weight takes a bfloat16 matrix whose K is a multiple of 8, got {w.dtype} {tuple(w.shape)}")
+    n, k = w.shape
+    data = torch.empty(packed_weight_elems(n, k), dtype=torch.bfloat16, device=w.device)
+    lib = core()
+    _check(lib, lib.nnis_pack_weight(w.data_ptr(), data.data_ptr(), n, k, _stream()))
+    return PackedWeight(data, n, k)
+
+
+def _packed(w, what: str) -> None:
+    if not isinstance(w, PackedWeight):
+        raise KernelError(f"{what}: the weight must be packed (pack_weight) for the matrix-core kernels")
+
+
 # Where the tiled product cuts K among blocks (few tiles, a long K) the parts meet in this scratch: 256 blocks
 # of 64 x 64 sums at most.  Kept per device; calls on one device share it, so they follow one another on one
 # stream.  It is made outside a graph capture only: a capture that finds none goes without the cut.
@@ -298,8 +355,9 @@ def _gemm_workspace(device) -> Optional[torch.Tensor]:
 
 def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, split: int = 0) -> torch.Tensor:
     """out[M, N] = x[M, K] @ w[N, K]^T on the matrix cores: bfloat16 operands,
-    32-bit accumulation, bfloat16 or float32 output.  K must be a multiple of 8."""
-    _dev(x, "x"), _dev(w, "weight"), _dev(out, "out")
+    32-bit accumulation, bfloat16 or float32 output.  ``w``: a ``PackedWeight``."""
+    _packed(w, "gemm_bf16")
+    _dev(x, "x"), _dev(out, "out")
     m, k = x.shape
     n = w.shape[0]
     if w.shape[1] != k or out.shape != (m, n):
@@ -325,9 +383,10 @@ def gemm_fused(x_in: torch.Tensor, delta: Optional[torch.Tensor], x_out: Optiona
     up for a weight of gate rows followed by up rows; or rotate-half RoPE with
     the write of keys and values into the cache (``rope``: cos, sin, tok_slot,
     tok_pos, k_pages, v_pages, block_table, heads, kv_heads, head_dim)."""
+    _packed(w, "gemm_fused")
     m, k = x_in.shape
     n = w.shape[0]
-    _dev(x_in, "x"), _dev(norm_weight, "norm weight"), _dev(w, "weight"), _dev(y, "y")
+    _dev(x_in, "x"), _dev(norm_weight, "norm weight"), _dev(y, "y")
     if x_in.dtype != torch.float32 or w.dtype != torch.bfloat16 or y.dtype != torch.bfloat16 or w.shape[1] != k:
         raise KernelError("gemm_fused: x must be float32 [m, k], the weight bfloat16 [n, k] and y bfloat16")
     if norm_weight.numel() != k:
@@ -385,10 +444,11 @@ def gemm_residual(x: torch.Tensor, w: torch.Tensor, resid: torch.Tensor, gain: t
     norm's 1 / sqrt(mean + eps) is taken by ``gemm_scaled``, which reads them.
     ``x`` may be the ``KeyRuns`` of a decode attention (where ``fits``): the
     kernel then adds the runs up itself on its way."""
+    _packed(w, "gemm_residual")
     m, k = x.shape
     n = w.shape[0]
     runs = x if isinstance(x, KeyRuns) else None
-    for t, what in ((x if runs is None else x.partial, "x"), (w, "weight"), (resid, "resid"), (gain, "gain"), (scaled, "scaled"),
+    for t, what in ((x if runs is None else x.partial, "x"), (resid, "resid"), (gain, "gain"), (scaled, "scaled"),
                     (ss, "ss")):
         _dev(t, what)
         if not t.is_contiguous():
@@ -422,9 +482,10 @@ def gemm_scaled(scaled: torch.Tensor, ss: torch.Tensor, parts: int, eps: float, 
     """y = epilogue( (W . scaled) / sqrt(sum of the parts of ss / k + eps) ):
     the second half of an RMSNorm whose first half ``gemm_residual`` took, with
     the epilogues of ``gemm_fused``."""
+    _packed(w, "gemm_scaled")
     m, k = scaled.shape
     n = w.shape[0]
-    for t, what in ((scaled, "scaled"), (ss, "ss"), (w, "weight"), (y, "y")):
+    for t, what in ((scaled, "scaled"), (ss, "ss"), (y, "y")):
         _dev(t, what)
     if scaled.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or w.shape[1] != k or not scaled.is_contiguous():
         raise KernelError("gemm_scaled: scaled must be bfloat16 [m, k] and the weight bfloat16 [n, k]")
@@ -443,16 +504,13 @@ def gemm_scaled(scaled: torch.Tensor, ss: torch.Tensor, parts: int, eps: float, 
     return y
 
 
-def _mfma_ok(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> bool:
-    return (x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and x.shape[1] % 8 == 0
-            and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0 and out.data_ptr() % 16 == 0)
-
-
-def linear(x: torch.Tensor, weight: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
-    """out = x @ weight^T.  bfloat16 operands take the matrix-core kernels;
-    32-bit operands (and widths the 16-byte loads cannot take) the ordered
-    32-bit product."""
-    if _mfma_ok(x, weight, out):
+def linear(x: torch.Tensor, weight, out: torch.Tensor) -> torch.Tensor:
+    """out = x @ weight^T.  A packed weight (bfloat16) takes the matrix-core
+    kernels; a weight as the checkpoint has it (32-bit, or a width the 16-byte
+    loads cannot take) the ordered 32-bit product."""
+    if isinstance(weight, PackedWeight):
+        if x.dtype != torch.bfloat16 or x.data_ptr() % 16 != 0 or out.data_ptr() % 16 != 0:
+            raise KernelError(f"linear: a packed weight multiplies bfloat16 rows on 16-byte boundaries, got {x.dtype}")
         return gemm_bf16(x, weight, out)
     return gemm_ordered(x, weight, out)
 

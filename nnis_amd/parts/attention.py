@@ -46,8 +46,8 @@ class CausalSelfAttention(Mixer):
 
     def bind(self, weights, rt):
         # one projection for queries, keys and values: rows q heads, k heads, v heads
-        self.qkv = Projection(torch.cat([weights[self.names["q"]], weights[self.names["k"]], weights[self.names["v"]]], dim=0))
-        self.out = Projection(weights[self.names["o"]])
+        self.qkv = Projection(torch.cat([weights[self.names["q"]], weights[self.names["k"]], weights[self.names["v"]]], dim=0), rt)
+        self.out = Projection(weights[self.names["o"]], rt)
 
     def weight_bytes(self):
         return self.qkv.weight_bytes() + self.out.weight_bytes()

@@ -42,7 +42,7 @@ class LinearHead(Part):
 
     def bind(self, weights, rt):
         # a tied head is the same device tensor as the embedding table
-        self.projection = Projection(weights[self.weight_name])
+        self.projection = Projection(weights[self.weight_name], rt)
 
     def weight_bytes(self):
         return self.projection.weight_bytes()

@@ -31,8 +31,8 @@ class GatedFeedForward(FeedForward):
         ]
 
     def bind(self, weights, rt):
-        self.gate_up = Projection(torch.cat([weights[self.names["gate"]], weights[self.names["up"]]], dim=0))
-        self.down = Projection(weights[self.names["down"]])
+        self.gate_up = Projection(torch.cat([weights[self.names["gate"]], weights[self.names["up"]]], dim=0), rt)
+        self.down = Projection(weights[self.names["down"]], rt)
 
     def weight_bytes(self):
         return self.gate_up.weight_bytes() + self.down.weight_bytes()

@@ -49,22 +49,20 @@ class PendingNorm:
         self.residual = self.x
         return out
 
-    def can_fuse(self, weight: torch.Tensor) -> bool:
+    def can_fuse(self, weight) -> bool:
         """True when ``fused`` may be called with this projection weight."""
         ops = self.rt.ops
         fits = (
             getattr(self.norm, "fusable_rms", False)
             and self.x.dtype == torch.float32
-            and weight.dtype == torch.bfloat16
+            and isinstance(weight, ops.PackedWeight)
             and self.rt.dtype == torch.bfloat16
-            and weight.shape[1] % 8 == 0
-            and weight.data_ptr() % 16 == 0
         )
         if self.scaled is not None:
             return fits
         return fits and self.rows <= ops.FUSED_MAX_TOKENS and (self.delta is None or self.delta.dtype == torch.bfloat16)
 
-    def fused(self, weight: torch.Tensor, y: torch.Tensor, epilogue: int, rope=None) -> torch.Tensor:
+    def fused(self, weight, y: torch.Tensor, epilogue: int, rope=None) -> torch.Tensor:
         """y = epilogue(weight . norm(x + delta)) in one kernel."""
         if self.scaled is not None:
             return self.rt.ops.gemm_scaled(self.scaled, self.ss, self.parts, self.norm.eps, weight, y, epilogue, rope)
@@ -87,7 +85,7 @@ class ResidualInto:
         self.norm = norm
         self.rt = rt
 
-    def can_take(self, x: torch.Tensor, weight: torch.Tensor) -> bool:
+    def can_take(self, x: torch.Tensor, weight) -> bool:
         residual = self.source.residual
         return (
             getattr(self.norm, "fusable_rms", False)
@@ -96,13 +94,11 @@ class ResidualInto:
             and residual.is_contiguous()
             and self.rt.dtype == torch.bfloat16
             and x.dtype == torch.bfloat16
-            and weight.dtype == torch.bfloat16
+            and isinstance(weight, self.rt.ops.PackedWeight)
             and weight.shape[0] == residual.shape[1]
-            and weight.shape[1] % 8 == 0
-            and weight.data_ptr() % 16 == 0
         )
 
-    def take(self, x: torch.Tensor, weight: torch.Tensor) -> PendingNorm:
+    def take(self, x: torch.Tensor, weight) -> PendingNorm:
         """residual += x @ weight^T; returns the next norm, prepared."""
         rt, residual = self.rt, self.source.residual
         rows, width = residual.shape

@@ -1,7 +1,8 @@
 """A projection y = W x with the checkpoint's [out, in] weight and no bias
 (/root/reference/crates/nnis-model/src/runtime.rs:402-426).  The kernel is
-chosen by the types at hand: 32-bit operands take the ordered 32-bit product;
-bfloat16 operands take the matrix-core kernels.
+chosen by the types at hand: a 32-bit weight takes the ordered 32-bit product;
+a bfloat16 weight is packed once, when it is bound, into the order the
+matrix-core kernels read, and takes those.
 """
 
 from __future__ import annotations
@@ -12,14 +13,23 @@ import torch
 
 
 class Projection:
-    def __init__(self, weight: torch.Tensor):
+    def __init__(self, weight: torch.Tensor, rt=None):
+        """``rt``: the runtime the projection will run under; with a bfloat16
+        one, a bfloat16 weight is kept packed only (the checkpoint's order is
+        dropped).  Without it the weight stays as it is and takes the ordered
+        product."""
         if weight.dim() != 2:
             raise ValueError(f"a projection weight is a matrix, got shape {tuple(weight.shape)}")
-        self.weight = weight.contiguous()
-        self.out_features, self.in_features = self.weight.shape
+        self.out_features, self.in_features = weight.shape
+        self._bytes = weight.numel() * weight.element_size()
+        if rt is not None and rt.dtype == torch.bfloat16 and rt.ops.packs(weight):
+            self.weight = rt.ops.pack_weight(weight.contiguous())
+        else:
+            self.weight = weight.contiguous()
 
     def weight_bytes(self) -> int:
-        return self.weight.numel() * self.weight.element_size()
+        """The weight's own bytes: what a step has to read of it."""
+        return self._bytes
 
     def __call__(self, x: torch.Tensor, rt, out_dtype: Optional[torch.dtype] = None,
                  out: Optional[torch.Tensor] = None) -> torch.Tensor:

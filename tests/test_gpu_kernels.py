@@ -95,7 +95,7 @@ def test_gemm_bf16_on_the_matrix_cores(m, n, k, y_dtype):
     x = torch.randint(-3, 4, (m, k)).to(torch.bfloat16)
     w = torch.randint(-3, 4, (n, k)).to(torch.bfloat16)
     y = torch.full((m, n), 7.0, dtype=DT[y_dtype], device="cuda")
-    ops.gemm_bf16(x.cuda(), w.cuda(), y)
+    ops.gemm_bf16(x.cuda(), ops.pack_weight(w.cuda()), y)
     want = x.double() @ w.double().t()
     if y_dtype == "float32":
         assert torch.equal(y.cpu().double(), want)
@@ -104,11 +104,27 @@ def test_gemm_bf16_on_the_matrix_cores(m, n, k, y_dtype):
     # and with ordinary values, against the 64-bit product
     x = torch.randn(m, k).to(torch.bfloat16)
     w = torch.randn(n, k).to(torch.bfloat16)
-    ops.gemm_bf16(x.cuda(), w.cuda(), y)
+    ops.gemm_bf16(x.cuda(), ops.pack_weight(w.cuda()), y)
     want = x.double() @ w.double().t()
     scale = x.double().abs() @ w.double().abs().t()
     tol = 1e-6 * math.sqrt(k) if y_dtype == "float32" else 4e-3
     assert ((y.cpu().double() - want).abs() <= tol * scale + 1e-30).all()
+
+
+@pytest.mark.parametrize("n,k", [(16, 64), (5, 8), (37, 88), (130, 200), (960, 576)])
+def test_packed_weight_order(n, k):
+    """Element (row, c) of a weight lies in strip row / 16, chunk c / 64, half c % 16 / 8, lane
+    16 * (c % 64 / 16) + row % 16, place c % 8; what pads the last strip and chunk is zeros."""
+    ops = _ops()
+    w = torch.randn(n, k).bfloat16()
+    packed = ops.pack_weight(w.cuda())
+    assert packed.shape == (n, k) and packed.data.numel() == ops.packed_weight_elems(n, k)
+    strips, chunks = (n + 15) // 16, ((k + 63) // 64) | 1  # a strip is padded to an odd number of chunks
+    got = packed.data.cpu().view(strips, chunks, 2, 4, 16, 8)  # [strip][chunk][half][k group][row][8]
+    padded = torch.zeros(strips * 16, chunks * 64, dtype=torch.bfloat16)
+    padded[:n, :k] = w
+    want = padded.view(strips, 16, chunks, 4, 2, 8).permute(0, 2, 4, 3, 1, 5)  # [strip][row][chunk][k group][half][8] ->
+    assert torch.equal(got, want.contiguous())
 
 
 def test_gemm_bf16_refuses_what_it_cannot_load():
@@ -116,9 +132,12 @@ def test_gemm_bf16_refuses_what_it_cannot_load():
     x = torch.zeros(4, 12, dtype=torch.bfloat16, device="cuda")
     w = torch.zeros(6, 12, dtype=torch.bfloat16, device="cuda")
     with pytest.raises(KernelError, match="multiple of 8"):
+        ops.pack_weight(w)
+    assert not ops.packs(w)
+    with pytest.raises(KernelError, match="must be packed"):  # a weight in the checkpoint's order is not taken for a packed one
         ops.gemm_bf16(x, w, torch.zeros(4, 6, dtype=torch.bfloat16, device="cuda"))
     out = torch.zeros(4, 6, dtype=torch.bfloat16, device="cuda")
-    ops.linear(x + 1, w + 1, out)  # the dispatcher falls back to the ordered product
+    ops.linear(x + 1, w + 1, out)  # a weight that is not packed takes the ordered product
     assert (out == 12).all()
 
 
@@ -248,6 +267,7 @@ def test_residual_projection_adds_up_key_runs(heads, kv_heads, head_dim, splits,
                                      1.0 / math.sqrt(head_dim), 0, splits, partial, waves, keep_runs=True)
     assert isinstance(runs, ops.KeyRuns) and runs.shape == (m, k) and runs.fits(rows_out)
     w = (torch.randn(rows_out, k) / math.sqrt(k)).bfloat16().cuda()
+    packed = ops.pack_weight(w)
     gain = (1 + 0.3 * torch.randn(rows_out)).bfloat16().cuda()
     resid = torch.randn(m, rows_out).cuda()
 
@@ -255,7 +275,7 @@ def test_residual_projection_adds_up_key_runs(heads, kv_heads, head_dim, splits,
         mine = resid.clone()
         scaled = torch.zeros(m, rows_out, dtype=torch.bfloat16, device="cuda")
         ss = torch.zeros(ops.gemm_residual_parts(m, rows_out), m, device="cuda")
-        parts = ops.gemm_residual(x, w, mine, gain, scaled, ss)
+        parts = ops.gemm_residual(x, packed, mine, gain, scaled, ss)
         return mine[live].cpu(), scaled[live].cpu(), ss[:parts][:, live].cpu()
 
     fused = project(runs)
@@ -327,7 +347,7 @@ def test_gemm_tiled_over_many_blocks(hint):
     x = torch.randint(-3, 4, (m, k)).to(torch.bfloat16)
     w = torch.randint(-3, 4, (n, k)).to(torch.bfloat16)
     y = torch.full((m, n), 7.0, dtype=torch.float32, device="cuda")
-    ops.gemm_bf16(x.cuda(), w.cuda(), y, hint)
+    ops.gemm_bf16(x.cuda(), ops.pack_weight(w.cuda()), y, hint)
     assert torch.equal(y.cpu().double(), x.double() @ w.double().t())
 
 
@@ -348,7 +368,7 @@ def test_residual_projection_prepares_the_norm(m, n, k, gain_dtype):
     scaled = torch.full((m, n), 9.0, dtype=torch.bfloat16, device="cuda")
     rows = ops.gemm_residual_parts(m, n)
     ss = torch.full((rows + 1, m), 7.0, device="cuda")
-    parts = ops.gemm_residual(x.cuda(), w.cuda(), resid_gpu, gain.cuda(), scaled, ss)
+    parts = ops.gemm_residual(x.cuda(), ops.pack_weight(w.cuda()), resid_gpu, gain.cuda(), scaled, ss)
     assert 0 < parts <= rows
     assert (ss[parts:] == 7.0).all()  # nothing beyond the parts it names
     got = resid_gpu.cpu().double()
@@ -387,15 +407,15 @@ def test_fused_norm_projection(m, k, with_delta, gain_dtype):
         resid = x.cuda()
         scaled = torch.empty(m, k, dtype=torch.bfloat16, device="cuda")
         ss = torch.empty(ops.gemm_residual_parts(m, k), m, device="cuda")
-        parts = ops.gemm_residual(delta.cuda(), torch.eye(k).bfloat16().cuda(), resid, gain.cuda(), scaled, ss)
+        parts = ops.gemm_residual(delta.cuda(), ops.pack_weight(torch.eye(k).bfloat16().cuda()), resid, gain.cuda(), scaled, ss)
         assert torch.equal(resid.cpu(), summed)
 
     def run(w, y, epilogue, rope=None):
         if prepared:
-            ops.gemm_scaled(scaled, ss, parts, eps, w.cuda(), y, epilogue, rope)
+            ops.gemm_scaled(scaled, ss, parts, eps, ops.pack_weight(w.cuda()), y, epilogue, rope)
             return y.cpu().double()
         x_out = torch.full((m, k), 9.0, device="cuda") if with_delta else None
-        ops.gemm_fused(x.cuda(), delta.cuda() if with_delta else None, x_out, gain.cuda(), eps, w.cuda(), y, epilogue, rope)
+        ops.gemm_fused(x.cuda(), delta.cuda() if with_delta else None, x_out, gain.cuda(), eps, ops.pack_weight(w.cuda()), y, epilogue, rope)
         if with_delta:
             assert torch.equal(x_out.cpu(), summed)  # the residual sum, exactly, written once
         return y.cpu().double()
@@ -458,7 +478,7 @@ def test_scaled_projection_with_every_tile(hint, m):
     resid = v.cuda()
     scaled = torch.empty(m, k, dtype=torch.bfloat16, device="cuda")
     ss = torch.empty(ops.gemm_residual_parts(m, k), m, device="cuda")
-    parts = ops.gemm_residual(torch.zeros(m, 8, dtype=torch.bfloat16, device="cuda"), torch.zeros(k, 8, dtype=torch.bfloat16, device="cuda"),
+    parts = ops.gemm_residual(torch.zeros(m, 8, dtype=torch.bfloat16, device="cuda"), ops.pack_weight(torch.zeros(k, 8, dtype=torch.bfloat16, device="cuda")),
                               resid, gain.cuda(), scaled, ss)
 
     def close(got, want, what):
@@ -467,12 +487,12 @@ def test_scaled_projection_with_every_tile(hint, m):
     n = 300
     w = (torch.randn(n, k) / math.sqrt(k)).bfloat16()
     y = torch.empty(m, n, dtype=torch.bfloat16, device="cuda")
-    close(ops.gemm_scaled(scaled, ss, parts, eps, w.cuda(), y, ops.EPILOGUE_STORE, None, hint).cpu().double(), normed @ w.double().t(), "store")
+    close(ops.gemm_scaled(scaled, ss, parts, eps, ops.pack_weight(w.cuda()), y, ops.EPILOGUE_STORE, None, hint).cpu().double(), normed @ w.double().t(), "store")
     inner = 200
     w = (torch.randn(2 * inner, k) / math.sqrt(k)).bfloat16()
     both = normed @ w.double().t()
     y = torch.empty(m, inner, dtype=torch.bfloat16, device="cuda")
-    close(ops.gemm_scaled(scaled, ss, parts, eps, w.cuda(), y, ops.EPILOGUE_SILU, None, hint).cpu().double(),
+    close(ops.gemm_scaled(scaled, ss, parts, eps, ops.pack_weight(w.cuda()), y, ops.EPILOGUE_SILU, None, hint).cpu().double(),
           P.silu(both[:, :inner]) * both[:, inner:], "silu")
     heads, kv_heads, head_dim = 5, 2, 64
     w = (torch.randn((heads + 2 * kv_heads) * head_dim, k) / math.sqrt(k)).bfloat16()
@@ -486,7 +506,7 @@ def test_scaled_projection_with_every_tile(hint, m):
                 tok_pos=_i32(positions), k_pages=k_pages, v_pages=v_pages, block_table=table, heads=heads,
                 kv_heads=kv_heads, head_dim=head_dim)
     y = torch.empty(m, heads * head_dim, dtype=torch.bfloat16, device="cuda")
-    got_q = ops.gemm_scaled(scaled, ss, parts, eps, w.cuda(), y, ops.EPILOGUE_ROPE, rope, hint).cpu().double()
+    got_q = ops.gemm_scaled(scaled, ss, parts, eps, ops.pack_weight(w.cuda()), y, ops.EPILOGUE_ROPE, rope, hint).cpu().double()
     pos = torch.tensor(positions)
     turned = P.rope_rotate_half(qkv[:, :heads + kv_heads], torch.from_numpy(cos_np)[pos].double(), torch.from_numpy(sin_np)[pos].double())
     close(got_q.view(m, heads, head_dim), turned[:, :heads], "queries")
@@ -699,7 +719,7 @@ def test_refusals():
     ops = _ops()
     f = lambda *shape, dtype=torch.float32: torch.zeros(*shape, dtype=dtype, device="cuda")  # noqa: E731
     with pytest.raises(KernelError, match="ss has 1 rows"):  # scratch too small for the parts it would write
-        ops.gemm_residual(f(70, 176, dtype=torch.bfloat16), f(64, 176, dtype=torch.bfloat16), f(70, 64),
+        ops.gemm_residual(f(70, 176, dtype=torch.bfloat16), ops.pack_weight(f(64, 176, dtype=torch.bfloat16)), f(70, 64),
                           f(64, dtype=torch.bfloat16), f(70, 64, dtype=torch.bfloat16), f(1, 70))
     with pytest.raises(KernelError):
         ops.gemm_ordered(f(3, 8), f(5, 9), f(3, 5))

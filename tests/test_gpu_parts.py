@@ -157,7 +157,7 @@ def _register_toy():
             return [TensorSpec(self.weight_name, (self.width, self.width))]
 
         def bind(self, weights, rt):
-            self.proj = Projection(weights[self.weight_name])
+            self.proj = Projection(weights[self.weight_name], rt)
 
         def cache_request(self):
             return StateRequest((self.width,), "float32")
