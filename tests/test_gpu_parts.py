@@ -286,3 +286,195 @@ def test_toy_architecture_with_a_stateful_mixer(tmp_path, dtype):
     assert again == sa
     rows = engine.step([StepEntry(again, b, list(range(13)))]).cpu()
     assert_close(rows, want_b, dtype, "toy reused slot")
+
+
+# ---------------------------------------------------------------------------
+# a second toy architecture: a feed-forward that routes each token to one of
+# several experts, positions learned and added to the embedding (no rotation),
+# and a norm of another kind (centred) -- all three defined here
+# ---------------------------------------------------------------------------
+
+def _register_routed_toy():
+    from nnis_amd.config import register_architecture
+    from nnis_amd.models import ModelSpec, ScheduleEntry
+    from nnis_amd.parts import FeedForward, Norm, PositionEncoding, TensorSpec, register_part
+    from nnis_amd.parts.linear import Projection
+
+    class RoutedFeedForward(FeedForward):
+        """y = p_e * W2_e relu(W1_e x) for the expert e with the largest router logit, p its softmax weight."""
+
+        def __init__(self, width, inner, experts, router, first, second):
+            self.width, self.inner, self.experts = width, inner, experts
+            self.names = (router, first, second)
+
+        def tensors(self):
+            router, first, second = self.names
+            specs = [TensorSpec(router, (self.experts, self.width))]
+            for e in range(self.experts):
+                specs += [TensorSpec(f"{first}.{e}", (self.inner, self.width)), TensorSpec(f"{second}.{e}", (self.width, self.inner))]
+            return specs
+
+        def bind(self, weights, rt):
+            router, first, second = self.names
+            self.router = weights[router].float()  # router logits are taken in 32-bit
+            self.first = [Projection(weights[f"{first}.{e}"], rt) for e in range(self.experts)]
+            self.second = [Projection(weights[f"{second}.{e}"], rt) for e in range(self.experts)]
+
+        def forward(self, x, ctx, rt):
+            logits = x.float() @ self.router.t()
+            weight, chosen = torch.softmax(logits, dim=-1).max(dim=-1)
+            y = torch.zeros(x.shape, dtype=torch.float32, device=x.device)
+            for e in range(self.experts):
+                rows = (chosen == e).nonzero().flatten()
+                if rows.numel():
+                    hidden = torch.relu(self.first[e](x[rows].contiguous(), rt))
+                    y[rows] = self.second[e](hidden, rt).float() * weight[rows, None]
+            return y.to(rt.dtype)
+
+    class LearnedPositions(PositionEncoding):
+        """x_t += table[position of t]."""
+
+        def __init__(self, width, max_positions, weight):
+            self.width, self.max_positions, self.weight_name = width, max_positions, weight
+
+        def tensors(self):
+            return [TensorSpec(self.weight_name, (self.max_positions, self.width))]
+
+        def bind(self, weights, rt):
+            self.table = weights[self.weight_name].float()
+
+        def embed(self, x, ctx, rt):
+            live = ctx.tok_slot[:x.shape[0]] >= 0
+            rows = self.table[ctx.tok_pos[:x.shape[0]].long().clamp(min=0)]
+            return x + rows * live[:, None]
+
+    class CentredNorm(Norm):
+        """(x - mean) / sqrt(var + eps) * weight."""
+
+        def __init__(self, width, eps, weight):
+            self.width, self.eps, self.weight_name = width, eps, weight
+
+        def tensors(self):
+            return [TensorSpec(self.weight_name, (self.width,), init="gain")]
+
+        def bind(self, weights, rt):
+            self.gain = weights[self.weight_name].float()
+
+        def forward(self, x, rt, rows=None):
+            x = x.float() if rows is None else x.float()[rows.long()]
+            centred = x - x.mean(dim=-1, keepdim=True)
+            return (centred * torch.rsqrt(centred.pow(2).mean(dim=-1, keepdim=True) + self.eps) * self.gain).to(rt.dtype)
+
+        def add_forward(self, residual, delta, rt, rows=None):
+            residual += delta.float()
+            return self.forward(residual, rt, rows)
+
+    @dataclass(frozen=True)
+    class RoutedConfig:
+        width: int
+        vocab_size: int
+        layers: int
+        experts: int
+        raw: dict
+
+        @classmethod
+        def from_dict(cls, raw):
+            return cls(raw["width"], raw["vocab_size"], raw["layers"], raw["experts"], dict(raw))
+
+    def routed_spec(cfg):
+        w = cfg.width
+        layers = []
+        for index in range(cfg.layers):
+            p = f"h.{index}."
+            layers.append({
+                "kind": "pre_norm", "width": w,
+                "norm1": {"kind": "centred", "width": w, "eps": 1e-4, "weight": p + "ln1"},
+                "mixer": {"kind": "causal_attention", "width": w, "heads": 3, "kv_heads": 3, "head_dim": 16, "position": None,
+                          "q": p + "q", "k": p + "k", "v": p + "v", "o": p + "o"},
+                "norm2": {"kind": "centred", "width": w, "eps": 1e-4, "weight": p + "ln2"},
+                # dense in the even layers, routed in the odd ones
+                "feed_forward": ({"kind": "gated", "width": w, "inner": 72, "gate": p + "g", "up": p + "u", "down": p + "d"}
+                                 if index % 2 == 0 else
+                                 {"kind": "routed_relu", "width": w, "inner": 40, "experts": cfg.experts, "router": p + "router",
+                                  "first": p + "w1", "second": p + "w2"})})
+        return ModelSpec(
+            architecture="RoutedToyForCausalLM", width=w, vocab_size=cfg.vocab_size, max_positions=128, stored_dtype="bfloat16",
+            embedding={"kind": "table", "vocab_size": cfg.vocab_size, "width": w, "weight": "wte"},
+            positions={"learned": {"kind": "learned", "width": w, "max_positions": 128, "weight": "wpe"}},
+            layers=layers, schedule=[ScheduleEntry(i) for i in range(cfg.layers)],
+            final_norm={"kind": "centred", "width": w, "eps": 1e-4, "weight": "ln_f"},
+            head={"kind": "linear", "vocab_size": cfg.vocab_size, "width": w, "weight": "head", "tied_to": "wte"},
+            config_json=cfg.raw)
+
+    register_part("feed_forward", "routed_relu", RoutedFeedForward, replace=True)
+    register_part("position", "learned", LearnedPositions, replace=True)
+    register_part("norm", "centred", CentredNorm, replace=True)
+    register_architecture("RoutedToyForCausalLM", RoutedConfig, routed_spec, replace=True)
+
+
+def _plain_routed_toy(folder, ids, layers, experts):
+    from safetensors import safe_open
+
+    with safe_open(folder + "/model.safetensors", framework="pt") as handle:
+        w = {n: handle.get_tensor(n).float() for n in handle.keys()}
+    t = len(ids)
+
+    def norm(x, gain):
+        centred = x - x.mean(dim=-1, keepdim=True)
+        return centred * torch.rsqrt(centred.pow(2).mean(dim=-1, keepdim=True) + 1e-4) * gain
+
+    x = P.embedding(w["wte"], ids) + w["wpe"][:t]
+    chosen_all = []
+    for layer in range(layers):
+        p = f"h.{layer}."
+        h = norm(x, w[p + "ln1"])
+        q, k, v = (P.linear(h, w[p + n]).view(t, 3, 16) for n in "qkv")
+        x = x + P.linear(P.causal_attention(q, k, v, 0.25).reshape(t, 48), w[p + "o"])
+        h = norm(x, w[p + "ln2"])
+        if layer % 2 == 0:
+            x = x + P.swiglu(h, w[p + "g"], w[p + "u"], w[p + "d"])
+        else:
+            weight, chosen = torch.softmax(P.linear(h, w[p + "router"]), dim=-1).max(dim=-1)
+            chosen_all.append(chosen)
+            y = torch.stack([P.linear(torch.relu(P.linear(h[i:i + 1], w[f"{p}w1.{int(e)}"])), w[f"{p}w2.{int(e)}"])[0]
+                             for i, e in enumerate(chosen)])
+            x = x + y * weight[:, None]
+    return P.linear(norm(x, w["ln_f"]), w["wte"]), chosen_all
+
+
+def test_toy_architecture_with_routing_and_learned_positions(tmp_path):
+    """A feed-forward with routing in some layers and a dense one in others, positions added to the
+    embedding, attention without rotation and a norm of another kind: registered, built, loaded and
+    stepped (whole prompts of unequal lengths, then token by token) without a change to the library."""
+    import nnis_amd
+    from nnis_amd.api import load_engine
+    from nnis_amd.engine.batch import StepEntry
+
+    _register_routed_toy()
+    folder = str(tmp_path / "routed")
+    raw = {"architectures": ["RoutedToyForCausalLM"], "model_type": "routed_toy", "width": 48, "vocab_size": 157, "layers": 4,
+           "experts": 3}
+    nnis_amd.write_random_model(folder, raw, seed=11)
+    # random routers of N(0, 0.02) would leave every choice a near tie: make them decisive
+    from nnis_amd.weights.safetensors_io import SafetensorsFile, write_safetensors
+
+    stored = SafetensorsFile(folder + "/model.safetensors")
+    tensors = {name: stored.tensor(name).clone() for name in stored.names()}
+    stored.close()
+    for name in tensors:
+        if name.endswith("router"):
+            tensors[name] = (tensors[name].float() * 200).to(tensors[name].dtype)
+    write_safetensors(folder + "/model.safetensors", tensors.items())
+    engine = load_engine(folder, dtype="float32", max_tokens=512)
+    rng = np.random.default_rng(5)
+    a, b = rng.integers(0, 157, size=37).tolist(), rng.integers(0, 157, size=9).tolist()
+    (want_a, chosen_a), (want_b, _) = _plain_routed_toy(folder, a, 4, 3), _plain_routed_toy(folder, b, 4, 3)
+    assert all(len(set(c.tolist())) > 1 for c in chosen_a), "the test's tokens must reach more than one expert"
+    sa, sb = engine.start_sequence(), engine.start_sequence()
+    rows = engine.step([StepEntry(sa, a[:30], list(range(30))), StepEntry(sb, b[:2], [0, 1])]).cpu()
+    assert_close(rows[:30], want_a[:30], "float32", "routed prompt a")
+    assert_close(rows[30:], want_b[:2], "float32", "routed prompt b")
+    for i in range(7):
+        rows = engine.step([StepEntry(sb, [b[2 + i]], [0]), StepEntry(sa, [a[30 + i]], [0])]).cpu()
+        assert_close(rows[0], want_b[2 + i], "float32", f"routed decode b {i}")
+        assert_close(rows[1], want_a[30 + i], "float32", f"routed decode a {i}")
