@@ -71,6 +71,8 @@ def main() -> int:
     parser.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     parser.add_argument("--seed", type=int, default=0)
     parser.add_argument("--no-points", action="store_true", help="skip the batch-1 and batch-64 decode points")
+    parser.add_argument("--prompt-min", type=int, default=128, help="shortest prompt of the decode batches")
+    parser.add_argument("--prompt-max", type=int, default=2048, help="longest prompt of the decode batches (within the context)")
     args = parser.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this library runs on one GPU; --gpus {args.gpus} is not supported")
@@ -78,7 +80,8 @@ def main() -> int:
     SHAPE.clear()
     SHAPE.update(SHAPES[args.shape])
     args.layers = args.layers or SHAPE["layers"]
-    longest_prompt = min(2048, SHAPE["context"] - args.steps - args.warmup - 1)
+    longest_prompt = min(args.prompt_max, SHAPE["context"] - args.steps - args.warmup - 1)
+    shortest_prompt = max(1, min(args.prompt_min, longest_prompt))
 
     import numpy as np
     import torch
@@ -95,7 +98,7 @@ def main() -> int:
 
         def decode_run(batch, steps, warmup):
             """Prefills ``batch`` prompts in one step, then times ``steps`` decode steps."""
-            lengths = rng.integers(128, longest_prompt + 1, size=batch).tolist()
+            lengths = rng.integers(shortest_prompt, longest_prompt + 1, size=batch).tolist()
             room = batch * SHAPE["context"]  # every sequence may grow to the model's context
             engine = load_engine(folder, dtype=args.dtype, max_tokens=room)
             selector = DeviceSelector(engine)
@@ -188,7 +191,7 @@ def main() -> int:
             "model": f"{SHAPE['name']} shape (Llama)", "layers": args.layers, "layers_of_model": SHAPE["layers"],
             "hidden": SHAPE["hidden"], "heads": SHAPE["heads"], "kv_heads": SHAPE["kv_heads"], "head_dim": SHAPE["head_dim"],
             "inner": SHAPE["inner"], "vocab": SHAPE["vocab"], "tied_head": SHAPE["tied"], "context": SHAPE["context"],
-            "global_batch": args.batch, "seq_len": SHAPE["context"], "prompt_min": 128, "prompt_max": longest_prompt,
+            "global_batch": args.batch, "seq_len": SHAPE["context"], "prompt_min": shortest_prompt, "prompt_max": longest_prompt,
             "mean_prompt": round(float(np.mean(lengths)), 1), "parallelism": "single GPU", "sampling": "greedy on device",
         },
         "prefill": {
