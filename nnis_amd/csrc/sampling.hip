@@ -71,7 +71,7 @@ __device__ int count_at_least(const RowView& r, unsigned t, int* scratch) {
 __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
     const float* __restrict__ logits, double* __restrict__ weights, int vocab, const int* __restrict__ row_slot,
     unsigned long long* __restrict__ rng, const float* __restrict__ temperature, const int* __restrict__ top_k,
-    const float* __restrict__ top_p, int* __restrict__ out) {
+    const float* __restrict__ top_p, int by_slot, int* __restrict__ out) {
   __shared__ double scratch_d[kSampleThreads / kWave];
   __shared__ int scratch_i[kSampleThreads / kWave];
   __shared__ int found;
@@ -108,7 +108,8 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
   __syncthreads();
   for (int i = 0; i < kSampleThreads / kWave; ++i) key_max = wave_keys[i] > key_max ? wave_keys[i] : key_max;
   const unsigned max_bits = (key_max & 0x80000000u) ? (key_max & 0x7fffffffu) : ~key_max;
-  const double inv_t = 1.0 / (double)temperature[row];
+  const int at = by_slot ? slot : row;  // where the row's options lie: per sequence (kept with its slot) or per row
+  const double inv_t = 1.0 / (double)temperature[at];
   const double max_scaled = (double)__uint_as_float(max_bits) * inv_t;
   for (int c = threadIdx.x; c < vocab; c += kSampleThreads) w[c] = exp((double)r.logits[c] * inv_t - max_scaled);
   __syncthreads();
@@ -119,7 +120,7 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
   bool limited = false;
   double total = mass_at_least(r, 0u, scratch_d);
 
-  const int k = top_k[row];
+  const int k = top_k[at];
   if (k > 0 && k < vocab) {
     unsigned t = 0;
     for (int bit = 31; bit >= 0; --bit) {
@@ -134,7 +135,7 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
     total = mass_at_least(r, t + 1u, scratch_d) + (double)cut_ties * weight_at;
   }
 
-  const float p = top_p[row];
+  const float p = top_p[at];
   if (p > 0.0f && p <= 1.0f) {
     const double threshold = (double)p * total;
     unsigned t = 0;
@@ -226,12 +227,12 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
 
 extern "C" int nnis_sample(const float* logits, double* weights, int rows, int vocab, const int* row_slot,
                            unsigned long long* rng, const float* temperature, const int* top_k, const float* top_p,
-                           int* out, void* stream) {
+                           int by_slot, int* out, void* stream) {
   NNIS_REQUIRE(rows >= 0 && vocab > 0, "sample: bad sizes rows=%d vocab=%d", rows, vocab);
   NNIS_REQUIRE((long long)vocab <= 65535LL * kSampleThreads, "sample: vocabulary %d is too large for this kernel", vocab);
   if (rows == 0) return 0;
   hipLaunchKernelGGL(sample_kernel, dim3(rows), dim3(kSampleThreads), 0, (hipStream_t)stream, logits, weights, vocab,
-                     row_slot, rng, temperature, top_k, top_p, out);
+                     row_slot, rng, temperature, top_k, top_p, by_slot, out);
   NNIS_LAUNCH_CHECK("sample");
   return 0;
 }

@@ -165,7 +165,7 @@ def generate(engine, requests: Sequence[GenerationRequest], selector=None, max_b
 
 
 def _run_ahead(engine, selector, requests, results, slot_of, rows, pending, take) -> None:
-    """The decode steps of a batch of greedy sequences, a step ahead of the
+    """The decode steps of a batch, greedy or sampled, a step ahead of the
     host.  ``pending``: the selection of the tokens that come next, asked for
     but not read; its row j belongs to request ``rows[j]``.  Before the host
     reads them, the step that feeds them back is put on the stream, with their
@@ -188,7 +188,8 @@ def _run_ahead(engine, selector, requests, results, slot_of, rows, pending, take
             if len(onward) != len(rows):
                 ids = ids.index_select(0, torch.tensor(onward, dtype=torch.long, device=ids.device)).contiguous()
             logits = engine.step_from_device([slot_of[rows[j]] for j in onward], ids)
-            following = selector.select_start(logits, [slot_of[rows[j]] for j in onward], [None] * len(onward))
+            following = selector.select_start(logits, [slot_of[rows[j]] for j in onward],
+                                              [requests[rows[j]].sampling for j in onward])
         tokens = pending.result()
         for j, index in enumerate(rows):
             if index in slot_of:  # (else ended by an earlier token: this row ran for nothing)

@@ -1,20 +1,22 @@
 """Token selection on the device for a batch of logit rows: argmax for greedy
-rows, the sampling kernel for seeded rows.  Each sequence's generator state
-lives in the cache's per-slot state region, so a sequence's draws do not
-depend on what else is in the batch
-(/root/reference/crates/nnis-model/src/session_batch.rs:7-8)."""
+rows, the sampling kernel for seeded rows.  Each sequence's generator state and
+its sampling options live in the cache's per-slot state regions, so a
+sequence's draws do not depend on what else is in the batch
+(/root/reference/crates/nnis-model/src/session_batch.rs:7-8) and a step's
+selection needs nothing from the host but the rows' slots."""
 
 from __future__ import annotations
 
 from typing import List, Optional, Sequence
 
-import numpy as np
 import torch
 
 from ..errors import InvalidInput
 from .params import SamplingParams
 
 RNG_REGION = "sampler.rng"
+# the options of a sequence that samples, set when it starts (``DeviceSelector.start``)
+OPTION_REGIONS = {"sampler.temperature": torch.float32, "sampler.top_k": torch.int32, "sampler.top_p": torch.float32}
 
 
 class PendingTokens:
@@ -28,7 +30,11 @@ class PendingTokens:
 
     def result(self) -> List[int]:
         self._event.synchronize()
-        return self._host.tolist()
+        tokens = self._host.tolist()
+        for row, token in enumerate(tokens):
+            if token < 0:  # what the sampling kernel leaves in place of a token it will not draw
+                raise InvalidInput(f"sampling refused row {row}: a logit is not finite")
+        return tokens
 
 
 class DeviceSelector:
@@ -37,34 +43,45 @@ class DeviceSelector:
         self.rt = engine.rt
         self.vocab_size = engine.vocab_size
         cache = engine.cache
-        if RNG_REGION not in cache.state_regions:
-            cache.add_state_region(RNG_REGION, (), torch.int64)
+        for name, dtype in {RNG_REGION: torch.int64, **OPTION_REGIONS}.items():
+            if name not in cache.state_regions:
+                cache.add_state_region(name, (), dtype)
         self.rng = cache.state_regions[RNG_REGION]
+        self.temperature, self.top_k, self.top_p = (cache.state_regions[name] for name in OPTION_REGIONS)
         self._weights = None
-        self._picked = None       # int32 on the device, reused from step to step
-        self._picked_host = None  # its pinned twin: the copy back needs no staging
         self._pairs = [None, None]  # (device, pinned host, event) of select_start, used in turn
         self._turn = 0
+        self._row_slots = (None, None)  # the slots of the rows that sample (-1: a greedy row), as last asked for, and on the device
 
-    def _to_host(self, picked: torch.Tensor, rows: int) -> List[int]:
-        if self._picked_host is None or self._picked_host.numel() < rows:
-            self._picked_host = torch.empty(max(rows, 64), dtype=torch.int32, pin_memory=True)
-        host = self._picked_host[:rows]
-        host.copy_(picked[:rows], non_blocking=True)
-        torch.cuda.current_stream().synchronize()
-        return host.tolist()
+    def start(self, slot: int, params: Optional[SamplingParams]) -> None:
+        """Called when a sequence starts: seeds its generator and keeps its options with its slot."""
+        if params is not None:
+            params.validate(self.vocab_size)
+            seed = params.seed if params.seed < (1 << 63) else params.seed - (1 << 64)
+            self.rng[slot] = seed
+            self.temperature[slot] = float(params.temperature)
+            self.top_k[slot] = int(params.top_k or 0)
+            self.top_p[slot] = float(params.top_p or 0.0)
+
+    def _sampling_rows(self, slots: Sequence[int], params: Sequence[Optional[SamplingParams]]) -> torch.Tensor:
+        """int32 on the device: a row's slot if it samples, -1 if it is greedy.  Copied only when it changes
+        (a batch's rows change when a sequence ends, not from step to step)."""
+        key = tuple(int(s) if p is not None else -1 for s, p in zip(slots, params))
+        if self._row_slots[0] != key:
+            self._row_slots = (key, torch.tensor(key, dtype=torch.int32, device=self.rt.device))
+        return self._row_slots[1]
 
     def select_start(self, logits: torch.Tensor, slots: Sequence[int], params: Sequence[Optional[SamplingParams]]):
-        """Greedy rows only: the selection is put on the stream and the copy of
-        the tokens to the host behind it; nothing waits.  Returns a
-        ``PendingTokens`` -- the tokens on the device (for a step that starts
-        before the host has read them) and ``result()``, which waits for the
-        copy -- or None when a row samples (then ``select`` is the way).  Two
-        results may be outstanding at a time: the third call reuses the first's
-        buffers."""
-        if any(p is not None for p in params):
-            return None
+        """The selection of one token per row of ``logits`` (float32 [rows,
+        vocab] on the device) is put on the stream and the copy of the tokens
+        to the host behind it; nothing waits.  ``params[j]`` says whether row j
+        samples (its options are those its sequence started with) or is greedy
+        (None).  Returns a ``PendingTokens``: the tokens on the device (for a
+        step that starts before the host has read them) and ``result()``, which
+        waits for the copy.  Two results may be outstanding at a time: the
+        third call reuses the first's buffers."""
         rows = logits.shape[0]
+        ops = self.rt.ops
         self._turn ^= 1
         pair = self._pairs[self._turn]
         if pair is None or pair[0].numel() < rows:
@@ -72,49 +89,17 @@ class DeviceSelector:
             pair = self._pairs[self._turn] = (torch.empty(size, dtype=torch.int32, device=self.rt.device),
                                               torch.empty(size, dtype=torch.int32, pin_memory=True), torch.cuda.Event())
         device, host, event = pair
-        self.rt.ops.argmax(logits, device[:rows])
+        ops.argmax(logits, device[:rows])
+        if any(p is not None for p in params):
+            if self._weights is None or self._weights.shape[0] < rows:
+                self._weights = torch.empty((max(rows, 8), self.vocab_size), dtype=torch.float64, device=self.rt.device)
+            # the rows that sample are written over; a greedy row keeps its argmax
+            ops.sample(logits, self._weights, self._sampling_rows(slots, params), self.rng, self.temperature, self.top_k,
+                       self.top_p, device[:rows], by_slot=True)
         host[:rows].copy_(device[:rows], non_blocking=True)
         event.record()
         return PendingTokens(device[:rows], host[:rows], event)
 
-    def start(self, slot: int, params: Optional[SamplingParams]) -> None:
-        """Called when a sequence starts: seeds its generator."""
-        if params is not None:
-            params.validate(self.vocab_size)
-            seed = params.seed if params.seed < (1 << 63) else params.seed - (1 << 64)
-            self.rng[slot] = seed
-
     def select(self, logits: torch.Tensor, slots: Sequence[int], params: Sequence[Optional[SamplingParams]]) -> List[int]:
-        """One token per row of ``logits`` (float32 [rows, vocab] on the device)."""
-        rows = logits.shape[0]
-        ops = self.rt.ops
-        if self._picked is None or self._picked.numel() < rows:
-            self._picked = torch.empty(max(rows, 64), dtype=torch.int32, device=self.rt.device)
-        picked = self._picked[:rows]
-        ops.argmax(logits, picked)
-        if any(p is not None for p in params):
-            row_slot = np.asarray([s if p is not None else -1 for s, p in zip(slots, params)], dtype=np.int32)
-            temperature = np.asarray([p.temperature if p is not None else 1.0 for p in params], dtype=np.float32)
-            top_k = np.asarray([(p.top_k or 0) if p is not None else 0 for p in params], dtype=np.int32)
-            top_p = np.asarray([(p.top_p or 0.0) if p is not None else 0.0 for p in params], dtype=np.float32)
-            if self._weights is None or self._weights.shape[0] < rows:
-                self._weights = torch.empty((max(rows, 8), self.vocab_size), dtype=torch.float64, device=self.rt.device)
-            sampled = torch.full((rows,), -3, dtype=torch.int32, device=self.rt.device)
-            ops.sample(
-                logits, self._weights,
-                torch.from_numpy(row_slot).to(self.rt.device), self.rng,
-                torch.from_numpy(temperature).to(self.rt.device), torch.from_numpy(top_k).to(self.rt.device),
-                torch.from_numpy(top_p).to(self.rt.device), sampled,
-            )
-            sampled_host = sampled.cpu().tolist()
-            picked_host = picked.cpu().tolist()
-            out = []
-            for row, p in enumerate(params):
-                if p is None:
-                    out.append(picked_host[row])
-                else:
-                    if sampled_host[row] < 0:
-                        raise InvalidInput(f"sampling refused row {row}: a logit is not finite")
-                    out.append(sampled_host[row])
-            return out
-        return self._to_host(picked, rows)
+        """One token per row of ``logits``, on the host."""
+        return self.select_start(logits, slots, params).result()

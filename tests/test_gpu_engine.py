@@ -173,6 +173,67 @@ def test_running_a_step_ahead_changes_nothing(model_dirs, dtype):
     assert len(got[0][0]) <= 4 and len(got[4][0]) <= 2
 
 
+def test_sampled_batches_run_a_step_ahead_too(model_dirs):
+    """A batch whose rows sample (each with options and a seed of its own), next to greedy rows, runs a
+    step ahead of the host like a greedy one: the tokens are those of the loop that waits for every token,
+    with a stop token met on the way, requests that end early and slots used again by a second batch."""
+    from nnis_amd.engine.generate import GenerationRequest, generate
+    from nnis_amd.sampling import SamplingParams
+    from nnis_amd.sampling.device import DeviceSelector
+
+    engine = _engine(model_dirs, "B", "bfloat16", max_tokens=16 * 64)
+    assert engine.use_graphs
+    config, _ = TINY_CONFIGS["B"]
+    rng = np.random.default_rng(3)
+    prompts = [rng.integers(0, config["vocab_size"], size=n).tolist() for n in (4, 19, 1, 33, 8)]
+    sampling = [SamplingParams(seed=11, temperature=0.7), None, SamplingParams(seed=12, temperature=1.3, top_k=5),
+                SamplingParams(seed=13, temperature=0.9, top_p=0.8), SamplingParams(seed=2 ** 64 - 5, temperature=1.0)]
+    limits = [10, 6, 3, 10, 1]
+
+    class StepByStep:
+        def __init__(self, inner):
+            self.start, self.select = inner.start, inner.select
+
+    def run(selector, stops):
+        requests = [GenerationRequest(p, max_new_tokens=n, stop_token_ids=stops[i], sampling=sampling[i])
+                    for i, (p, n) in enumerate(zip(prompts, limits))]
+        out = generate(engine, requests, selector=selector, max_batch=3)
+        assert engine.free_slots() == engine.cache.max_slots
+        return [(r.tokens, r.finish_reason) for r in out]
+
+    none = [[] for _ in prompts]
+    free = run(StepByStep(DeviceSelector(engine)), none)
+    assert run(DeviceSelector(engine), none) == free
+    assert [len(tokens) for tokens, _ in free] == limits
+    stops = [[] for _ in prompts]
+    stops[0], stops[3] = [free[0][0][4]], [free[3][0][2]]  # the 5th sampled token of request 0, the 3rd of request 3
+    want = run(StepByStep(DeviceSelector(engine)), stops)
+    got = run(DeviceSelector(engine), stops)
+    assert got == want
+    assert got[0][1] == "stop" and len(got[0][0]) <= 5 and got[3][1] == "stop" and got[1][1] == "length"
+
+
+def test_selector_refuses_a_row_that_is_not_finite(model_dirs):
+    from nnis_amd.errors import InvalidInput
+    from nnis_amd.sampling import SamplingParams
+    from nnis_amd.sampling.device import DeviceSelector
+
+    engine = _engine(model_dirs, "A", "float32", max_tokens=4 * 64)
+    selector = DeviceSelector(engine)
+    slots = [engine.start_sequence(), engine.start_sequence()]
+    params = [SamplingParams(seed=1), None]
+    selector.start(slots[0], params[0])
+    selector.start(slots[1], params[1])
+    logits = torch.zeros(2, engine.vocab_size, device="cuda")
+    logits[1, 5] = 3.0
+    assert selector.select(logits, slots, params)[1] == 5  # the greedy row, next to a row that samples
+    logits[0, 7] = float("inf")
+    with pytest.raises(InvalidInput, match="row 0"):
+        selector.select(logits, slots, params)
+    for slot in slots:
+        engine.end_sequence(slot)
+
+
 def test_command_line(model_dirs):
     plain = P.PlainLlama(model_dirs["B"])
     prompt = [3, 141, 59, 26, 535]
