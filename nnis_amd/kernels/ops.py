@@ -6,7 +6,6 @@ runs hand-written device code; none has a host or library stand-in.
 from __future__ import annotations
 
 import ctypes
-import os
 from typing import Optional
 
 import torch
@@ -599,7 +598,7 @@ def attention_decode_bf16(q, out, k_pages, v_pages, block_table, tok_slot, tok_p
 
 # Up to this many tokens a decode step leaves its runs of keys to the output projection; beyond, every block of
 # the projection making the same activations again costs more than the kernel between the two.
-KEY_RUNS_MOST_TOKENS = int(os.environ.get("NNIS_KEY_RUNS_TOKENS", "4"))
+KEY_RUNS_MOST_TOKENS = 4
 
 
 class KeyRuns:
