@@ -11,7 +11,7 @@ import pytest
 import torch
 
 import plain_llama as P
-from gpu_helpers import assert_close, cache_for, context, runtime
+from gpu_helpers import assert_close, cache_for, context, runtime, tolerance
 
 pytestmark = pytest.mark.gpu
 DTYPES = ["float32", "bfloat16"]
@@ -478,3 +478,124 @@ def test_toy_architecture_with_routing_and_learned_positions(tmp_path):
         rows = engine.step([StepEntry(sb, [b[2 + i]], [0]), StepEntry(sa, [a[30 + i]], [0])]).cpu()
         assert_close(rows[0], want_b[2 + i], "float32", f"routed decode b {i}")
         assert_close(rows[1], want_a[30 + i], "float32", f"routed decode a {i}")
+
+
+# ---------------------------------------------------------------------------
+# a third toy architecture: layers that read all keys next to layers that read
+# a window of them, with head sizes of their own -- two groups of the cache
+# ---------------------------------------------------------------------------
+
+_WINDOW = 40
+
+
+def _register_windowed_toy():
+    from nnis_amd.config import register_architecture
+    from nnis_amd.models import ModelSpec, ScheduleEntry
+
+    @dataclass(frozen=True)
+    class WindowedConfig:
+        width: int
+        vocab_size: int
+        layers: int
+        raw: dict
+
+        @classmethod
+        def from_dict(cls, raw):
+            return cls(raw["width"], raw["vocab_size"], raw["layers"], dict(raw))
+
+    def windowed_spec(cfg):
+        w = cfg.width
+        layers = []
+        for index in range(cfg.layers):
+            p = f"l.{index}."
+            wide = index % 2 == 0  # even layers: all keys, 4 heads of 16 on 2; odd: a window, 2 heads of 32 on 1
+            layers.append({
+                "kind": "pre_norm", "width": w,
+                "norm1": {"kind": "rms", "width": w, "eps": 1e-5, "weight": p + "n1"},
+                "mixer": {"kind": "causal_attention", "width": w, "heads": 4 if wide else 2, "kv_heads": 2 if wide else 1,
+                          "head_dim": 16 if wide else 32, "position": "rope16" if wide else "rope32",
+                          "window": None if wide else _WINDOW, "q": p + "q", "k": p + "k", "v": p + "v", "o": p + "o"},
+                "norm2": {"kind": "rms", "width": w, "eps": 1e-5, "weight": p + "n2"},
+                "feed_forward": {"kind": "gated", "width": w, "inner": 88, "gate": p + "g", "up": p + "u", "down": p + "d"}})
+        return ModelSpec(
+            architecture="WindowedToyForCausalLM", width=w, vocab_size=cfg.vocab_size, max_positions=256, stored_dtype="bfloat16",
+            embedding={"kind": "table", "vocab_size": cfg.vocab_size, "width": w, "weight": "emb"},
+            positions={"rope16": {"kind": "rotary_half", "rot_dim": 16, "theta": 10000.0, "max_positions": 256},
+                       "rope32": {"kind": "rotary_half", "rot_dim": 32, "theta": 500.0, "max_positions": 256}},
+            layers=layers, schedule=[ScheduleEntry(i) for i in range(cfg.layers)],
+            final_norm={"kind": "rms", "width": w, "eps": 1e-5, "weight": "norm"},
+            head={"kind": "linear", "vocab_size": cfg.vocab_size, "width": w, "weight": "head", "tied_to": "emb"},
+            config_json=cfg.raw)
+
+    register_architecture("WindowedToyForCausalLM", WindowedConfig, windowed_spec, replace=True)
+
+
+def _plain_windowed_toy(folder, ids, layers, window=_WINDOW):
+    from safetensors import safe_open
+
+    with safe_open(folder + "/model.safetensors", framework="pt") as handle:
+        w = {n: handle.get_tensor(n).float() for n in handle.keys()}
+    t = len(ids)
+    x = P.embedding(w["emb"], ids)
+    for layer in range(layers):
+        p = f"l.{layer}."
+        wide = layer % 2 == 0
+        heads, kv_heads, hd, theta = (4, 2, 16, 10000.0) if wide else (2, 1, 32, 500.0)
+        cos, sin = (torch.from_numpy(a)[:t] for a in P.rope_tables(256, hd, theta))
+        h = P.rms_norm(x, w[p + "n1"], 1e-5)
+        q = P.rope_rotate_half(P.linear(h, w[p + "q"]).view(t, heads, hd), cos, sin)
+        k = P.rope_rotate_half(P.linear(h, w[p + "k"]).view(t, kv_heads, hd), cos, sin)
+        v = P.linear(h, w[p + "v"]).view(t, kv_heads, hd)
+        if wide:
+            mixed = P.causal_attention(q, k, v, hd ** -0.5)
+        else:  # the query at p reads keys p - window + 1 .. p
+            k_all, v_all = (a.repeat_interleave(heads // kv_heads, dim=1) for a in (k, v))
+            scores = torch.einsum("qhd,khd->hqk", q, k_all) * hd ** -0.5
+            place = torch.arange(t)
+            seen = (place[None, :] <= place[:, None]) & (place[None, :] > place[:, None] - window)
+            scores = scores.masked_fill(~seen[None], float("-inf"))
+            mixed = torch.einsum("hqk,khd->qhd", torch.softmax(scores, dim=-1), v_all)
+        x = x + P.linear(mixed.reshape(t, heads * hd), w[p + "o"])
+        x = x + P.swiglu(P.rms_norm(x, w[p + "n2"], 1e-5), w[p + "g"], w[p + "u"], w[p + "d"])
+    return P.linear(P.rms_norm(x, w["norm"], 1e-5), w["emb"])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_toy_architecture_with_windowed_layers(tmp_path, dtype):
+    """Layers that keep all keys and layers that read a window of 40, with head sizes of their own: the cache
+    gives each kind storage of its own, and prompts longer than the window, cut before and behind the
+    window's edge, then decoded one by one across a page's edge, give the plain model's logits."""
+    import nnis_amd
+    from nnis_amd.api import load_engine
+    from nnis_amd.engine.batch import StepEntry
+
+    _register_windowed_toy()
+    folder = str(tmp_path / "windowed")
+    raw = {"architectures": ["WindowedToyForCausalLM"], "model_type": "windowed_toy", "width": 64, "vocab_size": 301, "layers": 4}
+    nnis_amd.write_random_model(folder, raw, seed=21)
+    engine = load_engine(folder, dtype=dtype, max_tokens=512)
+    groups = engine.cache.kv_groups
+    assert len(groups) == 2 and sorted(g.request.window or 0 for g in groups) == [0, _WINDOW]
+    assert sorted(len(g.entries) for g in groups) == [2, 2]
+    rng = np.random.default_rng(9)
+    a, b = rng.integers(0, 301, size=150).tolist(), rng.integers(0, 301, size=45).tolist()
+    want_a, want_b = _plain_windowed_toy(folder, a, 4), _plain_windowed_toy(folder, b, 4)
+    # the window matters: with one key more or less in it the plain logits move by far more than the 32-bit
+    # bound (the window's edge in bfloat16 is the kernel tests' matter: a loud key just outside and just inside)
+    for other in (_WINDOW - 1, _WINDOW + 1):
+        moved = (_plain_windowed_toy(folder, a, 4, window=other)[_WINDOW:] - want_a[_WINDOW:]).abs().max(dim=-1).values
+        assert moved.min().item() > 20 * tolerance("float32")[0], moved.min().item()
+    sa, sb = engine.start_sequence(), engine.start_sequence()
+    rows = engine.step([StepEntry(sa, a[:30], list(range(30))), StepEntry(sb, b[:41], list(range(41)))]).cpu()
+    assert_close(rows[:30], want_a[:30], dtype, "windowed prompt a, inside the window")
+    assert_close(rows[30:], want_b[:41], dtype, "windowed prompt b, one token beyond the window")
+    rows = engine.step([StepEntry(sa, a[30:120], list(range(90)))]).cpu()  # a second run of tokens, across the window and a page
+    assert_close(rows, want_a[30:120], dtype, "windowed continuation of a")
+    for i in range(4):
+        rows = engine.step([StepEntry(sb, [b[41 + i]], [0]), StepEntry(sa, [a[120 + i]], [0])]).cpu()
+        assert_close(rows[0], want_b[41 + i], dtype, f"windowed decode b {i}")
+        assert_close(rows[1], want_a[120 + i], dtype, f"windowed decode a {i}")
+    engine.end_sequence(sb)
+    for i in range(124, 150):  # alone, over the edge of the second page
+        rows = engine.step([StepEntry(sa, [a[i]], [0])]).cpu()
+        assert_close(rows[0], want_a[i], dtype, f"windowed decode a {i}")
