@@ -650,22 +650,33 @@ def decode_max_waves(heads: int, kv_heads: int, head_dim: int) -> int:
     return attention_module(head_dim).nnis_attention_decode_max_waves(heads, kv_heads)
 
 
-def decode_plan(batch: int, kv_heads: int, longest: int, max_waves: int = 4):
+def decode_plan(batch: int, kv_heads: int, longest: int, max_waves: int = 4, width: int = 0):
     """(splits, waves) of a decode step's attention.  A block of 4 waves deals
     a sequence's pages among its waves.  Cutting the keys into runs for more
     blocks costs a second kernel that sums the runs (dearer the more runs), so
-    it pays only from about 16 pages on; then a wave gets 2 to 4 pages, in at
+    it pays only from about 9 pages on; then a wave gets 1 to 2 pages, in at
     most 8 runs and about a thousand waves on the chip.  Powers of two.
+    ``width`` (query heads x head size, 0: unknown) says what a run costs to
+    sum: beyond 1024 runs pay from 17 pages on and a wave gets 2 to 4 pages
+    (32 heads of 64, 128 to 2k keys, tokens/s with the one rule and the other:
+    batch 8 on 4 key-value heads 5,654 against 5,497, batch 1 862 against 852;
+    batch 1 on 32 key-value heads 700 against 682).
     Measured on 9 query / 3 key-value heads of 64 (microseconds a layer, runs
     of 1/2/4/8/16): batch 1 at 1k keys 7.9/8.3/8.7/10.7, at 8k 30/20/15/14/17;
-    batch 8 at 2k 11.6/11.0/9.5/9.3/13.6; batch 32 at 4k 27/25/31/34/45."""
+    batch 8 at 2k 11.6/11.0/9.5/9.3/13.6; batch 32 at 4k 27/25/31/34/45.  And
+    on whole decode steps of 30 such layers (milliseconds, runs of 1/2/4/8 with
+    4 waves): batch 1 at 1k keys 0.839/0.822/0.790/0.775, at 128 to 2k
+    0.957/0.882/0.823/0.790, at 256 keys 0.724/0.742/0.741/0.749; batch 8 at 1k
+    0.943/0.952/0.919/0.914, at 128 to 2k 1.051/0.968/0.910/0.890, at 512 keys
+    0.874/0.900/0.881/0.893."""
     pages = (longest + 63) // 64
     waves = 1
     while waves * 2 <= min(max_waves, pages):
         waves *= 2
     splits = 1
-    if pages > 16:
-        wanted = min(8, (pages + 7) // 8)
+    first, each = (8, 4) if 0 < width <= 1024 else (16, 8)  # runs from more than `first` pages on, about `each` pages a run
+    if pages > first:
+        wanted = min(8, (pages + each - 1) // each)
         room = max(1, 1024 // max(1, batch * kv_heads * waves))
         while splits * 2 <= room and splits < wanted:
             splits *= 2
@@ -704,7 +715,7 @@ def attention(q: torch.Tensor, out: torch.Tensor, view, ctx, heads: int, kv_head
         if ctx.splits:
             splits, waves = ctx.splits, ctx.waves
         else:
-            splits, waves = decode_plan(ctx.batch, kv_heads, ctx.max_len)
+            splits, waves = decode_plan(ctx.batch, kv_heads, ctx.max_len, width=heads * head_dim)
         waves = min(waves, decode_max_waves(heads, kv_heads, head_dim))
         partial = None
         if splits > 1:

@@ -57,7 +57,7 @@ class DecoderModel:
     def decode_plan(self, batch: int, longest: int, rt):
         """(splits, waves) of a decode step's attention kernels, one plan for all layers."""
         kv_heads = [request.kv_heads for _, request in self.cache_requests()[0] if hasattr(request, "kv_heads")]
-        return rt.ops.decode_plan(batch, min(kv_heads), longest) if kv_heads else (1, 1)
+        return rt.ops.decode_plan(batch, min(kv_heads), longest, width=self.spec.width) if kv_heads else (1, 1)
 
     # ---- cache ---------------------------------------------------------------
     def cache_requests(self) -> Tuple[List[Tuple[int, Any]], Dict[int, int]]:
