@@ -18,7 +18,7 @@
 
 namespace {
 
-constexpr int kSampleThreads = 1024;
+constexpr int kSampleThreads = 512;  // 8 waves: a thread may keep up to 128 keys of its row in registers
 
 __device__ __forceinline__ unsigned ordered_key(float v) {
   if (v == 0.0f) v = 0.0f;  // -0 and +0 compare equal
@@ -53,21 +53,70 @@ struct RowView {
   int vocab;
 };
 
+// A thread's elements are threadIdx.x + i * kSampleThreads.  With PER > 0 it keeps their ordered keys in
+// registers (vocab <= PER * kSampleThreads; 0 for an element beyond the row, which is below every finite
+// value's key) and a pass over the row reads the weights only, every load asked for before the first is used;
+// PER == 0 reads keys and weights from memory, for rows of any length.  The sums are the same term by term
+// either way: an element that does not count adds 0.
+template <int PER>
+struct Keys {
+  unsigned held[PER > 0 ? PER : 1];
+};
+
+template <int PER>
+__device__ __forceinline__ void load_keys(Keys<PER>& keys, const RowView& r) {
+  if constexpr (PER > 0) {
+#pragma clang loop unroll(full)
+    for (int i = 0; i < PER; ++i) {
+      const int c = threadIdx.x + i * kSampleThreads;
+      keys.held[i] = c < r.vocab ? ordered_key(r.logits[c]) : 0u;
+    }
+  }
+}
+
 // weight of all tokens whose key is >= t
-__device__ double mass_at_least(const RowView& r, unsigned t, double* scratch) {
+template <int PER>
+__device__ __forceinline__ double mass_at_least(const RowView& r, const Keys<PER>& keys, unsigned t, double* scratch) {
   double sum = 0.0;
-  for (int c = threadIdx.x; c < r.vocab; c += kSampleThreads)
-    if (ordered_key(r.logits[c]) >= t) sum += r.weights[c];
+  if constexpr (PER > 0) {
+    constexpr int kBatch = 8;
+    const unsigned from = t > 1u ? t : 1u;  // an element beyond the row has key 0 and never counts
+    int first = threadIdx.x;
+    asm volatile("" : "+v"(first));  // each pass works out its addresses again: kept from pass to pass they would take the keys' registers
+#pragma clang loop unroll(full)
+    for (int i0 = 0; i0 < PER; i0 += kBatch) {
+      double w[kBatch];
+#pragma clang loop unroll(full)
+      for (int j = 0; j < kBatch; ++j) {
+        const int c = first + (i0 + j) * kSampleThreads;
+        w[j] = i0 + j < PER ? r.weights[c < r.vocab ? c : r.vocab - 1] : 0.0;  // (beyond the row: the last again, not counted)
+      }
+#pragma clang loop unroll(full)
+      for (int j = 0; j < kBatch; ++j)
+        if (i0 + j < PER) sum += keys.held[i0 + j] >= from ? w[j] : 0.0;
+      __builtin_amdgcn_sched_barrier(0);  // a batch's loads at a time: the registers hold the keys
+    }
+  } else {
+    for (int c = threadIdx.x; c < r.vocab; c += kSampleThreads)
+      if (ordered_key(r.logits[c]) >= t) sum += r.weights[c];
+  }
   return block_total(sum, scratch);
 }
 
-__device__ int count_at_least(const RowView& r, unsigned t, int* scratch) {
+template <int PER>
+__device__ __forceinline__ int count_at_least(const RowView& r, const Keys<PER>& keys, unsigned t, int* scratch) {
   int count = 0;
-  for (int c = threadIdx.x; c < r.vocab; c += kSampleThreads)
-    if (ordered_key(r.logits[c]) >= t) ++count;
+  if constexpr (PER > 0) {
+#pragma clang loop unroll(full)
+    for (int i = 0; i < PER; ++i) count += (keys.held[i] >= t && keys.held[i] != 0u) ? 1 : 0;
+  } else {
+    for (int c = threadIdx.x; c < r.vocab; c += kSampleThreads)
+      if (ordered_key(r.logits[c]) >= t) ++count;
+  }
   return block_total(count, scratch);
 }
 
+template <int PER>
 __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
     const float* __restrict__ logits, double* __restrict__ weights, int vocab, const int* __restrict__ row_slot,
     unsigned long long* __restrict__ rng, const float* __restrict__ temperature, const int* __restrict__ top_k,
@@ -83,6 +132,8 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
   double* w = weights + (size_t)row * vocab;
   r.weights = w;
   r.vocab = vocab;
+  Keys<PER> keys;
+  load_keys<PER>(keys, r);
 
   // maximum key, and a check that every logit is finite
   unsigned key_max = 0;
@@ -118,21 +169,21 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
   unsigned cut_key = 0;
   int cut_ties = 0;          // meaningful only when limited
   bool limited = false;
-  double total = mass_at_least(r, 0u, scratch_d);
+  double total = mass_at_least<PER>(r, keys, 0u, scratch_d);
 
   const int k = top_k[at];
   if (k > 0 && k < vocab) {
     unsigned t = 0;
     for (int bit = 31; bit >= 0; --bit) {
       const unsigned probe = t | (1u << bit);
-      if (count_at_least(r, probe, scratch_i) >= k) t = probe;
+      if (count_at_least<PER>(r, keys, probe, scratch_i) >= k) t = probe;
     }
-    const int above = count_at_least(r, t + 1u, scratch_i);
+    const int above = count_at_least<PER>(r, keys, t + 1u, scratch_i);
     cut_key = t;
     cut_ties = k - above;
     limited = true;
     const double weight_at = exp((double)__uint_as_float((t & 0x80000000u) ? (t & 0x7fffffffu) : ~t) * inv_t - max_scaled);
-    total = mass_at_least(r, t + 1u, scratch_d) + (double)cut_ties * weight_at;
+    total = mass_at_least<PER>(r, keys, t + 1u, scratch_d) + (double)cut_ties * weight_at;
   }
 
   const float p = top_p[at];
@@ -141,14 +192,14 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
     unsigned t = 0;
     for (int bit = 31; bit >= 0; --bit) {
       const unsigned probe = t | (1u << bit);
-      const double mass = (limited && probe <= cut_key) ? total : mass_at_least(r, probe, scratch_d);
+      const double mass = (limited && probe <= cut_key) ? total : mass_at_least<PER>(r, keys, probe, scratch_d);
       if (mass >= threshold) t = probe;
     }
     // t >= cut_key when limited, because the whole kept mass reaches the threshold
-    const double base = mass_at_least(r, t + 1u, scratch_d);
+    const double base = mass_at_least<PER>(r, keys, t + 1u, scratch_d);
     const double weight_at = exp((double)__uint_as_float((t & 0x80000000u) ? (t & 0x7fffffffu) : ~t) * inv_t - max_scaled);
     int available = (limited && t == cut_key) ? cut_ties
-                                              : count_at_least(r, t, scratch_i) - count_at_least(r, t + 1u, scratch_i);
+                                              : count_at_least<PER>(r, keys, t, scratch_i) - count_at_least<PER>(r, keys, t + 1u, scratch_i);
     int need = 1;
     double reached = base + weight_at;
     while (need < available && reached < threshold) {
@@ -169,13 +220,13 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
   unsigned t = 0;
   for (int bit = 31; bit >= 0; --bit) {
     const unsigned probe = t | (1u << bit);
-    const double mass = (limited && probe <= cut_key) ? total : mass_at_least(r, probe, scratch_d);
+    const double mass = (limited && probe <= cut_key) ? total : mass_at_least<PER>(r, keys, probe, scratch_d);
     if (mass > draw) t = probe;
   }
-  const double base = mass_at_least(r, t + 1u, scratch_d);
+  const double base = mass_at_least<PER>(r, keys, t + 1u, scratch_d);
   const double weight_at = exp((double)__uint_as_float((t & 0x80000000u) ? (t & 0x7fffffffu) : ~t) * inv_t - max_scaled);
   const int available = (limited && t == cut_key) ? cut_ties
-                                                  : count_at_least(r, t, scratch_i) - count_at_least(r, t + 1u, scratch_i);
+                                                  : count_at_least<PER>(r, keys, t, scratch_i) - count_at_least<PER>(r, keys, t + 1u, scratch_i);
   int index = 0;
   double reached = base + weight_at;
   while (index + 1 < available && !(draw < reached)) {
@@ -231,8 +282,18 @@ extern "C" int nnis_sample(const float* logits, double* weights, int rows, int v
   NNIS_REQUIRE(rows >= 0 && vocab > 0, "sample: bad sizes rows=%d vocab=%d", rows, vocab);
   NNIS_REQUIRE((long long)vocab <= 65535LL * kSampleThreads, "sample: vocabulary %d is too large for this kernel", vocab);
   if (rows == 0) return 0;
-  hipLaunchKernelGGL(sample_kernel, dim3(rows), dim3(kSampleThreads), 0, (hipStream_t)stream, logits, weights, vocab,
-                     row_slot, rng, temperature, top_k, top_p, by_slot, out);
+  const dim3 grid(rows), block(kSampleThreads);
+  hipStream_t s = (hipStream_t)stream;
+#define NNIS_SAMPLE(PER) hipLaunchKernelGGL(sample_kernel<PER>, grid, block, 0, s, logits, weights, vocab, row_slot, rng, temperature, top_k, top_p, by_slot, out)
+  // elements a thread keeps in registers: the least that covers the row
+  if (vocab <= 8 * kSampleThreads) NNIS_SAMPLE(8);
+  else if (vocab <= 16 * kSampleThreads) NNIS_SAMPLE(16);
+  else if (vocab <= 32 * kSampleThreads) NNIS_SAMPLE(32);
+  else if (vocab <= 64 * kSampleThreads) NNIS_SAMPLE(64);
+  else if (vocab <= 96 * kSampleThreads) NNIS_SAMPLE(96);
+  else if (vocab <= 128 * kSampleThreads) NNIS_SAMPLE(128);
+  else NNIS_SAMPLE(0);
+#undef NNIS_SAMPLE
   NNIS_LAUNCH_CHECK("sample");
   return 0;
 }
