@@ -48,13 +48,16 @@ class TensorSpec:
     """A tensor a part reads from the checkpoint.
 
     ``init`` tells the random-weights writer how to draw it: ``"matrix"`` is
-    N(0, 0.02) and ``"gain"`` is 1 + N(0, 0.01).  ``fallback`` names another
-    checkpoint tensor that stands in when this one is absent (a tied head)."""
+    N(0, 0.02) and ``"gain"`` is 1 + N(0, 0.01); ``"index"`` marks a table of
+    integers, uniform in [0, ``high``), which is stored and kept as int32
+    whatever the activation type.  ``fallback`` names another checkpoint
+    tensor that stands in when this one is absent (a tied head)."""
 
     name: str
     shape: Tuple[int, ...]
     init: str = "matrix"
     fallback: Optional[str] = None
+    high: Optional[int] = None
 
 
 @dataclass(frozen=True)

@@ -5,7 +5,8 @@ looks each one up in ``model.safetensors`` (or the shards named by
 ``model.safetensors.index.json``), checks shape and stored type, and puts it
 on the device.  A tensor stored in bfloat16 stays bfloat16 and one stored in
 32-bit stays 32-bit; only the 32-bit path widens (exactly, ``bits << 16``:
-/root/reference/crates/nnis-model/src/safetensors_loader.rs:610-624).
+/root/reference/crates/nnis-model/src/safetensors_loader.rs:610-624).  A table
+of integers (a part declares it so) is kept as int32 on either path.
 Everything wrong with a folder is reported in one error: missing tensors,
 tensors nobody asked for, wrong shapes, unsupported stored types
 (the reference's checks: safetensors_loader.rs:711-724,831-874).
@@ -26,6 +27,7 @@ from .safetensors_io import SafetensorsFile
 SINGLE = "model.safetensors"
 INDEX = "model.safetensors.index.json"
 _STORED = {"F32": torch.float32, "BF16": torch.bfloat16}
+_STORED_INTEGERS = {"I32": torch.int32, "I64": torch.int64}  # what a table of integers may be stored as
 # buffers that older checkpoints carry beside the weights
 _IGNORED_SUFFIXES = ("rotary_emb.inv_freq",)
 
@@ -82,6 +84,7 @@ def load_weights(model_dir: str, specs: Sequence[TensorSpec], device, widen_to_f
     wrong_shape: List[str] = []
     wrong_type: List[str] = []
     consumed = set()
+    integer_tables = set()  # checkpoint names
     plan = []  # (spec name, checkpoint name)
     seen = set()
     for spec in specs:
@@ -99,7 +102,12 @@ def load_weights(model_dir: str, specs: Sequence[TensorSpec], device, widen_to_f
         if tuple(shape) != tuple(spec.shape):
             wrong_shape.append(f"{source}: expected {list(spec.shape)}, file has {list(shape)}")
             continue
-        if stored not in _STORED:
+        if spec.init == "index":
+            if stored not in _STORED_INTEGERS:
+                wrong_type.append(f"{source}: stored as {stored}; a table of integers is stored as I32 or I64")
+                continue
+            integer_tables.add(source)
+        elif stored not in _STORED:
             wrong_type.append(f"{source}: stored as {stored}; supported are F32 and BF16")
             continue
         plan.append((spec.name, source))
@@ -126,9 +134,14 @@ def load_weights(model_dir: str, specs: Sequence[TensorSpec], device, widen_to_f
     for name, source in plan:
         if source not in on_device:
             host = where[source].tensor(source)
-            tensor = host.to(device)
-            if widen_to_float32 and tensor.dtype != torch.float32:
-                tensor = tensor.to(torch.float32)
+            if source in integer_tables:
+                if host.numel() and (int(host.min()) < -(1 << 31) or int(host.max()) >= (1 << 31)):
+                    raise WeightError(f"{source}: a value does not fit the 32-bit integers the table is kept in")
+                tensor = host.to(torch.int32).to(device)
+            else:
+                tensor = host.to(device)
+                if widen_to_float32 and tensor.dtype != torch.float32:
+                    tensor = tensor.to(torch.float32)
             on_device[source] = tensor.contiguous()
         out[name] = on_device[source]
     for handle in files:

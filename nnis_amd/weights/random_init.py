@@ -1,6 +1,6 @@
 """Random-weights mode: writes a model folder (config.json, model.safetensors)
-from a configuration and a seed.  Every matrix is N(0, 0.02) and every norm
-gain 1 + N(0, 0.01), drawn in the order the model declares its tensors from
+from a configuration and a seed.  Every matrix is N(0, 0.02), every norm
+gain 1 + N(0, 0.01) and every table of integers uniform in its range, drawn in the order the model declares its tensors from
 one seeded generator.  The reference has no such mode; it downloads a pinned
 random checkpoint (/root/reference/tools/tiny_random_llama_fixture.py:29-31).
 """
@@ -38,6 +38,11 @@ def write_random_model(model_dir: str, raw_config: Dict[str, Any], seed: int) ->
             if tensor.name in done or tensor.fallback is not None:
                 continue  # a tensor with a stand-in (tied head) is not drawn
             done.add(tensor.name)
+            if tensor.init == "index":
+                if not tensor.high or tensor.high <= 0:
+                    raise InvalidInput(f"tensor {tensor.name}: a table of integers needs the end of its range (high)")
+                yield tensor.name, torch.randint(0, int(tensor.high), tuple(tensor.shape), generator=generator, dtype=torch.int32)
+                continue
             noise = torch.randn(tensor.shape, generator=generator, dtype=torch.float32)
             if tensor.init == "gain":
                 value = 1.0 + 0.01 * noise

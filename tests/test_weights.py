@@ -166,3 +166,79 @@ def test_malformed_container(tmp_path):
     path.write_bytes(struct.pack("<Q", len(header)) + header + b"\0" * 8)
     with pytest.raises(WeightError, match="does not fit"):
         SafetensorsFile(str(path))
+
+
+def test_tables_of_integers_are_kept_as_int32(tmp_path):
+    """A part may declare a table of integers (here a toy embedding that maps token ids through a table
+    before the lookup): the random model holds it as I32, the loader keeps it int32 on the bfloat16 path
+    and on the 32-bit path (which widens everything else), takes I64 too, and names a float in its place
+    as a wrong type."""
+    from dataclasses import dataclass
+
+    from nnis_amd.config import register_architecture
+    from nnis_amd.models import ModelSpec, ScheduleEntry
+    from nnis_amd.parts import Part, TensorSpec, register_part
+
+    class RemappedTable(Part):
+        def __init__(self, vocab_size, width, weight, remap):
+            self.vocab_size, self.width, self.weight_name, self.remap_name = vocab_size, width, weight, remap
+
+        def tensors(self):
+            return [TensorSpec(self.weight_name, (self.vocab_size, self.width)),
+                    TensorSpec(self.remap_name, (self.vocab_size,), init="index", high=self.vocab_size)]
+
+    @dataclass(frozen=True)
+    class RemapConfig:
+        raw: dict
+
+        @classmethod
+        def from_dict(cls, raw):
+            return cls(dict(raw))
+
+    def remap_spec(cfg):
+        return ModelSpec(
+            architecture="RemapToyForCausalLM", width=32, vocab_size=97, max_positions=64, stored_dtype="bfloat16",
+            embedding={"kind": "remapped_table", "vocab_size": 97, "width": 32, "weight": "emb", "remap": "remap"},
+            positions={},
+            layers=[{"kind": "pre_norm", "width": 32,
+                     "norm1": {"kind": "rms", "width": 32, "eps": 1e-5, "weight": "n1"},
+                     "mixer": {"kind": "causal_attention", "width": 32, "heads": 2, "kv_heads": 1, "head_dim": 16, "position": None,
+                               "q": "q", "k": "k", "v": "v", "o": "o"},
+                     "norm2": {"kind": "rms", "width": 32, "eps": 1e-5, "weight": "n2"},
+                     "feed_forward": {"kind": "gated", "width": 32, "inner": 48, "gate": "g", "up": "u", "down": "d"}}],
+            schedule=[ScheduleEntry(0)],
+            final_norm={"kind": "rms", "width": 32, "eps": 1e-5, "weight": "norm"},
+            head={"kind": "linear", "vocab_size": 97, "width": 32, "weight": "head", "tied_to": "emb"},
+            config_json=cfg.raw)
+
+    register_part("embedding", "remapped_table", RemappedTable, replace=True)
+    register_architecture("RemapToyForCausalLM", RemapConfig, remap_spec, replace=True)
+    folder = str(tmp_path / "remap")
+    raw = {"architectures": ["RemapToyForCausalLM"], "model_type": "remap_toy"}
+    nnis_amd.write_random_model(folder, raw, seed=4)
+    stored = SafetensorsFile(os.path.join(folder, "model.safetensors"))
+    assert stored.entries["remap"] == ("I32", (97,)) and stored.entries["emb"][0] == "BF16"
+    table = stored.tensor("remap").clone()
+    everything = {name: stored.tensor(name).clone() for name in stored.names()}
+    stored.close()
+    assert table.dtype == torch.int32 and 0 <= int(table.min()) and int(table.max()) < 97 and len(set(table.tolist())) > 20
+    specs = DecoderModel(spec_from_config(raw)[1]).tensors()
+    for widen in (False, True):
+        loaded = load_weights(folder, specs, "cpu", widen_to_float32=widen)
+        assert loaded["remap"].dtype == torch.int32 and torch.equal(loaded["remap"], table)
+        assert loaded["emb"].dtype == (torch.float32 if widen else torch.bfloat16)
+    # stored in 64 bits: taken, narrowed; a value that does not fit is refused
+    wide = dict(everything, remap=table.to(torch.int64))
+    write_safetensors(os.path.join(folder, "model.safetensors"), wide.items())
+    assert torch.equal(load_weights(folder, specs, "cpu", widen_to_float32=False)["remap"], table)
+    wide["remap"][3] = 1 << 40
+    write_safetensors(os.path.join(folder, "model.safetensors"), wide.items())
+    with pytest.raises(WeightError, match="does not fit"):
+        load_weights(folder, specs, "cpu", widen_to_float32=False)
+    # a float where the table of integers should be, and integers where a matrix should be
+    write_safetensors(os.path.join(folder, "model.safetensors"), dict(everything, remap=table.float()).items())
+    with pytest.raises(WeightError, match="remap: stored as F32; a table of integers"):
+        load_weights(folder, specs, "cpu", widen_to_float32=False)
+    write_safetensors(os.path.join(folder, "model.safetensors"), dict(everything, norm=torch.ones(32, dtype=torch.int32)).items())
+    with pytest.raises(WeightError, match="norm: stored as I32; supported are F32 and BF16"):
+        load_weights(folder, specs, "cpu", widen_to_float32=False)
