@@ -62,6 +62,7 @@ class KVGroup:
         pinned = torch.device(device).type == "cuda"
         self.block_table_host = torch.zeros((slots, per_slot), dtype=torch.int32, pin_memory=pinned)
         self.block_table = torch.zeros((slots, per_slot), dtype=torch.int32, device=device)
+        self._table_rows = self.block_table_host.numpy()  # the same memory: an entry is written without a tensor operation
         self._dirty = set()
 
     def bytes_per_token(self) -> int:
@@ -71,8 +72,7 @@ class KVGroup:
         changed = self.table.grow(slot, new_length)
         if changed:
             row = self.table.rows[slot]
-            for index in changed:
-                self.block_table_host[slot, index] = row[index]
+            self._table_rows[slot, changed[0]:changed[-1] + 1] = row[changed[0]:changed[-1] + 1]  # (the new pages follow one another)
             self._dirty.add(slot)
 
     def flush(self) -> None:

@@ -57,9 +57,9 @@ def _validate(request: GenerationRequest, index: int, vocab_size: int, max_posit
         raise InvalidInput(f"request {index}: the prompt is empty")
     if request.max_new_tokens <= 0:
         raise InvalidInput(f"request {index}: max_new_tokens must be positive; got {request.max_new_tokens}")
-    for token in request.prompt:
-        if not 0 <= int(token) < vocab_size:
-            raise InvalidInput(f"request {index}: token id {token} is out of range for vocabulary {vocab_size}")
+    if not all(0 <= int(t) < vocab_size for t in request.prompt):
+        token = next(t for t in request.prompt if not 0 <= int(t) < vocab_size)
+        raise InvalidInput(f"request {index}: token id {token} is out of range for vocabulary {vocab_size}")
     if len(request.prompt) + request.max_new_tokens > max_positions:
         raise InvalidInput(
             f"request {index}: prompt of {len(request.prompt)} tokens plus {request.max_new_tokens} new tokens "

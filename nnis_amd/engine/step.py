@@ -31,6 +31,7 @@ class Engine:
         self.cache = SequenceCache(requests, shared, max_tokens, model.spec.max_positions, rt.dtype, rt.device, max_slots)
         self._staging = None
         self._staging_dev = None
+        self._staged = None  # recorded behind the staging copy
         # decode steps are replayed from HIP graphs when every part of the model
         # runs only kernels that read the step's metadata from device memory
         self._borrowed = False
@@ -60,6 +61,7 @@ class Engine:
             raise InvalidInput("a step needs at least one sequence")
         seen = set()
         growth = {}
+        arrays = []  # each entry's token ids, as checked
         for entry in entries:
             if entry.slot in seen:
                 raise InvalidInput(f"slot {entry.slot} appears twice in one step")
@@ -68,17 +70,23 @@ class Engine:
             count = len(entry.tokens)
             if count == 0:
                 raise InvalidInput(f"slot {entry.slot}: a step needs at least one token per sequence")
-            for token in entry.tokens:
-                if not 0 <= int(token) < self.vocab_size:
-                    # runtime.rs:1155-1163
-                    raise InvalidInput(f"token id {token} is out of range for vocabulary {self.vocab_size}")
-            if entry.want is not None:
-                for place in entry.want:
-                    if not 0 <= int(place) < count:
-                        raise InvalidInput(f"slot {entry.slot}: wanted place {place} is not among its {count} tokens")
+            try:
+                ids = np.asarray(entry.tokens, dtype=np.int64)  # a prompt of thousands: checked as an array, not one by one
+            except (TypeError, ValueError, OverflowError):
+                raise InvalidInput(f"slot {entry.slot}: token ids must be integers") from None
+            if ids.ndim != 1 or int(ids.min()) < 0 or int(ids.max()) >= self.vocab_size:
+                bad = next((t for t in entry.tokens if not 0 <= int(t) < self.vocab_size), entry.tokens)
+                # runtime.rs:1155-1163
+                raise InvalidInput(f"token id {bad} is out of range for vocabulary {self.vocab_size}")
+            arrays.append(ids)
+            if entry.want is not None and len(entry.want):
+                places = np.asarray(entry.want, dtype=np.int64)
+                if int(places.min()) < 0 or int(places.max()) >= count:
+                    place = next(p for p in entry.want if not 0 <= int(p) < count)
+                    raise InvalidInput(f"slot {entry.slot}: wanted place {place} is not among its {count} tokens")
             growth[entry.slot] = count
         self.cache.check_room(growth)
-        return growth
+        return growth, arrays
 
     def _stage(self, arrays: List[np.ndarray]) -> List[torch.Tensor]:
         """One pinned buffer, one copy to the device, views per array."""
@@ -87,6 +95,9 @@ class Engine:
             size = max(1024, 1 << (total - 1).bit_length())
             self._staging = torch.empty(size, dtype=torch.int32, pin_memory=True)
             self._staging_dev = torch.empty(size, dtype=torch.int32, device=self.rt.device)
+            self._staged = torch.cuda.Event()
+        else:
+            self._staged.synchronize()  # the pinned buffer is reused: the previous step's copy has left it
         host = self._staging.numpy()
         offset = 0
         spans = []
@@ -97,6 +108,7 @@ class Engine:
         # the previous step's kernels may still read the device buffer: the
         # copy is ordered after them on the same stream
         self._staging_dev[:total].copy_(self._staging[:total], non_blocking=True)
+        self._staged.record()
         return [self._staging_dev[o:o + n] for o, n in spans]
 
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
@@ -111,7 +123,7 @@ class Engine:
         self._borrowed = False
         if self.use_graphs and entries and all(len(e.tokens) == 1 for e in entries):
             return self._decode_step(entries)
-        growth = self._validate(entries)
+        growth, token_arrays = self._validate(entries)
         pos0 = [self.cache.length(e.slot) for e in entries]
         counts = [len(e.tokens) for e in entries]
         total = sum(counts)
@@ -123,7 +135,7 @@ class Engine:
         row = 0
         for index, entry in enumerate(entries):
             n = counts[index]
-            ids[row:row + n] = np.asarray(entry.tokens, dtype=np.int32)
+            ids[row:row + n] = token_arrays[index]
             tok_slot[row:row + n] = entry.slot
             tok_pos[row:row + n] = np.arange(pos0[index], pos0[index] + n, dtype=np.int32)
             places = [n - 1] if entry.want is None else entry.want
@@ -132,8 +144,6 @@ class Engine:
             seq_start[index + 1] = row
         self.cache.grow(growth)
 
-        # the staging buffer is reused: wait until the previous step's copy has left it
-        torch.cuda.current_stream().synchronize() if self._staging is not None else None
         dev = self._stage([
             ids, tok_slot, tok_pos,
             np.asarray([e.slot for e in entries], dtype=np.int32), seq_start,
