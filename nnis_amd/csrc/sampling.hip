@@ -186,15 +186,44 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
     total = mass_at_least<PER>(r, keys, t + 1u, scratch_d) + (double)cut_ties * weight_at;
   }
 
+  // The largest key t at which `holds(weight of all kept tokens with key >= t)` is still true, by bits from the
+  // top.  With the keys in registers a probe first counts (no memory): a probe that holds the same tokens as
+  // the bound above it (which failed) or as the bound below (which held) needs no sum -- among 49,152 keys that
+  // is about half of the 32 probes, the upper bits that all keys share and the lower ones between neighbours.
+  auto find_cut = [&](auto holds) -> unsigned {
+    unsigned t = 0;
+    int count_below = -1;  // tokens with key >= t, where known (not at the start: with a limit `total` is not all tokens' weight)
+    int count_above = 0;   // tokens at and above the lowest probe that failed; at first none, whose weight 0 never holds
+    for (int bit = 31; bit >= 0; --bit) {
+      const unsigned probe = t | (1u << bit);
+      if (limited && probe <= cut_key) {  // everything kept lies at or above the limit: the whole kept weight, which holds
+        t = probe;
+        count_below = -1;
+        continue;
+      }
+      int count = -2;
+      if constexpr (PER > 0) {
+        count = count_at_least<PER>(r, keys, probe, scratch_i);
+        if (count == count_above) continue;
+        if (count == count_below) {
+          t = probe;
+          continue;
+        }
+      }
+      if (holds(mass_at_least<PER>(r, keys, probe, scratch_d))) {
+        t = probe;
+        count_below = count;
+      } else {
+        count_above = count;
+      }
+    }
+    return t;
+  };
+
   const float p = top_p[at];
   if (p > 0.0f && p <= 1.0f) {
     const double threshold = (double)p * total;
-    unsigned t = 0;
-    for (int bit = 31; bit >= 0; --bit) {
-      const unsigned probe = t | (1u << bit);
-      const double mass = (limited && probe <= cut_key) ? total : mass_at_least<PER>(r, keys, probe, scratch_d);
-      if (mass >= threshold) t = probe;
-    }
+    const unsigned t = find_cut([&](double mass) { return mass >= threshold; });
     // t >= cut_key when limited, because the whole kept mass reaches the threshold
     const double base = mass_at_least<PER>(r, keys, t + 1u, scratch_d);
     const double weight_at = exp((double)__uint_as_float((t & 0x80000000u) ? (t & 0x7fffffffu) : ~t) * inv_t - max_scaled);
@@ -217,12 +246,7 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
   const double unit = (double)(raw >> 11) * (1.0 / 9007199254740992.0);
   const double draw = unit * total;
 
-  unsigned t = 0;
-  for (int bit = 31; bit >= 0; --bit) {
-    const unsigned probe = t | (1u << bit);
-    const double mass = (limited && probe <= cut_key) ? total : mass_at_least<PER>(r, keys, probe, scratch_d);
-    if (mass > draw) t = probe;
-  }
+  const unsigned t = find_cut([&](double mass) { return mass > draw; });
   const double base = mass_at_least<PER>(r, keys, t + 1u, scratch_d);
   const double weight_at = exp((double)__uint_as_float((t & 0x80000000u) ? (t & 0x7fffffffu) : ~t) * inv_t - max_scaled);
   const int available = (limited && t == cut_key) ? cut_ties
