@@ -519,8 +519,8 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
   // newest NS - 2 steps' loads of this wave have arrived (loads arrive in the order they were
   // asked for), and for the other waves' at the barrier.  A step beyond the end of K is asked for all the
   // same, so that the count holds: from the row's last whole chunk, a valid address, and nobody reads it.
-  // In the last step of a K that is no multiple of BK the same holds for the chunks beyond K; the lanes
-  // that hold them as the first operand make them zeros.
+  // In the last step of a K that is no multiple of BK the same holds for the activations' chunks beyond K;
+  // they meet the zeros that pad the packed weights' last chunk (finite times zero: the row's own last values).
   const int steps = (k + BK - 1) / BK;
   const int steps_a_part = (steps + ksplit - 1) / ksplit;
   const int step0 = part * steps_a_part;  // this block multiplies steps step0 .. step1 - 1 (none, for a part beyond the end)
@@ -539,7 +539,6 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
     for (int o = 0; o < B_LOADS; ++o)
       __builtin_amdgcn_global_load_lds((global_ptr_t)(b_src[o] + from_chunk), (lds_ptr_t)(base + A_BYTES + o * 4096), 16, 0, 0);
   };
-  const bool ragged = (k % BK) != 0;
 
 #pragma unroll
   for (int s = 0; s < NS - 1; ++s) ask(step0 + s, s);
@@ -608,10 +607,6 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
       for (int i = 0; i < TM; ++i) a_frag[i] = a_tile[swizzled<CH>(wave_m * WM + i * 16 + r, g * 2 + half)];  // k as the weights are packed
 #pragma unroll
       for (int jj = 0; jj < TN; ++jj) b_frag[jj] = b_tile[((wave_n * TN + jj) * 2 + half) * kWave + lane];
-      if (ragged && step == steps - 1 && step * BK + (g * 2 + half) * 8 + 8 > k) {
-#pragma unroll
-        for (int i = 0; i < TM; ++i) a_frag[i] = zero_chunk();
-      }
 #pragma unroll
       for (int i = 0; i < TM; ++i)
 #pragma unroll
