@@ -600,18 +600,30 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
     ask(step + NS - 1, stage == 0 ? NS - 1 : stage - 1);
     const bf16x8* a_tile = (const bf16x8*)(tile_lds + stage * STAGE_BYTES);
     const bf16x8* b_tile = (const bf16x8*)(tile_lds + stage * STAGE_BYTES + A_BYTES);
+    static_assert(BK == 64, "two halves of 32 k a step");
+    bf16x8 a_frag[2][TM], b_frag[2][TN];  // an instruction takes 32 k: the operands of both halves of the step
 #pragma unroll
-    for (int half = 0; half < BK / 32; ++half) {  // an instruction takes 32 k
-      bf16x8 a_frag[TM], b_frag[TN];
+    for (int half = 0; half < 2; ++half) {
 #pragma unroll
-      for (int i = 0; i < TM; ++i) a_frag[i] = a_tile[swizzled<CH>(wave_m * WM + i * 16 + r, g * 2 + half)];  // k as the weights are packed
+      for (int i = 0; i < TM; ++i) a_frag[half][i] = a_tile[swizzled<CH>(wave_m * WM + i * 16 + r, g * 2 + half)];  // k as the weights are packed
 #pragma unroll
-      for (int jj = 0; jj < TN; ++jj) b_frag[jj] = b_tile[((wave_n * TN + jj) * 2 + half) * kWave + lane];
+      for (int jj = 0; jj < TN; ++jj) b_frag[half][jj] = b_tile[((wave_n * TN + jj) * 2 + half) * kWave + lane];
+    }
+#pragma unroll
+    for (int half = 0; half < 2; ++half)
 #pragma unroll
       for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int jj = 0; jj < TN; ++jj) acc[i][jj] = mfma(b_frag[jj], a_frag[i], acc[i][jj]);
+        for (int jj = 0; jj < TN; ++jj) acc[i][jj] = mfma(b_frag[half][jj], a_frag[half][i], acc[i][jj]);
+    // the order for the compiler's scheduler: the first half's reads, then the first half's products each with a read of
+    // the second half behind it, then the rest of the products -- so that no wave waits for all its reads before it multiplies
+    __builtin_amdgcn_sched_group_barrier(0x100, TM + TN, 0);
+#pragma unroll
+    for (int n = 0; n < TM + TN; ++n) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
     }
+    __builtin_amdgcn_sched_group_barrier(0x008, 2 * TM * TN - (TM + TN), 0);
     // what this wave read of its stage has arrived too: the stage is the next step's to fill
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     wait_loads_but<(NS - 2) * LOADS>();

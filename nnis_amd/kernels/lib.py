@@ -41,6 +41,10 @@ FLAGS = [
     "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
 ]
+# Per source: the matrix instructions of the products keep their sums in the ordinary vector registers.  Left to
+# itself the compiler puts them into the accumulation registers and, in the tiled kernel's loop, moves them to and
+# fro every step (48 moves for 16 matrix instructions).
+SOURCE_FLAGS = {"gemm_mfma.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]}
 HEADERS = {"core": ["common.h", "epilogue.h"], "attention": ["common.h"]}  # what a module's sources include
 CORE_SOURCES = ["elementwise.hip", "gemm.hip", "gemm_mfma.hip", "gemm_fused.hip", "sampling.hip"]
 ATTENTION_SOURCES = ["attention.hip"]
@@ -72,6 +76,7 @@ def _module_hash(sources: List[str], defines: Dict[str, str]) -> str:
             digest.update(name.encode())
             digest.update(handle.read())
     digest.update(" ".join(FLAGS).encode())
+    digest.update(repr(sorted((name, flags) for name, flags in SOURCE_FLAGS.items() if name in sources)).encode())
     digest.update(repr(sorted(defines.items())).encode())
     return digest.hexdigest()[:12]
 
@@ -164,7 +169,7 @@ def build_module(module: str, force: bool = False) -> str:
             obj = os.path.join(work, source + ".o")
             objects.append(obj)
             commands.append(
-                (f"{source} [{module}]", [hipcc] + FLAGS + define_flags + ["-I", CSRC, "-c", os.path.join(CSRC, source), "-o", obj])
+                (f"{source} [{module}]", [hipcc] + FLAGS + SOURCE_FLAGS.get(source, []) + define_flags + ["-I", CSRC, "-c", os.path.join(CSRC, source), "-o", obj])
             )
         _run_with_heartbeat(commands, env)
         tmp_out = os.path.join(work, name)
