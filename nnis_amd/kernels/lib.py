@@ -41,10 +41,12 @@ FLAGS = [
     "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
 ]
-# Per source: the matrix instructions of the products keep their sums in the ordinary vector registers.  Left to
-# itself the compiler puts them into the accumulation registers and, in the tiled kernel's loop, moves them to and
-# fro every step (48 moves for 16 matrix instructions).
-SOURCE_FLAGS = {"gemm_mfma.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]}
+# Per source: the matrix instructions keep their sums in the ordinary vector registers.  Left to itself the
+# compiler puts them into the accumulation registers and moves them to and fro: in the tiled product's loop 48
+# moves a step for 16 matrix instructions, in the decode attention with keys on lanes 336 for 144 (no kernel
+# of either file spills with the sums in vector registers, at any head size).
+_VECTOR_SUMS = ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]
+SOURCE_FLAGS = {"gemm_mfma.hip": _VECTOR_SUMS, "attention.hip": _VECTOR_SUMS}
 HEADERS = {"core": ["common.h", "epilogue.h"], "attention": ["common.h"]}  # what a module's sources include
 CORE_SOURCES = ["elementwise.hip", "gemm.hip", "gemm_mfma.hip", "gemm_fused.hip", "sampling.hip"]
 ATTENTION_SOURCES = ["attention.hip"]
