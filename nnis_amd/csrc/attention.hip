@@ -905,6 +905,33 @@ __global__ void attention_combine_kernel(const float* __restrict__ partial, bf16
   const int token = blockIdx.x, head = blockIdx.y;
   if (tok_slot[token] < 0) return;
   const float* base = partial + ((size_t)token * heads + head) * splits * kPartial;
+  constexpr int kAtOnce = 8;  // runs whose references, sums and outputs a thread asks for together: one round trip
+  if (splits <= kAtOnce) {
+    for (int d = threadIdx.x; d < HD; d += blockDim.x) {
+      float m[kAtOnce], l[kAtOnce], o[kAtOnce];
+#pragma unroll
+      for (int s = 0; s < kAtOnce; ++s) {
+        const float* p = base + (size_t)(s < splits ? s : splits - 1) * kPartial;  // (beyond the last: the last again, not counted)
+        m[s] = p[HD];
+        l[s] = p[HD + 1];
+        o[s] = p[d];
+      }
+      float m_all = -INFINITY;
+#pragma unroll
+      for (int s = 0; s < kAtOnce; ++s) m_all = s < splits ? fmaxf(m_all, m[s]) : m_all;
+      float num = 0.0f, den = 0.0f;
+#pragma unroll
+      for (int s = 0; s < kAtOnce; ++s) {
+        if (s < splits) {
+          const float w = m[s] == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(m[s] - m_all);
+          num += o[s] * w;
+          den += l[s] * w;
+        }
+      }
+      out[((size_t)token * heads + head) * HD + d] = (bf16_t)(num / den);
+    }
+    return;
+  }
   float m_all = -INFINITY;
   for (int s = 0; s < splits; ++s) m_all = fmaxf(m_all, base[(size_t)s * kPartial + HD]);
   for (int d = threadIdx.x; d < HD; d += blockDim.x) {
