@@ -690,6 +690,12 @@ PREFILL_NARROW_FROM = 1024
 PREFILL_COLUMNS = 0
 
 
+# The work list of a prefill step goes to the device through pinned memory, so that the copy does not make the
+# host wait for the kernels already on the stream (a copy from ordinary memory does: 70 to 100 us a step).  One
+# buffer per device, grown when a step needs more; the event says when the last copy has left it.
+_tile_staging = {}
+
+
 def _prefill_tiles(ctx, rows: int, device):
     """Work items of a prefill step for tiles of ``rows`` query rows, longest first."""
     cached = ctx.tiles.get(rows)
@@ -697,8 +703,21 @@ def _prefill_tiles(ctx, rows: int, device):
         items = [(pos0 + min(row0 + rows, count), seq, row0)
                  for seq, (count, pos0) in enumerate(zip(ctx.host_new, ctx.host_pos0)) for row0 in range(0, count, rows)]
         items.sort(reverse=True)
-        packed = torch.tensor([[seq for _, seq, _ in items], [row0 for _, _, row0 in items]], dtype=torch.int32)
-        packed = packed.to(device, non_blocking=True)
+        count = len(items)
+        key = (device.type, device.index)
+        held = _tile_staging.get(key)
+        if held is None or held[0].shape[1] < count:
+            size = max(256, 1 << (count - 1).bit_length())
+            held = _tile_staging[key] = (torch.empty((2, size), dtype=torch.int32, pin_memory=True), torch.cuda.Event())
+        else:
+            held[1].synchronize()
+        host, copied = held
+        view = host.numpy()
+        view[0, :count] = [seq for _, seq, _ in items]
+        view[1, :count] = [row0 for _, _, row0 in items]
+        packed = torch.empty((2, count), dtype=torch.int32, device=device)
+        packed.copy_(host[:, :count], non_blocking=True)
+        copied.record()
         cached = ctx.tiles[rows] = (packed[0], packed[1])
     return cached
 
