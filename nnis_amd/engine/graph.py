@@ -115,3 +115,128 @@ class DecodeGraphs:
             graph.capture()
             self.graphs[key] = graph
         return graph
+
+
+# ---------------------------------------------------------------------------------------------
+# Prompt steps whose shape comes again
+# ---------------------------------------------------------------------------------------------
+# A step over a few thousand tokens launches 150 kernels and more; where the model is small the host
+# needs as long to launch them as the GPU to run them.  A step's *shape* -- how many new tokens each of
+# its sequences brings, how many logit rows are wanted, and the class of its longest sequence (which
+# picks the attention kernels' plan) -- fixes every launch; tokens, slots, positions and the order of the
+# attention's work items are data.  The second time a shape comes it is captured into a graph whose
+# kernels read that data from fixed buffers; from the third time on the step is a copy into the buffers
+# and a replay.  Only shapes of up to PREFILL_GRAPH_MOST_TOKENS tokens are kept, the most recently used
+# PREFILL_GRAPHS_KEPT of them (a graph keeps its activations' memory), and only where the step's kernels are
+# short enough for the host to matter: tokens x width^2 up to PREFILL_GRAPH_MOST_WORK.  (Measured, a
+# 2,048-token step: width 576 2.32 ms replayed against 2.35 to 2.65 launched, by the host's speed; width 2048
+# 7.65 against 7.45 and 11.4 against 11.0 -- a replay leaves a gap of a microsecond between kernels that
+# launches keeping ahead of the GPU do not.)
+PREFILL_GRAPH_MOST_TOKENS = 4096
+PREFILL_GRAPH_MOST_WORK = 1.5e9
+PREFILL_GRAPHS_KEPT = 4
+
+
+class PrefillGraph:
+    def __init__(self, engine, counts: Sequence[int], wanted: int, plan_class: int, tile_rows: Sequence[int]):
+        self.engine = engine if isinstance(engine, weakref.ProxyTypes) else weakref.proxy(engine)
+        ops = engine.rt.ops
+        device = engine.rt.device
+        self.counts = list(counts)
+        total, batch = sum(counts), len(counts)
+        # the step's arrays in one buffer, in the order the step function stages them
+        self.sizes = [total, total, total, batch, batch + 1, batch, wanted]
+        self.tile_rows = list(tile_rows)
+        self.tile_counts = [sum((n + rows - 1) // rows for n in counts) for rows in self.tile_rows]
+        sizes = self.sizes + [2 * n for n in self.tile_counts]
+        self.spans, offset = [], 0
+        for size in sizes:
+            self.spans.append((offset, size))
+            offset += size
+        self.meta = torch.zeros(offset, dtype=torch.int32, device=device)
+        self.host = torch.empty(offset, dtype=torch.int32, pin_memory=True)
+        self.copied = torch.cuda.Event()
+        self.copied.record()
+        views = [self.meta[o:o + n] for o, n in self.spans]
+        tiles = {rows: (views[7 + i][:n], views[7 + i][n:]) for i, (rows, n) in enumerate(zip(self.tile_rows, self.tile_counts))}
+        self.ids, self.want_rows = views[0], views[6]
+        self.ctx = StepContext(
+            tokens=total, batch=batch, tok_slot=views[1], tok_pos=views[2], seq_slot=views[3], seq_start=views[4],
+            seq_pos0=views[5], decode=False, max_new=max(counts), max_len=ops.PREFILL_CLASS_LENGTH[plan_class],
+            host_new=list(counts), tiles=tiles)
+        self.graph = None
+        self.logits = None
+
+    def fill(self, arrays, first_positions: Sequence[int]) -> None:
+        """The step's data into the buffers: ``arrays`` as the step function stages them (ids, slot and position
+        of each token, slot, first row and first position of each sequence, wanted rows)."""
+        ops = self.engine.rt.ops
+        self.copied.synchronize()  # the previous copy has left the pinned buffer
+        host = self.host.numpy()
+        for (offset, size), array in zip(self.spans, arrays):
+            host[offset:offset + size] = array
+        for (offset, _), rows, n in zip(self.spans[7:], self.tile_rows, self.tile_counts):
+            seqs, row0s = ops.prefill_tile_items(self.counts, first_positions, rows)
+            host[offset:offset + n] = seqs
+            host[offset + n:offset + 2 * n] = row0s
+        self.meta.copy_(self.host, non_blocking=True)
+        self.copied.record()
+
+    def _forward(self) -> torch.Tensor:
+        engine = self.engine
+        return engine.model.forward(self.ids, self.ctx, engine.cache, self.want_rows, engine.rt)
+
+    def first_run(self) -> torch.Tensor:
+        """Runs the step that the buffers hold as any step runs, then captures its launches.  Returns that
+        run's logits (the caller's to keep)."""
+        logits = self._forward()
+        torch.cuda.synchronize()
+        self.graph = torch.cuda.CUDAGraph()
+        gc.collect()  # (as for the decode graphs: no graph may be destroyed while one is captured)
+        collecting = gc.isenabled()
+        gc.disable()
+        try:
+            with torch.cuda.graph(self.graph):
+                self.logits = self._forward()
+        finally:
+            if collecting:
+                gc.enable()
+        return logits
+
+    def run(self) -> torch.Tensor:
+        """Replays the step on what the buffers hold; the rows returned view the graph's output buffer."""
+        self.graph.replay()
+        return self.logits
+
+
+class PrefillGraphs:
+    """The prompt-step graphs of one engine: counts how often a shape has come, captures it the second time."""
+
+    def __init__(self, engine):
+        self.engine = weakref.proxy(engine)
+        self.seen: Dict[tuple, int] = {}
+        self.graphs: Dict[tuple, PrefillGraph] = {}  # in the order of their last use
+
+    def step(self, key: tuple, arrays, first_positions: Sequence[int], tile_rows):
+        """(logits, borrowed) if this step is replayed or captured; None if it is to run as any step.
+        ``tile_rows``: called for the row counts of the attention's work lists the shape's eager run made."""
+        graph = self.graphs.pop(key, None)
+        if graph is not None:
+            self.graphs[key] = graph  # the most recently used is last
+            graph.fill(arrays, first_positions)
+            return graph.run(), True
+        times = self.seen.get(key, 0) + 1
+        self.seen[key] = times
+        if len(self.seen) > 1024:
+            self.seen.clear()
+        rows = tile_rows()
+        if times < 2 or rows is None:
+            return None
+        counts, wanted, plan_class = key
+        graph = PrefillGraph(self.engine, counts, wanted, plan_class, rows)
+        graph.fill(arrays, first_positions)
+        logits = graph.first_run()
+        while len(self.graphs) >= PREFILL_GRAPHS_KEPT:
+            self.graphs.pop(next(iter(self.graphs)))
+        self.graphs[key] = graph
+        return logits, False

@@ -17,6 +17,7 @@ import torch
 from ..cache import SequenceCache
 from ..errors import InvalidInput
 from .batch import StepContext, StepEntry
+from .graph import PREFILL_GRAPH_MOST_TOKENS, PREFILL_GRAPH_MOST_WORK, PrefillGraphs
 
 
 class Engine:
@@ -37,6 +38,8 @@ class Engine:
         self._borrowed = False
         self.use_graphs = model.graph_safe() if use_graphs is None else (use_graphs and model.graph_safe())
         self._graphs = None
+        self._prefill_graphs = None  # prompt steps whose shape comes again
+        self._tile_rows = {}  # per shape: rows a tile of the attention's work lists, as the eager run made them
 
     # ---- sequences -----------------------------------------------------------
     def start_sequence(self) -> int:
@@ -144,10 +147,25 @@ class Engine:
             seq_start[index + 1] = row
         self.cache.grow(growth)
 
-        dev = self._stage([
+        arrays = [
             ids, tok_slot, tok_pos,
             np.asarray([e.slot for e in entries], dtype=np.int32), seq_start,
             np.asarray(pos0, dtype=np.int32), np.asarray(want_rows, dtype=np.int32),
+        ]
+        longest = max(p + n for p, n in zip(pos0, counts))
+        shape = None
+        if (self.use_graphs and total <= PREFILL_GRAPH_MOST_TOKENS and want_rows
+                and total * float(self.model.spec.width) ** 2 <= PREFILL_GRAPH_MOST_WORK):
+            # a shape that comes again is replayed from a graph (engine/graph.py)
+            shape = (tuple(counts), len(want_rows), self.rt.ops.prefill_plan_class(longest))
+            if self._prefill_graphs is None:
+                self._prefill_graphs = PrefillGraphs(self)
+            done = self._prefill_graphs.step(shape, arrays, pos0, lambda: self._tile_rows.get(shape))
+            if done is not None:
+                logits, self._borrowed = done
+                return logits
+        dev = self._stage([
+            *arrays,
         ])
         ctx = StepContext(
             tokens=total,
@@ -159,12 +177,17 @@ class Engine:
             seq_pos0=dev[5],
             decode=all(n == 1 for n in counts),
             max_new=max(counts),
-            max_len=max(p + n for p, n in zip(pos0, counts)),
+            max_len=longest,
             host_slots=[e.slot for e in entries],
             host_new=counts,
             host_pos0=pos0,
         )
-        return self.model.forward(dev[0], ctx, self.cache, dev[6], self.rt)
+        logits = self.model.forward(dev[0], ctx, self.cache, dev[6], self.rt)
+        if shape is not None:
+            self._tile_rows[shape] = sorted(ctx.tiles)  # the attention's work lists this shape needs
+            if len(self._tile_rows) > 1024:
+                self._tile_rows.clear()
+        return logits
 
     def step_from_device(self, slots: Sequence[int], ids_device: torch.Tensor) -> torch.Tensor:
         """A step of one token per sequence whose ids are on the device already

@@ -685,8 +685,8 @@ def decode_plan(batch: int, kv_heads: int, longest: int, max_waves: int = 4, wid
 
 # One column tile a wave (and so up to 8 waves a block) for long sequences was measured slower than the full
 # group a wave with 4 waves (2,048 tokens, 9/3 heads of 64: 5.5 ms a step against 4.6): keys and values are read
-# once per query head then.  The switch stays for other shapes; 0 is off.
-PREFILL_NARROW_FROM = 1024
+# once per query head then.  The switch (for steps whose longest sequence has 1,024 tokens and more) stays for other
+# shapes; 0 is off.
 PREFILL_COLUMNS = 0
 
 
@@ -696,14 +696,30 @@ PREFILL_COLUMNS = 0
 _tile_staging = {}
 
 
+def prefill_plan_class(longest: int) -> int:
+    """Steps whose longest sequence falls into the same class launch the same prefill attention kernels
+    (``attention`` picks the waves of a block, and the column option, by these thresholds)."""
+    return 3 if longest >= 1024 else (2 if longest >= 512 else (1 if longest >= 128 else 0))
+
+
+PREFILL_CLASS_LENGTH = (1, 128, 512, 1024)  # a length of each class
+
+
+def prefill_tile_items(new_tokens, first_positions, rows: int):
+    """Work items (sequence of the step, first row) of a prefill step for tiles of ``rows`` query rows: those
+    with the most keys first."""
+    items = [(pos0 + min(row0 + rows, count), seq, row0)
+             for seq, (count, pos0) in enumerate(zip(new_tokens, first_positions)) for row0 in range(0, count, rows)]
+    items.sort(reverse=True)
+    return [seq for _, seq, _ in items], [row0 for _, _, row0 in items]
+
+
 def _prefill_tiles(ctx, rows: int, device):
     """Work items of a prefill step for tiles of ``rows`` query rows, longest first."""
     cached = ctx.tiles.get(rows)
     if cached is None:
-        items = [(pos0 + min(row0 + rows, count), seq, row0)
-                 for seq, (count, pos0) in enumerate(zip(ctx.host_new, ctx.host_pos0)) for row0 in range(0, count, rows)]
-        items.sort(reverse=True)
-        count = len(items)
+        seqs, row0s = prefill_tile_items(ctx.host_new, ctx.host_pos0, rows)
+        count = len(seqs)
         key = (device.type, device.index)
         held = _tile_staging.get(key)
         if held is None or held[0].shape[1] < count:
@@ -713,8 +729,8 @@ def _prefill_tiles(ctx, rows: int, device):
             held[1].synchronize()
         host, copied = held
         view = host.numpy()
-        view[0, :count] = [seq for _, seq, _ in items]
-        view[1, :count] = [row0 for _, _, row0 in items]
+        view[0, :count] = seqs
+        view[1, :count] = row0s
         packed = torch.empty((2, count), dtype=torch.int32, device=device)
         packed.copy_(host[:, :count], non_blocking=True)
         copied.record()
@@ -745,9 +761,10 @@ def attention(q: torch.Tensor, out: torch.Tensor, view, ctx, heads: int, kv_head
     if fast and not ctx.decode:
         # A tile's keys are a chain of dependent loads: the longest tile sets the kernel's time.  The waves of
         # a block deal the keys among themselves (their merge lives in LDS).
-        columns = PREFILL_COLUMNS if ctx.max_len >= PREFILL_NARROW_FROM else 0
+        plan_class = prefill_plan_class(ctx.max_len)
+        columns = PREFILL_COLUMNS if plan_class == 3 else 0
         most = prefill_max_waves(heads, kv_heads, head_dim, columns)
-        waves = min(most, 8 if ctx.max_len >= 1024 else (4 if ctx.max_len >= 512 else (2 if ctx.max_len >= 128 else 1)))
+        waves = min(most, (1, 2, 4, 8)[plan_class])
         tile_seq, tile_row0 = _prefill_tiles(ctx, prefill_tile_rows(heads, kv_heads, head_dim, columns), q.device)
         return attention_prefill_bf16(q, out, view.k_pages, view.v_pages, view.block_table, tile_seq, tile_row0,
                                       ctx.seq_slot, ctx.seq_start, ctx.seq_pos0, heads, kv_heads, head_dim, scale, window,

@@ -234,6 +234,74 @@ def test_selector_refuses_a_row_that_is_not_finite(model_dirs):
         engine.end_sequence(slot)
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_prompt_steps_whose_shape_comes_again(model_dirs, dtype):
+    """The second time a step's shape comes (new tokens per sequence, wanted rows, class of the longest
+    sequence) it is captured, from the third time on replayed: with other tokens, other slots, other first
+    positions (a prompt's second run of tokens) and other wanted places each time, the logits are the plain
+    model's; shapes beyond the kept few push the oldest out, and a shape that comes back is captured again."""
+    from nnis_amd.engine import graph as G
+    from nnis_amd.engine.batch import StepEntry
+
+    engine = _engine(model_dirs, "B", dtype, max_tokens=64 * 64)
+    assert engine.use_graphs
+    config, _ = TINY_CONFIGS["B"]
+    plain = P.PlainLlama(model_dirs["B"])
+    rng = np.random.default_rng(17)
+    vocab = config["vocab_size"]
+
+    def run(counts, starts, wants):
+        """Sequences with ``starts[i]`` tokens already in the cache (put there in one step) bring ``counts[i]``
+        more; returns nothing, checks the wanted rows against the plain model."""
+        tokens = [rng.integers(0, vocab, size=s + n).tolist() for s, n in zip(starts, counts)]
+        slots = [engine.start_sequence() for _ in counts]
+        for slot, t, s in zip(slots, tokens, starts):
+            if s:
+                engine.step([StepEntry(slot, t[:s], [])])
+        rows = engine.step([StepEntry(slot, t[s:], want) for slot, t, s, want in zip(slots, tokens, starts, wants)]).cpu()
+        at = 0
+        for t, s, n, want in zip(tokens, starts, counts, wants):
+            places = [n - 1] if want is None else want
+            whole = plain.logits(t)
+            for place in places:
+                _close(rows[at], whole[s + place], dtype, f"counts {counts} starts {starts} place {place}")
+                at += 1
+        assert at == rows.shape[0]
+        for slot in slots:
+            engine.end_sequence(slot)
+
+    # the same shape five times: eager, captured, replayed three times -- other slots each time (a sequence is left
+    # running between the steps), first positions 0 and beyond, wanted places that differ in where but not in how many
+    keeper = engine.start_sequence()
+    engine.step([StepEntry(keeper, [1, 2, 3], None)])
+    run([37, 5, 70], [0, 0, 0], [[0, 36], None, [69]])
+    run([37, 5, 70], [0, 0, 0], [[1, 2], None, [3]])
+    graphs = engine._prefill_graphs.graphs
+    assert len(graphs) == 1
+    other = engine.start_sequence()
+    engine.step([StepEntry(other, [4, 5], None)])
+    run([37, 5, 70], [3, 20, 0], [[36, 0], None, [10]])
+    run([37, 5, 70], [0, 9, 30], [None, [4], [0, 69]])
+    engine.end_sequence(keeper)
+    run([37, 5, 70], [11, 0, 1], [[5], [0, 4], None])
+    assert len(graphs) == 1
+    # a longer first position puts the step into another class of the attention's plan: a shape of its own
+    run([37, 5, 70], [0, 0, 100], [[0, 36], None, [69]])
+    run([37, 5, 70], [0, 0, 100], [[0, 36], None, [69]])
+    assert len(graphs) == 2
+    # more shapes than are kept: the oldest goes, and comes back through a new capture
+    first = next(iter(graphs))
+    for n in range(G.PREFILL_GRAPHS_KEPT):
+        for _ in range(3):
+            run([3 + n], [0], [None])
+    assert len(graphs) == G.PREFILL_GRAPHS_KEPT and first not in graphs
+    for _ in range(3):
+        run([37, 5, 70], [0, 0, 0], [[0, 36], None, [69]])
+    assert first in graphs
+    engine.end_sequence(other)
+    assert engine.free_slots() == engine.cache.max_slots
+
+
 def test_command_line(model_dirs):
     plain = P.PlainLlama(model_dirs["B"])
     prompt = [3, 141, 59, 26, 535]
