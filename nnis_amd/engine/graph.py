@@ -21,6 +21,7 @@ from typing import Dict, List, Sequence, Tuple
 import numpy as np
 import torch
 
+from ..errors import KernelError
 from .batch import StepContext
 
 BUCKETS = (1, 2, 4, 8, 12, 16, 24, 32, 48, 64)
@@ -163,7 +164,7 @@ class PrefillGraph:
         self.ctx = StepContext(
             tokens=total, batch=batch, tok_slot=views[1], tok_pos=views[2], seq_slot=views[3], seq_start=views[4],
             seq_pos0=views[5], decode=False, max_new=max(counts), max_len=ops.PREFILL_CLASS_LENGTH[plan_class],
-            host_new=list(counts), tiles=tiles)
+            host_new=None, host_pos0=None, tiles=tiles)  # (no host lists: a work list that is not in `tiles` is an error)
         self.graph = None
         self.logits = None
 
@@ -186,18 +187,26 @@ class PrefillGraph:
         engine = self.engine
         return engine.model.forward(self.ids, self.ctx, engine.cache, self.want_rows, engine.rt)
 
-    def first_run(self) -> torch.Tensor:
+    def first_run(self):
         """Runs the step that the buffers hold as any step runs, then captures its launches.  Returns that
-        run's logits (the caller's to keep)."""
-        logits = self._forward()
+        run's logits (the caller's to keep), or None if the step cannot run from these buffers; ``graph`` is
+        None afterwards if it could not be captured."""
+        try:
+            logits = self._forward()
+        except KernelError:
+            return None  # (a work list that the shape's record does not name: the caller runs the step as any step)
         torch.cuda.synchronize()
-        self.graph = torch.cuda.CUDAGraph()
+        graph = torch.cuda.CUDAGraph()
         gc.collect()  # (as for the decode graphs: no graph may be destroyed while one is captured)
         collecting = gc.isenabled()
         gc.disable()
         try:
-            with torch.cuda.graph(self.graph):
+            with torch.cuda.graph(graph):
                 self.logits = self._forward()
+            self.graph = graph
+        except KernelError:
+            # a part that cannot run under capture: the shape goes on being launched
+            self.graph = self.logits = None
         finally:
             if collecting:
                 gc.enable()
@@ -215,6 +224,7 @@ class PrefillGraphs:
     def __init__(self, engine):
         self.engine = weakref.proxy(engine)
         self.seen: Dict[tuple, int] = {}
+        self.refused = set()  # shapes whose capture failed
         self.graphs: Dict[tuple, PrefillGraph] = {}  # in the order of their last use
 
     def step(self, key: tuple, arrays, first_positions: Sequence[int], tile_rows):
@@ -225,6 +235,8 @@ class PrefillGraphs:
             self.graphs[key] = graph  # the most recently used is last
             graph.fill(arrays, first_positions)
             return graph.run(), True
+        if key in self.refused:
+            return None
         times = self.seen.get(key, 0) + 1
         self.seen[key] = times
         if len(self.seen) > 1024:
@@ -236,6 +248,9 @@ class PrefillGraphs:
         graph = PrefillGraph(self.engine, counts, wanted, plan_class, rows)
         graph.fill(arrays, first_positions)
         logits = graph.first_run()
+        if graph.graph is None:
+            self.refused.add(key)
+            return None if logits is None else (logits, False)
         while len(self.graphs) >= PREFILL_GRAPHS_KEPT:
             self.graphs.pop(next(iter(self.graphs)))
         self.graphs[key] = graph

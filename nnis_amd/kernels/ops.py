@@ -718,6 +718,10 @@ def _prefill_tiles(ctx, rows: int, device):
     """Work items of a prefill step for tiles of ``rows`` query rows, longest first."""
     cached = ctx.tiles.get(rows)
     if cached is None:
+        if ctx.host_new is None or torch.cuda.is_current_stream_capturing():
+            # (a step that runs from fixed buffers brings its lists; a copy recorded under capture would bring
+            # this step's list to every replay)
+            raise KernelError(f"a prompt step from fixed buffers has no work list for tiles of {rows} rows")
         seqs, row0s = prefill_tile_items(ctx.host_new, ctx.host_pos0, rows)
         count = len(seqs)
         key = (device.type, device.index)

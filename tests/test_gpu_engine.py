@@ -298,6 +298,16 @@ def test_prompt_steps_whose_shape_comes_again(model_dirs, dtype):
     for _ in range(3):
         run([37, 5, 70], [0, 0, 0], [[0, 36], None, [69]])
     assert first in graphs
+    # a step that cannot be captured (here: a work list that the record of the shape's first run does not name)
+    # is launched as any step, this time and from then on
+    run([21, 40], [0, 0], [None, None])
+    (shape,) = [key for key in engine._tile_rows if key[0] == (21, 40)]
+    if engine._tile_rows[shape]:  # (the 32-bit attention has no work lists)
+        engine._tile_rows[shape] = []
+        kept = list(graphs)
+        for _ in range(3):
+            run([21, 40], [0, 0], [[0], [5]])
+        assert shape in engine._prefill_graphs.refused and list(graphs) == kept
     engine.end_sequence(other)
     assert engine.free_slots() == engine.cache.max_slots
 
