@@ -63,14 +63,51 @@ struct Keys {
   unsigned held[PER > 0 ? PER : 1];
 };
 
+// Returns whether one of this thread's logits is not finite.
 template <int PER>
-__device__ __forceinline__ void load_keys(Keys<PER>& keys, const RowView& r) {
+__device__ __forceinline__ int load_keys(Keys<PER>& keys, const RowView& r) {
+  int bad = 0;
   if constexpr (PER > 0) {
 #pragma clang loop unroll(full)
     for (int i = 0; i < PER; ++i) {
       const int c = threadIdx.x + i * kSampleThreads;
-      keys.held[i] = c < r.vocab ? ordered_key(r.logits[c]) : 0u;
+      const float v = c < r.vocab ? r.logits[c] : 0.0f;
+      bad |= isfinite(v) ? 0 : 1;
+      keys.held[i] = c < r.vocab ? ordered_key(v) : 0u;
     }
+  } else {
+    for (int c = threadIdx.x; c < r.vocab; c += kSampleThreads) bad |= isfinite(r.logits[c]) ? 0 : 1;
+  }
+  return bad;
+}
+
+// The weights exp((l - l_max) / T) of every row that samples, 64-bit, with all of the chip (a row's own block
+// would take 49,152 of them 40 us and more).  `best` holds an index of each row's maximum.
+constexpr int kWeightThreads = 256, kWeightsEach = 8;
+__global__ __launch_bounds__(kWeightThreads) void sample_weights_kernel(
+    const float* __restrict__ logits, double* __restrict__ weights, int vocab, const int* __restrict__ row_slot,
+    const float* __restrict__ temperature, int by_slot, const int* __restrict__ best) {
+  const int row = blockIdx.y;
+  const int slot = row_slot[row];
+  if (slot < 0) return;
+  const float* l = logits + (size_t)row * vocab;
+  double* w = weights + (size_t)row * vocab;
+  const double inv_t = 1.0 / (double)temperature[by_slot ? slot : row];
+  const int best_at = best[row];
+  float top = l[best_at < 0 ? 0 : (best_at < vocab ? best_at : vocab - 1)];  // (in range for a row of finite logits; never read outside)
+  if (top == 0.0f) top = 0.0f;
+  const double max_scaled = (double)top * inv_t;
+  const int c0 = blockIdx.x * (kWeightThreads * kWeightsEach) + threadIdx.x;
+  float v[kWeightsEach];
+#pragma unroll
+  for (int j = 0; j < kWeightsEach; ++j) {
+    const int c = c0 + j * kWeightThreads;
+    v[j] = l[c < vocab ? c : vocab - 1];
+  }
+#pragma unroll
+  for (int j = 0; j < kWeightsEach; ++j) {
+    const int c = c0 + j * kWeightThreads;
+    if (c < vocab) w[c] = exp((double)v[j] * inv_t - max_scaled);
   }
 }
 
@@ -103,24 +140,30 @@ __device__ __forceinline__ double mass_at_least(const RowView& r, const Keys<PER
   return block_total(sum, scratch);
 }
 
+// number of tokens whose key is >= t
 template <int PER>
 __device__ __forceinline__ int count_at_least(const RowView& r, const Keys<PER>& keys, unsigned t, int* scratch) {
-  int count = 0;
   if constexpr (PER > 0) {
+    // a comparison and an add with carry an element (counting the lanes' bits with the scalar unit instead was
+    // slower at 96 keys a thread: 239 against 182 us for a whole draw)
+    const unsigned from = t > 1u ? t : 1u;  // an element beyond the row has key 0 and never counts
+    int count = 0;
 #pragma clang loop unroll(full)
-    for (int i = 0; i < PER; ++i) count += (keys.held[i] >= t && keys.held[i] != 0u) ? 1 : 0;
+    for (int i = 0; i < PER; ++i) count += keys.held[i] >= from ? 1 : 0;
+    return block_total(count, scratch);
   } else {
+    int count = 0;
     for (int c = threadIdx.x; c < r.vocab; c += kSampleThreads)
       if (ordered_key(r.logits[c]) >= t) ++count;
+    return block_total(count, scratch);
   }
-  return block_total(count, scratch);
 }
 
 template <int PER>
 __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
     const float* __restrict__ logits, double* __restrict__ weights, int vocab, const int* __restrict__ row_slot,
     unsigned long long* __restrict__ rng, const float* __restrict__ temperature, const int* __restrict__ top_k,
-    const float* __restrict__ top_p, int by_slot, int* __restrict__ out) {
+    const float* __restrict__ top_p, int by_slot, const int* best, int* out) {  // (`best` may be `out`)
   __shared__ double scratch_d[kSampleThreads / kWave];
   __shared__ int scratch_i[kSampleThreads / kWave];
   __shared__ int found;
@@ -133,37 +176,17 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
   r.weights = w;
   r.vocab = vocab;
   Keys<PER> keys;
-  load_keys<PER>(keys, r);
-
-  // maximum key, and a check that every logit is finite
-  unsigned key_max = 0;
-  int bad = 0;
-  for (int c = threadIdx.x; c < vocab; c += kSampleThreads) {
-    const float v = r.logits[c];
-    if (!isfinite(v)) bad = 1;
-    const unsigned key = ordered_key(v);
-    key_max = key > key_max ? key : key_max;
-  }
-  bad = block_total(bad, scratch_i);
-  if (bad) {
+  // a check that every logit is finite, on the way
+  if (block_total(load_keys<PER>(keys, r), scratch_i)) {
     if (threadIdx.x == 0) out[row] = -1;  // the host raises: a non-finite logit is refused
     return;
   }
-#pragma unroll
-  for (int offset = kWave / 2; offset > 0; offset >>= 1) {
-    const unsigned other = __shfl_xor(key_max, offset, kWave);
-    key_max = other > key_max ? other : key_max;
-  }
-  __shared__ unsigned wave_keys[kSampleThreads / kWave];
-  if (threadIdx.x % kWave == 0) wave_keys[threadIdx.x / kWave] = key_max;
-  __syncthreads();
-  for (int i = 0; i < kSampleThreads / kWave; ++i) key_max = wave_keys[i] > key_max ? wave_keys[i] : key_max;
-  const unsigned max_bits = (key_max & 0x80000000u) ? (key_max & 0x7fffffffu) : ~key_max;
   const int at = by_slot ? slot : row;  // where the row's options lie: per sequence (kept with its slot) or per row
   const double inv_t = 1.0 / (double)temperature[at];
-  const double max_scaled = (double)__uint_as_float(max_bits) * inv_t;
-  for (int c = threadIdx.x; c < vocab; c += kSampleThreads) w[c] = exp((double)r.logits[c] * inv_t - max_scaled);
-  __syncthreads();
+  const int best_at = best[row];
+  float top = r.logits[best_at < 0 ? 0 : (best_at < vocab ? best_at : vocab - 1)];  // (as sample_weights_kernel took it)
+  if (top == 0.0f) top = 0.0f;
+  const double max_scaled = (double)top * inv_t;
 
   // the kept prefix: everything with key > cut_key plus `cut_ties` tokens at cut_key
   unsigned cut_key = 0;
@@ -190,10 +213,72 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
   // top.  With the keys in registers a probe first counts (no memory): a probe that holds the same tokens as
   // the bound above it (which failed) or as the bound below (which held) needs no sum -- among 49,152 keys that
   // is about half of the 32 probes, the upper bits that all keys share and the lower ones between neighbours.
-  auto find_cut = [&](auto holds) -> unsigned {
+  // And once the kept tokens between the two bounds are few (kNear), their keys and weights are put into LDS, in
+  // a fixed order, and a probe sums those on top of the upper bound's weight: a sum over the row's weights in
+  // memory takes 6 to 8 us, one over the near ones under 1.
+  constexpr int kNear = 2048;
+  __shared__ unsigned near_key[kNear];
+  __shared__ int near_at[kNear];
+  __shared__ double near_weight[kNear];
+  __shared__ int wave_near[kSampleThreads / kWave];
+  bool near = false;         // the search's state, for `mass_from` after it too
+  int near_count = 0;
+  double mass_above = 0.0;   // weight of the tokens at and above the lowest probe that failed before the near ones were taken
+
+  auto gather_near = [&](unsigned lower, unsigned upper, bool has_upper) __attribute__((always_inline)) {
+    const unsigned from = lower > 1u ? lower : 1u;
+    int mine = 0;
+    if constexpr (PER > 0) {
+#pragma clang loop unroll(full)
+      for (int i = 0; i < PER; ++i) mine += (keys.held[i] >= from && (!has_upper || keys.held[i] < upper)) ? 1 : 0;
+    }
+    const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+    int upto = mine;  // with this thread's
+#pragma unroll
+    for (int offset = 1; offset < kWave; offset <<= 1) {
+      const int other = __shfl_up(upto, offset, kWave);
+      upto += lane >= offset ? other : 0;
+    }
+    __syncthreads();
+    if (lane == kWave - 1) wave_near[wave] = upto;
+    __syncthreads();
+    int place = upto - mine, all = 0;
+    for (int w = 0; w < kSampleThreads / kWave; ++w) {
+      place += w < wave ? wave_near[w] : 0;
+      all += wave_near[w];
+    }
+    if constexpr (PER > 0) {
+#pragma clang loop unroll(full)
+      for (int i = 0; i < PER; ++i) {
+        if (keys.held[i] >= from && (!has_upper || keys.held[i] < upper)) {
+          near_key[place] = keys.held[i];
+          near_at[place] = threadIdx.x + i * kSampleThreads;
+          ++place;
+        }
+      }
+    }
+    __syncthreads();
+    for (int j = threadIdx.x; j < all; j += kSampleThreads) near_weight[j] = r.weights[near_at[j]];
+    __syncthreads();
+    near = true;
+    near_count = all;
+  };
+  // weight of the kept tokens with key >= probe (above the limit, if there is one)
+  auto mass_from = [&](unsigned probe) __attribute__((always_inline)) -> double {
+    if (!near) return mass_at_least<PER>(r, keys, probe, scratch_d);
+    double sum = 0.0;
+    for (int j = threadIdx.x; j < near_count; j += kSampleThreads) sum += near_key[j] >= probe ? near_weight[j] : 0.0;
+    return mass_above + block_total(sum, scratch_d);
+  };
+
+  auto find_cut = [&](auto holds) __attribute__((always_inline)) -> unsigned {
     unsigned t = 0;
     int count_below = -1;  // tokens with key >= t, where known (not at the start: with a limit `total` is not all tokens' weight)
     int count_above = 0;   // tokens at and above the lowest probe that failed; at first none, whose weight 0 never holds
+    unsigned upper = 0;    // the lowest probe that failed, if one has
+    bool has_upper = false;
+    near = false;
+    mass_above = 0.0;
     for (int bit = 31; bit >= 0; --bit) {
       const unsigned probe = t | (1u << bit);
       if (limited && probe <= cut_key) {  // everything kept lies at or above the limit: the whole kept weight, which holds
@@ -209,12 +294,23 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
           t = probe;
           continue;
         }
+        if (!near) {
+          const unsigned lower = (limited && t <= cut_key) ? cut_key + 1u : t;  // (cut_key < probe <= 2^32 - 1)
+          const int between = (count_below >= 0 && lower == t ? count_below : count_at_least<PER>(r, keys, lower, scratch_i)) - count_above;
+          if (between <= kNear) gather_near(lower, upper, has_upper);
+        }
       }
-      if (holds(mass_at_least<PER>(r, keys, probe, scratch_d))) {
+      const double mass = mass_from(probe);
+      if (holds(mass)) {
         t = probe;
         count_below = count;
       } else {
         count_above = count;
+        if (!near) {  // (the near tokens were taken below the bound of that moment: its weight stays their base)
+          mass_above = mass;
+          upper = probe;
+          has_upper = true;
+        }
       }
     }
     return t;
@@ -225,7 +321,7 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
     const double threshold = (double)p * total;
     const unsigned t = find_cut([&](double mass) { return mass >= threshold; });
     // t >= cut_key when limited, because the whole kept mass reaches the threshold
-    const double base = mass_at_least<PER>(r, keys, t + 1u, scratch_d);
+    const double base = mass_from(t + 1u);
     const double weight_at = exp((double)__uint_as_float((t & 0x80000000u) ? (t & 0x7fffffffu) : ~t) * inv_t - max_scaled);
     int available = (limited && t == cut_key) ? cut_ties
                                               : count_at_least<PER>(r, keys, t, scratch_i) - count_at_least<PER>(r, keys, t + 1u, scratch_i);
@@ -247,10 +343,11 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
   const double draw = unit * total;
 
   const unsigned t = find_cut([&](double mass) { return mass > draw; });
-  const double base = mass_at_least<PER>(r, keys, t + 1u, scratch_d);
+  const double base = mass_from(t + 1u);
   const double weight_at = exp((double)__uint_as_float((t & 0x80000000u) ? (t & 0x7fffffffu) : ~t) * inv_t - max_scaled);
-  const int available = (limited && t == cut_key) ? cut_ties
-                                                  : count_at_least<PER>(r, keys, t, scratch_i) - count_at_least<PER>(r, keys, t + 1u, scratch_i);
+  int same = -1;  // tokens whose key equals t, where it is known or cheap to know
+  if (PER > 0 || !(limited && t == cut_key)) same = count_at_least<PER>(r, keys, t, scratch_i) - count_at_least<PER>(r, keys, t + 1u, scratch_i);
+  const int available = (limited && t == cut_key) ? cut_ties : same;
   int index = 0;
   double reached = base + weight_at;
   while (index + 1 < available && !(draw < reached)) {
@@ -258,6 +355,15 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
     reached += weight_at;
   }
 
+  if constexpr (PER > 0) {
+    if (same == 1) {  // the usual case, no ties at t: the thread that holds the key names the token
+#pragma clang loop unroll(full)
+      for (int i = 0; i < PER; ++i)
+        if (keys.held[i] == t) out[row] = threadIdx.x + i * kSampleThreads;
+      if (threadIdx.x == 0) rng[slot] = state;
+      return;
+    }
+  }
   // the index-th token (by id) whose key equals t: contiguous chunks per thread, then a scan
   const int chunk = (vocab + kSampleThreads - 1) / kSampleThreads;
   const int begin = threadIdx.x * chunk;
@@ -302,13 +408,17 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
 
 extern "C" int nnis_sample(const float* logits, double* weights, int rows, int vocab, const int* row_slot,
                            unsigned long long* rng, const float* temperature, const int* top_k, const float* top_p,
-                           int by_slot, int* out, void* stream) {
+                           int by_slot, const int* best, int* out, void* stream) {
   NNIS_REQUIRE(rows >= 0 && vocab > 0, "sample: bad sizes rows=%d vocab=%d", rows, vocab);
+  NNIS_REQUIRE(best != nullptr, "sample: needs an index of each row's maximum");
+  NNIS_REQUIRE(rows <= 65535, "sample: %d rows are more than a launch takes", rows);
   NNIS_REQUIRE((long long)vocab <= 65535LL * kSampleThreads, "sample: vocabulary %d is too large for this kernel", vocab);
   if (rows == 0) return 0;
   const dim3 grid(rows), block(kSampleThreads);
   hipStream_t s = (hipStream_t)stream;
-#define NNIS_SAMPLE(PER) hipLaunchKernelGGL(sample_kernel<PER>, grid, block, 0, s, logits, weights, vocab, row_slot, rng, temperature, top_k, top_p, by_slot, out)
+  hipLaunchKernelGGL(sample_weights_kernel, dim3((vocab + kWeightThreads * kWeightsEach - 1) / (kWeightThreads * kWeightsEach), rows),
+                     dim3(kWeightThreads), 0, s, logits, weights, vocab, row_slot, temperature, by_slot, best);
+#define NNIS_SAMPLE(PER) hipLaunchKernelGGL(sample_kernel<PER>, grid, block, 0, s, logits, weights, vocab, row_slot, rng, temperature, top_k, top_p, by_slot, best, out)
   // elements a thread keeps in registers: the least that covers the row
   if (vocab <= 8 * kSampleThreads) NNIS_SAMPLE(8);
   else if (vocab <= 16 * kSampleThreads) NNIS_SAMPLE(16);

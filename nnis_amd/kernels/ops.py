@@ -42,7 +42,7 @@ _CORE_SIGNATURES = {
     "nnis_gemm_residual_runs": [_VOID, _INT, _INT, _INT, _VOID, _VOID, _VOID, _VOID, _INT, _VOID, _VOID, _INT, _INT, _INT, _VOID,
                                 _VOID],
     "nnis_pack_weight": [_VOID, _VOID, _INT, _INT, _VOID],
-    "nnis_sample": [_VOID, _VOID, _INT, _INT, _VOID, _VOID, _VOID, _VOID, _VOID, _INT, _VOID, _VOID],
+    "nnis_sample": [_VOID, _VOID, _INT, _INT, _VOID, _VOID, _VOID, _VOID, _VOID, _INT, _VOID, _VOID, _VOID],
 }
 _ATTN_SIGNATURES = {
     "nnis_attention_rows": [_VOID, _INT, _VOID, _INT, _VOID, _VOID, _INT, _VOID, _INT, _VOID, _VOID, _INT, _INT, _INT,
@@ -778,12 +778,16 @@ def attention(q: torch.Tensor, out: torch.Tensor, view, ctx, heads: int, kv_head
 
 
 def sample(logits: torch.Tensor, weights: torch.Tensor, row_slot: torch.Tensor, rng: torch.Tensor,
-           temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor, out: torch.Tensor, by_slot: bool = False) -> torch.Tensor:
+           temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor, out: torch.Tensor, by_slot: bool = False,
+           best: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Seeded sampling per row; rows whose slot is negative are skipped (their
     ``out`` stays as it is).  ``rng`` is int64 [slots] holding each sequence's
     SplitMix64 state; ``weights`` is float64 scratch of at least [rows, vocab].
     ``temperature``, ``top_k`` and ``top_p`` hold a value per row, or, with
-    ``by_slot``, per slot (like ``rng``).  A row with a non-finite logit gets -1."""
+    ``by_slot``, per slot (like ``rng``).  ``best`` (int32 [rows], may be
+    ``out``) holds an index of each row's maximum where the caller has it
+    (``argmax``); without it the maxima are found here.  A row with a
+    non-finite logit gets -1."""
     for t, what in ((logits, "logits"), (weights, "weights"), (row_slot, "row_slot"), (rng, "rng"),
                     (temperature, "temperature"), (top_k, "top_k"), (top_p, "top_p"), (out, "out")):
         _dev(t, what)
@@ -799,8 +803,14 @@ def sample(logits: torch.Tensor, weights: torch.Tensor, row_slot: torch.Tensor, 
     needed = rng.numel() if by_slot else rows
     if min(temperature.numel(), top_k.numel(), top_p.numel()) < needed:
         raise KernelError("sample: temperature, top_k and top_p need a value per " + ("slot" if by_slot else "row"))
+    if best is None:
+        best = argmax(logits, torch.empty(rows, dtype=torch.int32, device=logits.device))
+    else:
+        _dev(best, "best")
+        if best.dtype != torch.int32 or best.numel() < rows:
+            raise KernelError("sample: best must be int32 [rows]")
     lib = core()
     _check(lib, lib.nnis_sample(logits.data_ptr(), weights.data_ptr(), rows, vocab, row_slot.data_ptr(), rng.data_ptr(),
-                                temperature.data_ptr(), top_k.data_ptr(), top_p.data_ptr(), 1 if by_slot else 0, out.data_ptr(),
-                                _stream()))
+                                temperature.data_ptr(), top_k.data_ptr(), top_p.data_ptr(), 1 if by_slot else 0,
+                                best.data_ptr(), out.data_ptr(), _stream()))
     return out

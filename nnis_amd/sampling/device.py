@@ -95,7 +95,7 @@ class DeviceSelector:
                 self._weights = torch.empty((max(rows, 8), self.vocab_size), dtype=torch.float64, device=self.rt.device)
             # the rows that sample are written over; a greedy row keeps its argmax
             ops.sample(logits, self._weights, self._sampling_rows(slots, params), self.rng, self.temperature, self.top_k,
-                       self.top_p, device[:rows], by_slot=True)
+                       self.top_p, device[:rows], by_slot=True, best=device[:rows])
         host[:rows].copy_(device[:rows], non_blocking=True)
         event.record()
         return PendingTokens(device[:rows], host[:rows], event)
