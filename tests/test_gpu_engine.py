@@ -369,19 +369,25 @@ def test_command_line_with_text(model_dirs, tmp_path):
 
 @pytest.mark.parametrize("options", [dict(), dict(temperature=0.8), dict(top_k=40), dict(top_p=0.7),
                                      dict(temperature=1.3, top_k=200, top_p=0.95), dict(top_k=1)])
-def test_device_sampling_matches_the_host_sampler(options):
+@pytest.mark.parametrize("vocab", [1000, 5003, 20011, 49152, 70001])
+def test_device_sampling_matches_the_host_sampler(options, vocab):
     """Same logits, same seeds: the kernel picks what the reference's host
-    procedure picks, draw after draw (the generator state lives per slot)."""
+    procedure picks, draw after draw (the generator state lives per slot).
+    The vocabularies take the kernel's variants: keys in registers, 8 to 128 a
+    thread, and read from memory (70,001); from 5,003 on a search starts with
+    sums over the whole row and goes on with the tokens near the draw."""
     from nnis_amd.kernels import ops
     from nnis_amd.sampling import HostSampler, SamplingParams
 
-    vocab, rows, draws = 1000, 6, 40
+    rows, draws = 6, 40 if vocab == 1000 else 8
     rng = np.random.default_rng(3)
     logits = (rng.standard_normal((rows, vocab)) * 2.5).astype(np.float32)
     logits[0, 5] = logits[0, 900] = logits[0].max() + 0.5  # a tie at the top
     logits[1, :] = 0.25  # all equal
     logits[2, 17] = -0.0
     logits[2, 18] = 0.0
+    logits[3] = np.round(logits[3] * 4) / 4  # many ties everywhere: a draw's key is shared by hundreds
+    logits[4] *= 0.02  # nearly flat: the tokens near a draw stay many for most of the search
     dev = torch.from_numpy(logits).cuda()
     slots = [4, 0, 7, 2, 5, -1]  # the last row is skipped
     state = torch.zeros(8, dtype=torch.int64, device="cuda")
