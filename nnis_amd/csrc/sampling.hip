@@ -192,23 +192,6 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
   unsigned cut_key = 0;
   int cut_ties = 0;          // meaningful only when limited
   bool limited = false;
-  double total = mass_at_least<PER>(r, keys, 0u, scratch_d);
-
-  const int k = top_k[at];
-  if (k > 0 && k < vocab) {
-    unsigned t = 0;
-    for (int bit = 31; bit >= 0; --bit) {
-      const unsigned probe = t | (1u << bit);
-      if (count_at_least<PER>(r, keys, probe, scratch_i) >= k) t = probe;
-    }
-    const int above = count_at_least<PER>(r, keys, t + 1u, scratch_i);
-    cut_key = t;
-    cut_ties = k - above;
-    limited = true;
-    const double weight_at = exp((double)__uint_as_float((t & 0x80000000u) ? (t & 0x7fffffffu) : ~t) * inv_t - max_scaled);
-    total = mass_at_least<PER>(r, keys, t + 1u, scratch_d) + (double)cut_ties * weight_at;
-  }
-
   // The largest key t at which `holds(weight of all kept tokens with key >= t)` is still true, by bits from the
   // top.  With the keys in registers a probe first counts (no memory): a probe that holds the same tokens as
   // the bound above it (which failed) or as the bound below (which held) needs no sum -- among 49,152 keys that
@@ -286,6 +269,10 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
         count_below = -1;
         continue;
       }
+      if (near) {  // the sums decide by themselves: over the same tokens they are the same sums
+        if (holds(mass_from(probe))) t = probe;
+        continue;
+      }
       int count = -2;
       if constexpr (PER > 0) {
         count = count_at_least<PER>(r, keys, probe, scratch_i);
@@ -315,6 +302,46 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
     }
     return t;
   };
+
+  // top-k: the k-th largest key by a search over counts; once the tokens between its bounds are few, over those
+  const int k = top_k[at];
+  double total;
+  if (k > 0 && k < vocab) {
+    unsigned t = 0, upper = 0;
+    bool has_upper = false;
+    int above = 0, below = vocab;  // tokens at and above `upper`, at and above t (while the search counts the whole row)
+    for (int bit = 31; bit >= 0; --bit) {
+      const unsigned probe = t | (1u << bit);
+      int count;
+      if (near) {
+        int some = 0;
+        for (int j = threadIdx.x; j < near_count; j += kSampleThreads) some += near_key[j] >= probe ? 1 : 0;
+        count = above + block_total(some, scratch_i);
+      } else {
+        count = count_at_least<PER>(r, keys, probe, scratch_i);
+      }
+      if (count >= k) {
+        t = probe;
+        if (!near) below = count;
+      } else if (!near) {
+        above = count;
+        upper = probe;
+        has_upper = true;
+      }
+      if constexpr (PER > 0) {
+        if (!near && below - above <= kNear) gather_near(t, upper, has_upper);
+      }
+    }
+    near = false;
+    const int over = count_at_least<PER>(r, keys, t + 1u, scratch_i);
+    cut_key = t;
+    cut_ties = k - over;
+    limited = true;
+    const double weight_at = exp((double)__uint_as_float((t & 0x80000000u) ? (t & 0x7fffffffu) : ~t) * inv_t - max_scaled);
+    total = mass_at_least<PER>(r, keys, t + 1u, scratch_d) + (double)cut_ties * weight_at;
+  } else {
+    total = mass_at_least<PER>(r, keys, 0u, scratch_d);
+  }
 
   const float p = top_p[at];
   if (p > 0.0f && p <= 1.0f) {
