@@ -129,10 +129,10 @@ class DecodeGraphs:
 # kernels read that data from fixed buffers; from the third time on the step is a copy into the buffers
 # and a replay.  Only shapes of up to PREFILL_GRAPH_MOST_TOKENS tokens are kept, the most recently used
 # PREFILL_GRAPHS_KEPT of them (a graph keeps its activations' memory), and only where the step's kernels are
-# short enough for the host to matter: tokens x width^2 up to PREFILL_GRAPH_MOST_WORK.  (Measured, a
-# 2,048-token step: width 576 2.32 ms replayed against 2.35 to 2.65 launched, by the host's speed; width 2048
-# 7.65 against 7.45 and 11.4 against 11.0 -- a replay leaves a gap of a microsecond between kernels that
-# launches keeping ahead of the GPU do not.)
+# short enough for the host to matter: tokens x width^2 up to PREFILL_GRAPH_MOST_WORK.  Measured, one prompt a
+# step, launched against replayed, milliseconds: width 576, 30 layers: 64 tokens 2.27 / 0.83, 256 2.33 / 1.33,
+# 1,024 2.41 / 1.64, 2,048 2.42 / 2.24; width 2048, 22 layers: 64 tokens 1.79 / 1.38, 256 2.16 / 2.08, 512
+# 2.77 / 2.75, from 1,024 on equal (4.24, 7.28): there the kernels bound the step and a graph would only hold memory.
 PREFILL_GRAPH_MOST_TOKENS = 4096
 PREFILL_GRAPH_MOST_WORK = 1.5e9
 PREFILL_GRAPHS_KEPT = 4
