@@ -1,0 +1,47 @@
+"""The host-side choices of the attention kernels' shapes: pure functions of
+the step's sizes, checked for their invariants (what a kernel's launch
+assumes) and for the measured cases their docstrings name."""
+
+import pytest
+
+from nnis_amd.kernels.ops import PREFILL_CLASS_LENGTH, decode_plan, prefill_plan_class, prefill_tile_items
+
+
+@pytest.mark.parametrize("batch", [1, 2, 8, 33, 64, 256])
+@pytest.mark.parametrize("kv_heads", [1, 3, 8, 32])
+@pytest.mark.parametrize("longest", [1, 63, 64, 65, 600, 1100, 2048, 8191])
+@pytest.mark.parametrize("width", [0, 576, 2048, 4096])
+def test_decode_plan_invariants(batch, kv_heads, longest, width):
+    splits, waves = decode_plan(batch, kv_heads, longest, max_waves=4, width=width)
+    pages = (longest + 63) // 64
+    for n in (splits, waves):
+        assert n >= 1 and n & (n - 1) == 0  # powers of two
+    assert waves <= 4 and waves <= max(1, pages)  # no wave without a page
+    assert splits <= 8
+    if pages <= 8:
+        assert splits == 1  # short sequences are never cut into runs
+    if splits > 1:
+        assert batch * kv_heads * waves * splits <= 2048  # runs only while the chip has room for their blocks
+    assert decode_plan(batch, kv_heads, longest, max_waves=1, width=width)[1] == 1
+
+
+def test_decode_plan_measured_cases():
+    assert decode_plan(8, 3, 2048, width=576) == (8, 4)      # a narrow model: a page or two a wave
+    assert decode_plan(64, 3, 2048, width=576) == (1, 4)     # no room for runs
+    assert decode_plan(16, 32, 2048, width=2048) == (1, 4)
+    assert decode_plan(64, 32, 2048, width=2048) == (1, 2)   # four and more blocks a compute unit: two waves a block
+    assert decode_plan(8, 3, 64, width=576) == (1, 1)
+
+
+def test_prefill_plan_class_and_work_lists():
+    assert [prefill_plan_class(n) for n in (1, 127, 128, 511, 512, 1023, 1024, 5000)] == [0, 0, 1, 1, 2, 2, 3, 3]
+    for plan_class, least in enumerate(PREFILL_CLASS_LENGTH):
+        assert prefill_plan_class(least) == plan_class
+    # every row of every sequence lies in exactly one tile; longest tiles (by the keys they read) first
+    counts, first = [37, 5, 70, 1], [0, 100, 3, 64]
+    for rows in (16, 32, 64):
+        seqs, row0s = prefill_tile_items(counts, first, rows)
+        seen = sorted((s, r) for s, r in zip(seqs, row0s))
+        assert seen == sorted((s, r) for s, n in enumerate(counts) for r in range(0, n, rows))
+        ends = [first[s] + min(r + rows, counts[s]) for s, r in zip(seqs, row0s)]
+        assert ends == sorted(ends, reverse=True)
