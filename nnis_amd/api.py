@@ -13,28 +13,33 @@ from .models.decoder import DecoderModel
 from .weights.loader import load_weights
 
 
-def load_model(model_dir: str, dtype="bfloat16", device="cuda:0"):
+def load_model(model_dir: str, dtype="bfloat16", device="cuda:0", narrow_to_bfloat16: bool = False):
     """Reads config.json, picks the model by its architecture name, loads the
-    tensors by name and binds them to the parts.  Returns (model, runtime)."""
+    tensors by name and binds them to the parts.  Returns (model, runtime).
+    ``narrow_to_bfloat16``: a checkpoint stored in 32-bit is rounded to
+    bfloat16 as it is loaded (only with ``dtype`` bfloat16); without it its
+    weights stay 32-bit and take the slow ordered product."""
     raw = read_config_json(model_dir)
     _, spec = spec_from_config(raw)
     rt = Runtime(device=device, dtype=dtype)
     model = DecoderModel(spec)
-    weights = load_weights(model_dir, model.tensors(), rt.device, widen_to_float32=rt.is_fp32)
+    weights = load_weights(model_dir, model.tensors(), rt.device, widen_to_float32=rt.is_fp32,
+                           declared_dtype=spec.stored_dtype, narrow_to_bfloat16=narrow_to_bfloat16)
     model.bind(weights, rt)
     return model, rt
 
 
 def load_engine(model_dir: str, dtype="bfloat16", max_tokens: int = 8192, device="cuda:0",
-                max_slots: Optional[int] = None) -> Engine:
-    model, rt = load_model(model_dir, dtype=dtype, device=device)
+                max_slots: Optional[int] = None, narrow_to_bfloat16: bool = False) -> Engine:
+    model, rt = load_model(model_dir, dtype=dtype, device=device, narrow_to_bfloat16=narrow_to_bfloat16)
     return Engine(model, rt, max_tokens=max_tokens, max_slots=max_slots)
 
 
 def generate(model, prompts: Sequence[Sequence[int]], max_new_tokens: int = 16, sample: bool = False,
              seed: Union[int, Sequence[int], None] = None, temperature: float = 1.0, top_k: Optional[int] = None,
              top_p: Optional[float] = None, stop_token_ids: Optional[Sequence[int]] = None, dtype="bfloat16",
-             device="cuda:0", max_tokens: Optional[int] = None, max_batch: int = 64) -> List[List[int]]:
+             device="cuda:0", max_tokens: Optional[int] = None, max_batch: int = 64,
+             narrow_to_bfloat16: bool = False) -> List[List[int]]:
     """The Python entry point, with the command line's option names and
     meanings (/root/reference/crates/nnis-cli/src/main.rs:179-365): greedy
     unless ``sample``; ``sample`` requires a seed (one per prompt, or one
@@ -63,7 +68,7 @@ def generate(model, prompts: Sequence[Sequence[int]], max_new_tokens: int = 16, 
         engine = model
     else:
         need = max_tokens or sum(((len(p) + max_new_tokens + 63) // 64) * 64 for p in prompts)
-        engine = load_engine(model, dtype=dtype, max_tokens=need, device=device)
+        engine = load_engine(model, dtype=dtype, max_tokens=need, device=device, narrow_to_bfloat16=narrow_to_bfloat16)
     stops = engine.model.spec.stop_token_ids if stop_token_ids is None else tuple(stop_token_ids)
     requests = [
         GenerationRequest(p, max_new_tokens, stops,

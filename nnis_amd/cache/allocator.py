@@ -12,6 +12,7 @@ because the length says where the data ends.
 
 from __future__ import annotations
 
+import heapq
 from typing import Dict, List
 
 from ..errors import CacheFull, InvalidInput
@@ -32,7 +33,7 @@ class FreeList:
             raise InvalidInput(f"a cache needs at least one {what}")
         self.count = count
         self.what = what
-        self._free = list(range(count - 1, -1, -1))  # pop() gives the lowest
+        self._free = list(range(count))  # a heap: the lowest comes first, whatever order items came back in
         self._held = set()
 
     @property
@@ -46,7 +47,7 @@ class FreeList:
     def take(self) -> int:
         if not self._free:
             raise CacheFull(f"no free {self.what} (all {self.count} are held)")
-        item = self._free.pop()
+        item = heapq.heappop(self._free)
         self._held.add(item)
         return item
 
@@ -54,9 +55,7 @@ class FreeList:
         if item not in self._held:
             raise InvalidInput(f"{self.what} {item} is not held (released twice, or never acquired)")
         self._held.remove(item)
-        self._free.append(item)
-        # keep lowest-first order so reuse is deterministic
-        self._free.sort(reverse=True)
+        heapq.heappush(self._free, item)  # lowest-first reuse stays deterministic without a sort per item
 
 
 class PageTable:
@@ -92,3 +91,17 @@ class PageTable:
     def release(self, slot: int) -> None:
         for page in self.rows.pop(slot, []):
             self.pool.give_back(page)
+
+    def shrink(self, slot: int, new_length: int) -> int:
+        """Gives back the pages of ``slot`` beyond those that ``new_length``
+        tokens need; returns how many.  The row's first pages stay where they
+        are, so the block table's entries for the tokens kept do not change."""
+        row = self.rows.get(slot)
+        keep = pages_for(new_length)
+        if not row or len(row) <= keep:
+            return 0
+        gone = row[keep:]
+        del row[keep:]
+        for page in gone:
+            self.pool.give_back(page)
+        return len(gone)

@@ -58,7 +58,7 @@ class KVGroup:
         self.table = PageTable(pages, slots, per_slot)
         # zero at first: a page's unwritten tail is multiplied by zero weights, so it must hold numbers
         self.k = torch.zeros((len(entries), pages) + k_page_shape(request.kv_heads, request.head_dim), dtype=dtype, device=device)
-        self.v = torch.zeros((len(entries), pages) + v_page_shape(request.kv_heads, request.head_dim), dtype=dtype, device=device)
+        self.v = torch.zeros((len(entries), pages) + v_page_shape(request.kv_heads, request.value_head_dim), dtype=dtype, device=device)
         pinned = torch.device(device).type == "cuda"
         self.block_table_host = torch.zeros((slots, per_slot), dtype=torch.int32, pin_memory=pinned)
         self.block_table = torch.zeros((slots, per_slot), dtype=torch.int32, device=device)
@@ -66,7 +66,8 @@ class KVGroup:
         self._dirty = set()
 
     def bytes_per_token(self) -> int:
-        return 2 * len(self.entries) * self.request.kv_heads * self.request.head_dim * self.k.element_size()
+        return (len(self.entries) * self.request.kv_heads * (self.request.head_dim + self.request.value_head_dim)
+                * self.k.element_size())
 
     def grow(self, slot: int, new_length: int) -> None:
         changed = self.table.grow(slot, new_length)
@@ -105,6 +106,7 @@ class SequenceCache:
 
         self.kv_groups: List[KVGroup] = []
         self.state_regions: Dict[str, torch.Tensor] = {}
+        self._layer_state: List[str] = []  # regions that a mixer's StateRequest asked for
         self._views: Dict[int, Any] = {}
         grouped: Dict[KVRequest, List[int]] = {}
         for index, request in requests:
@@ -112,6 +114,7 @@ class SequenceCache:
                 grouped.setdefault(request, []).append(index)
             elif isinstance(request, StateRequest):
                 region = self.add_state_region(f"entry{index}", request.shape, getattr(torch, request.dtype))
+                self._layer_state.append(f"entry{index}")
                 self._views[index] = StateView(region, read_only=False)
             elif request is not None:
                 raise InvalidInput(f"schedule entry {index}: unknown cache request {request!r}")
@@ -157,6 +160,39 @@ class SequenceCache:
             return self.lengths[slot]
         except KeyError:
             raise InvalidInput(f"cache slot {slot} is not held") from None
+
+    def truncate(self, slot: int, length: int) -> None:
+        """Shortens a sequence to its first ``length`` tokens: the pages beyond
+        go back to their pools at once, the tokens kept stay where they are, and
+        the next step appends at ``length``
+        (/root/reference/crates/nnis-rt/src/kv_cache.rs:181-192: a length above
+        the current one is an error and nothing changes).  What the given-up
+        part of the last page kept holds is never read: the length says where
+        the data ends.  Refused where the model keeps fixed-size state per
+        sequence (``StateRequest``): such state has consumed the dropped
+        tokens and cannot be wound back."""
+        current = self.length(slot)
+        if not 0 <= int(length) <= current:
+            raise InvalidInput(f"slot {slot} holds {current} tokens; it cannot be truncated to {length}")
+        if length == current:
+            return
+        if self._layer_state:
+            raise InvalidInput(
+                f"slot {slot}: a model that keeps fixed-size state per sequence ({', '.join(self._layer_state)}) cannot be "
+                "truncated; release the slot and run the tokens again")
+        for group in self.kv_groups:
+            group.table.shrink(slot, int(length))
+        self.lengths[slot] = int(length)
+
+    def reset(self, slot: int) -> None:
+        """The slot as it was when acquired: no tokens, no pages, state zero
+        (kv_cache.rs:170-172).  The slot stays held."""
+        self.length(slot)  # raises if the slot is not held
+        for group in self.kv_groups:
+            group.table.shrink(slot, 0)
+        self.lengths[slot] = 0
+        for region in self.state_regions.values():
+            region[slot].zero_()
 
     def check_room(self, growth: Dict[int, int]) -> None:
         """Raises before anything changes if the slots cannot grow by the given

@@ -5,8 +5,11 @@ running, :1348-1391 exit codes: 0 success, 1 runtime failure, 2 usage error).
 
 Additions of this library, because a model folder made from random weights has
 no tokenizer: ``--prompt-ids 5,17,3`` gives a prompt as token ids (the output
-is then ids too), ``--dtype`` picks the precision and ``--max-tokens`` sizes
-the cache.  ``--tokenizer`` defaults to MODEL/tokenizer.json, as in the
+is then ids too), ``--dtype`` picks the precision, ``--narrow-to-bfloat16``
+rounds a checkpoint stored in 32-bit to bfloat16 as it is loaded (the
+reference refuses to narrow implicitly,
+/root/reference/crates/nnis-model/src/safetensors_loader.rs:610-624: here it
+is the caller's explicit choice) and ``--max-tokens`` sizes the cache.  ``--tokenizer`` defaults to MODEL/tokenizer.json, as in the
 reference's Hugging Face front end
 (/root/reference/docs/HF_GENERATION_PROCESS.md:31).
 """
@@ -26,14 +29,14 @@ SAMPLING_POLICY_VERSION = 1
 GENERATE_BATCH_JSON_SCHEMA_VERSION = 1
 
 USAGE = """Usage:
-  nnis generate --model DIR [--tokenizer FILE] (--prompt TEXT | --prompt-ids IDS) [--device N] [--max-new-tokens N] [--sample --seed U64] [--temperature F] [--top-k N] [--top-p F] [--stream] [--dtype bfloat16|float32] [--max-tokens N]
-  nnis generate-batch --model DIR [--tokenizer FILE] (--prompt TEXT | --prompt-ids IDS) [--prompt ...] --seed U64 [--seed U64 ...] [--device N] [--max-new-tokens N] [--temperature F] [--top-k N] [--top-p F] [--json] [--dtype bfloat16|float32] [--max-tokens N]
+  nnis generate --model DIR [--tokenizer FILE] (--prompt TEXT | --prompt-ids IDS) [--device N] [--max-new-tokens N] [--sample --seed U64] [--temperature F] [--top-k N] [--top-p F] [--stream] [--dtype bfloat16|float32] [--narrow-to-bfloat16] [--max-tokens N]
+  nnis generate-batch --model DIR [--tokenizer FILE] (--prompt TEXT | --prompt-ids IDS) [--prompt ...] --seed U64 [--seed U64 ...] [--device N] [--max-new-tokens N] [--temperature F] [--top-k N] [--top-p F] [--json] [--dtype bfloat16|float32] [--narrow-to-bfloat16] [--max-tokens N]
 
 Default decoding on `generate` is greedy. Opt-in `--sample` requires `--seed`. Optional `--temperature`, `--top-k`, and `--top-p` apply only with `--sample`. `--stream` is valid only with `--sample` and prints each token as it is emitted. The device ordinal defaults to 0.
 
 `generate-batch` is always sampled and requires one `--seed` per prompt (no silent seed reuse). Shared optional `--temperature` / `--top-k` / `--top-p` apply to every request. The prompts are prefilled together in one step and decoded as one batch; a request that ends earlier leaves the batch. Human text by default; `--json` emits versioned JSON.
 
-`--prompt-ids` takes comma-separated token ids instead of text; the output is then token ids."""
+`--prompt-ids` takes comma-separated token ids instead of text; the output is then token ids. `--narrow-to-bfloat16` rounds weights stored in 32-bit to bfloat16 at load (with `--dtype bfloat16`)."""
 
 
 class UsageError(Exception):
@@ -56,6 +59,7 @@ class GenerateArgs:
     top_p: Optional[float] = None
     json: bool = False
     dtype: str = "bfloat16"
+    narrow_to_bfloat16: bool = False
     max_tokens: Optional[int] = None
     batch: bool = False
 
@@ -166,6 +170,8 @@ def parse_args(argv: List[str]):
             args.dtype = value("--dtype", "bfloat16 or float32")
             if args.dtype not in ("bfloat16", "float32"):
                 raise UsageError(f"--dtype must be bfloat16 or float32; got {args.dtype}")
+        elif argument == "--narrow-to-bfloat16":
+            args.narrow_to_bfloat16 = True
         elif argument == "--max-tokens":
             args.max_tokens = _int("--max-tokens", value("--max-tokens", "an integer"), 1)
         elif argument in ("--help", "-h"):
@@ -239,7 +245,8 @@ def run(args: GenerateArgs, out=sys.stdout) -> int:
         prompts = [ids if ids else text.encode(prompt) for prompt, ids in zip(args.prompts, args.prompt_ids)]
         as_ids = [bool(ids) for ids in args.prompt_ids]
         max_tokens = args.max_tokens or sum(((len(p) + args.max_new_tokens + 63) // 64) * 64 for p in prompts)
-        engine = load_engine(args.model_dir, dtype=args.dtype, max_tokens=max_tokens, device=f"cuda:{args.device_ordinal}")
+        engine = load_engine(args.model_dir, dtype=args.dtype, max_tokens=max_tokens, device=f"cuda:{args.device_ordinal}",
+                             narrow_to_bfloat16=args.narrow_to_bfloat16)
         stops = engine.model.spec.stop_token_ids  # from the model's metadata (main.rs:1291-1296)
 
         def show(ids: List[int], ids_out: bool) -> str:

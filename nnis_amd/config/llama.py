@@ -105,6 +105,53 @@ class LlamaConfig:
             return "MQA"
         return "GQA"
 
+    def capability_record(self) -> str:
+        """The reference's canonical capability record, line for line
+        (decoder_capabilities.rs:72-91; its fixtures for the two pinned
+        checkpoints: exact_checkpoint_spec.rs:10-30)."""
+        topology = {"MHA": "multi_head", "GQA": "grouped_query", "MQA": "multi_query"}[self.attention_topology()]
+        stored = {"float32": "f32", "bfloat16": "bf16"}[self.torch_dtype]
+        return (f"NNIS-DECODER-CAPABILITY-V1\nattention={topology}\nrope=llama_rotate_half_unscaled\nmlp=swiglu_silu\n"
+                f"weight_dtype={stored}\nq_heads={self.num_attention_heads}\nkv_heads={self.num_key_value_heads}\n"
+                f"head_dim={self.head_dim}\n")
+
+    def describe(self) -> Dict[str, Any]:
+        """What this configuration asks of the engine, with the sizes a caller
+        plans memory by: parameters, bytes of weights as stored, bytes of cache
+        a token takes in each runtime type."""
+        h, inner, layers = self.hidden_size, self.intermediate_size, self.num_hidden_layers
+        per_layer = (self.q_width + 2 * self.kv_width) * h + h * self.q_width + 3 * h * inner + 2 * h
+        table = self.vocab_size * h
+        parameters = layers * per_layer + h + table * (1 if self.tie_word_embeddings else 2)
+        stored_bytes = 2 if self.torch_dtype == "bfloat16" else 4
+        cache_elements = 2 * layers * self.kv_width
+        return {
+            "architecture": self.architecture,
+            "attention": self.attention_topology(),
+            "query_heads": self.num_attention_heads,
+            "key_value_heads": self.num_key_value_heads,
+            "group_size": self.group_size,
+            "head_dim": self.head_dim,
+            "position_encoding": "rotary, rotate-half, unscaled",
+            "rope_theta": self.rope_theta,
+            "feed_forward": "gated (SiLU on the gate)",
+            "norm": "RMSNorm",
+            "rms_norm_eps": self.rms_norm_eps,
+            "layers": layers,
+            "width": h,
+            "inner": inner,
+            "vocab_size": self.vocab_size,
+            "max_positions": self.max_position_embeddings,
+            "tied_head": self.tie_word_embeddings,
+            "stored_dtype": self.torch_dtype,
+            "runtime_dtypes": ["bfloat16", "float32"],
+            "parameters": parameters,
+            "weight_bytes": parameters * stored_bytes,
+            "cache_bytes_per_token": {"bfloat16": 2 * cache_elements, "float32": 4 * cache_elements},
+            "stop_token_ids": list(self.eos_token_ids),
+            "capability_record": self.capability_record(),
+        }
+
     # ---- construction --------------------------------------------------
     @classmethod
     def from_dict(cls, raw: Dict[str, Any]) -> "LlamaConfig":

@@ -37,6 +37,43 @@ extern "C" int nnis_embed(const int* ids, const void* table, int table_dtype, fl
   return 0;
 }
 
+// The same row copy out of a table kept in the packed order of the matrix-core products (common.h): a head
+// that shares the table needs that order, and the table is then kept once.  8 consecutive channels of a row lie
+// together (16 bytes); a thread copies one such piece.
+__global__ void embed_packed_kernel(const int* __restrict__ ids, const bf16_t* __restrict__ packed,
+                                    float* __restrict__ out, int width, int vocab) {
+  const int token = blockIdx.x;
+  const int id = ids[token];
+  float* dst = out + (size_t)token * width;
+  const bool inside = id >= 0 && id < vocab;
+  const size_t strip = inside ? (size_t)(id >> 4) * nnis_packed_strip_elems(width) : 0;
+  for (int k = threadIdx.x * 8; k < width; k += blockDim.x * 8) {
+    uint4 piece = make_uint4(0, 0, 0, 0);
+    if (inside) {
+      const size_t at = strip + (size_t)(k / 64) * kPackedChunkElems + (size_t)((k % 16) / 8) * kPackedHalfElems +
+                        (size_t)(16 * ((k % 64) / 16) + (id & 15)) * 8;
+      piece = *(const uint4*)(packed + at);
+    }
+    const uint32_t words[4] = {piece.x, piece.y, piece.z, piece.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {  // bfloat16 widens by a shift
+      dst[k + 2 * i] = __uint_as_float(words[i] << 16);
+      dst[k + 2 * i + 1] = __uint_as_float(words[i] & 0xffff0000u);
+    }
+  }
+}
+
+extern "C" int nnis_embed_packed(const int* ids, const void* packed, float* out, int tokens, int width, int vocab,
+                                 void* stream) {
+  NNIS_REQUIRE(tokens >= 0 && width > 0 && vocab > 0, "embed: bad sizes tokens=%d width=%d vocab=%d", tokens, width, vocab);
+  NNIS_REQUIRE(width % 8 == 0, "embed: a packed table has a width that is a multiple of 8, got %d", width);
+  if (tokens == 0) return 0;
+  hipLaunchKernelGGL(embed_packed_kernel, dim3(tokens), dim3(64 * ((width / 8 + 63) / 64 > 4 ? 4 : (width / 8 + 63) / 64)), 0,
+                     (hipStream_t)stream, ids, (const bf16_t*)packed, out, width, vocab);
+  NNIS_LAUNCH_CHECK("embed_packed");
+  return 0;
+}
+
 // -----------------------------------------------------------------------------
 // RMSNorm: y[c] = (x[c] * (1/sqrt(mean(x^2) + eps))) * w[c]
 // (/root/reference/crates/nnis-model/src/kernels.rs:15-48: eps inside the

@@ -35,4 +35,5 @@ class StepContext:
     host_pos0: List[int] = field(default_factory=list)
     splits: int = 0  # runs the keys of a decode step are cut into; 0: chosen by the kernel's wrapper
     waves: int = 1  # waves of a block of the decode attention kernel (used when splits is given)
+    plan_len: int = 0  # the length each mixer plans its decode kernels for, where it is not max_len (a captured step)
     tiles: dict = field(default_factory=dict)  # work lists of prefill kernels, by tile size, made on first use

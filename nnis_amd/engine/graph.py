@@ -2,7 +2,7 @@
 
 A decode step launches a few hundred small kernels; issued one by one from the
 host the step is bound by launch overhead, not by the GPU.  For a batch size
-(padded up to a bucket) and a plan of the attention kernels (splits, waves), the step is captured once
+(padded up to a bucket) and the plans of the layers' kernels for it (each mixer's own), the step is captured once
 into a graph whose kernels read their token ids, slots and positions from
 fixed device buffers; each later step copies three small arrays into those
 buffers and replays the graph.  Padding rows carry slot -1: kernels that touch
@@ -35,12 +35,13 @@ def bucket(batch: int) -> int:
 
 
 class DecodeGraph:
-    def __init__(self, engine, padded: int, plan: Tuple[int, int]):
+    def __init__(self, engine, padded: int, plan_len: int):
+        """``plan_len``: a length whose plans (``DecoderModel.decode_plan`` for ``padded`` sequences) are the
+        ones this graph is captured with and replayed for."""
         # not a strong reference: engine -> graphs -> engine would keep both alive until the cycle
         # collector runs, and that may be in the middle of another engine's capture
         self.engine = engine if isinstance(engine, weakref.ProxyTypes) else weakref.proxy(engine)
         self.padded = padded
-        splits, waves = plan
         device = engine.rt.device
         # rows: 0 token ids, 1 slots, 2 positions
         self.meta = torch.zeros((3, padded), dtype=torch.int32, device=device)
@@ -52,9 +53,10 @@ class DecodeGraph:
         self.copied.record()
         self.ctx = StepContext(
             tokens=padded, batch=padded, tok_slot=self.meta[1], tok_pos=self.meta[2], seq_slot=self.meta[1],
-            seq_start=self.rows, seq_pos0=self.meta[2], decode=True, max_new=1, max_len=0, splits=splits, waves=waves)
+            seq_start=self.rows, seq_pos0=self.meta[2], decode=True, max_new=1, max_len=0, plan_len=plan_len)
         self.graph = None
         self.logits = None
+        self.scratch = None  # the kernels' shared scratch whose address the capture baked in: held as long as the graph
 
     def _forward(self) -> torch.Tensor:
         engine = self.engine
@@ -80,6 +82,10 @@ class DecodeGraph:
         finally:
             if collecting:
                 gc.enable()
+        # The split attention's partial sums go through a scratch tensor that the kernels' wrapper keeps per
+        # device.  The eager run above sized it and the capture baked its address in, so the graph holds it:
+        # whatever the wrapper does later, a replay never writes into memory that has gone back to the allocator.
+        self.scratch = self.engine.rt.ops.decode_scratch_held(self.engine.rt.device)
 
     def run(self, ids, slots: Sequence[int], positions: Sequence[int], ids_device: torch.Tensor = None) -> torch.Tensor:
         """``ids``: the step's token ids, or None when they are on the device
@@ -101,20 +107,31 @@ class DecodeGraph:
         return self.logits
 
 
+DECODE_GRAPHS_KEPT = 24  # a graph keeps its activations' memory; a batch that shrinks walks through a few buckets and plans
+
+
 class DecodeGraphs:
-    """The graphs of one engine, made on first use."""
+    """The graphs of one engine, made on first use; the ``DECODE_GRAPHS_KEPT`` used last are kept."""
 
     def __init__(self, engine):
         self.engine = weakref.proxy(engine)
-        self.graphs: Dict[Tuple[int, Tuple[int, int]], DecodeGraph] = {}
+        self.graphs: Dict[tuple, DecodeGraph] = {}  # in the order of their last use
 
-    def get(self, batch: int, plan: Tuple[int, int]) -> DecodeGraph:
-        key = (bucket(batch), plan)
-        graph = self.graphs.get(key)
+    def get(self, batch: int, longest: int) -> DecodeGraph:
+        """The graph for ``batch`` sequences, the longest of ``longest`` tokens after the step: one per
+        (bucket of the batch, the layers' plans for that bucket and length)."""
+        padded = bucket(batch)
+        engine = self.engine
+        key = (padded, engine.model.decode_plan(padded, longest, engine.rt))
+        graph = self.graphs.pop(key, None)
         if graph is None:
-            graph = DecodeGraph(self.engine, key[0], plan)
+            graph = DecodeGraph(engine, padded, longest)
             graph.capture()
-            self.graphs[key] = graph
+            while len(self.graphs) >= DECODE_GRAPHS_KEPT:
+                # (the stream may still replay the oldest: it is destroyed only when the GPU has left it)
+                torch.cuda.synchronize()
+                self.graphs.pop(next(iter(self.graphs)))
+        self.graphs[key] = graph  # the most recently used is last
         return graph
 
 

@@ -51,6 +51,15 @@ class Engine:
     def length(self, slot: int) -> int:
         return self.cache.length(slot)
 
+    def truncate(self, slot: int, length: int) -> None:
+        """Shortens a sequence to its first ``length`` tokens; the next step
+        appends there.  Pages beyond go back to the cache at once."""
+        self.cache.truncate(slot, length)
+
+    def reset(self, slot: int) -> None:
+        """Empties a sequence's slot without giving the slot back."""
+        self.cache.reset(slot)
+
     def free_slots(self) -> int:
         return self.cache.slots.free
 
@@ -222,11 +231,12 @@ class Engine:
                 for place in entry.want:
                     if int(place) != 0:
                         raise InvalidInput(f"slot {entry.slot}: wanted place {place} is not among its 1 tokens")
-        pos0 = self.cache.grow_by_one(slots)
         if self._graphs is None:
             self._graphs = DecodeGraphs(self)
-        plan = self.model.decode_plan(len(entries), max(pos0) + 1, self.rt)
-        graph = self._graphs.get(len(entries), plan)
+        # the graph first (its capture may fail), the cache's growth after it: a refused step changes nothing
+        longest = max(self.cache.length(slot) for slot in slots) + 1
+        graph = self._graphs.get(len(entries), longest)
+        pos0 = self.cache.grow_by_one(slots)
         logits = graph.run(ids, slots, pos0, ids_device)
         wanted = [i for i, e in enumerate(entries) if e.want is None or len(e.want) > 0]
         if len(wanted) == len(entries):

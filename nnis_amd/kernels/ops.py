@@ -24,6 +24,7 @@ _U64 = ctypes.c_uint64
 
 _CORE_SIGNATURES = {
     "nnis_embed": [_VOID, _VOID, _INT, _VOID, _INT, _INT, _INT, _VOID],
+    "nnis_embed_packed": [_VOID, _VOID, _VOID, _INT, _INT, _INT, _VOID],
     "nnis_rmsnorm": [_VOID, _INT, _VOID, _INT, _VOID, _INT, _VOID, _INT, _VOID, _INT, _INT, _FLT, _VOID],
     "nnis_rope_kv_write": [_VOID, _INT, _VOID, _INT, _VOID, _VOID, _INT, _INT, _VOID, _VOID, _VOID, _VOID, _INT,
                            _VOID, _INT, _INT, _INT, _INT, _INT, _VOID],
@@ -136,12 +137,19 @@ def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
 
 # ---------------------------------------------------------------------------
 
-def embed(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
-    """out[t, :] = table[ids[t], :] widened to 32-bit; ids outside the table give a zero row."""
+def embed(ids: torch.Tensor, table, out: torch.Tensor) -> torch.Tensor:
+    """out[t, :] = table[ids[t], :] widened to 32-bit; ids outside the table give a zero row.
+    ``table``: a matrix [vocab, width], or the ``PackedWeight`` of one (a table that a head shares)."""
     _dev(ids, "ids"), _dev(table, "embedding table"), _dev(out, "out")
     tokens, width = out.shape
     if ids.dtype != torch.int32 or ids.numel() < tokens:
         raise KernelError(f"embed: ids must be int32 with at least {tokens} entries")
+    if isinstance(table, PackedWeight):
+        if table.shape[1] != width or out.dtype != torch.float32:
+            raise KernelError(f"embed: packed table {table.shape} / out {tuple(out.shape)} {out.dtype} do not fit")
+        lib = core()
+        _check(lib, lib.nnis_embed_packed(ids.data_ptr(), table.data_ptr(), out.data_ptr(), tokens, width, table.shape[0], _stream()))
+        return out
     if table.dim() != 2 or table.shape[1] != width or out.dtype != torch.float32:
         raise KernelError(f"embed: table {tuple(table.shape)} / out {tuple(out.shape)} {out.dtype} do not fit")
     lib = core()
@@ -183,9 +191,10 @@ def rope_kv_write(qkv: torch.Tensor, q_out: torch.Tensor, cos: Optional[torch.Te
                   v_pages: Optional[torch.Tensor], block_table: Optional[torch.Tensor], heads: int, kv_heads: int,
                   head_dim: int) -> torch.Tensor:
     """Rotates queries and keys by their positions and writes keys and values
-    into the pages of each token's slot.  ``k_pages`` is
-    ``[pages, kv_heads, 64, head_dim]``, ``v_pages`` ``[pages, kv_heads,
-    head_dim, 64]``; both ``None`` for a run that keeps no cache of its own."""
+    into the pages of each token's slot.  ``k_pages`` and ``v_pages`` are
+    ``[pages, *k_page_shape(kv_heads, head_dim)]`` and ``[pages,
+    *v_page_shape(kv_heads, head_dim)]`` (``cache/layout.py``); both ``None``
+    for a run that keeps no cache of its own."""
     _dev(qkv, "qkv"), _dev(q_out, "q_out"), _dev(tok_slot, "tok_slot"), _dev(tok_pos, "tok_pos")
     tokens = qkv.shape[0]
     if qkv.shape[1] != (heads + 2 * kv_heads) * head_dim or q_out.shape != (tokens, heads * head_dim):
@@ -377,7 +386,8 @@ FUSED_MAX_TOKENS = 16  # beyond a tile of 16 tokens every wave re-reads too much
 def gemm_fused(x_in: torch.Tensor, delta: Optional[torch.Tensor], x_out: Optional[torch.Tensor], norm_weight: torch.Tensor,
                eps: float, w: torch.Tensor, y: torch.Tensor, epilogue: int = EPILOGUE_STORE, rope: Optional[dict] = None,
                split: int = 0):
-    """y = epilogue( W . rmsnorm(x_in + delta) ) for up to 64 tokens, in one
+    """y = epilogue( W . rmsnorm(x_in + delta) ) for a few tokens (callers
+    keep to ``FUSED_MAX_TOKENS``; the kernel itself takes up to 64), in one
     kernel; ``x_out`` receives x_in + delta.  ``epilogue``: store; SiLU(gate) *
     up for a weight of gate rows followed by up rows; or rotate-half RoPE with
     the write of keys and values into the cache (``rope``: cos, sin, tok_slot,
@@ -628,22 +638,30 @@ class KeyRuns:
 
 
 _DECODE_KERNELS = {"auto": 0, "columns": 1, "keys": 2}
-_decode_scratch = {}
+_decode_scratch = {}  # per device: every scratch made so far, the largest last
 
 
 def decode_scratch(device, floats: int) -> torch.Tensor:
-    """Scratch of the split decode attention, kept per device and grown when a
-    call needs more.  Calls on one device share it, so they must follow one
-    another on one stream; it grows outside a graph capture only (the run that
-    warms a graph up sizes it)."""
+    """Scratch of the split decode attention, kept per device.  Calls on one
+    device share it, so they must follow one another on one stream.  A call
+    that needs more gets a larger tensor, made outside a graph capture only
+    (the run that warms a graph up sizes it); the smaller ones are kept until
+    the process ends, because a captured graph has the address it was captured
+    with baked in and goes on writing there on every replay.  (A graph also
+    holds the tensor it captured: ``engine/graph.py``.)"""
     key = (device.type, device.index)
-    held = _decode_scratch.get(key)
-    if held is None or held.numel() < floats:
+    held = _decode_scratch.setdefault(key, [])
+    if not held or held[-1].numel() < floats:
         if torch.cuda.is_current_stream_capturing():
             raise KernelError("attention: the decode scratch would have to grow inside a graph capture")
-        held = torch.empty(max(floats, 2 * held.numel() if held is not None else 1 << 16), dtype=torch.float32, device=device)
-        _decode_scratch[key] = held
-    return held
+        held.append(torch.empty(max(floats, 2 * held[-1].numel() if held else 1 << 16), dtype=torch.float32, device=device))
+    return held[-1]
+
+
+def decode_scratch_held(device):
+    """The scratch a decode attention launched now would use (None: none made yet)."""
+    held = _decode_scratch.get((device.type, device.index))
+    return held[-1] if held else None
 
 
 def decode_max_waves(heads: int, kv_heads: int, head_dim: int) -> int:
@@ -758,7 +776,7 @@ def attention(q: torch.Tensor, out: torch.Tensor, view, ctx, heads: int, kv_head
         if ctx.splits:
             splits, waves = ctx.splits, ctx.waves
         else:
-            splits, waves = decode_plan(ctx.batch, kv_heads, ctx.max_len, width=heads * head_dim)
+            splits, waves = decode_plan(ctx.batch, kv_heads, ctx.plan_len or ctx.max_len, width=heads * head_dim)
         waves = min(waves, decode_max_waves(heads, kv_heads, head_dim))
         partial = None
         if splits > 1:

@@ -24,6 +24,7 @@ class DecoderModel:
         self.final_norm = build_part("norm", spec.final_norm)
         self.head = build_part("head", spec.head)
         self.bound = False
+        self._plans = {}
 
     # ---- weights -------------------------------------------------------------
     def parts(self):
@@ -39,8 +40,15 @@ class DecoderModel:
         return out
 
     def bind(self, weights: Dict[str, torch.Tensor], rt) -> None:
-        for part in self.parts():
+        parts = self.parts()
+        for part in parts:
             part.bind(weights, rt)
+        # a tensor that two parts share (a tied head's table) is kept once: whoever packed it offers the copy
+        for owner in parts:
+            for source, packed in owner.packed_sources():
+                for part in parts:
+                    if part is not owner:
+                        part.adopt_packed(source, packed)
         self.bound = True
 
     def step_weight_bytes(self) -> int:
@@ -55,9 +63,16 @@ class DecoderModel:
         return all(getattr(part, "graph_safe", False) for part in self.parts())
 
     def decode_plan(self, batch: int, longest: int, rt):
-        """(splits, waves) of a decode step's attention kernels, one plan for all layers."""
-        kv_heads = [request.kv_heads for _, request in self.cache_requests()[0] if hasattr(request, "kv_heads")]
-        return rt.ops.decode_plan(batch, min(kv_heads), longest, width=self.spec.width) if kv_heads else (1, 1)
+        """The plans of every run of the schedule for a step of one token
+        each (``Block.decode_plan``): each layer plans for its own heads and
+        sizes.  Plans depend on a length through its pages only."""
+        key = (batch, (longest + 63) // 64)
+        plans = self._plans.get(key)
+        if plans is None:
+            if len(self._plans) > 4096:
+                self._plans.clear()
+            plans = self._plans[key] = tuple(self.layers[entry.layer].decode_plan(batch, longest, rt) for entry in self.spec.schedule)
+        return plans
 
     # ---- cache ---------------------------------------------------------------
     def cache_requests(self) -> Tuple[List[Tuple[int, Any]], Dict[int, int]]:

@@ -55,6 +55,10 @@ class CausalSelfAttention(Mixer):
     def cache_request(self):
         return KVRequest(self.kv_heads, self.head_dim, self.window)
 
+    def decode_plan(self, batch, longest, rt):
+        # what ``ops.attention`` picks for a step of single tokens with these sizes
+        return rt.ops.decode_plan(batch, self.kv_heads, longest, width=self.heads * self.head_dim)
+
     takes_pending_norm = True
     adds_to_residual = True
 

@@ -47,10 +47,12 @@ from ..errors import InvalidInput
 class TensorSpec:
     """A tensor a part reads from the checkpoint.
 
-    ``init`` tells the random-weights writer how to draw it: ``"matrix"`` is
-    N(0, 0.02) and ``"gain"`` is 1 + N(0, 0.01); ``"index"`` marks a table of
-    integers, uniform in [0, ``high``), which is stored and kept as int32
-    whatever the activation type.  ``fallback`` names another checkpoint
+    ``init`` names the rule by which the random-weights writer draws it
+    (``weights/random_init.py``: ``register_init_rule``): ``"matrix"`` is
+    N(0, 0.02), ``"gain"`` is 1 + N(0, 0.01), ``"zeros"`` is zeros; ``"index"``
+    marks a table of integers, uniform in [0, ``high``), which is stored and
+    kept as int32 whatever the activation type.  A part may register a rule
+    of its own.  ``fallback`` names another checkpoint
     tensor that stands in when this one is absent (a tied head)."""
 
     name: str
@@ -63,11 +65,17 @@ class TensorSpec:
 @dataclass(frozen=True)
 class KVRequest:
     """Keys and values of every token (``window is None``) or of the last
-    ``window`` tokens, for ``kv_heads`` heads of ``head_dim``."""
+    ``window`` tokens, for ``kv_heads`` heads whose keys have ``head_dim``
+    channels and whose values ``value_dim`` (None: as many as the keys)."""
 
     kv_heads: int
     head_dim: int
     window: Optional[int] = None
+    value_dim: Optional[int] = None
+
+    @property
+    def value_head_dim(self) -> int:
+        return self.head_dim if self.value_dim is None else self.value_dim
 
 
 @dataclass(frozen=True)
@@ -101,6 +109,19 @@ class Part:
     def weight_bytes(self) -> int:
         """Bytes of weights one step has to read through this part."""
         return 0
+
+    def packed_sources(self):
+        """[((address, shape) of a loaded tensor, its packed copy)] for the
+        tensors this part packed when it was bound and no longer keeps in the
+        checkpoint's order.  The model offers each to every other part
+        (``adopt_packed``), so that a tensor two parts share is kept once."""
+        return []
+
+    def adopt_packed(self, source, packed) -> bool:
+        """Takes another part's packed copy in place of the tensor at
+        ``source`` if this part holds that tensor and can work from the
+        packed order; says whether it did."""
+        return False
 
 
 class Norm(Part):
@@ -136,6 +157,14 @@ class Mixer(Part):
     def cache_request(self):
         return None
 
+    def decode_plan(self, batch: int, longest: int, rt):
+        """How this mixer would launch a step of one token for each of
+        ``batch`` sequences, the longest of ``longest`` tokens: anything that
+        can be hashed and compared, or None if its launches do not depend on
+        the lengths.  A captured step is replayed only for steps whose plans
+        equal those it was captured with."""
+        return None
+
     def forward(self, x, ctx, view, rt):
         raise NotImplementedError
 
@@ -147,6 +176,9 @@ class FeedForward(Part):
 
 class Block(Part):
     def cache_request(self):
+        return None
+
+    def decode_plan(self, batch: int, longest: int, rt):
         return None
 
     def forward(self, stream, ctx, view, rt):

@@ -42,6 +42,9 @@ class PreNormBlock(Block):
     def cache_request(self):
         return self.mixer.cache_request()
 
+    def decode_plan(self, batch, longest, rt):
+        return self.mixer.decode_plan(batch, longest, rt)
+
     @property
     def entry_norm(self):
         """The norm a stream meets first here: a block before this one may prepare it."""

@@ -25,6 +25,16 @@ class TokenEmbedding(Part):
     def bind(self, weights, rt):
         self.table = weights[self.weight_name].contiguous()
 
+    def adopt_packed(self, source, packed) -> bool:
+        """A part of the model has packed the tensor at ``source`` (address,
+        shape) for the matrix cores.  If that tensor is this table (a tied
+        head), rows are gathered from the packed copy from now on and the
+        table in the checkpoint's order is let go: the table is kept once."""
+        if isinstance(self.table, torch.Tensor) and source == (self.table.data_ptr(), tuple(self.table.shape)):
+            self.table = packed
+            return True
+        return False
+
     def forward(self, ids, tokens, rt):
         """ids: int32 on the device -> the 32-bit residual stream [tokens, width]."""
         return rt.ops.embed(ids, self.table, rt.empty(tokens, self.width, dtype=torch.float32))
@@ -43,6 +53,9 @@ class LinearHead(Part):
     def bind(self, weights, rt):
         # a tied head is the same device tensor as the embedding table
         self.projection = Projection(weights[self.weight_name], rt)
+
+    def packed_sources(self):
+        return [(self.projection.packed_from, self.projection.weight)] if self.projection.packed_from else []
 
     def weight_bytes(self):
         return self.projection.weight_bytes()

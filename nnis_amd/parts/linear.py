@@ -22,8 +22,11 @@ class Projection:
             raise ValueError(f"a projection weight is a matrix, got shape {tuple(weight.shape)}")
         self.out_features, self.in_features = weight.shape
         self._bytes = weight.numel() * weight.element_size()
+        self.packed_from = None  # (address, shape) of the tensor a packed weight was made from
         if rt is not None and rt.dtype == torch.bfloat16 and rt.ops.packs(weight):
-            self.weight = rt.ops.pack_weight(weight.contiguous())
+            weight = weight.contiguous()
+            self.weight = rt.ops.pack_weight(weight)
+            self.packed_from = (weight.data_ptr(), tuple(weight.shape))
         else:
             self.weight = weight.contiguous()
 

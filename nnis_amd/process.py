@@ -21,6 +21,7 @@ import os
 import subprocess
 import sys
 import tempfile
+import threading
 from typing import Any, Dict, List, Optional
 
 SCHEMA_VERSION = 1
@@ -38,38 +39,71 @@ class RequestError(ValueError):
 def validate_request(model: str, tokenizer: Optional[str], prompt: Optional[str], prompt_ids: Optional[str], device: int,
                      max_new_tokens: int, result: str) -> None:
     if os.path.islink(model) or not os.path.isdir(model):
-        raise RequestError(f"model path must be a directory, not a symlink: {model}")
+        raise RequestError(f"--model must name a real folder (symbolic links are refused): {model}")
     if (prompt is None) == (prompt_ids is None):
         raise RequestError("exactly one of --prompt and --prompt-ids is required")
     if prompt is not None:
         if "\0" in prompt:
-            raise RequestError("prompt must not contain NUL bytes")
+            raise RequestError("the prompt holds a NUL byte")
         size = len(prompt.encode("utf-8"))
         if not 1 <= size <= MAX_PROMPT_BYTES:
-            raise RequestError(f"prompt must encode to 1..={MAX_PROMPT_BYTES} UTF-8 bytes; got {size}")
+            raise RequestError(f"the prompt is {size} bytes of UTF-8; between 1 and {MAX_PROMPT_BYTES} are taken")
         path = tokenizer or os.path.join(model, "tokenizer.json")
         if os.path.islink(path) or not os.path.isfile(path):
-            raise RequestError(f"tokenizer path must be a regular file, not a symlink: {path}")
+            raise RequestError(f"the tokenizer must be an ordinary file (symbolic links are refused): {path}")
     if not 0 <= device <= 2**31 - 1:
-        raise RequestError("device ordinal must be a non-negative integer")
+        raise RequestError("--device takes a device number from 0 up")
     if not 1 <= max_new_tokens <= MAX_NEW_TOKENS:
-        raise RequestError(f"max-new-tokens must be in 1..={MAX_NEW_TOKENS}; got {max_new_tokens}")
+        raise RequestError(f"--max-new-tokens {max_new_tokens} is outside 1 to {MAX_NEW_TOKENS}")
     if os.path.lexists(result):
         raise RequestError(f"result path already exists: {result}")
 
 
-def run_child(command: List[str], timeout: float) -> Dict[str, Any]:
-    """Runs the command without a shell; output beyond the cap fails the run."""
+def run_child(command: List[str], timeout: float, capture_limit: int = MAX_CAPTURE_BYTES) -> Dict[str, Any]:
+    """Runs the command without a shell.  Both output channels are drained as
+    the child writes them, each by a thread of its own, and never more than
+    ``capture_limit`` bytes of a channel are kept: a child that writes more is
+    stopped there and the run fails, whatever it would have printed after."""
     try:
-        done = subprocess.run(command, stdin=subprocess.DEVNULL, capture_output=True, timeout=timeout, check=False)
-    except subprocess.TimeoutExpired:
-        return {"status": "timeout", "exit_code": None, "stdout": b"", "stderr": f"no result within {timeout} s".encode()}
+        child = subprocess.Popen(command, stdin=subprocess.DEVNULL, stdout=subprocess.PIPE, stderr=subprocess.PIPE)
     except OSError as error:
         return {"status": "not_started", "exit_code": None, "stdout": b"", "stderr": str(error).encode()}
-    if len(done.stdout) > MAX_CAPTURE_BYTES or len(done.stderr) > MAX_CAPTURE_BYTES:
-        return {"status": "output_too_large", "exit_code": done.returncode, "stdout": b"", "stderr": b"output exceeds the capture limit"}
-    return {"status": "generated" if done.returncode == 0 else "failed", "exit_code": done.returncode,
-            "stdout": done.stdout, "stderr": done.stderr}
+    kept = {"stdout": bytearray(), "stderr": bytearray()}
+    over = threading.Event()
+
+    def drain(pipe, name: str) -> None:
+        with pipe:
+            while True:
+                piece = pipe.read1(65536)
+                if not piece:
+                    return
+                room = capture_limit - len(kept[name])
+                if len(piece) > room:
+                    kept[name] += piece[:room]
+                    over.set()
+                    child.kill()  # nothing more is wanted from it
+                    return
+                kept[name] += piece
+
+    readers = [threading.Thread(target=drain, args=(pipe, name), daemon=True)
+               for pipe, name in ((child.stdout, "stdout"), (child.stderr, "stderr"))]
+    for reader in readers:
+        reader.start()
+    try:
+        code = child.wait(timeout=timeout)
+    except subprocess.TimeoutExpired:
+        child.kill()
+        child.wait()
+        for reader in readers:
+            reader.join(timeout=5)
+        return {"status": "timeout", "exit_code": None, "stdout": b"", "stderr": f"no result within {timeout} s".encode()}
+    for reader in readers:
+        reader.join(timeout=5)
+    if over.is_set():
+        return {"status": "output_too_large", "exit_code": code, "stdout": b"",
+                "stderr": f"the child wrote more than {capture_limit} bytes to one channel and was stopped".encode()}
+    return {"status": "generated" if code == 0 else "failed", "exit_code": code,
+            "stdout": bytes(kept["stdout"]), "stderr": bytes(kept["stderr"])}
 
 
 def build_result(inputs: Dict[str, Any], child: Dict[str, Any]) -> Dict[str, Any]:

@@ -3,9 +3,16 @@
 The parts of a model declare the tensors they read (name, shape); the loader
 looks each one up in ``model.safetensors`` (or the shards named by
 ``model.safetensors.index.json``), checks shape and stored type, and puts it
-on the device.  A tensor stored in bfloat16 stays bfloat16 and one stored in
-32-bit stays 32-bit; only the 32-bit path widens (exactly, ``bits << 16``:
-/root/reference/crates/nnis-model/src/safetensors_loader.rs:610-624).  A table
+on the device.  Every tensor's stored type must be the one config.json
+declares (``torch_dtype``; safetensors_loader.rs:718-724).  A tensor stored in
+bfloat16 stays bfloat16 and one stored in 32-bit stays 32-bit; the 32-bit path
+widens (exactly, ``bits << 16``:
+/root/reference/crates/nnis-model/src/safetensors_loader.rs:610-624), and
+nothing narrows unless the caller asks for it: ``narrow_to_bfloat16`` rounds
+32-bit tensors to bfloat16 (nearest, ties to even) as they are loaded, so that
+a 32-bit checkpoint under a bfloat16 runtime runs on the matrix cores.  Without
+it such a checkpoint keeps its 32-bit weights and every projection takes the
+ordered 32-bit product, much slower; the loader says so in one line.  A table
 of integers (a part declares it so) is kept as int32 on either path.
 Everything wrong with a folder is reported in one error: missing tensors,
 tensors nobody asked for, wrong shapes, unsupported stored types
@@ -16,7 +23,8 @@ from __future__ import annotations
 
 import json
 import os
-from typing import Dict, List, Sequence
+import sys
+from typing import Dict, List, Optional, Sequence
 
 import torch
 
@@ -70,7 +78,19 @@ def open_weight_files(model_dir: str) -> List[SafetensorsFile]:
     raise WeightError(f"{model_dir} holds neither {SINGLE} nor {INDEX}")
 
 
-def load_weights(model_dir: str, specs: Sequence[TensorSpec], device, widen_to_float32: bool) -> Dict[str, torch.Tensor]:
+_DECLARED = {"float32": "F32", "bfloat16": "BF16"}
+
+
+def load_weights(model_dir: str, specs: Sequence[TensorSpec], device, widen_to_float32: bool,
+                 declared_dtype: Optional[str] = None, narrow_to_bfloat16: bool = False) -> Dict[str, torch.Tensor]:
+    """``declared_dtype``: config.json's ``torch_dtype`` ("float32" or
+    "bfloat16"; None skips the check, for callers without a config.json).
+    ``narrow_to_bfloat16``: round tensors stored in 32-bit to bfloat16 at load
+    (not with ``widen_to_float32``)."""
+    if narrow_to_bfloat16 and widen_to_float32:
+        raise WeightError("narrow_to_bfloat16 is for a bfloat16 runtime; the 32-bit path keeps 32-bit weights")
+    if declared_dtype is not None and declared_dtype not in _DECLARED:
+        raise WeightError(f"config.json declares torch_dtype {declared_dtype!r}; supported are float32 and bfloat16")
     files = open_weight_files(model_dir)
     where: Dict[str, SafetensorsFile] = {}
     duplicates: List[str] = []
@@ -110,6 +130,9 @@ def load_weights(model_dir: str, specs: Sequence[TensorSpec], device, widen_to_f
         elif stored not in _STORED:
             wrong_type.append(f"{source}: stored as {stored}; supported are F32 and BF16")
             continue
+        elif declared_dtype is not None and stored != _DECLARED[declared_dtype]:
+            wrong_type.append(f"{source}: stored as {stored}; config.json declares {declared_dtype}")
+            continue
         plan.append((spec.name, source))
     unexpected = sorted(
         name for name in where if name not in consumed and not name.endswith(_IGNORED_SUFFIXES)
@@ -124,11 +147,12 @@ def load_weights(model_dir: str, specs: Sequence[TensorSpec], device, widen_to_f
         if wrong_shape:
             lines.append(f"  wrong shapes ({len(wrong_shape)}): " + "; ".join(wrong_shape))
         if wrong_type:
-            lines.append(f"  unsupported stored types ({len(wrong_type)}): " + "; ".join(wrong_type))
+            lines.append(f"  wrong stored types ({len(wrong_type)}): " + "; ".join(wrong_type))
         if duplicates:
             lines.append(f"  tensors in more than one shard ({len(duplicates)}): " + "; ".join(sorted(duplicates)))
         raise WeightError("\n".join(lines))
 
+    kept_wide = 0
     on_device: Dict[str, torch.Tensor] = {}  # by checkpoint name: a tied head shares the table's memory
     out: Dict[str, torch.Tensor] = {}
     for name, source in plan:
@@ -142,8 +166,17 @@ def load_weights(model_dir: str, specs: Sequence[TensorSpec], device, widen_to_f
                 tensor = host.to(device)
                 if widen_to_float32 and tensor.dtype != torch.float32:
                     tensor = tensor.to(torch.float32)
+                elif tensor.dtype == torch.float32 and not widen_to_float32:
+                    if narrow_to_bfloat16:
+                        tensor = tensor.to(torch.bfloat16)  # round to nearest, ties to even
+                    else:
+                        kept_wide += 1
             on_device[source] = tensor.contiguous()
         out[name] = on_device[source]
     for handle in files:
         handle.close()
+    if kept_wide:
+        print(f"[nnis_amd] {model_dir}: {kept_wide} tensors are stored in 32-bit and stay so; under bfloat16 their products "
+              "take the ordered 32-bit kernel (slow).  narrow_to_bfloat16 / --narrow-to-bfloat16 rounds them at load.",
+              file=sys.stderr, flush=True)
     return out

@@ -177,3 +177,97 @@ def test_one_more_token_each_is_all_or_nothing():
     with pytest.raises(CacheFull, match="positions end at 70"):
         lone.grow_by_one([s])
     assert lone.length(s) == 70
+
+
+def test_truncate_gives_pages_back_and_keeps_the_rest():
+    # the rules of /root/reference/crates/nnis-rt/src/kv_cache.rs:69-83,170-192,509-545 on pages
+    cache = _cache(max_tokens=512)  # 8 pages
+    a, b = cache.acquire(), cache.acquire()
+    cache.grow({a: 200, b: 65})
+    full = cache.kv_groups[0]
+    first_pages = list(full.table.rows[a])
+    assert len(first_pages) == 4 and full.table.pool.free == 2
+    # longer than what is held: refused, nothing changes
+    with pytest.raises(InvalidInput, match="cannot be truncated to 201"):
+        cache.truncate(a, 201)
+    with pytest.raises(InvalidInput):
+        cache.truncate(a, -1)
+    assert cache.length(a) == 200 and full.table.pool.free == 2
+    cache.truncate(a, 200)  # to its own length: nothing to do
+    assert full.table.rows[a] == first_pages
+    cache.truncate(a, 70)  # 4 pages -> 2, in every group
+    assert cache.length(a) == 70 and cache.length(b) == 65
+    assert full.table.rows[a] == first_pages[:2]
+    assert all(g.table.pool.free == 4 for g in cache.kv_groups)
+    assert not set(first_pages[2:]) & set(full.table.pool.held)
+    # the next tokens are appended at the new length, on pages taken anew (lowest first: those just given back)
+    cache.grow({a: 100})
+    assert cache.length(a) == 170 and full.table.rows[a][:2] == first_pages[:2]
+    assert sorted(full.table.rows[a][2:]) == sorted(first_pages[2:])[:1]
+    assert full.block_table[a, :3].tolist() == full.table.rows[a]
+    # within a page: no page moves
+    cache.truncate(a, 129)
+    assert len(full.table.rows[a]) == 3
+    cache.truncate(a, 128)
+    assert len(full.table.rows[a]) == 2
+    with pytest.raises(InvalidInput, match="not held"):
+        cache.truncate(7, 0)
+    # nothing is lost, held twice or freed twice
+    for slot in (a, b):
+        cache.release(slot)
+    assert all(g.table.pool.free == 8 and not g.table.pool.held for g in cache.kv_groups)
+
+
+def test_reset_empties_a_slot_that_stays_held():
+    cache = _cache(max_tokens=256)
+    region = cache.add_state_region("extra", (2,), torch.float32)
+    a = cache.acquire()
+    cache.grow({a: 130})
+    region[a] = 3.0
+    cache.reset(a)
+    assert cache.length(a) == 0 and a in cache.slots.held
+    assert all(g.table.pool.free == 4 for g in cache.kv_groups)
+    assert region[a].abs().sum() == 0
+    cache.grow({a: 256})  # the whole cache again
+    assert cache.length(a) == 256
+    cache.release(a)
+    with pytest.raises(InvalidInput):
+        cache.reset(a)
+
+
+def test_fixed_size_state_refuses_truncation():
+    cache = _cache(extra=[(4, StateRequest((3,)))])
+    a = cache.acquire()
+    cache.grow({a: 10})
+    with pytest.raises(InvalidInput, match="fixed-size state"):
+        cache.truncate(a, 5)
+    assert cache.length(a) == 10
+    cache.truncate(a, 10)  # nothing is wound back: allowed
+    cache.reset(a)  # starts the sequence over, state zeroed
+    assert cache.length(a) == 0
+
+
+def test_free_list_hands_out_the_lowest_whatever_came_back():
+    from nnis_amd.cache.allocator import FreeList
+
+    pool = FreeList(6, "thing")
+    taken = [pool.take() for _ in range(6)]
+    assert taken == [0, 1, 2, 3, 4, 5]
+    for item in (4, 1, 5, 2):
+        pool.give_back(item)
+    assert [pool.take() for _ in range(4)] == [1, 2, 4, 5]
+    with pytest.raises(CacheFull):
+        pool.take()
+    pool.give_back(3)
+    with pytest.raises(InvalidInput):
+        pool.give_back(3)
+    assert pool.free == 1 and pool.held == frozenset({0, 1, 2, 4, 5})
+
+
+def test_values_may_be_narrower_than_keys():
+    cache = SequenceCache([(0, KVRequest(2, 32, value_dim=16)), (1, KVRequest(2, 32))], {}, max_tokens=128, max_positions=128,
+                          dtype=torch.float32, device="cpu")
+    assert len(cache.kv_groups) == 2  # a need of its own, storage of its own
+    narrow = cache.kv_groups[0]
+    assert narrow.k.shape[2:] == (2, 4, 64, 8) and narrow.v.shape[2:] == (2, 1, 2, 4, 16, 8)
+    assert narrow.bytes_per_token() == 2 * (32 + 16) * 4 and cache.kv_groups[1].bytes_per_token() == 2 * 64 * 4

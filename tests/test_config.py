@@ -103,3 +103,33 @@ def test_no_size_stands_in_code():
     assert a.layers[0]["norm1"]["eps"] != b.layers[0]["norm1"]["eps"]
     assert a.positions["rope"]["theta"] != b.positions["rope"]["theta"]
     assert a.vocab_size != b.vocab_size and a.max_positions != b.max_positions
+
+
+def test_presets_and_the_capability_record():
+    """The named shapes read back as configurations, and the two checkpoints
+    the reference pins give its capability records letter for letter
+    (/root/reference/crates/nnis-model/src/exact_checkpoint_spec.rs:10-30,219-259)."""
+    from nnis_amd.config import preset, preset_names
+
+    assert {"smollm2-135m", "smollm2-1.7b", "tinyllama-1.1b", "tiny-a", "tiny-b"} <= set(preset_names())
+    small = LlamaConfig.from_dict(preset("smollm2-135m"))
+    assert small.capability_record() == ("NNIS-DECODER-CAPABILITY-V1\nattention=grouped_query\nrope=llama_rotate_half_unscaled\n"
+                                         "mlp=swiglu_silu\nweight_dtype=bf16\nq_heads=9\nkv_heads=3\nhead_dim=64\n")
+    tiny = LlamaConfig.from_dict(preset("tinyllama-1.1b"))
+    assert tiny.capability_record() == ("NNIS-DECODER-CAPABILITY-V1\nattention=grouped_query\nrope=llama_rotate_half_unscaled\n"
+                                        "mlp=swiglu_silu\nweight_dtype=bf16\nq_heads=32\nkv_heads=4\nhead_dim=64\n")
+    assert tiny.kv_width == 256 and tiny.eos_token_ids == (2,) and small.eos_token_ids == (0,)
+    wide = LlamaConfig.from_dict(preset("smollm2-1.7b"))
+    assert "attention=multi_head" in wide.capability_record()
+    assert "attention=multi_query" in LlamaConfig.from_dict(preset("tiny-b")).capability_record()
+    # the record a caller plans by: parameter counts of the published sizes, bytes of cache a token
+    described = small.describe()
+    assert described["parameters"] == 134_515_008 and described["weight_bytes"] == 2 * 134_515_008
+    assert described["cache_bytes_per_token"] == {"bfloat16": 23_040, "float32": 46_080}
+    assert described["attention"] == "GQA" and described["group_size"] == 3 and described["tied_head"]
+    assert tiny.describe()["parameters"] == 1_100_048_384
+    # overrides replace keys and leave the preset as it was
+    assert preset("smollm2-135m", num_hidden_layers=2)["num_hidden_layers"] == 2
+    assert preset("smollm2-135m")["num_hidden_layers"] == 30
+    with pytest.raises(InvalidInput, match="unknown preset"):
+        preset("llama-70b")

@@ -25,7 +25,7 @@ def test_request_rules(tmp_path):
             process.validate_request(**{**ok, **change})
     link = tmp_path / "link"
     link.symlink_to(model)
-    with pytest.raises(process.RequestError, match="symlink"):
+    with pytest.raises(process.RequestError, match="symbolic links are refused"):
         process.validate_request(**{**ok, "model": str(link)})
 
 
@@ -35,6 +35,14 @@ def test_child_and_result_file(tmp_path):
     assert process.run_child([sys.executable, "-c", "import sys; sys.exit(3)"], 30)["status"] == "failed"
     assert process.run_child([sys.executable, "-c", "import time; time.sleep(5)"], 0.2)["status"] == "timeout"
     assert process.run_child([str(tmp_path / "no-such-binary")], 5)["status"] == "not_started"
+    # the cap holds while the child is read: a child that would write without end is stopped at the cap
+    endless = "import sys\nwhile True: sys.stdout.write('x' * 65536)"
+    cut = process.run_child([sys.executable, "-c", endless], 60, capture_limit=1 << 20)
+    assert cut["status"] == "output_too_large" and cut["stdout"] == b"" and b"1048576" in cut["stderr"]
+    noisy = process.run_child([sys.executable, "-c", "import sys; sys.stderr.write('e' * 5000); print('ok')"], 30, capture_limit=4096)
+    assert noisy["status"] == "output_too_large"
+    exact = process.run_child([sys.executable, "-c", "import sys; sys.stdout.write('y' * 4096)"], 30, capture_limit=4096)
+    assert exact["status"] == "generated" and len(exact["stdout"]) == 4096
     result = process.build_result({"prompt": "x"}, child)
     assert result["stdout"]["bytes"] == 6 and len(result["stdout"]["sha256"]) == 64 and result["sampling"] == "greedy"
     path = tmp_path / "out" / "r.json"

@@ -97,7 +97,7 @@ def test_one_error_lists_everything(model_dirs, tmp_path):
     assert "missing tensors (1)" in text and "model.layers.1.mlp.up_proj.weight [256, 96]" in text
     assert "unexpected tensors (1)" in text and "model.layers.7.extra.weight" in text
     assert "wrong shapes (1)" in text and "expected [32, 96], file has [32, 95]" in text
-    assert "unsupported stored types (1)" in text and "F16" in text
+    assert "wrong stored types (1)" in text and "F16" in text
     assert "inv_freq" not in text
 
 
@@ -242,3 +242,56 @@ def test_tables_of_integers_are_kept_as_int32(tmp_path):
     write_safetensors(os.path.join(folder, "model.safetensors"), dict(everything, norm=torch.ones(32, dtype=torch.int32)).items())
     with pytest.raises(WeightError, match="norm: stored as I32; supported are F32 and BF16"):
         load_weights(folder, specs, "cpu", widen_to_float32=False)
+
+
+def test_stored_types_must_be_the_declared_one(model_dirs, tmp_path, capsys):
+    """Every tensor is stored in config.json's torch_dtype
+    (/root/reference/crates/nnis-model/src/safetensors_loader.rs:718-724); nothing is narrowed unless the
+    caller says so (safetensors_loader.rs:610-624), and then to the nearest bfloat16, ties to even."""
+    folder = str(tmp_path / "mixed")
+    shutil.copytree(model_dirs["A"], folder)
+    handle = SafetensorsFile(os.path.join(folder, "model.safetensors"))
+    tensors = [(n, handle.tensor(n).clone().float() if n == "model.norm.weight" else handle.tensor(n).clone()) for n in handle.names()]
+    write_safetensors(os.path.join(folder, "model.safetensors"), tensors)
+    with pytest.raises(WeightError) as info:
+        load_weights(folder, _specs(TINY_A), "cpu", widen_to_float32=False, declared_dtype="bfloat16")
+    assert "wrong stored types (1)" in str(info.value) and "model.norm.weight: stored as F32; config.json declares bfloat16" in str(info.value)
+    load_weights(folder, _specs(TINY_A), "cpu", widen_to_float32=False)  # without a declaration the mix is taken as stored
+    with pytest.raises(WeightError, match="declares torch_dtype"):
+        load_weights(folder, _specs(TINY_A), "cpu", False, declared_dtype="float16")
+
+    # a 32-bit checkpoint: stays 32-bit (and says so), widens to itself, narrows only when asked
+    capsys.readouterr()
+    kept = load_weights(model_dirs["C"], _specs(TINY_C), "cpu", widen_to_float32=False, declared_dtype="float32")
+    assert all(t.dtype == torch.float32 for t in kept.values())
+    assert "stay so" in capsys.readouterr().err
+    narrowed = load_weights(model_dirs["C"], _specs(TINY_C), "cpu", widen_to_float32=False, declared_dtype="float32",
+                            narrow_to_bfloat16=True)
+    assert capsys.readouterr().err == ""
+    assert all(t.dtype == torch.bfloat16 for t in narrowed.values())
+    name = "model.layers.0.mlp.up_proj.weight"
+    # nearest, ties to even, worked on the bits: add 0x7fff + the kept part's lowest bit, drop the low half
+    bits = kept[name].view(torch.int32).to(torch.int64) & 0xFFFFFFFF
+    want = (((bits + 0x7FFF + ((bits >> 16) & 1)) >> 16) & 0xFFFF).to(torch.int32)
+    assert torch.equal(narrowed[name].view(torch.int16).to(torch.int32) & 0xFFFF, want)
+    with pytest.raises(WeightError, match="bfloat16 runtime"):
+        load_weights(model_dirs["C"], _specs(TINY_C), "cpu", widen_to_float32=True, narrow_to_bfloat16=True)
+
+
+def test_init_rules_are_a_registry(tmp_path):
+    from nnis_amd.errors import InvalidInput
+    from nnis_amd.parts.base import TensorSpec
+    from nnis_amd.weights.random_init import _INIT_RULES, register_init_rule, registered_init_rules
+
+    assert {"matrix", "gain", "zeros", "index"} <= set(registered_init_rules())
+    with pytest.raises(InvalidInput, match="already registered"):
+        register_init_rule("matrix", lambda spec, generator, dtype: None)
+    register_init_rule("test_sevens", lambda spec, generator, dtype: torch.full(tuple(spec.shape), 7.0, dtype=dtype))
+    try:
+        generator = torch.Generator().manual_seed(0)
+        drawn = _INIT_RULES["test_sevens"](TensorSpec("x", (2, 3), init="test_sevens"), generator, torch.bfloat16)
+        assert drawn.dtype == torch.bfloat16 and bool((drawn == 7).all())
+        zeros = _INIT_RULES["zeros"](TensorSpec("b", (4,), init="zeros"), generator, torch.float32)
+        assert zeros.dtype == torch.float32 and not zeros.any()
+    finally:
+        del _INIT_RULES["test_sevens"]
