@@ -36,13 +36,59 @@ def cache_for(requests, rt, max_tokens=1024, max_positions=1024, shared=None):
     return SequenceCache(list(enumerate(requests)), shared or {}, max_tokens, max_positions, rt.dtype, rt.device)
 
 
+class Bf16Yardstick:
+    """What bfloat16 alone does to a model's logits: the plain model run with
+    its activations rounded to bfloat16 where the engine keeps them so (its
+    twin), against the plain model in full precision, over sequences of the
+    test's own.  The engine in bfloat16 may be off the plain logits by at most
+    1.5 times the twin's error in root mean square (over sets of at least
+    ``RMS_FROM`` logits) and twice its worst logit.  A fault -- a key missed,
+    a mask off by one, a stale slot -- moves logits by several times that."""
+
+    RMS_FROM = 16384
+
+    def __init__(self, plain, sequences):
+        errors = []
+        for ids in sequences:
+            ids = list(ids)
+            errors.append((plain.logits(ids, _bf16_round) - plain.logits(ids)).flatten().double())
+        error = torch.cat(errors)
+        self.rms = float(error.pow(2).mean().sqrt())
+        self.worst = float(error.abs().max())
+        assert self.rms > 0 and self.worst < 0.25, (self.rms, self.worst)  # rounding: not nothing, and not a fault
+
+    def check(self, got, want, what=""):
+        """``got`` and ``want``: logits of the same shape (tensors or arrays)."""
+        error = (torch.as_tensor(np.asarray(got)).double() - torch.as_tensor(np.asarray(want)).double()).flatten()
+        worst = float(error.abs().max())
+        assert worst <= 2.0 * self.worst, f"{what}: worst logit off by {worst:.3g}; the bfloat16 twin's worst is {self.worst:.3g}"
+        if error.numel() >= self.RMS_FROM:
+            rms = float(error.pow(2).mean().sqrt())
+            assert rms <= 1.5 * self.rms, f"{what}: rms error {rms:.3g}; the bfloat16 twin's is {self.rms:.3g}"
+
+    def margin(self) -> float:
+        """How far below the plain model's best logit a token that the engine
+        picks greedily may lie: both logits may move by the worst error."""
+        return 4.0 * self.worst
+
+
+def _bf16_round(x):
+    return x.to(torch.bfloat16).to(x.dtype)
+
+
 def tolerance(dtype):
     return (2e-5, 2e-5) if dtype in ("float32", torch.float32) else (2e-2, 2e-2)
 
 
 def assert_close(got, want, dtype, what=""):
+    """32-bit: rounding of sums.  bfloat16: 2e-2 of a value plus an absolute
+    part that follows the size of the values compared (4e-2 of their root
+    mean square, at most 2e-2): logits of a tiny model are far smaller than 1,
+    and a flat bound would let a fault of their own size pass."""
     atol, rtol = tolerance(dtype)
     got, want = got.detach().float().cpu(), want.detach().float().cpu()
+    if atol > 1e-3 and want.numel():
+        atol = min(atol, 4e-2 * float(want.double().pow(2).mean().sqrt()))
     error = (got - want).abs()
     bound = atol + rtol * want.abs()
-    assert bool((error <= bound).all()), f"{what}: max error {error.max().item():.3g} (bound {atol}+{rtol}*|x|)"
+    assert bool((error <= bound).all()), f"{what}: max error {error.max().item():.3g} (bound {atol:.3g}+{rtol}*|x|)"

@@ -12,11 +12,22 @@ import torch
 
 import plain_llama as P
 from configs import TINY_CONFIGS
+from gpu_helpers import Bf16Yardstick
 
 pytestmark = pytest.mark.gpu
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-TOL = {"float32": (2e-5, 2e-5), "bfloat16": (2e-2, 2e-2)}
+_YARDS = {}
+
+
+def _yard(model_dirs, name):
+    """What bfloat16 alone does to the logits of tiny model ``name``, over sequences of several pages."""
+    if name not in _YARDS:
+        config, seed = TINY_CONFIGS[name]
+        rng = np.random.default_rng(900 + seed)
+        sequences = [rng.integers(0, config["vocab_size"], size=n).tolist() for n in (40, 97, 130, min(250, config["max_position_embeddings"]))]
+        _YARDS[name] = Bf16Yardstick(P.PlainLlama(model_dirs[name]), sequences)
+    return _YARDS[name]
 
 
 def _engine(model_dirs, name, dtype, max_tokens=1024):
@@ -25,10 +36,13 @@ def _engine(model_dirs, name, dtype, max_tokens=1024):
     return load_engine(model_dirs[name], dtype=dtype, max_tokens=max_tokens)
 
 
-def _close(got, want, dtype, what):
-    atol, rtol = TOL[dtype]
+def _close(got, want, dtype, what, yard=None):
+    """32-bit: rounding of sums.  bfloat16: within the model's yardstick (``_yard``)."""
+    if dtype == "bfloat16":
+        yard.check(got.float().cpu(), want.float().cpu(), what)
+        return
     error = (got - want).abs()
-    bound = atol + rtol * want.abs()
+    bound = 2e-5 + 2e-5 * want.abs()
     assert bool((error <= bound).all()), f"{what}: max error {error.max().item():.3g}"
 
 
@@ -50,7 +64,7 @@ def test_long_decoding(model_dirs, name, dtype):
         rows.append(engine.step([StepEntry(slot, [token], [0])]))
     got = torch.cat(rows).cpu()
     assert engine.length(slot) == total
-    _close(got, want, dtype, f"tiny {name} {dtype} long decoding")
+    _close(got, want, dtype, f"tiny {name} {dtype} long decoding", _yard(model_dirs, name))
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -65,13 +79,14 @@ def test_first_tokens(model_dirs, dtype):
     plain = P.PlainLlama(model_dirs["C"])
     engine = _engine(model_dirs, "C", dtype)
     a, b = engine.start_sequence(), engine.start_sequence()
+    yard = _yard(model_dirs, "C")
     first = engine.step([StepEntry(a, short[:1], [0]), StepEntry(b, long[:67], [66])]).cpu()
-    _close(first[0], plain.logits(short[:1])[0], dtype, "first token")
-    _close(first[1], plain.logits(long[:67])[66], dtype, "neighbour")
+    _close(first[0], plain.logits(short[:1])[0], dtype, "first token", yard)
+    _close(first[1], plain.logits(long[:67])[66], dtype, "neighbour", yard)
     for i in range(1, 4):
         rows = engine.step([StepEntry(b, [long[66 + i]], [0]), StepEntry(a, [short[i]], None)]).cpu()
-        _close(rows[1], plain.logits(short[:i + 1])[i], dtype, f"token {i}")
-        _close(rows[0], plain.logits(long[:67 + i])[66 + i], dtype, f"neighbour {i}")
+        _close(rows[1], plain.logits(short[:i + 1])[i], dtype, f"token {i}", yard)
+        _close(rows[0], plain.logits(long[:67 + i])[66 + i], dtype, f"neighbour {i}", yard)
 
 
 def test_refused_steps_change_nothing(model_dirs):
@@ -111,14 +126,19 @@ def test_greedy_generation_through_the_entry_point(model_dirs, name):
     # a cache of 6 pages and batches of at most 3: two batches, slots used again
     got = nnis_amd.generate(model_dirs[name], prompts, max_new_tokens=8, dtype="float32", max_tokens=6 * 64, max_batch=3)
     assert got == want
-    # bfloat16 may leave the 32-bit path at a near tie: every token it picks must be
-    # (nearly) the plain model's best continuation of what it has picked so far
+    # bfloat16 may leave the 32-bit path at a near tie: every token it picks must be the plain model's best
+    # continuation of what it has picked so far, or lie below the best by no more than rounding moves two logits
+    margin = _yard(model_dirs, name).margin()
     got16 = nnis_amd.generate(model_dirs[name], prompts, max_new_tokens=8, dtype="bfloat16", max_tokens=6 * 64, max_batch=3)
+    at_best = total = 0
     for prompt, tokens in zip(prompts, got16):
         assert 1 <= len(tokens) <= 8
         logits = plain.logits(prompt + tokens)[len(prompt) - 1:-1]
         for row, token in zip(logits, tokens):
-            assert row[token].item() >= row.max().item() - 3e-2
+            assert row[token].item() >= row.max().item() - margin, (token, row[token].item(), row.max().item(), margin)
+            at_best += int(token == int(row.argmax()))
+            total += 1
+    assert at_best >= 0.8 * total, (at_best, total)  # and near ties are the exception
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -264,7 +284,7 @@ def test_prompt_steps_whose_shape_comes_again(model_dirs, dtype):
             places = [n - 1] if want is None else want
             whole = plain.logits(t)
             for place in places:
-                _close(rows[at], whole[s + place], dtype, f"counts {counts} starts {starts} place {place}")
+                _close(rows[at], whole[s + place], dtype, f"counts {counts} starts {starts} place {place}", _yard(model_dirs, "B"))
                 at += 1
         assert at == rows.shape[0]
         for slot in slots:
@@ -438,3 +458,78 @@ def test_sampled_generation_is_seeded_and_per_sequence(model_dirs):
         assert sampler.sample(plain.logits(ids)[-1].numpy()) == token
         ids.append(token)
     assert engine.free_slots() == engine.cache.max_slots and engine.free_pages() == engine.cache.pages
+
+
+def test_a_captured_step_keeps_the_scratch_it_was_captured_with(tmp_path):
+    """The split decode attention leaves its partial sums in a scratch tensor
+    that the kernels' wrapper keeps per device and replaces by a larger one
+    when a step needs more.  A graph captured before has the first one's
+    address baked in: it must still own that memory when it is replayed, or it
+    writes into whatever the allocator has handed the block to since."""
+    import nnis_amd
+    from configs import SHAPE_CONFIGS
+    from nnis_amd.api import load_engine
+    from nnis_amd.engine.batch import StepEntry
+    from nnis_amd.kernels import ops
+
+    config, seed = SHAPE_CONFIGS["tinyllama-1.1b"]  # 32 query heads on 4: a batch of 8 at 1,100 keys needs 69,632 floats
+    folder = tmp_path / "model"
+    folder.mkdir()
+    nnis_amd.write_random_model(str(folder), config, seed)
+    plain = P.PlainLlama(str(folder))
+    rng = np.random.default_rng(5)
+    vocab = config["vocab_size"]
+    sequences = [rng.integers(0, vocab, size=1104).tolist() for _ in range(8)]
+    want = [plain.logits(sequences[i]) for i in (0, 1)]
+    yard = Bf16Yardstick(plain, [sequences[0][:600]])
+
+    ops._decode_scratch.clear()  # as in a fresh process (graphs captured by earlier tests hold what they use)
+    engine = load_engine(str(folder), dtype="bfloat16", max_tokens=8 * 1152)
+    assert engine.use_graphs
+    a = engine.start_sequence()
+    engine.step([StepEntry(a, sequences[0][:1100], [])])
+    row = engine.step([StepEntry(a, [sequences[0][1100]], [0])])  # captured: one sequence, its keys in 4 runs
+    yard.check(row.cpu(), want[0][1100:1101], "one sequence, first step")
+    small = ops.decode_scratch_held(engine.rt.device)
+    assert small is not None and small.numel() == 1 << 16
+    graph = next(iter(engine._graphs.graphs.values()))
+    assert graph.scratch.data_ptr() == small.data_ptr()
+
+    others = [engine.start_sequence() for _ in range(7)]
+    engine.step([StepEntry(s, t[:1100], []) for s, t in zip(others, sequences[1:])])
+    engine.step([StepEntry(s, [t[1100]], [0]) for s, t in zip([a] + others, sequences)])  # 8 sequences: a larger scratch
+    large = ops.decode_scratch_held(engine.rt.device)
+    assert large.numel() > small.numel() and large.data_ptr() != small.data_ptr()
+    del small
+    torch.cuda.synchronize()
+    sentinels = [torch.full((1 << 16,), 7.0, device="cuda") for _ in range(6)]  # what would take a freed block of that size
+    assert all(s.data_ptr() != graph.scratch.data_ptr() for s in sentinels)
+
+    for slot in others[1:]:
+        engine.end_sequence(slot)
+    b = others[0]
+    # the first graph again, for each of two sequences alone
+    row_a = engine.step([StepEntry(a, [sequences[0][1101]], [0])]).cpu()
+    row_b = engine.step([StepEntry(b, [sequences[1][1101]], [0])]).cpu()
+    torch.cuda.synchronize()
+    assert all(bool((s == 7.0).all()) for s in sentinels)
+    yard.check(row_a, want[0][1101:1102], "one sequence, replayed after the scratch grew")
+    yard.check(row_b, want[1][1101:1102], "another sequence through the same graph")
+
+
+def test_a_tied_head_keeps_the_table_once(model_dirs):
+    """In bfloat16 the head multiplies the table in the matrix cores' packed
+    order; the embedding gathers its rows from that same copy, and the table
+    in the checkpoint's order is let go
+    (/root/reference/crates/nnis-model/src/safetensors_loader.rs:755-786: a
+    tied head shares the embedding's buffer).  32-bit: one tensor for both."""
+    from nnis_amd.api import load_model
+    from nnis_amd.kernels.ops import PackedWeight
+
+    model, _ = load_model(model_dirs["A"], dtype="bfloat16")
+    assert isinstance(model.embedding.table, PackedWeight)
+    assert model.embedding.table is model.head.projection.weight
+    untied, _ = load_model(model_dirs["B"], dtype="bfloat16")  # a head of its own: the table stays as loaded
+    assert isinstance(untied.embedding.table, torch.Tensor) and isinstance(untied.head.projection.weight, PackedWeight)
+    wide, _ = load_model(model_dirs["A"], dtype="float32")
+    assert wide.embedding.table.data_ptr() == wide.head.projection.weight.data_ptr()

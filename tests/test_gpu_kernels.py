@@ -336,6 +336,62 @@ def test_prefill_attention_with_more_items_than_compute_units(heads, kv_heads, h
             assert (got[packed, 0] - vs[slot][key, 0]).abs().max().item() < 0.05
 
 
+@pytest.mark.parametrize("heads, kv_heads, head_dim", [(9, 3, 64), (32, 4, 64), (4, 4, 32)])
+def test_attention_beyond_64_pages(heads, kv_heads, head_dim):
+    """A sequence of 4,500 tokens (71 pages: a wave that walks them all comes
+    to the end of its first run of page numbers and has to fetch the next),
+    with a loud key in the very first page and one beyond page 64, for one
+    token of a decode step (one wave and one run, several waves, several runs,
+    both kernels) and for the last rows of a prompt step."""
+    ops = _ops()
+    torch.manual_seed(heads + head_dim)
+    length = 4500
+    scale = 1.0 / math.sqrt(head_dim)
+    ks = [torch.randn(length, kv_heads, head_dim).bfloat16().float(), torch.randn(70, kv_heads, head_dim).bfloat16().float()]
+    vs = [torch.randn(length, kv_heads, head_dim).bfloat16().float(), torch.randn(70, kv_heads, head_dim).bfloat16().float()]
+    group = heads // kv_heads
+    q_last = torch.randn(heads, head_dim).bfloat16().float()
+    # head 0 finds key 5 (page 0); the first head of the last group finds key 4,230 (page 66)
+    far_head = heads - group
+    ks[0][5, 0] = (q_last[0] * (14.0 / scale / q_last[0].pow(2).sum())).bfloat16().float()
+    ks[0][4230, kv_heads - 1] = (q_last[far_head] * (14.0 / scale / q_last[far_head].pow(2).sum())).bfloat16().float()
+    k_pages, v_pages, table = _paged(ks, vs, torch.bfloat16, kv_heads, head_dim, pages=80, max_pages=72)
+    rows = [(0, length - 1, q_last), (1, 69, torch.randn(heads, head_dim).bfloat16().float())]
+    q = torch.stack([q for _, _, q in rows]).bfloat16().reshape(len(rows), -1).cuda()
+    want = _plain_rows(rows, ks, vs, scale)
+    kernels = ["columns"] + (["keys"] if group <= 4 else [])
+    for kernel in kernels:
+        for splits, waves in ((1, 1), (1, 4), (8, 4), (2, 1)):
+            waves = min(waves, ops.decode_max_waves(heads, kv_heads, head_dim))
+            out = torch.full((len(rows), heads * head_dim), 3.0, dtype=torch.bfloat16, device="cuda")
+            partial = torch.full((len(rows) * heads * splits * (head_dim + 4),), float("nan"), dtype=torch.float32, device="cuda")
+            ops.attention_decode_bf16(q, out, k_pages, v_pages, table, _i32([0, 1]), _i32([length - 1, 69]), heads, kv_heads,
+                                      head_dim, scale, 0, splits, partial, waves, kernel)
+            got = out.cpu().float().view(len(rows), heads, head_dim)
+            assert (got - want).abs().max().item() <= 2e-2, (kernel, splits, waves, (got - want).abs().max().item())
+            assert (got[0, 0] - vs[0][5, 0]).abs().max().item() < 0.05, (kernel, splits, waves)
+            assert (got[0, far_head] - vs[0][4230, kv_heads - 1]).abs().max().item() < 0.05, (kernel, splits, waves)
+    # a prompt step: the sequence's last 40 tokens are new, the 4,460 before them are in the cache
+    new = 40
+    pos0 = length - new
+    q_rows = torch.randn(new, heads, head_dim).bfloat16().float()
+    q_rows[-1] = q_last
+    prompt_rows = [(0, pos0 + i, q_rows[i]) for i in range(new)]
+    want = _plain_rows(prompt_rows, ks, vs, scale)
+    qp = q_rows.bfloat16().reshape(new, -1).cuda()
+    for waves in (1, 8):
+        waves = min(waves, ops.prefill_max_waves(heads, kv_heads, head_dim))
+        tile = ops.prefill_tile_rows(heads, kv_heads, head_dim)
+        items = [(0, row0) for row0 in range(0, new, tile)]
+        out = torch.full((new, heads * head_dim), 3.0, dtype=torch.bfloat16, device="cuda")
+        ops.attention_prefill_bf16(qp, out, k_pages, v_pages, table, _i32([s for s, _ in items]), _i32([r for _, r in items]),
+                                   _i32([0]), _i32([0, new]), _i32([pos0]), heads, kv_heads, head_dim, scale, 0, waves)
+        got = out.cpu().float().view(new, heads, head_dim)
+        assert (got - want).abs().max().item() <= 2e-2, (waves, (got - want).abs().max().item())
+        assert (got[-1, 0] - vs[0][5, 0]).abs().max().item() < 0.05
+        assert (got[-1, far_head] - vs[0][4230, kv_heads - 1]).abs().max().item() < 0.05
+
+
 @pytest.mark.parametrize("hint", [32, 48])
 def test_gemm_tiled_over_many_blocks(hint):
     """Both tiles of the tiled kernel over a grid of hundreds of blocks in

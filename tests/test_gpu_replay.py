@@ -11,6 +11,7 @@ import torch
 import plain_llama as P
 import replay
 from configs import SHAPE_CONFIGS, TINY_CONFIGS
+from gpu_helpers import Bf16Yardstick
 
 pytestmark = pytest.mark.gpu
 
@@ -45,9 +46,9 @@ def test_schedules_agree_with_the_plain_model(model_dirs, tmp_path, name, dtype)
     requests = _requests(vocab, 100 + seed)
     plain = P.PlainLlama(model_dirs[name], torch.float32)
     plain_logits = {n: plain.logits(t) for n, t in requests.items()}
-    # 32-bit: rounding of sums only.  bfloat16: activations and cache keep 8 bits
-    # of mantissa; logits here are of order 1.
-    atol, rtol = (2e-5, 2e-5) if dtype == "float32" else (2e-2, 2e-2)
+    # 32-bit: rounding of sums only.  bfloat16: measured against what bfloat16 alone does to this model's
+    # logits (the plain model with its activations rounded where the engine keeps them so).
+    yard = Bf16Yardstick(plain, requests.values()) if dtype == "bfloat16" else None
 
     # every schedule in one process, one after another, with a cache too small
     # to hold them side by side: 8 pages, the largest batch needs 7
@@ -60,14 +61,26 @@ def test_schedules_agree_with_the_plain_model(model_dirs, tmp_path, name, dtype)
         renamed.append({"entries": [dict(e, id=tag + e["id"]) for e in step["entries"]], "end": [tag + n for n in step.get("end", [])]})
     rows = replay.run_trace(model_dirs[name], dtype, renamed, str(tmp_path), max_tokens=8 * 64, vocab=vocab)
     assert len(rows) == 3 * sum(LENGTHS)
+    keys = sorted((n, p) for n, t in requests.items() for p in range(len(t)))
+    want = np.stack([plain_logits[n][p].numpy() for n, p in keys])
+    stacked = {}
     for tag, what in (("w", "whole"), ("t", "last 32 one by one"), ("b", "unequal batches")):
         part = {(n[1:], p): row for (n, p), row in rows.items() if n[0] == tag}
         assert len(part) == sum(LENGTHS)
-        _compare(part, plain_logits, atol, rtol, f"tiny {name} {dtype} {what}")
-    # the schedules agree with each other far more closely than with the plain model's rounding
-    between = max(float(np.abs(rows[("w" + n, p)] - rows[(tag + n, p)]).max())
-                  for tag in "tb" for n, t in requests.items() for p in range(len(t)))
-    assert between <= (1e-5 if dtype == "float32" else 2e-2), between
+        if yard is None:
+            _compare(part, plain_logits, 2e-5, 2e-5, f"tiny {name} {dtype} {what}")
+        else:
+            stacked[tag] = np.stack([part[key] for key in keys])
+            yard.check(stacked[tag], want, f"tiny {name} {dtype} {what}")
+    if yard is None:
+        # the schedules agree with each other far more closely than with the plain model's rounding
+        between = max(float(np.abs(rows[("w" + n, p)] - rows[(tag + n, p)]).max())
+                      for tag in "tb" for n, t in requests.items() for p in range(len(t)))
+        assert between <= 1e-5, between
+    else:
+        # and in bfloat16 as closely as each agrees with the plain model
+        for tag in "tb":
+            yard.check(stacked[tag], stacked["w"], f"tiny {name} {dtype} schedule {tag} against whole")
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
