@@ -497,7 +497,8 @@ def test_a_captured_step_keeps_the_scratch_it_was_captured_with(tmp_path):
 
     others = [engine.start_sequence() for _ in range(7)]
     engine.step([StepEntry(s, t[:1100], []) for s, t in zip(others, sequences[1:])])
-    engine.step([StepEntry(s, [t[1100]], [0]) for s, t in zip([a] + others, sequences)])  # 8 sequences: a larger scratch
+    engine.step([StepEntry(a, [sequences[0][1101]], [0])]
+                + [StepEntry(s, [t[1100]], [0]) for s, t in zip(others, sequences[1:])])  # 8 sequences: a larger scratch
     large = ops.decode_scratch_held(engine.rt.device)
     assert large.numel() > small.numel() and large.data_ptr() != small.data_ptr()
     del small
@@ -509,11 +510,11 @@ def test_a_captured_step_keeps_the_scratch_it_was_captured_with(tmp_path):
         engine.end_sequence(slot)
     b = others[0]
     # the first graph again, for each of two sequences alone
-    row_a = engine.step([StepEntry(a, [sequences[0][1101]], [0])]).cpu()
+    row_a = engine.step([StepEntry(a, [sequences[0][1102]], [0])]).cpu()
     row_b = engine.step([StepEntry(b, [sequences[1][1101]], [0])]).cpu()
     torch.cuda.synchronize()
     assert all(bool((s == 7.0).all()) for s in sentinels)
-    yard.check(row_a, want[0][1101:1102], "one sequence, replayed after the scratch grew")
+    yard.check(row_a, want[0][1102:1103], "one sequence, replayed after the scratch grew")
     yard.check(row_b, want[1][1101:1102], "another sequence through the same graph")
 
 

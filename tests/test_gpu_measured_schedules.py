@@ -152,14 +152,15 @@ def test_the_head_at_real_vocabularies(m, n, k):
         else:
             assert torch.equal(y.cpu(), want.to(torch.bfloat16))
     # the same product on a prepared operand (the norm's second half in the kernel): the parts of the sums of
-    # squares are chosen so that every row's scale is exactly 1/2 or 1/4
+    # squares are chosen so that every row's mean square plus eps is 4 or 16, its scale 1/2 or 1/4
     parts = 3
     ss = torch.zeros(parts, m)
-    ss[0] = torch.where(torch.arange(m) % 2 == 0, 4.0 * k, 16.0 * k) - 2.0
+    eps = 2.0 ** -10
+    ss[0] = torch.where(torch.arange(m) % 2 == 0, (4.0 - eps) * k, (16.0 - eps) * k) - 2.0
     ss[1], ss[2] = 1.5, 0.5
     scale = torch.where(torch.arange(m) % 2 == 0, 0.5, 0.25).double()
     y = torch.full((m, n), 7.0, dtype=torch.bfloat16, device="cuda")
-    ops.gemm_scaled(x.cuda(), ss.cuda(), parts, 0.0, packed, y, ops.EPILOGUE_STORE)
+    ops.gemm_scaled(x.cuda(), ss.cuda(), parts, eps, packed, y, ops.EPILOGUE_STORE)
     scaled = want * scale[:, None]
     error = (y.cpu().double() - scaled).abs()
     assert bool((error <= 2.0 ** -8 * scaled.abs() + 1e-6).all()), error.max().item()  # one rounding to bfloat16, a root of 1 ulp
