@@ -4,6 +4,9 @@
 // Storage types are chosen at run time (32-bit float or bfloat16); every sum,
 // statistic and rotation is computed in 32-bit.
 #include "common.h"
+#include "nnis_noalloc.h"
+
+#include <mutex>
 
 thread_local char g_nnis_error[512] = {0};
 
@@ -597,5 +600,59 @@ extern "C" int nnis_argmax(const float* logits, int* out, int rows, int vocab, v
   NNIS_LAUNCH_CHECK("argmax");
   hipLaunchKernelGGL(argmax_rows_kernel, dim3(rows), dim3(64), 0, (hipStream_t)stream, part_v, part_i, out, chunks);
   NNIS_LAUNCH_CHECK("argmax");
+  return 0;
+}
+
+// -----------------------------------------------------------------------------
+// The same argmax from a fixed array in device memory (nnis_noalloc.h): no allocation anywhere on the way.
+// Host code never uses the array's name for its memory: the name is a host-side stand-in, and each GPU has a
+// copy of the array at an address of its own, asked for once per device with that device current.
+// -----------------------------------------------------------------------------
+static __device__ __align__(256) unsigned int nnis_static_scratch[NNIS_STATIC_SCRATCH_WORDS];
+
+constexpr int kStaticScratchDevices = 64;
+static void* g_static_scratch_ptr[kStaticScratchDevices] = {nullptr};
+static std::mutex g_static_scratch_mutex;
+
+// the current device's copy of the array (nullptr with a message left on failure)
+static void* nnis_static_scratch_address() {
+  int device = -1;
+  hipError_t status = hipGetDevice(&device);
+  if (status != hipSuccess || device < 0 || device >= kStaticScratchDevices) {
+    nnis_fail("argmax_static: no current device (%s)", status != hipSuccess ? hipGetErrorString(status) : "index out of range");
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> guard(g_static_scratch_mutex);
+  if (g_static_scratch_ptr[device] == nullptr) {
+    void* address = nullptr;
+    status = hipGetSymbolAddress(&address, HIP_SYMBOL(nnis_static_scratch));
+    if (status != hipSuccess || address == nullptr) {
+      nnis_fail("argmax_static: the fixed array has no address on device %d (%s)", device, hipGetErrorString(status));
+      return nullptr;
+    }
+    g_static_scratch_ptr[device] = address;
+  }
+  return g_static_scratch_ptr[device];
+}
+
+extern "C" int nnis_argmax_static(const float* logits, int* out, int rows, int vocab, void* stream) {
+  NNIS_REQUIRE(rows >= 0 && vocab > 0, "argmax_static: bad sizes rows=%d vocab=%d", rows, vocab);
+  if (rows == 0) return 0;
+  NNIS_REQUIRE(logits != nullptr && out != nullptr, "argmax_static: logits and out must be given");
+  NNIS_REQUIRE(rows <= 65535, "argmax_static: %d rows exceed the grid limit", rows);
+  const long long chunks = ((long long)vocab + kArgmaxChunk - 1) / kArgmaxChunk;
+  const long long words = 2LL * rows * chunks;
+  NNIS_REQUIRE(words <= NNIS_STATIC_SCRATCH_WORDS,
+               "argmax_static: %d rows of %d columns need %lld words of scratch; the fixed array holds %d "
+               "(use nnis_argmax with scratch of the caller's)", rows, vocab, words, NNIS_STATIC_SCRATCH_WORDS);
+  void* scratch = nnis_static_scratch_address();
+  if (scratch == nullptr) return 1;
+  float* part_v = (float*)scratch;
+  int* part_i = (int*)(part_v + (size_t)rows * chunks);
+  hipLaunchKernelGGL(argmax_chunk_kernel, dim3((int)chunks, rows), dim3(256), 0, (hipStream_t)stream, logits, part_v, part_i,
+                     vocab, (int)chunks);
+  NNIS_LAUNCH_CHECK("argmax_static");
+  hipLaunchKernelGGL(argmax_rows_kernel, dim3(rows), dim3(64), 0, (hipStream_t)stream, part_v, part_i, out, (int)chunks);
+  NNIS_LAUNCH_CHECK("argmax_static");
   return 0;
 }

@@ -47,7 +47,7 @@ FLAGS = [
 # of either file spills with the sums in vector registers, at any head size).
 _VECTOR_SUMS = ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]
 SOURCE_FLAGS = {"gemm_mfma.hip": _VECTOR_SUMS, "attention.hip": _VECTOR_SUMS}
-HEADERS = {"core": ["common.h", "epilogue.h"], "attention": ["common.h"]}  # what a module's sources include
+HEADERS = {"core": ["common.h", "epilogue.h", "nnis_noalloc.h"], "attention": ["common.h"]}  # what a module's sources include
 CORE_SOURCES = ["elementwise.hip", "gemm.hip", "gemm_mfma.hip", "gemm_fused.hip", "sampling.hip"]
 ATTENTION_SOURCES = ["attention.hip"]
 PREBUILT_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 112, 128)

@@ -31,6 +31,7 @@ _CORE_SIGNATURES = {
     "nnis_silu_mul": [_VOID, _INT, _VOID, _INT, _INT, _INT, _VOID],
     "nnis_argmax": [_VOID, _VOID, _INT, _INT, _VOID, _VOID],
     "nnis_argmax_scratch": [_INT, _INT],
+    "nnis_argmax_static": [_VOID, _VOID, _INT, _INT, _VOID],
     "nnis_gemm_ordered": [_VOID, _INT, _VOID, _INT, _VOID, _INT, _INT, _INT, _INT, _VOID],
     "nnis_gemm_bf16": [_VOID, _VOID, _VOID, _INT, _INT, _INT, _INT, _INT, _VOID, _SIZE, _VOID],
     "nnis_gemm_fused": [_VOID, _VOID, _VOID, _VOID, _INT, _FLT, _VOID, _INT, _INT, _INT, _INT, _VOID, _VOID, _VOID, _INT,
@@ -246,6 +247,24 @@ def argmax(logits: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     lib = core()
     scratch = torch.empty(max(1, lib.nnis_argmax_scratch(rows, vocab)), dtype=torch.float32, device=logits.device)
     _check(lib, lib.nnis_argmax(logits.data_ptr(), out.data_ptr(), rows, vocab, scratch.data_ptr(), _stream()))
+    return out
+
+
+STATIC_SCRATCH_WORDS = 65536  # NNIS_STATIC_SCRATCH_WORDS of csrc/nnis_noalloc.h
+
+
+def argmax_no_alloc(logits: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """``argmax`` for callers that cannot allocate: the first pass's results go
+    through a fixed array that the library holds on the GPU (256 KB; enough
+    for 2 * rows * ceil(vocab / 4096) <= 65,536 words, beyond that the call
+    is refused).  Calls on one GPU share the array: keep them in order on one
+    stream."""
+    _dev(logits, "logits"), _dev(out, "out")
+    rows, vocab = logits.shape
+    if logits.dtype != torch.float32 or out.dtype != torch.int32 or out.numel() < rows:
+        raise KernelError("argmax: logits must be float32 [rows, vocab] and out int32 [rows]")
+    lib = core()
+    _check(lib, lib.nnis_argmax_static(logits.data_ptr(), out.data_ptr(), rows, vocab, _stream()))
     return out
 
 
