@@ -319,6 +319,7 @@ struct MfmaArgs {
   const bf16_t* v_pages;
   const int* block_table;
   int max_pages;
+  int rows_by_token;  // decode: block_table holds a row per token of the step (the step's tables), not per slot
   int heads, kv_heads;
   int window;
   float scale_log2;
@@ -681,12 +682,18 @@ __global__ __launch_bounds__(64 * kBlockWaves) void attention_decode_kernel(Mfma
   extern __shared__ float merge[];  // [waves / 2][C][kTilesD * 4 + 2][64]
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave, r = lane % 16, g = lane / 16;
   const int token = blockIdx.x, kv_head = blockIdx.y, split = blockIdx.z;
-  const int slot = a.tok_slot[token];
-  if (slot < 0) return;  // a padding row (the whole block leaves): its output is never read
+  // With the step's tables a token's pages are a row of its own and nothing is asked of its slot: the first
+  // pages' numbers are one round trip away, not two.  (A padding row then reads the page its row names, 0,
+  // and leaves a result that nobody reads.)
+  int slot = 0;
+  if (!a.rows_by_token) {
+    slot = a.tok_slot[token];
+    if (slot < 0) return;  // a padding row (the whole block leaves): its output is never read
+  }
   const int group = a.heads / a.kv_heads;
   const int pos = a.tok_pos[token];
   const int first_key = (a.window > 0 && pos + 1 > a.window) ? pos + 1 - a.window : 0;
-  const int* pages = a.block_table + (size_t)slot * a.max_pages;
+  const int* pages = a.block_table + (size_t)(a.rows_by_token ? token : slot) * a.max_pages;
 
   QFrag q[C];
   int lo[C], hi[C];
@@ -750,12 +757,15 @@ __global__ __launch_bounds__(64 * kKeysWaves) void attention_decode_keys_kernel(
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave, r = lane % 16, g = lane / 16;
   const int blk = lane / 4, j = lane % 4;  // the scores' layout: keys 4 blk .. 4 blk + 3 of a page, head j of the group
   const int token = blockIdx.x, kv_head = blockIdx.y, split = blockIdx.z;
-  const int slot = a.tok_slot[token];
-  if (slot < 0) return;  // a padding row (the whole block leaves): its output is never read
+  int slot = 0;
+  if (!a.rows_by_token) {  // (see attention_decode_kernel)
+    slot = a.tok_slot[token];
+    if (slot < 0) return;  // a padding row (the whole block leaves): its output is never read
+  }
   const int group = a.heads / a.kv_heads;
   const int pos = a.tok_pos[token];
   const int first_key = (a.window > 0 && pos + 1 > a.window) ? pos + 1 - a.window : 0;
-  const int* pages = a.block_table + (size_t)slot * a.max_pages;
+  const int* pages = a.block_table + (size_t)(a.rows_by_token ? token : slot) * a.max_pages;
 
   // the query of head j, all channels (heads beyond the group: zeros, their columns are never written)
   bf16x8 q[HD / 8];
@@ -903,10 +913,12 @@ __global__ __launch_bounds__(64 * kKeysWaves) void attention_decode_keys_kernel(
 __global__ void attention_combine_kernel(const float* __restrict__ partial, bf16_t* __restrict__ out,
                                          const int* __restrict__ tok_slot, int heads, int splits) {
   const int token = blockIdx.x, head = blockIdx.y;
-  if (tok_slot[token] < 0) return;
   const float* base = partial + ((size_t)token * heads + head) * splits * kPartial;
   constexpr int kAtOnce = 8;  // runs whose references, sums and outputs a thread asks for together: one round trip
   if (splits <= kAtOnce) {
+    // a padding row's runs hold whatever the scratch held: they are read like any (the slot is asked for in the
+    // same round trip, not before it) and nothing is stored for them
+    const int slot = tok_slot[token];
     for (int d = threadIdx.x; d < HD; d += blockDim.x) {
       float m[kAtOnce], l[kAtOnce], o[kAtOnce];
 #pragma unroll
@@ -928,10 +940,11 @@ __global__ void attention_combine_kernel(const float* __restrict__ partial, bf16
           den += l[s] * w;
         }
       }
-      out[((size_t)token * heads + head) * HD + d] = (bf16_t)(num / den);
+      if (slot >= 0) out[((size_t)token * heads + head) * HD + d] = (bf16_t)(num / den);
     }
     return;
   }
+  if (tok_slot[token] < 0) return;
   float m_all = -INFINITY;
   for (int s = 0; s < splits; ++s) m_all = fmaxf(m_all, base[(size_t)s * kPartial + HD]);
   for (int d = threadIdx.x; d < HD; d += blockDim.x) {
@@ -997,7 +1010,7 @@ int fill_common(MfmaArgs& a, const void* q, void* out, const void* k_pages, cons
   a.block_table = block_table; a.max_pages = max_pages; a.heads = heads; a.kv_heads = kv_heads; a.window = window;
   a.scale_log2 = scale * kLog2e;
   a.tile_seq = a.tile_row0 = a.seq_slot = a.seq_start = a.seq_pos0 = a.tok_slot = a.tok_pos = nullptr;
-  a.splits = 1; a.partial = nullptr;
+  a.splits = 1; a.partial = nullptr; a.rows_by_token = 0;
   return 0;
 }
 }  // namespace
@@ -1120,9 +1133,11 @@ extern "C" int nnis_attention_decode_max_waves(int heads, int kv_heads) {
 extern "C" int nnis_attention_decode_bf16(const void* q, void* out, const void* k_pages, const void* v_pages,
                                           const int* block_table, int max_pages, const int* tok_slot, const int* tok_pos,
                                           int tokens, int heads, int kv_heads, int head_dim, int window, float scale,
-                                          int splits, int waves, float* partial, int kind, int combine, void* stream) {
+                                          int splits, int waves, float* partial, int kind, int combine, int rows_by_token,
+                                          void* stream) {
   MfmaArgs a;
   if (fill_common(a, q, out, k_pages, v_pages, block_table, max_pages, heads, kv_heads, head_dim, window, scale)) return 1;
+  a.rows_by_token = rows_by_token ? 1 : 0;
   NNIS_REQUIRE(splits >= 1 && splits <= 65535, "attention: bad number of splits %d", splits);
   NNIS_REQUIRE(splits == 1 || partial != nullptr, "attention: splits need scratch memory");
   NNIS_REQUIRE((uintptr_t)partial % 16 == 0, "attention: scratch memory must be 16-byte aligned");
@@ -1193,7 +1208,7 @@ extern "C" int nnis_attention_combine(const float*, void*, const int*, int, int,
   return nnis_fail("attention: the matrix-core kernels need a head size in steps of 16; this module has %d", NNIS_HEAD_DIM);
 }
 extern "C" int nnis_attention_decode_bf16(const void*, void*, const void*, const void*, const int*, int, const int*, const int*,
-                                          int, int, int, int, int, float, int, int, float*, int, int, void*) {
+                                          int, int, int, int, int, float, int, int, float*, int, int, int, void*) {
   return nnis_fail("attention: the matrix-core kernels need a head size in steps of 16; this module has %d", NNIS_HEAD_DIM);
 }
 #endif

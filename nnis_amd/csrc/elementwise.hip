@@ -78,6 +78,55 @@ extern "C" int nnis_embed_packed(const int* ids, const void* packed, float* out,
 }
 
 // -----------------------------------------------------------------------------
+// The step's tables: what every layer's kernels would otherwise look up again through each token's slot and
+// position, gathered once per step by token: its rows of the rotation tables, the cache page that takes its
+// key and value, and (for a step of single tokens) the pages of its sequence.  A kernel that reads them has
+// nothing to wait for before it can ask for its data.  A padding row (negative slot) gets the identity
+// rotation, page -1 and, as its sequence's only page, page 0 (read by nobody who stores a result).
+// -----------------------------------------------------------------------------
+__global__ __launch_bounds__(64) void step_tables_kernel(const int* __restrict__ tok_slot, const int* __restrict__ tok_pos,
+                                                         const float* __restrict__ cos_table, const float* __restrict__ sin_table,
+                                                         int half, int table_positions, const int* __restrict__ block_table,
+                                                         int max_pages, float* __restrict__ tok_cos, float* __restrict__ tok_sin,
+                                                         int* __restrict__ tok_page, int* __restrict__ tok_pages) {
+  const int token = blockIdx.x;
+  const int slot = tok_slot[token];
+  int pos = tok_pos[token];
+  const bool live = slot >= 0 && pos >= 0;
+  if (cos_table) {
+    const int row = live && pos < table_positions ? pos : 0;
+    for (int c = threadIdx.x; c < half; c += blockDim.x) {
+      tok_cos[(size_t)token * half + c] = live ? cos_table[(size_t)row * half + c] : 1.0f;
+      tok_sin[(size_t)token * half + c] = live ? sin_table[(size_t)row * half + c] : 0.0f;
+    }
+  }
+  if (block_table) {
+    const int* row = block_table + (size_t)(live ? slot : 0) * max_pages;
+    int last = live ? pos / kPageTokens : 0;
+    last = last < max_pages ? last : max_pages - 1;
+    if (threadIdx.x == 0) tok_page[token] = live ? row[last] : -1;
+    if (tok_pages)
+      for (int i = threadIdx.x; i <= last; i += blockDim.x) tok_pages[(size_t)token * max_pages + i] = live ? row[i] : 0;
+  }
+}
+
+// tok_cos / tok_sin: [tokens, half] (with cos_table); tok_page: [tokens] and tok_pages: [tokens, max_pages] or
+// null (with block_table).  Either half of the work may be left out (null tables).
+extern "C" int nnis_step_tables(const int* tok_slot, const int* tok_pos, int tokens, const float* cos_table,
+                                const float* sin_table, int half, int table_positions, const int* block_table, int max_pages,
+                                float* tok_cos, float* tok_sin, int* tok_page, int* tok_pages, void* stream) {
+  NNIS_REQUIRE(tokens >= 0 && tok_slot && tok_pos, "step_tables: the tokens' slots and positions are missing");
+  NNIS_REQUIRE((cos_table == nullptr) == (sin_table == nullptr), "step_tables: cos and sin tables come together");
+  NNIS_REQUIRE(cos_table == nullptr || (half > 0 && table_positions > 0 && tok_cos && tok_sin), "step_tables: rotation rows need a place and sizes");
+  NNIS_REQUIRE(block_table == nullptr || (max_pages > 0 && tok_page), "step_tables: pages need a place and the table's width");
+  if (tokens == 0 || (cos_table == nullptr && block_table == nullptr)) return 0;
+  hipLaunchKernelGGL(step_tables_kernel, dim3(tokens), dim3(64), 0, (hipStream_t)stream, tok_slot, tok_pos, cos_table, sin_table,
+                     half, table_positions, block_table, max_pages, tok_cos, tok_sin, tok_page, tok_pages);
+  NNIS_LAUNCH_CHECK("step_tables");
+  return 0;
+}
+
+// -----------------------------------------------------------------------------
 // RMSNorm: y[c] = (x[c] * (1/sqrt(mean(x^2) + eps))) * w[c]
 // (/root/reference/crates/nnis-model/src/kernels.rs:15-48: eps inside the
 // root, mean over the row, x*scale*weight in that order).

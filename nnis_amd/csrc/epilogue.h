@@ -45,7 +45,26 @@ struct RopeTarget {
   const int* block_table;
   int max_pages;
   int heads, kv_heads, head_dim;
+  // The step's tables, where the caller brings them (all three, or none): each token's rows of the rotation
+  // tables [tokens, head_dim / 2] and the cache page of its position [tokens] (< 0: a padding row).  With them
+  // nothing the epilogue needs hangs on a value that has to be loaded first.
+  const float* tok_cos;
+  const float* tok_sin;
+  const int* tok_page;
 };
+
+__device__ __forceinline__ const float* rope_cos_row(const RopeTarget& a, int token, int pos) {
+  return a.tok_cos ? a.tok_cos + (size_t)token * (a.head_dim / 2) : a.cos_table + (size_t)pos * (a.head_dim / 2);
+}
+__device__ __forceinline__ const float* rope_sin_row(const RopeTarget& a, int token, int pos) {
+  return a.tok_sin ? a.tok_sin + (size_t)token * (a.head_dim / 2) : a.sin_table + (size_t)pos * (a.head_dim / 2);
+}
+// the cache page that takes the token's key and value, or < 0 (a padding row, or a run that keeps no cache)
+__device__ __forceinline__ int rope_page(const RopeTarget& a, int token, int slot, int pos) {
+  if (!a.k_pages) return -1;
+  if (a.tok_page) return a.tok_page[token];
+  return slot >= 0 ? a.block_table[(size_t)slot * a.max_pages + pos / kPageTokens] : -1;
+}
 
 // Rotate-half RoPE as /root/reference/crates/nnis-model/src/runtime_kernels.rs:38-66; keys stored rotated,
 // values as they are (runtime.rs:997-1016).  head: index among queries, then keys, then values; f0: the

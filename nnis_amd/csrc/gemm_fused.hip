@@ -128,18 +128,28 @@ __global__ __launch_bounds__(KSPLIT > 4 ? 64 * KSPLIT : 256) void gemm_fused_ker
   constexpr int kPartRegs = 8;  // parts of a row's sum of squares a lane keeps in flight (4 lane groups share a row)
   float ss_held[MT][kPartRegs];
   const bool ends_unit = active && part == 0;
+  const bool tables = EPI == EPI_ROPE && a.rope.tok_cos != nullptr;  // the step's tables: nothing hangs on a loaded value
   if (EPI == EPI_ROPE && ends_unit) {
+    const int head = row0 / a.rope.head_dim;
+    const int f0 = row0 % a.rope.head_dim + g * 4;
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
       int token = token0 + t * 16 + r;
       token = token < m ? token : m - 1;
-      tok_slot[t] = a.rope.tok_slot[token];
+      tok_slot[t] = tables ? 0 : a.rope.tok_slot[token];
       tok_pos[t] = a.rope.tok_pos[token];
       tok_page[t] = -1;
+      if (tables) {
+        if (head < a.rope.heads + a.rope.kv_heads) {
+          tok_cos[t] = *(const f32x4*)(a.rope.tok_cos + (size_t)token * (a.rope.head_dim / 2) + f0);
+          tok_sin[t] = *(const f32x4*)(a.rope.tok_sin + (size_t)token * (a.rope.head_dim / 2) + f0);
+        }
+        if (head >= a.rope.heads && a.rope.k_pages) tok_page[t] = a.rope.tok_page[token];
+      }
     }
   }
   auto dependent = [&]() {
-    if (EPI == EPI_ROPE && ends_unit) {
+    if (EPI == EPI_ROPE && ends_unit && !tables) {
       const int head = row0 / a.rope.head_dim;
       const int f0 = row0 % a.rope.head_dim + g * 4;
 #pragma unroll
@@ -429,6 +439,9 @@ int run_fused(FusedArgs& a, int epilogue, int table_positions, int split_hint, f
     NNIS_REQUIRE((a.rope.k_pages == nullptr) == (a.rope.v_pages == nullptr), "gemm_fused: key and value pages must come together");
     NNIS_REQUIRE(a.rope.k_pages == nullptr || (a.rope.block_table && a.rope.max_pages > 0), "gemm_fused: cache without a block table");
     NNIS_REQUIRE(table_positions > 0, "gemm_fused: empty rotation tables");
+    NNIS_REQUIRE((a.rope.tok_cos != nullptr) == (a.rope.tok_sin != nullptr) && (a.rope.tok_cos != nullptr) == (a.rope.tok_page != nullptr),
+                 "gemm_fused: the step's tables (rotation rows and pages of the tokens) come together or not at all");
+    NNIS_REQUIRE((uintptr_t)a.rope.tok_cos % 16 == 0 && (uintptr_t)a.rope.tok_sin % 16 == 0, "gemm_fused: the step's tables must be 16-byte aligned");
     units = (a.rope.heads + 2 * a.rope.kv_heads) * (a.rope.head_dim / 32);
   } else {
     return nnis_fail("gemm_fused: unknown epilogue %d", epilogue);
@@ -468,7 +481,8 @@ extern "C" int nnis_gemm_fused(const float* x_in, const void* delta, float* x_ou
                                float eps, const void* w, int m, int n, int k, int epilogue, void* y, const float* cos_table,
                                const float* sin_table, int table_positions, const int* tok_slot, const int* tok_pos,
                                void* k_pages, void* v_pages, const int* block_table, int max_pages, int heads, int kv_heads,
-                               int head_dim, int split_hint, void* stream_ptr) {
+                               int head_dim, const float* tok_cos, const float* tok_sin, const int* tok_page, int split_hint,
+                               void* stream_ptr) {
   NNIS_REQUIRE(m > 0 && nnis_gemm_takes_few_tokens(m, n, k), "gemm_fused: %d tokens are too many for a weight of %d x %d", m, n, k);
   NNIS_REQUIRE(n > 0 && k > 0 && k % 8 == 0, "gemm_fused: bad sizes n=%d k=%d (K must be a multiple of 8)", n, k);
   NNIS_REQUIRE(nnis_dtype_ok(norm_w_dtype), "gemm_fused: unknown norm weight dtype %d", norm_w_dtype);
@@ -484,6 +498,7 @@ extern "C" int nnis_gemm_fused(const float* x_in, const void* delta, float* x_ou
   a.rope.q_out = (bf16_t*)y; a.rope.cos_table = cos_table; a.rope.sin_table = sin_table; a.rope.tok_slot = tok_slot; a.rope.tok_pos = tok_pos;
   a.rope.k_pages = (bf16_t*)k_pages; a.rope.v_pages = (bf16_t*)v_pages; a.rope.block_table = block_table; a.rope.max_pages = max_pages;
   a.rope.heads = heads; a.rope.kv_heads = kv_heads; a.rope.head_dim = head_dim;
+  a.rope.tok_cos = tok_cos; a.rope.tok_sin = tok_sin; a.rope.tok_page = tok_page;
   return run_fused(a, epilogue, table_positions, split_hint, nullptr, 0, (hipStream_t)stream_ptr);
 }
 
@@ -492,7 +507,8 @@ extern "C" int nnis_gemm_fused(const float* x_in, const void* delta, float* x_ou
 extern "C" int nnis_gemm_scaled(const void* scaled, const float* ss_parts, int parts, float eps, const void* w, int m, int n,
                                 int k, int epilogue, void* y, const float* cos_table, const float* sin_table,
                                 int table_positions, const int* tok_slot, const int* tok_pos, void* k_pages, void* v_pages,
-                                const int* block_table, int max_pages, int heads, int kv_heads, int head_dim, int split_hint,
+                                const int* block_table, int max_pages, int heads, int kv_heads, int head_dim,
+                                const float* tok_cos, const float* tok_sin, const int* tok_page, int split_hint,
                                 float* workspace, size_t workspace_bytes, void* stream_ptr) {
   NNIS_REQUIRE(m > 0, "gemm_scaled: no tokens");
   NNIS_REQUIRE((uintptr_t)workspace % 16 == 0, "gemm_scaled: the workspace must be 16-byte aligned");
@@ -508,5 +524,6 @@ extern "C" int nnis_gemm_scaled(const void* scaled, const float* ss_parts, int p
   a.rope.q_out = (bf16_t*)y; a.rope.cos_table = cos_table; a.rope.sin_table = sin_table; a.rope.tok_slot = tok_slot; a.rope.tok_pos = tok_pos;
   a.rope.k_pages = (bf16_t*)k_pages; a.rope.v_pages = (bf16_t*)v_pages; a.rope.block_table = block_table; a.rope.max_pages = max_pages;
   a.rope.heads = heads; a.rope.kv_heads = kv_heads; a.rope.head_dim = head_dim;
+  a.rope.tok_cos = tok_cos; a.rope.tok_sin = tok_sin; a.rope.tok_page = tok_page;
   return run_fused(a, epilogue, table_positions, split_hint, workspace, workspace_bytes, (hipStream_t)stream_ptr);
 }

@@ -568,9 +568,9 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
       for (int i = 0; i < TM; ++i) {
         int token = row0 + wave_m * WM + i * 16 + r;
         token = token < m ? token : m - 1;
-        const int slot = y.rope.tok_slot[token];
+        const int slot = y.rope.tok_page ? 0 : y.rope.tok_slot[token];
         tok_pos[i] = y.rope.tok_pos[token];
-        tok_page[i] = (slot >= 0 && y.rope.k_pages) ? y.rope.block_table[(size_t)slot * y.rope.max_pages + tok_pos[i] / kPageTokens] : -1;
+        tok_page[i] = rope_page(y.rope, token, slot, tok_pos[i]);
       }
     }
   }
@@ -681,8 +681,8 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
           const int hd = y.rope.head_dim, head = first / hd, f0 = first % hd + 4 * g;
           epi_f32x4 c = {1.0f, 1.0f, 1.0f, 1.0f}, sn = {0.0f, 0.0f, 0.0f, 0.0f};
           if (head < y.rope.heads + y.rope.kv_heads) {
-            c = *(const epi_f32x4*)(y.rope.cos_table + (size_t)tok_pos[i] * (hd / 2) + f0);
-            sn = *(const epi_f32x4*)(y.rope.sin_table + (size_t)tok_pos[i] * (hd / 2) + f0);
+            c = *(const epi_f32x4*)(rope_cos_row(y.rope, token, tok_pos[i]) + f0);
+            sn = *(const epi_f32x4*)(rope_sin_row(y.rope, token, tok_pos[i]) + f0);
           }
           epilogue_rope(y.rope, token, tok_pos[i], head >= y.rope.heads ? tok_page[i] : -1, head, f0, lo, hi, c, sn);
         }
@@ -776,9 +776,9 @@ __global__ __launch_bounds__(256) void gemm_reduce_scaled_kernel(const float* __
   }
   int pos = 0, page = -1;
   if constexpr (EPI == EPI_ROPE) {
-    const int slot = y.rope.tok_slot[safe_token];
+    const int slot = y.rope.tok_page ? 0 : y.rope.tok_slot[safe_token];
     pos = y.rope.tok_pos[safe_token];
-    if (slot >= 0 && y.rope.k_pages) page = y.rope.block_table[(size_t)slot * y.rope.max_pages + pos / kPageTokens];
+    page = rope_page(y.rope, safe_token, slot, pos);
   }
   const int column = unit * 32 + quad * 4;  // the lower four; the upper four are 16 on
   const bool inside = token < m && column + 16 < width;
@@ -822,8 +822,8 @@ __global__ __launch_bounds__(256) void gemm_reduce_scaled_kernel(const float* __
     const int head = unit / per_head, f0 = (unit % per_head) * 16 + quad * 4;
     epi_f32x4 c = {1.0f, 1.0f, 1.0f, 1.0f}, sn = {0.0f, 0.0f, 0.0f, 0.0f};
     if (head < y.rope.heads + y.rope.kv_heads) {
-      c = *(const epi_f32x4*)(y.rope.cos_table + (size_t)pos * (hd / 2) + f0);
-      sn = *(const epi_f32x4*)(y.rope.sin_table + (size_t)pos * (hd / 2) + f0);
+      c = *(const epi_f32x4*)(rope_cos_row(y.rope, token, pos) + f0);
+      sn = *(const epi_f32x4*)(rope_sin_row(y.rope, token, pos) + f0);
     }
     epilogue_rope(y.rope, token, pos, head >= y.rope.heads ? page : -1, head, f0, lo, hi, c, sn);
   }

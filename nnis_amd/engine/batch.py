@@ -37,3 +37,16 @@ class StepContext:
     waves: int = 1  # waves of a block of the decode attention kernel (used when splits is given)
     plan_len: int = 0  # the length each mixer plans its decode kernels for, where it is not max_len (a captured step)
     tiles: dict = field(default_factory=dict)  # work lists of prefill kernels, by tile size, made on first use
+    tables: dict = field(default_factory=dict)  # the step's tables, made by the first layer that asks (``step_tables``)
+
+    def step_tables(self, rt, rotary=None, block_table=None):
+        """Each token's rows of the rotation tables ``rotary`` and its pages
+        in ``block_table``, gathered once a step (``ops.StepTables``): layers
+        that share a rotation and a cache group share the tables."""
+        key = (None if rotary is None else rotary.cos.data_ptr(), None if block_table is None else block_table.data_ptr())
+        made = self.tables.get(key)
+        if made is None:
+            made = self.tables[key] = rt.ops.step_tables(
+                self.tok_slot, self.tok_pos, self.tokens, rotary.cos if rotary is not None else None,
+                rotary.sin if rotary is not None else None, block_table, sequence_pages=self.decode)
+        return made

@@ -60,6 +60,7 @@ class DecodeGraph:
 
     def _forward(self) -> torch.Tensor:
         engine = self.engine
+        self.ctx.tables = {}  # the step's tables are made anew by every run (a capture must hold the kernel that makes them)
         return engine.model.forward(self.meta[0], self.ctx, engine.cache, self.rows[: self.padded], engine.rt)
 
     def capture(self) -> None:
@@ -202,6 +203,7 @@ class PrefillGraph:
 
     def _forward(self) -> torch.Tensor:
         engine = self.engine
+        self.ctx.tables = {}  # (as for the decode graphs)
         return engine.model.forward(self.ids, self.ctx, engine.cache, self.want_rows, engine.rt)
 
     def first_run(self):

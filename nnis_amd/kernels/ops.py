@@ -25,6 +25,7 @@ _U64 = ctypes.c_uint64
 _CORE_SIGNATURES = {
     "nnis_embed": [_VOID, _VOID, _INT, _VOID, _INT, _INT, _INT, _VOID],
     "nnis_embed_packed": [_VOID, _VOID, _VOID, _INT, _INT, _INT, _VOID],
+    "nnis_step_tables": [_VOID, _VOID, _INT, _VOID, _VOID, _INT, _INT, _VOID, _INT, _VOID, _VOID, _VOID, _VOID, _VOID],
     "nnis_rmsnorm": [_VOID, _INT, _VOID, _INT, _VOID, _INT, _VOID, _INT, _VOID, _INT, _INT, _FLT, _VOID],
     "nnis_rope_kv_write": [_VOID, _INT, _VOID, _INT, _VOID, _VOID, _INT, _INT, _VOID, _VOID, _VOID, _VOID, _INT,
                            _VOID, _INT, _INT, _INT, _INT, _INT, _VOID],
@@ -35,11 +36,11 @@ _CORE_SIGNATURES = {
     "nnis_gemm_ordered": [_VOID, _INT, _VOID, _INT, _VOID, _INT, _INT, _INT, _INT, _VOID],
     "nnis_gemm_bf16": [_VOID, _VOID, _VOID, _INT, _INT, _INT, _INT, _INT, _VOID, _SIZE, _VOID],
     "nnis_gemm_fused": [_VOID, _VOID, _VOID, _VOID, _INT, _FLT, _VOID, _INT, _INT, _INT, _INT, _VOID, _VOID, _VOID, _INT,
-                        _VOID, _VOID, _VOID, _VOID, _VOID, _INT, _INT, _INT, _INT, _INT, _VOID],
+                        _VOID, _VOID, _VOID, _VOID, _VOID, _INT, _INT, _INT, _INT, _VOID, _VOID, _VOID, _INT, _VOID],
     "nnis_gemm_residual_parts": [_INT, _INT],
     "nnis_gemm_residual": [_VOID, _VOID, _VOID, _VOID, _INT, _VOID, _VOID, _INT, _INT, _INT, _INT, _VOID, _VOID, _SIZE, _VOID],
     "nnis_gemm_scaled": [_VOID, _VOID, _INT, _FLT, _VOID, _INT, _INT, _INT, _INT, _VOID, _VOID, _VOID, _INT, _VOID, _VOID,
-                         _VOID, _VOID, _VOID, _INT, _INT, _INT, _INT, _INT, _VOID, _SIZE, _VOID],
+                         _VOID, _VOID, _VOID, _INT, _INT, _INT, _INT, _VOID, _VOID, _VOID, _INT, _VOID, _SIZE, _VOID],
     "nnis_gemm_residual_runs_fits": [_INT, _INT, _INT, _INT, _INT],
     "nnis_gemm_residual_runs": [_VOID, _INT, _INT, _INT, _VOID, _VOID, _VOID, _VOID, _INT, _VOID, _VOID, _INT, _INT, _INT, _VOID,
                                 _VOID],
@@ -54,7 +55,7 @@ _ATTN_SIGNATURES = {
                                     _INT, _INT, _INT, _FLT, _INT, _INT, _VOID],
     "nnis_attention_prefill_max_waves": [_INT, _INT, _INT],
     "nnis_attention_decode_bf16": [_VOID, _VOID, _VOID, _VOID, _VOID, _INT, _VOID, _VOID, _INT, _INT, _INT, _INT, _INT, _FLT,
-                                   _INT, _INT, _VOID, _INT, _INT, _VOID],
+                                   _INT, _INT, _VOID, _INT, _INT, _INT, _VOID],
     "nnis_attention_combine": [_VOID, _VOID, _VOID, _INT, _INT, _INT, _INT, _VOID],
     "nnis_attention_decode_max_waves": [_INT, _INT],
 }
@@ -282,6 +283,52 @@ def gemm_ordered(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.T
     return out
 
 
+class StepTables:
+    """What a step's kernels would look up through each token's slot and
+    position, gathered once by token (``step_tables``): ``cos`` / ``sin``
+    float32 [tokens, rot_dim / 2], each token's rows of the rotation tables;
+    ``page`` int32 [tokens], the cache page of each token's position (-1 for a
+    padding row); ``pages`` int32 [tokens, pages a slot may hold], for a step
+    of single tokens the pages of each token's sequence up to its position.
+    Any of them is None where it was not asked for."""
+
+    def __init__(self, tokens, cos=None, sin=None, page=None, pages=None):
+        self.tokens, self.cos, self.sin, self.page, self.pages = tokens, cos, sin, page, pages
+
+
+def step_tables(tok_slot: torch.Tensor, tok_pos: torch.Tensor, tokens: int, cos: Optional[torch.Tensor] = None,
+                sin: Optional[torch.Tensor] = None, block_table: Optional[torch.Tensor] = None,
+                sequence_pages: bool = False) -> StepTables:
+    """One kernel at the start of a step; see ``StepTables``.  ``cos`` / ``sin``:
+    rotation tables [positions, half]; ``block_table``: int32 [slots, pages];
+    ``sequence_pages``: also each token's sequence's pages (a decode step)."""
+    _dev(tok_slot, "tok_slot"), _dev(tok_pos, "tok_pos")
+    if tok_slot.dtype != torch.int32 or tok_pos.dtype != torch.int32 or min(tok_slot.numel(), tok_pos.numel()) < tokens:
+        raise KernelError("step_tables: tok_slot / tok_pos must be int32 with one entry per token")
+    out = StepTables(tokens)
+    half = positions = max_pages = 0
+    if cos is not None:
+        _dev(cos, "cos"), _dev(sin, "sin")
+        if cos.dtype != torch.float32 or sin.dtype != torch.float32 or cos.shape != sin.shape or cos.dim() != 2:
+            raise KernelError("step_tables: rotation tables must be float32 [positions, half]")
+        positions, half = cos.shape
+        out.cos = torch.empty((tokens, half), dtype=torch.float32, device=cos.device)
+        out.sin = torch.empty((tokens, half), dtype=torch.float32, device=cos.device)
+    if block_table is not None:
+        _dev(block_table, "block_table")
+        if block_table.dtype != torch.int32 or block_table.dim() != 2:
+            raise KernelError("step_tables: block_table must be int32 [slots, pages]")
+        max_pages = block_table.shape[1]
+        out.page = torch.empty(tokens, dtype=torch.int32, device=block_table.device)
+        if sequence_pages:
+            out.pages = torch.empty((tokens, max_pages), dtype=torch.int32, device=block_table.device)
+    lib = core()
+    _check(lib, lib.nnis_step_tables(tok_slot.data_ptr(), tok_pos.data_ptr(), tokens, _ptr(cos), _ptr(sin), half, positions,
+                                     _ptr(block_table), max_pages, _ptr(out.cos), _ptr(out.sin), _ptr(out.page),
+                                     _ptr(out.pages), _stream()))
+    return out
+
+
 def attention_rows(q: torch.Tensor, out: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
                    block_table: torch.Tensor, tok_slot: torch.Tensor, tok_pos: torch.Tensor, heads: int, kv_heads: int,
                    head_dim: int, scale: float, window: int = 0) -> torch.Tensor:
@@ -431,8 +478,16 @@ def gemm_fused(x_in: torch.Tensor, delta: Optional[torch.Tensor], x_out: Optiona
         float(eps), w.data_ptr(), m, n, k, int(epilogue), y.data_ptr(), _ptr(r.get("cos")), _ptr(r.get("sin")),
         r["cos"].shape[0] if r.get("cos") is not None else 0, _ptr(r.get("tok_slot")), _ptr(r.get("tok_pos")),
         _ptr(r.get("k_pages")), _ptr(r.get("v_pages")), _ptr(bt), bt.shape[1] if bt is not None else 0,
-        r.get("heads", 0), r.get("kv_heads", 0), r.get("head_dim", 0), int(split), _stream()))
+        r.get("heads", 0), r.get("kv_heads", 0), r.get("head_dim", 0), *_step_table_pointers(r), int(split), _stream()))
     return y
+
+
+def _step_table_pointers(rope: dict):
+    """(tok_cos, tok_sin, tok_page) of a rotating epilogue's ``tables`` (a ``StepTables``), or three nulls."""
+    tables = rope.get("tables")
+    if tables is None or tables.cos is None or tables.page is None:
+        return None, None, None
+    return tables.cos.data_ptr(), tables.sin.data_ptr(), tables.page.data_ptr()
 
 
 def _check_epilogue(what: str, m: int, n: int, y: torch.Tensor, epilogue: int, rope: Optional[dict]) -> dict:
@@ -447,6 +502,11 @@ def _check_epilogue(what: str, m: int, n: int, y: torch.Tensor, epilogue: int, r
             raise KernelError(f"{what}: rotation tables must be float32 [positions, head_dim / 2]")
         if r["tok_slot"].dtype != torch.int32 or r["tok_pos"].dtype != torch.int32 or min(r["tok_slot"].numel(), r["tok_pos"].numel()) < m:
             raise KernelError(f"{what}: tok_slot / tok_pos must be int32 with one entry per token")
+        tables = r.get("tables")
+        if tables is not None and tables.cos is not None:
+            if (tables.tokens < m or tables.cos.shape[1] != r["head_dim"] // 2 or tables.cos.dtype != torch.float32
+                    or (r.get("k_pages") is not None and tables.page is None)):
+                raise KernelError(f"{what}: the step's tables do not fit {m} tokens with heads of {r['head_dim']}")
         if r.get("k_pages") is not None:
             kp, vp, bt = r["k_pages"], r["v_pages"], r["block_table"]
             _dev(kp, "k_pages"), _dev(vp, "v_pages"), _dev(bt, "block_table")
@@ -527,7 +587,7 @@ def gemm_scaled(scaled: torch.Tensor, ss: torch.Tensor, parts: int, eps: float, 
         scaled.data_ptr(), ss.data_ptr(), int(parts), float(eps), w.data_ptr(), m, n, k, int(epilogue), y.data_ptr(),
         _ptr(r.get("cos")), _ptr(r.get("sin")), r["cos"].shape[0] if r.get("cos") is not None else 0, _ptr(r.get("tok_slot")),
         _ptr(r.get("tok_pos")), _ptr(r.get("k_pages")), _ptr(r.get("v_pages")), _ptr(bt), bt.shape[1] if bt is not None else 0,
-        r.get("heads", 0), r.get("kv_heads", 0), r.get("head_dim", 0), int(split), _ptr(work),
+        r.get("heads", 0), r.get("kv_heads", 0), r.get("head_dim", 0), *_step_table_pointers(r), int(split), _ptr(work),
         GEMM_WORKSPACE_BYTES if work is not None else 0, _stream()))
     return y
 
@@ -592,7 +652,7 @@ def attention_prefill_bf16(q, out, k_pages, v_pages, block_table, tile_seq, tile
 
 
 def attention_decode_bf16(q, out, k_pages, v_pages, block_table, tok_slot, tok_pos, heads, kv_heads, head_dim, scale,
-                          window=0, splits=1, partial=None, waves=1, kernel="auto", keep_runs=False):
+                          window=0, splits=1, partial=None, waves=1, kernel="auto", keep_runs=False, token_pages=None):
     """One query token per sequence over its cached keys.  The keys are cut
     into ``splits`` runs, each a block of ``waves`` waves that deal its pages
     among themselves and merge in LDS; the runs are summed by a second kernel.
@@ -603,9 +663,17 @@ def attention_decode_bf16(q, out, k_pages, v_pages, block_table, tok_slot, tok_p
     up itself (``gemm_residual``), or ``KeyRuns.combine()`` does.  ``kernel``:
     "keys" (keys on lanes; groups of up to 4 heads of up to 128 channels),
     "columns" (heads in the columns of a tile; any group the head size
-    carries) or "auto", which takes "keys" where it fits."""
+    carries) or "auto", which takes "keys" where it fits.  ``token_pages``
+    (int32 [tokens, pages], ``StepTables.pages``): each token's sequence's
+    pages, read in place of the block table's row of the token's slot."""
     _check_pages(q, out, k_pages, v_pages, block_table, heads, kv_heads, head_dim)
     tokens = q.shape[0]
+    table = block_table
+    if token_pages is not None:
+        _dev(token_pages, "token_pages")
+        if token_pages.dtype != torch.int32 or token_pages.dim() != 2 or token_pages.shape[0] < tokens:
+            raise KernelError("attention: token_pages must be int32 [tokens, pages]")
+        table = token_pages
     for t in (tok_slot, tok_pos):
         _dev(t, "step metadata")
         if t.dtype != torch.int32 or t.numel() < tokens:
@@ -616,10 +684,11 @@ def attention_decode_bf16(q, out, k_pages, v_pages, block_table, tok_slot, tok_p
         _dev(partial, "partial")
     lib = attention_module(head_dim)
     _check(lib, lib.nnis_attention_decode_bf16(q.data_ptr(), out.data_ptr(), k_pages.data_ptr(), v_pages.data_ptr(),
-                                               block_table.data_ptr(), block_table.shape[1], tok_slot.data_ptr(),
+                                               table.data_ptr(), table.shape[1], tok_slot.data_ptr(),
                                                tok_pos.data_ptr(), tokens, heads, kv_heads, head_dim, int(window),
                                                float(scale), int(splits), int(waves), _ptr(partial) if splits > 1 else None,
-                                               _DECODE_KERNELS[kernel], 0 if (keep_runs and splits > 1) else 1, _stream()))
+                                               _DECODE_KERNELS[kernel], 0 if (keep_runs and splits > 1) else 1,
+                                               1 if token_pages is not None else 0, _stream()))
     if keep_runs and splits > 1:
         return KeyRuns(partial, int(splits), tokens, heads, head_dim, tok_slot, out)
     return out
@@ -784,7 +853,7 @@ def _prefill_tiles(ctx, rows: int, device):
 
 
 def attention(q: torch.Tensor, out: torch.Tensor, view, ctx, heads: int, kv_heads: int, head_dim: int, scale: float,
-              window: int = 0, keep_runs: bool = False):
+              window: int = 0, keep_runs: bool = False, tables: Optional[StepTables] = None):
     """Attention of the step's tokens over the cache ``view``: bfloat16 with a
     head size in steps of 16 runs on the matrix cores (one kernel for single
     tokens, one for runs of tokens); anything else takes the 32-bit kernel.
@@ -802,7 +871,8 @@ def attention(q: torch.Tensor, out: torch.Tensor, view, ctx, heads: int, kv_head
             partial = decode_scratch(q.device, q.shape[0] * heads * splits * (head_dim + 4))
         return attention_decode_bf16(q, out, view.k_pages, view.v_pages, view.block_table, ctx.tok_slot, ctx.tok_pos, heads,
                                      kv_heads, head_dim, scale, window, splits, partial, waves,
-                                     keep_runs=keep_runs and q.shape[0] <= KEY_RUNS_MOST_TOKENS)
+                                     keep_runs=keep_runs and q.shape[0] <= KEY_RUNS_MOST_TOKENS,
+                                     token_pages=tables.pages if tables is not None else None)
     if fast and not ctx.decode:
         # A tile's keys are a chain of dependent loads: the longest tile sets the kernel's time.  The waves of
         # a block deal the keys among themselves (their merge lives in LDS).

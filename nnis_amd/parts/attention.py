@@ -74,6 +74,7 @@ class CausalSelfAttention(Mixer):
                     and self.head_dim % 32 == 0 and view.k_pages.dtype == torch.bfloat16):
                 # residual sum, norm, the three projections, the rotation and the cache write in one kernel
                 rope = dict(cos=tables.cos, sin=tables.sin, tok_slot=ctx.tok_slot, tok_pos=ctx.tok_pos,
+                            tables=ctx.step_tables(rt, tables, view.block_table),
                             k_pages=view.k_pages if writes else None, v_pages=view.v_pages if writes else None,
                             block_table=view.block_table if writes else None, heads=self.heads,
                             kv_heads=self.kv_heads, head_dim=self.head_dim)
@@ -96,8 +97,11 @@ class CausalSelfAttention(Mixer):
         tokens = q.shape[0]
         attn = rt.empty(tokens, self.heads * self.head_dim)
         # a decode step over long sequences leaves its runs of keys to the output projection, if that takes them
+        step = None
+        if ctx.decode and q.dtype == torch.bfloat16:
+            step = ctx.step_tables(rt, self.position.rotary() if self.position is not None else None, view.block_table)
         attn = rt.ops.attention(q, attn, view, ctx, self.heads, self.kv_heads, self.head_dim, self.scale, self.window or 0,
-                                keep_runs=into is not None)
+                                keep_runs=into is not None, tables=step)
         if isinstance(attn, rt.ops.KeyRuns) and not (into.can_take(attn, self.out.weight) and attn.fits(self.out.weight.shape[0])):
             attn = attn.combine()
         if into is not None and into.can_take(attn, self.out.weight):

@@ -392,6 +392,67 @@ def test_attention_beyond_64_pages(heads, kv_heads, head_dim):
         assert (got[-1, far_head] - vs[0][4230, kv_heads - 1]).abs().max().item() < 0.05
 
 
+def test_step_tables_and_the_kernels_that_read_them():
+    """The step's tables against plain indexing, padding rows included; the decode attention reading each token's
+    pages from them gives what it gives through slots and the block table; the rotating projection that takes
+    rotation rows and pages from them writes the same queries and the same cache."""
+    ops = _ops()
+    torch.manual_seed(11)
+    heads, kv_heads, head_dim = 6, 2, 64
+    half = head_dim // 2
+    lengths = [300, 70, 1, 129]
+    ks = [torch.randn(n, kv_heads, head_dim).bfloat16().float() for n in lengths]
+    vs = [torch.randn(n, kv_heads, head_dim).bfloat16().float() for n in lengths]
+    k_pages, v_pages, table = _paged(ks, vs, torch.bfloat16, kv_heads, head_dim)
+    cos, sin = (torch.from_numpy(t).cuda() for t in P.rope_tables(512, head_dim, 10000.0))
+    slots, positions = [2, -1, 0, 3, 1, -1], [0, 0, 299, 128, 69, 0]
+    tables = ops.step_tables(_i32(slots), _i32(positions), len(slots), cos, sin, table, sequence_pages=True)
+    host_table = table.cpu()
+    for row, (slot, pos) in enumerate(zip(slots, positions)):
+        if slot < 0:
+            assert tables.page[row].item() == -1 and tables.pages[row, 0].item() == 0
+            assert bool((tables.cos[row] == 1).all()) and bool((tables.sin[row] == 0).all())
+            continue
+        assert torch.equal(tables.cos[row], cos[pos]) and torch.equal(tables.sin[row], sin[pos])
+        assert tables.page[row].item() == host_table[slot, pos // 64].item()
+        assert torch.equal(tables.pages[row, :pos // 64 + 1].cpu(), host_table[slot, :pos // 64 + 1])
+    only_pages = ops.step_tables(_i32(slots), _i32(positions), len(slots), block_table=table)
+    assert only_pages.cos is None and only_pages.pages is None and torch.equal(only_pages.page, tables.page)
+
+    scale = 1.0 / math.sqrt(head_dim)
+    q = torch.randn(len(slots), heads * head_dim).bfloat16().cuda()
+    for kernel in ("keys", "columns"):
+        for splits, waves in ((1, 1), (4, 2)):
+            outs = []
+            for token_pages in (None, tables.pages):
+                out = torch.zeros(len(slots), heads * head_dim, dtype=torch.bfloat16, device="cuda")
+                partial = torch.zeros(len(slots) * heads * splits * (head_dim + 4), dtype=torch.float32, device="cuda")
+                ops.attention_decode_bf16(q, out, k_pages, v_pages, table, _i32(slots), _i32(positions), heads, kv_heads, head_dim,
+                                          scale, 0, splits, partial, waves, kernel, token_pages=token_pages)
+                outs.append(out.cpu())
+            live = [i for i, s in enumerate(slots) if s >= 0]
+            assert torch.equal(outs[0][live], outs[1][live]), (kernel, splits, waves)
+
+    # the rotating projection: 6 tokens, one a padding row, written at the positions above
+    m, k, eps = len(slots), 96, 1e-5
+    n = (heads + 2 * kv_heads) * head_dim
+    x = torch.randn(m, k)
+    gain = (1 + 0.1 * torch.randn(k)).bfloat16()
+    w = ops.pack_weight((torch.randn(n, k) / math.sqrt(k)).bfloat16().cuda())
+    results = []
+    for with_tables in (False, True):
+        kp, vp = k_pages.clone(), v_pages.clone()
+        rope = dict(cos=cos, sin=sin, tok_slot=_i32(slots), tok_pos=_i32(positions), k_pages=kp, v_pages=vp, block_table=table,
+                    heads=heads, kv_heads=kv_heads, head_dim=head_dim, tables=tables if with_tables else None)
+        y = torch.zeros(m, heads * head_dim, dtype=torch.bfloat16, device="cuda")
+        ops.gemm_fused(x.cuda(), None, None, gain.cuda(), eps, w, y, ops.EPILOGUE_ROPE, rope)
+        results.append((y.cpu(), kp.cpu(), vp.cpu()))
+    live = [i for i, s in enumerate(slots) if s >= 0]
+    assert torch.equal(results[0][0][live], results[1][0][live])
+    assert torch.equal(results[0][1], results[1][1]) and torch.equal(results[0][2], results[1][2])
+    assert not torch.equal(results[1][1], k_pages.cpu())  # and the cache was written
+
+
 @pytest.mark.parametrize("hint", [32, 48])
 def test_gemm_tiled_over_many_blocks(hint):
     """Both tiles of the tiled kernel over a grid of hundreds of blocks in
