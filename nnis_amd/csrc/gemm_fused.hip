@@ -81,7 +81,7 @@ __device__ __forceinline__ void load_gain8(const void* base, int dtype, int inde
   }
 }
 
-template <int MT, int KSPLIT, int EPI, bool PREP>
+template <int MT, int KSPLIT, int EPI, bool PREP, bool DEAL = false>
 __global__ __launch_bounds__(KSPLIT > 4 ? 64 * KSPLIT : 256) void gemm_fused_kernel(FusedArgs a, int tiles) {
   constexpr bool PAIR = EPI != EPI_STORE;
   constexpr int NACC = PAIR ? 2 : 1;
@@ -128,6 +128,17 @@ __global__ __launch_bounds__(KSPLIT > 4 ? 64 * KSPLIT : 256) void gemm_fused_ker
   constexpr int kPartRegs = 8;  // parts of a row's sum of squares a lane keeps in flight (4 lane groups share a row)
   float ss_held[MT][kPartRegs];
   const bool ends_unit = active && part == 0;
+  // The parts of a prepared row's sum of squares: a narrow row's few (up to 64) are all asked for by the lane
+  // groups of the wave that ends the unit, eight in flight each.  DEAL: a wide row's (a hundred and more) are
+  // dealt to the lane groups of all the waves that share the unit's K, so that they are one round trip too and
+  // not a chain of them (2048 columns, 8 tokens: the gate/up product 24.9 -> 16 us, the QKV product 14.2 -> 9).
+  // The waves' sums meet in LDS with the products' (part_ss), the lane groups' in the shuffles below.  A
+  // variant of its own: on narrow rows the dealing, and even its code beside the other, was measured slower
+  // (576 columns: a decode step of 30 layers 0.896 and 0.882 against 0.859 ms).
+  static_assert(!DEAL || (PREP && KSPLIT > 1), "parts are dealt among the waves that share a prepared operand's K");
+  const bool takes_parts = DEAL ? active : ends_unit;
+  const int part_first = g + (DEAL ? 4 * part : 0);
+  constexpr int part_stride = DEAL ? 4 * KSPLIT : 4;
   const bool tables = EPI == EPI_ROPE && a.rope.tok_cos != nullptr;  // the step's tables: nothing hangs on a loaded value
   if (EPI == EPI_ROPE && ends_unit) {
     const int head = row0 / a.rope.head_dim;
@@ -162,14 +173,13 @@ __global__ __launch_bounds__(KSPLIT > 4 ? 64 * KSPLIT : 256) void gemm_fused_ker
           tok_page[t] = a.rope.block_table[(size_t)tok_slot[t] * a.rope.max_pages + tok_pos[t] / kPageTokens];
       }
     }
-    if (PREP && ends_unit) {
-      // lane group g takes every fourth part; the groups are added with the sums of squares below
+    if (PREP && takes_parts) {
 #pragma unroll
       for (int t = 0; t < MT; ++t) {
         const int token = token0 + t * 16 + r;
 #pragma unroll
         for (int i = 0; i < kPartRegs; ++i) {
-          const int p = g + 4 * i;
+          const int p = part_first + part_stride * i;
           ss_held[t][i] = (token < m && p < a.parts) ? a.ss_parts[(size_t)p * m + token] : 0.0f;
         }
       }
@@ -200,6 +210,7 @@ __global__ __launch_bounds__(KSPLIT > 4 ? 64 * KSPLIT : 256) void gemm_fused_ker
     }
     const bool writes_x = !PREP && a.delta != nullptr && unit == 0;  // the first unit's waves cover every k once
     const bool gain_f32 = a.norm_w_dtype == NNIS_F32;
+    if (DEAL && part >= chunks) dependent();  // a wave without a share of K still takes its share of the parts
     if constexpr (PREP) {
       for (int base = part; base < chunks; base += KSPLIT * DEPTH) {
         bf16x8 wa[DEPTH][2], wb[DEPTH][2], xs[DEPTH][2][MT];
@@ -317,14 +328,28 @@ __global__ __launch_bounds__(KSPLIT > 4 ? 64 * KSPLIT : 256) void gemm_fused_ker
         }
     }
   }
-  if (PREP && ends_unit) {
+  if (PREP && takes_parts) {
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
 #pragma unroll
       for (int i = 0; i < kPartRegs; ++i) ss[t] += ss_held[t][i];
       const int token = token0 + t * 16 + r;
-      if (token < m)
-        for (int p = g + 4 * kPartRegs; p < a.parts; p += 4) ss[t] += a.ss_parts[(size_t)p * m + token];  // wide rows
+      if (token < m) {  // more parts than the lanes that take them hold at once
+        if constexpr (DEAL) {  // eight more at a time
+          for (int p0 = part_first + part_stride * kPartRegs; p0 < a.parts; p0 += part_stride * kPartRegs) {
+            float more[kPartRegs];
+#pragma unroll
+            for (int i = 0; i < kPartRegs; ++i) {
+              const int p = p0 + part_stride * i;
+              more[i] = p < a.parts ? a.ss_parts[(size_t)p * m + token] : 0.0f;
+            }
+#pragma unroll
+            for (int i = 0; i < kPartRegs; ++i) ss[t] += more[i];
+          }
+        } else {
+          for (int p = g + 4 * kPartRegs; p < a.parts; p += 4) ss[t] += a.ss_parts[(size_t)p * m + token];
+        }
+      }
     }
   }
   // a token's sum of squares: over the four lane groups of this wave, then over the waves that share K
@@ -387,6 +412,8 @@ __global__ __launch_bounds__(KSPLIT > 4 ? 64 * KSPLIT : 256) void gemm_fused_ker
   }
 }
 
+constexpr int kDealPartsFrom = 64;  // rows of more parts than this take the variant that deals them to all waves
+
 template <int MT, int KSPLIT, int EPI>
 void launch_fused(const FusedArgs& a, int units, hipStream_t stream) {
   constexpr int kWaves = KSPLIT > 4 ? KSPLIT : 4;
@@ -394,6 +421,12 @@ void launch_fused(const FusedArgs& a, int units, hipStream_t stream) {
   const int unit_blocks = (units + kUnits - 1) / kUnits;
   const int tiles = (a.m + 16 * MT - 1) / (16 * MT);
   const dim3 grid(tiles == 1 ? unit_blocks : (unit_blocks + 7) / 8 * 8 * tiles), block(64 * kWaves);
+  if constexpr (KSPLIT > 1) {
+    if (a.scaled && a.parts > kDealPartsFrom) {
+      hipLaunchKernelGGL((gemm_fused_kernel<MT, KSPLIT, EPI, true, true>), grid, block, 0, stream, a, tiles);
+      return;
+    }
+  }
   if (a.scaled) hipLaunchKernelGGL((gemm_fused_kernel<MT, KSPLIT, EPI, true>), grid, block, 0, stream, a, tiles);
   else hipLaunchKernelGGL((gemm_fused_kernel<MT, KSPLIT, EPI, false>), grid, block, 0, stream, a, tiles);
 }
