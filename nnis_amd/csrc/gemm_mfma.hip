@@ -552,15 +552,28 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
     static_assert(BM == 64, "a lane per row of the tile");
     const int token = row0 + lane < m ? row0 + lane : m - 1;
     float total = 0.0f;
-    for (int p0 = wave; p0 < y.parts; p0 += 32) {
-      float part[8];
+    if (y.parts <= 32) {
+      for (int p0 = wave; p0 < y.parts; p0 += 32) {
+        float part[8];
 #pragma unroll
-      for (int u = 0; u < 8; ++u) {
-        const int p = p0 + 4 * u;
-        part[u] = y.ss_parts[(size_t)(p < y.parts ? p : y.parts - 1) * m + token];
+        for (int u = 0; u < 8; ++u) {
+          const int p = p0 + 4 * u;
+          part[u] = y.ss_parts[(size_t)(p < y.parts ? p : y.parts - 1) * m + token];
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) total += p0 + 4 * u < y.parts ? part[u] : 0.0f;
       }
+    } else {  // a wide row that the kernel for few tokens prepared (a part per 16 columns): 32 loads at a time
+      for (int p0 = wave; p0 < y.parts; p0 += 128) {
+        float part[32];
 #pragma unroll
-      for (int u = 0; u < 8; ++u) total += p0 + 4 * u < y.parts ? part[u] : 0.0f;
+        for (int u = 0; u < 32; ++u) {
+          const int p = p0 + 4 * u;
+          part[u] = y.ss_parts[(size_t)(p < y.parts ? p : y.parts - 1) * m + token];
+        }
+#pragma unroll
+        for (int u = 0; u < 32; ++u) total += p0 + 4 * u < y.parts ? part[u] : 0.0f;
+      }
     }
     row_scale[wave][lane] = total;
     if constexpr (EPI == EPI_ROPE) {
