@@ -216,3 +216,46 @@ def test_whole_model_invariants(model_dirs, name):
     # tied head: the embedding stands in
     if model.tied:
         assert "lm_head.weight" not in model.w
+
+
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_whole_model_from_library_routines(model_dirs, name):
+    """The same model put together a second time from the library's own
+    routines, each with its defaults: ``rms_norm`` (eps inside the root, a
+    mean), ``scaled_dot_product_attention`` (causal, its default scale
+    1/sqrt(head size), grouped heads by repetition), ``silu``, and a rotation
+    written as a complex product.  A scale taken before the dot product or
+    left out, a norm with eps outside the root, a gate without its
+    activation or heads grouped the other way round would all miss this."""
+    import torch.nn.functional as F
+
+    model = P.PlainLlama(model_dirs[name], torch.float64)
+    w, t = model.w, 29
+    torch.manual_seed(5)
+    ids = torch.randint(0, model.V, (t,))
+    x = F.embedding(ids, w["model.embed_tokens.weight"])
+    half = model.hd // 2
+    inv_freq = 1.0 / model.theta ** (torch.arange(half, dtype=torch.float64) * 2 / model.hd)
+    turn = torch.polar(torch.ones(t, half, dtype=torch.float64), torch.arange(t, dtype=torch.float64)[:, None] * inv_freq)
+
+    def rotate(v):  # [t, heads, hd]: (v[j] + i v[j + half]) * exp(i pos inv_freq_j)
+        z = torch.complex(v[..., :half], v[..., half:]) * turn[:, None, :]
+        return torch.cat([z.real, z.imag], -1)
+
+    for layer in range(model.L):
+        p = f"model.layers.{layer}."
+        h = F.rms_norm(x, (model.H,), w[p + "input_layernorm.weight"], model.eps)
+        q = rotate(F.linear(h, w[p + "self_attn.q_proj.weight"]).view(t, model.nh, model.hd))
+        k = rotate(F.linear(h, w[p + "self_attn.k_proj.weight"]).view(t, model.nkv, model.hd))
+        v = F.linear(h, w[p + "self_attn.v_proj.weight"]).view(t, model.nkv, model.hd)
+        group = model.nh // model.nkv
+        k, v = k.repeat_interleave(group, dim=1), v.repeat_interleave(group, dim=1)
+        attn = F.scaled_dot_product_attention(q.transpose(0, 1), k.transpose(0, 1), v.transpose(0, 1), is_causal=True)
+        x = x + F.linear(attn.transpose(0, 1).reshape(t, model.nh * model.hd), w[p + "self_attn.o_proj.weight"])
+        h = F.rms_norm(x, (model.H,), w[p + "post_attention_layernorm.weight"], model.eps)
+        x = x + F.linear(F.silu(F.linear(h, w[p + "mlp.gate_proj.weight"])) * F.linear(h, w[p + "mlp.up_proj.weight"]),
+                         w[p + "mlp.down_proj.weight"])
+    want = F.linear(F.rms_norm(x, (model.H,), w["model.norm.weight"], model.eps), model.lm_head_weight())
+    got = model.logits(ids.tolist())
+    # the rotation table is built in 32-bit as the reference builds it; in 64-bit here: angles differ by rounding
+    assert (got - want).abs().max().item() < 5e-6, (got - want).abs().max().item()
