@@ -534,3 +534,40 @@ def test_a_tied_head_keeps_the_table_once(model_dirs):
     assert isinstance(untied.embedding.table, torch.Tensor) and isinstance(untied.head.projection.weight, PackedWeight)
     wide, _ = load_model(model_dirs["A"], dtype="float32")
     assert wide.embedding.table.data_ptr() == wide.head.projection.weight.data_ptr()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_sequence_cut_back_goes_on_from_there(model_dirs, dtype):
+    """``truncate`` as the reference uses it to take back tokens a step ran
+    (/root/reference/crates/nnis-rt/src/kv_cache.rs:174-192): the sequence is
+    shortened across a page's edge and inside a page, goes on with other
+    tokens (in a prompt step and one token at a time, replayed from graphs in
+    bfloat16), and its logits are those of the sequence it now is."""
+    from nnis_amd.engine.batch import StepEntry
+
+    config, seed = TINY_CONFIGS["B"]
+    rng = np.random.default_rng(70 + seed)
+    first = rng.integers(0, config["vocab_size"], size=200).tolist()
+    plain = P.PlainLlama(model_dirs["B"])
+    yard = _yard(model_dirs, "B")
+    engine = _engine(model_dirs, "B", dtype, max_tokens=8 * 64)
+    slot, other = engine.start_sequence(), engine.start_sequence()
+    engine.step([StepEntry(slot, first[:190], []), StepEntry(other, first[:3], [])])
+    for token in first[190:]:
+        engine.step([StepEntry(slot, [token], [0])])
+    free = engine.free_pages()
+    engine.truncate(slot, 70)  # 4 pages -> 2
+    assert engine.length(slot) == 70 and engine.free_pages() == free + 2 and engine.length(other) == 3
+    second = first[:70] + rng.integers(0, config["vocab_size"], size=40).tolist()
+    want = plain.logits(second)
+    rows = engine.step([StepEntry(slot, second[70:100], list(range(30)))])
+    _close(rows.cpu(), want[70:100], dtype, "continued in one step", yard)
+    rows = torch.cat([engine.step([StepEntry(slot, [token], [0])]) for token in second[100:]])
+    _close(rows.cpu(), want[100:], dtype, "continued one by one", yard)
+    engine.truncate(slot, 100)  # inside its second page: no page moves
+    third = second[:100] + [5, 6, 7]
+    rows = torch.cat([engine.step([StepEntry(slot, [token], [0])]) for token in third[100:]])
+    _close(rows.cpu(), plain.logits(third)[100:], dtype, "cut back inside a page", yard)
+    engine.reset(slot)
+    rows = engine.step([StepEntry(slot, first[:5], [4])])
+    _close(rows.cpu(), plain.logits(first[:5])[4:5], dtype, "reset and used again", yard)

@@ -599,3 +599,163 @@ def test_toy_architecture_with_windowed_layers(tmp_path, dtype):
     for i in range(124, 150):  # alone, over the edge of the second page
         rows = engine.step([StepEntry(sa, [a[i]], [0])]).cpu()
         assert_close(rows[0], want_a[i], dtype, f"windowed decode a {i}")
+
+
+# ---------------------------------------------------------------------------
+# a fourth toy architecture: attention whose values are narrower than its keys
+# (a cache need of its own shape), with a bias drawn by an init rule the test
+# registers, a plan of its own for steps of single tokens, and a sequence that
+# is cut back and goes on differently
+# ---------------------------------------------------------------------------
+
+def _register_narrow():
+    from nnis_amd.cache.layout import k_offset, v_offset
+    from nnis_amd.config import register_architecture
+    from nnis_amd.models import ModelSpec, ScheduleEntry
+    from nnis_amd.parts import Mixer, TensorSpec, register_part
+    from nnis_amd.parts.base import KVRequest
+    from nnis_amd.weights import register_init_rule
+
+    register_init_rule("toy_tenth", lambda spec, generator, dtype: torch.full(tuple(spec.shape), 0.1, dtype=dtype), replace=True)
+    KD, VD = 32, 16
+    k_index = torch.tensor([[k_offset(t, c) for c in range(KD)] for t in range(64)])
+    v_index = torch.tensor([[v_offset(c, t) for c in range(VD)] for t in range(64)])
+
+    class NarrowValueAttention(Mixer):
+        """One head, no rotation: y = W_o softmax(q k^T / sqrt(32)) v + bias, keys of 32 channels, values of 16."""
+
+        planned = []  # what decode_plan was asked (the engine asks it only where steps are replayed from graphs)
+
+        def __init__(self, width, q, k, v, o, bias):
+            self.width, self.names, self.w = width, dict(q=q, k=k, v=v, o=o, bias=bias), None
+
+        def tensors(self):
+            n, w = self.names, self.width
+            return [TensorSpec(n["q"], (KD, w)), TensorSpec(n["k"], (KD, w)), TensorSpec(n["v"], (VD, w)),
+                    TensorSpec(n["o"], (w, VD)), TensorSpec(n["bias"], (w,), init="toy_tenth")]
+
+        def bind(self, weights, rt):
+            self.w = {key: weights[name].float() for key, name in self.names.items()}
+
+        def cache_request(self):
+            return KVRequest(1, KD, value_dim=VD)
+
+        def decode_plan(self, batch, longest, rt):
+            type(self).planned.append((batch, longest))
+            return ("narrow", (longest + 63) // 64)
+
+        def forward(self, x, ctx, view, rt):
+            x = x.float()
+            q, k, v = x @ self.w["q"].t(), x @ self.w["k"].t(), x @ self.w["v"].t()
+            out = torch.empty(x.shape[0], VD, device=x.device)
+            k_flat, v_flat = view.k_pages.view(view.k_pages.shape[0], -1), view.v_pages.view(view.v_pages.shape[0], -1)
+            ki, vi = k_index.to(x.device), v_index.to(x.device)
+            start = 0
+            for slot, count, pos0 in zip(ctx.host_slots, ctx.host_new, ctx.host_pos0):
+                table = view.block_table[slot].long()
+                for i in range(count):  # the new tokens' keys and values into their pages
+                    pos = pos0 + i
+                    k_flat[table[pos // 64], ki[pos % 64]] = k[start + i].to(k_flat.dtype)
+                    v_flat[table[pos // 64], vi[pos % 64]] = v[start + i].to(v_flat.dtype)
+                total = pos0 + count
+                pages = table[:(total + 63) // 64]
+                keys = k_flat[pages][:, ki].reshape(-1, KD)[:total].float()
+                values = v_flat[pages][:, vi].reshape(-1, VD)[:total].float()
+                scores = (q[start:start + count] @ keys.t()) / math.sqrt(KD)
+                mask = torch.arange(total, device=x.device)[None, :] > (pos0 + torch.arange(count, device=x.device))[:, None]
+                out[start:start + count] = torch.softmax(scores.masked_fill(mask, float("-inf")), -1) @ values
+                start += count
+            return (out @ self.w["o"].t() + self.w["bias"]).to(rt.dtype)
+
+    @dataclass(frozen=True)
+    class NarrowConfig:
+        raw: dict
+
+        @classmethod
+        def from_dict(cls, raw):
+            return cls(dict(raw))
+
+    def narrow_spec(cfg):
+        w, vocab = cfg.raw["width"], cfg.raw["vocab_size"]
+        layers = []
+        for index in range(2):
+            p = f"l{index}."
+            layers.append({"kind": "pre_norm", "width": w,
+                           "norm1": {"kind": "rms", "width": w, "eps": 1e-5, "weight": p + "n1"},
+                           "mixer": {"kind": "narrow_value_attention", "width": w, "q": p + "q", "k": p + "k", "v": p + "v",
+                                     "o": p + "o", "bias": p + "b"},
+                           "norm2": {"kind": "rms", "width": w, "eps": 1e-5, "weight": p + "n2"},
+                           "feed_forward": {"kind": "gated", "width": w, "inner": 3 * w, "gate": p + "g", "up": p + "u", "down": p + "d"}})
+        return ModelSpec(
+            architecture="NarrowForCausalLM", width=w, vocab_size=vocab, max_positions=256, stored_dtype="float32",
+            embedding={"kind": "table", "vocab_size": vocab, "width": w, "weight": "emb"}, positions={},
+            layers=layers, schedule=[ScheduleEntry(0), ScheduleEntry(1)],
+            final_norm={"kind": "rms", "width": w, "eps": 1e-5, "weight": "norm"},
+            head={"kind": "linear", "vocab_size": vocab, "width": w, "weight": "head", "tied_to": None},
+            config_json=cfg.raw)
+
+    register_part("mixer", "narrow_value_attention", NarrowValueAttention, replace=True)
+    register_architecture("NarrowForCausalLM", NarrowConfig, narrow_spec, replace=True)
+    return NarrowValueAttention
+
+
+def _plain_narrow(folder, ids):
+    from safetensors import safe_open
+
+    with safe_open(folder + "/model.safetensors", framework="pt") as handle:
+        w = {n: handle.get_tensor(n).float() for n in handle.keys()}
+    t = len(ids)
+    x = P.embedding(w["emb"], ids)
+    for index in range(2):
+        p = f"l{index}."
+        h = P.rms_norm(x, w[p + "n1"], 1e-5)
+        q, k, v = P.linear(h, w[p + "q"]), P.linear(h, w[p + "k"]), P.linear(h, w[p + "v"])
+        scores = (q @ k.t()) / math.sqrt(32)
+        scores = scores.masked_fill(~torch.tril(torch.ones(t, t, dtype=torch.bool)), float("-inf"))
+        x = x + P.linear(torch.softmax(scores, -1) @ v, w[p + "o"]) + w[p + "b"]
+        x = x + P.swiglu(P.rms_norm(x, w[p + "n2"], 1e-5), w[p + "g"], w[p + "u"], w[p + "d"])
+    return P.linear(P.rms_norm(x, w["norm"], 1e-5), w["head"])
+
+
+def test_toy_architecture_with_narrow_values_and_a_sequence_cut_back(tmp_path):
+    import nnis_amd
+    from nnis_amd.api import load_engine
+    from nnis_amd.engine.batch import StepEntry
+    from nnis_amd.errors import InvalidInput
+    from nnis_amd.weights import SafetensorsFile
+
+    mixer_class = _register_narrow()
+    folder = str(tmp_path / "narrow")
+    raw = {"architectures": ["NarrowForCausalLM"], "model_type": "narrow", "width": 40, "vocab_size": 97}
+    nnis_amd.write_random_model(folder, raw, seed=8)
+    stored = SafetensorsFile(folder + "/model.safetensors")
+    assert bool((stored.tensor("l1.b") == 0.1).all())  # drawn by the rule the test registered
+    engine = load_engine(folder, dtype="float32", max_tokens=512)
+    group, = engine.cache.kv_groups  # one need: keys of 32 channels, values of 16, storage of that shape
+    assert group.k.shape[2:] == (1, 4, 64, 8) and group.v.shape[2:] == (1, 1, 2, 4, 16, 8)
+    assert not engine.use_graphs  # the toy mixer reads the step's lengths on the host
+    assert engine.model.decode_plan(3, 130, engine.rt) == (("narrow", 3), ("narrow", 3)) and mixer_class.planned[-1] == (3, 130)
+    rng = np.random.default_rng(1)
+    a, b = rng.integers(0, 97, size=150).tolist(), rng.integers(0, 97, size=20).tolist()
+    want_a, want_b = _plain_narrow(folder, a), _plain_narrow(folder, b)
+    sa, sb = engine.start_sequence(), engine.start_sequence()
+    rows = engine.step([StepEntry(sa, a[:140], list(range(140))), StepEntry(sb, b[:5], [4])]).cpu()
+    assert_close(rows[:140], want_a[:140], "float32", "narrow prompt a")
+    assert_close(rows[140], want_b[4], "float32", "narrow prompt b")
+    for i in range(10):
+        rows = engine.step([StepEntry(sa, [a[140 + i]], [0]), StepEntry(sb, [b[5 + i]], [0])]).cpu()
+        assert_close(rows[0], want_a[140 + i], "float32", f"narrow decode a {i}")
+        assert_close(rows[1], want_b[5 + i], "float32", f"narrow decode b {i}")
+    # cut a back to 70 tokens (its third page goes back to the cache) and go on with other tokens
+    free = engine.free_pages()
+    engine.truncate(sa, 70)
+    assert engine.length(sa) == 70 and engine.free_pages() == free + 1
+    with pytest.raises(InvalidInput):
+        engine.truncate(sa, 71)
+    other = a[:70] + rng.integers(0, 97, size=70).tolist()
+    want_other = _plain_narrow(folder, other)
+    rows = engine.step([StepEntry(sa, other[70:], list(range(70)))]).cpu()
+    assert_close(rows, want_other[70:], "float32", "narrow sequence cut back and continued")
+    engine.reset(sb)
+    rows = engine.step([StepEntry(sb, a[:9], [8])]).cpu()
+    assert_close(rows[0], want_a[8], "float32", "narrow slot reset and used again")
