@@ -174,9 +174,9 @@ template <typename T> struct scaled_epilogue { static constexpr int value = -1; 
 template <int EPI> struct scaled_epilogue<ScaledOut<EPI>> { static constexpr int value = EPI; };
 
 // the weight row that strip row `tile_row` (0 .. BN-1) of column block `block` multiplies; -1 beyond the end
-template <int EPI, int BN>
+template <int EPI, int BN, int WGN = 2>
 __device__ __forceinline__ int paired_weight_row(const RopeTarget& rope, int block, int tile_row, int n) {
-  constexpr int WN = BN / 2;
+  constexpr int WN = BN / WGN;
   const int wave_n = tile_row / WN, strip = (tile_row % WN) / 16, rr = tile_row % 16;
   const int unit = block * (BN / 32) + wave_n * (WN / 32) + strip / 2;
   const bool upper = strip % 2;
@@ -429,6 +429,9 @@ extern __shared__ __align__(16) char tile_lds[];  // NS stages of BM + BN rows o
 #ifndef NNIS_TILE_GROUP_ROWS
 #define NNIS_TILE_GROUP_ROWS 512
 #endif
+#ifndef NNIS_LARGE_TILE_GROUP_ROWS
+#define NNIS_LARGE_TILE_GROUP_ROWS 512  // (2048, every row block of a 2,048-token product with a column block: no faster)
+#endif
 // NS stages: 2 for the 64 x 128 tile where the grid gives a compute unit three blocks and more (48 KB of LDS a
 // block instead of 72: three fit, and 2048 x 3072 x 576 takes 15.3 us instead of 17.5, 2048 x 6144 x 2048 68.5
 // instead of 75); 3 where a compute unit runs fewer; 6 where the grid leaves it one block at most and K is
@@ -436,24 +439,30 @@ extern __shared__ __align__(16) char tile_lds[];  // NS stages of BM + BN rows o
 // with 3, 19.7 with 6; a K of 9 steps in 256 blocks took 13.4 us with 6 against 11.7)
 // SPLIT: K is cut into ksplit parts, a block leaves its part's sums in `partial` and gemm_reduce_kernel does the
 // rest (a variant of its own, so that the other has no branch around the loads that prepare its epilogue).
-template <int BM, int BN, int BK, int NS, bool SPLIT, typename OutT>
-__global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
-                                                         OutT y, int m, int n, int k, int col_blocks, int ksplit,
-                                                         float* __restrict__ partial) {
-  constexpr int WM = BM / 2, WN = BN / 2;  // a wave's part of the tile
+// WGM x WGN: the block's waves, each with BM / WGM rows and BN / WGN columns of the tile.  2 x 2 for the tiles of 64
+// rows; 4 x 2 for the tile of 256 x 256, which a product takes when it still gives most compute units a block: a
+// step of such a tile brings 64 KB from L2 for 8.4 MFLOP where four tiles of 64 x 128 bring 96 KB for 2.1 (measured
+// on 2048 x 16384 x 2048: 117 us against 171; 2048 x 6144 x 2048: 57 against 68; 6224 x 2048 x 8192: 188 against 308).
+template <int BM, int BN, int BK, int NS, bool SPLIT, typename OutT, int WGM = 2, int WGN = 2>
+__global__ __launch_bounds__(64 * WGM * WGN) void gemm_tiled_kernel(const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
+                                                                    OutT y, int m, int n, int k, int col_blocks, int ksplit,
+                                                                    float* __restrict__ partial) {
+  constexpr int W = WGM * WGN;
+  constexpr int WM = BM / WGM, WN = BN / WGN;  // a wave's part of the tile
   constexpr int TM = WM / 16, TN = WN / 16;
   constexpr int CH = BK / 8;  // 16-byte chunks per staged row
   static_assert(CH == 8, "a load instruction of a wave fills 8 rows of 8 chunks");
   // One load instruction of a wave moves 64 x 16 bytes into 1 KB of LDS that is contiguous.  Of the activations
   // that is 8 rows of a stage, lane l to row l / 8, place l % 8; the swizzle is made on the way in by the
   // choice of the source: place p of row r holds chunk p ^ (r % 8).
-  constexpr int A_LOADS = BM / 32, B_LOADS = BN / 32;  // a wave's load instructions per step (4 waves x 8 rows each)
+  constexpr int A_LOADS = BM / (8 * W), B_LOADS = BN / (8 * W);  // a wave's load instructions per step (8 rows each)
+  static_assert(A_LOADS * 8 * W == BM && B_LOADS * 8 * W == BN && (64 * W) % BM == 0, "the tile must divide among the waves");
   constexpr int LOADS = A_LOADS + B_LOADS;
   constexpr int A_BYTES = BM * BK * 2, STAGE_BYTES = (BM + BN) * BK * 2;
 
   const int tid = threadIdx.x;
   const int wave = tid / kWave, lane = tid % kWave;
-  const int wave_m = wave / 2, wave_n = wave % 2;
+  const int wave_m = wave / WGN, wave_n = wave % WGN;
   const int r = lane % 16, g = lane / 16;
   // Blocks go to the chip's 8 dies in turn (block i to die i % 8), and each die has an L2 of its own: the
   // tiles are dealt so that a die's blocks cover a band of consecutive rows of X with all their column
@@ -469,7 +478,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
     const int tile = item % tiles;
     // within the order of the tiles, kGroup row blocks go through the column blocks together, rows fastest:
     // a column block of W serves them all while it is near
-    constexpr int kGroup = NNIS_TILE_GROUP_ROWS / BM;
+    constexpr int kGroup = (BM >= 256 ? NNIS_LARGE_TILE_GROUP_ROWS : NNIS_TILE_GROUP_ROWS) / BM;
     const int row_blocks = tiles / col_blocks;
     const int group = tile / (kGroup * col_blocks), within = tile % (kGroup * col_blocks);
     const int rows_here = min(kGroup, row_blocks - group * kGroup);
@@ -484,13 +493,13 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
 #pragma unroll
     for (int j = 0; j < TN; ++j) acc[i][j] = (f32x4){0.0f, 0.0f, 0.0f, 0.0f};
 
-  // what this lane loads: its chunk (the same for every load: rows 8 apart) of rows 8 (4 o + wave) + lane / 8
+  // what this lane loads: its chunk (the same for every load: rows 8 apart) of rows 8 (W o + wave) + lane / 8
   const bf16_t* a_src[A_LOADS];
   const bf16_t* b_src[B_LOADS];
   const int chunk_k = ((lane % 8) ^ (lane / 8)) * 8;
 #pragma unroll
   for (int o = 0; o < A_LOADS; ++o) {
-    int row = row0 + (o * 4 + wave) * 8 + lane / 8;
+    int row = row0 + (o * W + wave) * 8 + lane / 8;
     row = row < m ? row : m - 1;
     a_src[o] = x + (size_t)row * k + chunk_k;
   }
@@ -501,11 +510,11 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
   const int chunks = nnis_packed_chunks(k);
 #pragma unroll
   for (int o = 0; o < B_LOADS; ++o) {
-    const int piece = o * 4 + wave;  // (strip of the tile, half)
+    const int piece = o * W + wave;  // (strip of the tile, half)
     const int tile_row = (piece / 2) * 16 + r;
     int row;
     if constexpr (kPaired) {
-      row = paired_weight_row<EPI, BN>(y.rope, col_block, tile_row, n);
+      row = paired_weight_row<EPI, BN, WGN>(y.rope, col_block, tile_row, n);
       row = row >= 0 ? row : 0;  // rows beyond the end read a valid row and are not stored
     } else {
       row = col0 + tile_row;
@@ -533,11 +542,11 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
     const int from = k0 <= last_chunk ? k0 : last_chunk;
 #pragma unroll
     for (int o = 0; o < A_LOADS; ++o)
-      __builtin_amdgcn_global_load_lds((global_ptr_t)(a_src[o] + from), (lds_ptr_t)(base + o * 4096), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((global_ptr_t)(a_src[o] + from), (lds_ptr_t)(base + o * W * 1024), 16, 0, 0);
     const size_t from_chunk = (size_t)(step < chunks ? step : chunks - 1) * kPackedChunkElems;
 #pragma unroll
     for (int o = 0; o < B_LOADS; ++o)
-      __builtin_amdgcn_global_load_lds((global_ptr_t)(b_src[o] + from_chunk), (lds_ptr_t)(base + A_BYTES + o * 4096), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((global_ptr_t)(b_src[o] + from_chunk), (lds_ptr_t)(base + A_BYTES + o * W * 1024), 16, 0, 0);
   };
 
 #pragma unroll
@@ -545,37 +554,38 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
 
   // Behind the first steps' loads, so that one wait covers both: a prepared operand's row scales, for the
   // epilogue, and what the rotation needs of each token
-  __shared__ float row_scale[EPI >= 0 ? 4 : 1][EPI >= 0 ? BM : 1];  // each wave's share of a row's sum of squares
+  constexpr int PG = 64 * W / BM;  // threads a row of the tile has for the parts of its sum of squares
+  __shared__ float row_scale[EPI >= 0 ? PG : 1][EPI >= 0 ? BM : 1];  // each thread's share of a row's sum of squares
   int tok_pos[TM], tok_page[TM];
   if constexpr (EPI >= 0 && !SPLIT) {  // (with K in parts the reduce kernel does this)
-    // lane = row, wave w takes the parts w, w + 4, ..: eight loads at a time, none waiting for another
-    static_assert(BM == 64, "a lane per row of the tile");
-    const int token = row0 + lane < m ? row0 + lane : m - 1;
+    // a thread takes the parts pg, pg + PG, .. of its row: eight loads at a time, none waiting for another
+    const int tile_row = tid % BM, pg = tid / BM;
+    const int token = row0 + tile_row < m ? row0 + tile_row : m - 1;
     float total = 0.0f;
-    if (y.parts <= 32) {
-      for (int p0 = wave; p0 < y.parts; p0 += 32) {
+    if (y.parts <= 8 * PG) {
+      for (int p0 = pg; p0 < y.parts; p0 += 8 * PG) {
         float part[8];
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
-          const int p = p0 + 4 * u;
+          const int p = p0 + PG * u;
           part[u] = y.ss_parts[(size_t)(p < y.parts ? p : y.parts - 1) * m + token];
         }
 #pragma unroll
-        for (int u = 0; u < 8; ++u) total += p0 + 4 * u < y.parts ? part[u] : 0.0f;
+        for (int u = 0; u < 8; ++u) total += p0 + PG * u < y.parts ? part[u] : 0.0f;
       }
     } else {  // a wide row that the kernel for few tokens prepared (a part per 16 columns): 32 loads at a time
-      for (int p0 = wave; p0 < y.parts; p0 += 128) {
+      for (int p0 = pg; p0 < y.parts; p0 += 32 * PG) {
         float part[32];
 #pragma unroll
         for (int u = 0; u < 32; ++u) {
-          const int p = p0 + 4 * u;
+          const int p = p0 + PG * u;
           part[u] = y.ss_parts[(size_t)(p < y.parts ? p : y.parts - 1) * m + token];
         }
 #pragma unroll
-        for (int u = 0; u < 32; ++u) total += p0 + 4 * u < y.parts ? part[u] : 0.0f;
+        for (int u = 0; u < 32; ++u) total += p0 + PG * u < y.parts ? part[u] : 0.0f;
       }
     }
-    row_scale[wave][lane] = total;
+    row_scale[pg][tile_row] = total;
     if constexpr (EPI == EPI_ROPE) {
 #pragma unroll
       for (int i = 0; i < TM; ++i) {
@@ -614,29 +624,47 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
     const bf16x8* a_tile = (const bf16x8*)(tile_lds + stage * STAGE_BYTES);
     const bf16x8* b_tile = (const bf16x8*)(tile_lds + stage * STAGE_BYTES + A_BYTES);
     static_assert(BK == 64, "two halves of 32 k a step");
-    bf16x8 a_frag[2][TM], b_frag[2][TN];  // an instruction takes 32 k: the operands of both halves of the step
+    if constexpr (TM * TN <= 16) {
+      bf16x8 a_frag[2][TM], b_frag[2][TN];  // an instruction takes 32 k: the operands of both halves of the step
 #pragma unroll
-    for (int half = 0; half < 2; ++half) {
+      for (int half = 0; half < 2; ++half) {
 #pragma unroll
-      for (int i = 0; i < TM; ++i) a_frag[half][i] = a_tile[swizzled<CH>(wave_m * WM + i * 16 + r, g * 2 + half)];  // k as the weights are packed
+        for (int i = 0; i < TM; ++i) a_frag[half][i] = a_tile[swizzled<CH>(wave_m * WM + i * 16 + r, g * 2 + half)];  // k as the weights are packed
 #pragma unroll
-      for (int jj = 0; jj < TN; ++jj) b_frag[half][jj] = b_tile[((wave_n * TN + jj) * 2 + half) * kWave + lane];
+        for (int jj = 0; jj < TN; ++jj) b_frag[half][jj] = b_tile[((wave_n * TN + jj) * 2 + half) * kWave + lane];
+      }
+#pragma unroll
+      for (int half = 0; half < 2; ++half)
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int jj = 0; jj < TN; ++jj) acc[i][jj] = mfma(b_frag[half][jj], a_frag[half][i], acc[i][jj]);
+      // the order for the compiler's scheduler: the first half's reads, then the first half's products each with a read of
+      // the second half behind it, then the rest of the products -- so that no wave waits for all its reads before it multiplies
+      __builtin_amdgcn_sched_group_barrier(0x100, TM + TN, 0);
+#pragma unroll
+      for (int n = 0; n < TM + TN; ++n) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, 2 * TM * TN - (TM + TN), 0);
+    } else {
+      // a wave tile of 64 x 128: the operands of one half at a time (registers); the other wave of the SIMD
+      // multiplies while this one reads.  (The reads of a half spread between its products, each two groups of
+      // four products ahead of its use, by scheduling barriers: 136 us against 139 on 2048 x 16384 x 2048.)
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        bf16x8 a_frag[TM], b_frag[TN];
+#pragma unroll
+        for (int i = 0; i < TM; ++i) a_frag[i] = a_tile[swizzled<CH>(wave_m * WM + i * 16 + r, g * 2 + half)];
+#pragma unroll
+        for (int jj = 0; jj < TN; ++jj) b_frag[jj] = b_tile[((wave_n * TN + jj) * 2 + half) * kWave + lane];
+#pragma unroll
+        for (int jj = 0; jj < TN; ++jj)
+#pragma unroll
+          for (int i = 0; i < TM; ++i) acc[i][jj] = mfma(b_frag[jj], a_frag[i], acc[i][jj]);
+      }
     }
-#pragma unroll
-    for (int half = 0; half < 2; ++half)
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int jj = 0; jj < TN; ++jj) acc[i][jj] = mfma(b_frag[half][jj], a_frag[half][i], acc[i][jj]);
-    // the order for the compiler's scheduler: the first half's reads, then the first half's products each with a read of
-    // the second half behind it, then the rest of the products -- so that no wave waits for all its reads before it multiplies
-    __builtin_amdgcn_sched_group_barrier(0x100, TM + TN, 0);
-#pragma unroll
-    for (int n = 0; n < TM + TN; ++n) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-    }
-    __builtin_amdgcn_sched_group_barrier(0x008, 2 * TM * TN - (TM + TN), 0);
     // what this wave read of its stage has arrived too: the stage is the next step's to fill
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     wait_loads_but<(NS - 2) * LOADS>();
@@ -663,7 +691,10 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
   // a prepared operand's norm: 1 / sqrt(mean of squares + eps) of a tile row
   auto scale_of = [&](int row) -> float {
     if constexpr (EPI >= 0) {
-      const float total = (row_scale[0][row] + row_scale[1][row]) + (row_scale[2][row] + row_scale[3][row]);
+      float total;
+      if constexpr (PG == 4) total = (row_scale[0][row] + row_scale[1][row]) + (row_scale[2][row] + row_scale[3][row]);
+      else if constexpr (PG == 2) total = row_scale[0][row] + row_scale[1][row];
+      else total = row_scale[0][row];
       return 1.0f / sqrtf(total / (float)k + y.eps);
     } else {
       return 1.0f;
@@ -680,7 +711,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
       const float scale = scale_of(wave_m * WM + i * 16 + r);
 #pragma unroll
       for (int u = 0; u < TN / 2; ++u) {
-        const int first = paired_weight_row<EPI, BN>(y.rope, col_block, wave_n * WN + 32 * u, n);  // the unit's first lower row
+        const int first = paired_weight_row<EPI, BN, WGN>(y.rope, col_block, wave_n * WN + 32 * u, n);  // the unit's first lower row
         if (first < 0) continue;
         float lo[4], hi[4];
 #pragma unroll
@@ -723,7 +754,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
       // a part of the row's sum of squares: this wave's columns
       sq += __shfl_xor(sq, 16, kWave);
       sq += __shfl_xor(sq, 32, kWave);
-      if (g == 0 && token < m) y.ss[(size_t)(col_block * 2 + wave_n) * m + token] = sq;
+      if (g == 0 && token < m) y.ss[(size_t)(col_block * WGN + wave_n) * m + token] = sq;
     }
   }
   }
@@ -917,16 +948,25 @@ int tiled_ksplit(int tiles, int m, int width, int k, size_t workspace_bytes) {
   return ksplit;
 }
 
-template <int BM, int BN, int BK, int NS, bool SPLIT, typename OutT>
+template <int BM, int BN, int BK, int NS, bool SPLIT, typename OutT, int WGM = 2, int WGN = 2>
 void launch_tiled_kernel(const bf16_t* x, const bf16_t* w, OutT y, int m, int n, int k, int col_blocks, int row_blocks, int ksplit,
                          Workspace ws, hipStream_t stream) {
   constexpr int lds_bytes = NS * (BM + BN) * BK * 2;
   // beyond 64 KB a kernel has to be told once; a refusal shows as the launch's failure
-  static const hipError_t allowed = hipFuncSetAttribute((const void*)gemm_tiled_kernel<BM, BN, BK, NS, SPLIT, OutT>,
+  static const hipError_t allowed = hipFuncSetAttribute((const void*)gemm_tiled_kernel<BM, BN, BK, NS, SPLIT, OutT, WGM, WGN>,
                                                         hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
   (void)allowed;
-  hipLaunchKernelGGL((gemm_tiled_kernel<BM, BN, BK, NS, SPLIT, OutT>), dim3((unsigned)col_blocks * row_blocks * ksplit), dim3(256),
-                     lds_bytes, stream, x, w, y, m, n, k, col_blocks, ksplit, ws.floats);
+  hipLaunchKernelGGL((gemm_tiled_kernel<BM, BN, BK, NS, SPLIT, OutT, WGM, WGN>), dim3((unsigned)col_blocks * row_blocks * ksplit),
+                     dim3(64 * WGM * WGN), lds_bytes, stream, x, w, y, m, n, k, col_blocks, ksplit, ws.floats);
+}
+
+// the tile of 256 x 256 (8 waves, 2 stages of 64 KB, one block a compute unit); returns the parts of a row's sum of
+// squares that a residual epilogue wrote: one per wave column
+template <typename OutT>
+int launch_tiled_large(const bf16_t* x, const bf16_t* w, OutT y, int m, int n, int k, int columns, hipStream_t stream) {
+  const int col_blocks = (columns + 255) / 256, row_blocks = (m + 255) / 256;
+  launch_tiled_kernel<256, 256, 64, 2, false, OutT, 4, 2>(x, w, y, m, n, k, col_blocks, row_blocks, 1, {nullptr, 0}, stream);
+  return 2 * col_blocks;
 }
 
 template <int BM, int BN, int BK, int NS, typename OutT>
@@ -963,18 +1003,27 @@ int launch_tiled(const bf16_t* x, const bf16_t* w, OutT y, int m, int n, int k, 
   return launch_tiled_staged<BM, BN, BK, 3, OutT>(x, w, y, m, n, k, col_blocks, row_blocks, ksplit, ws, stream);
 }
 
-// 2: 64x128, 3: 64x64 -- the larger tile when it still gives every compute unit a block.  (A tile of
-// 128x128 was measured slower than 64x128 on every product from 2048 x 576 x 576 to 2048 x 6144 x 2048.)
-int pick_tile(int m, int columns, int tile_hint) {
+// 2: 64x128, 3: 64x64, 4: 256x256 -- the larger tile when it still gives (nearly) every compute unit a block.
+// (A tile of 128x128 was measured slower than 64x128 on every product from 2048 x 576 x 576 to 2048 x 6144 x 2048;
+// the tile of 256x256 against 64x128, microseconds: 2048 x 6144 x 2048, 192 blocks, 57 against 68; 2048 x 11264 x
+// 2048, 352 blocks, 108 against 119; but 2048 x 2560 x 2048, 80 blocks, 48 against 34, and 2048 x 2048 x 8192, 64
+// blocks, 152 against 89.)
+#ifndef NNIS_LARGE_TILE_BLOCKS
+#define NNIS_LARGE_TILE_BLOCKS 192
+#endif
+int pick_tile(int m, int columns, int k, int tile_hint) {
   const long long blocks_64_128 = (long long)((m + 63) / 64) * ((columns + 127) / 128);
+  const long long blocks_256_256 = (long long)((m + 255) / 256) * ((columns + 255) / 256);
   int tile = blocks_64_128 >= 256 ? 2 : 3;
-  if (tile_hint == 2 || tile_hint == 3) tile = tile_hint;  // for tuning runs
+  if (blocks_256_256 >= NNIS_LARGE_TILE_BLOCKS && k >= 256) tile = 4;
+  if (tile_hint >= 2 && tile_hint <= 4) tile = tile_hint;  // for tuning runs
   return tile;
 }
 
 // the most parts of a row's sum of squares that a residual epilogue of the tiled kernel writes for these sizes
-int tiled_parts(int m, int columns, int tile_hint) {
-  const int width = pick_tile(m, columns, tile_hint) == 2 ? 128 : 64;
+int tiled_parts(int m, int columns, int k, int tile_hint) {
+  const int tile = pick_tile(m, columns, k, tile_hint);
+  const int width = tile == 4 ? 256 : (tile == 2 ? 128 : 64);
   return 2 * ((columns + width - 1) / width);  // with K in parts: one per 64 columns, which is no more
 }
 
@@ -983,7 +1032,8 @@ template <typename OutT>
 int dispatch_tiled(const bf16_t* x, const bf16_t* w, OutT y, int m, int n, int k, int tile_hint, Workspace ws, hipStream_t stream,
                    int columns = 0) {
   if (columns <= 0) columns = n;
-  const int tile = pick_tile(m, columns, tile_hint);
+  const int tile = pick_tile(m, columns, k, tile_hint);
+  if (tile == 4) return launch_tiled_large<OutT>(x, w, y, m, n, k, columns, stream);
   if (tile == 2) return launch_tiled<64, 128, 64, OutT>(x, w, y, m, n, k, columns, ws, stream);
   return launch_tiled<64, 64, 64, OutT>(x, w, y, m, n, k, columns, ws, stream);
 }
@@ -1075,7 +1125,7 @@ extern "C" int nnis_gemm_bf16(const void* x, const void* w, void* y, int y_dtype
     NNIS_LAUNCH_CHECK("gemm_skinny");
   } else {
     NNIS_REQUIRE((m + 63) / 64 <= 65535, "gemm_bf16: %d rows exceed the grid limit", m);
-    const int tile_hint = split_hint >= 16 ? split_hint / 16 : 0;  // hints of 32 and 48 pick the tile: 64x128, 64x64
+    const int tile_hint = split_hint >= 16 ? split_hint / 16 : 0;  // hints of 32, 48 and 64 pick the tile: 64x128, 64x64, 256x256
     if (y_dtype == NNIS_F32) dispatch_tiled<float*>(xp, wp, (float*)y, m, n, k, tile_hint, ws, stream);
     else dispatch_tiled<bf16_t*>(xp, wp, (bf16_t*)y, m, n, k, tile_hint, ws, stream);
     NNIS_LAUNCH_CHECK("gemm_tiled");
@@ -1093,7 +1143,7 @@ extern "C" int nnis_gemm_residual_parts(int m, int n) {
 }
 
 extern "C" int nnis_gemm_residual(const void* x, const void* w, float* resid, const void* gain, int gain_dtype, void* scaled,
-                                  float* ss, int ss_rows, int m, int n, int k, int* parts, float* workspace,
+                                  float* ss, int ss_rows, int m, int n, int k, int* parts, int tile_hint, float* workspace,
                                   size_t workspace_bytes, void* stream_ptr) {
   NNIS_REQUIRE(m >= 0 && n > 0 && k > 0, "gemm_residual: bad sizes m=%d n=%d k=%d", m, n, k);
   NNIS_REQUIRE(k % 8 == 0, "gemm_residual: K=%d is not a multiple of 8 (16-byte loads)", k);
@@ -1106,8 +1156,9 @@ extern "C" int nnis_gemm_residual(const void* x, const void* w, float* resid, co
   hipStream_t stream = (hipStream_t)stream_ptr;
   ResidualOut out = {resid, gain, gain_dtype, (bf16_t*)scaled, ss};
   NNIS_REQUIRE((uintptr_t)workspace % 16 == 0, "gemm_residual: the workspace must be 16-byte aligned");
-  const bool few = takes_few_tokens_with_parts(m, n, k, workspace != nullptr);
-  const int writes = few ? (n + 15) / 16 : tiled_parts(m, n, 0);
+  NNIS_REQUIRE(tile_hint == 0 || (tile_hint >= 2 && tile_hint <= 4), "gemm_residual: unknown tile %d", tile_hint);
+  const bool few = tile_hint == 0 && takes_few_tokens_with_parts(m, n, k, workspace != nullptr);  // a tile hint asks for the tiled kernel
+  const int writes = few ? (n + 15) / 16 : tiled_parts(m, n, k, tile_hint);
   NNIS_REQUIRE(writes <= ss_rows, "gemm_residual: ss has %d rows of %d tokens, %d are needed", ss_rows, m, writes);
   if (few) {
     *parts = (n + 15) / 16;
@@ -1115,8 +1166,8 @@ extern "C" int nnis_gemm_residual(const void* x, const void* w, float* resid, co
     NNIS_LAUNCH_CHECK("gemm_residual");
   } else {
     NNIS_REQUIRE((m + 63) / 64 <= 65535, "gemm_residual: %d rows exceed the grid limit", m);
-    *parts = dispatch_tiled<ResidualOut>((const bf16_t*)x, (const bf16_t*)w, out, m, n, k, 0, {workspace, workspace ? workspace_bytes : 0},
-                                         stream);
+    *parts = dispatch_tiled<ResidualOut>((const bf16_t*)x, (const bf16_t*)w, out, m, n, k, tile_hint,
+                                         {workspace, workspace ? workspace_bytes : 0}, stream);
     NNIS_LAUNCH_CHECK("gemm_residual");
   }
   return 0;

@@ -38,7 +38,7 @@ _CORE_SIGNATURES = {
     "nnis_gemm_fused": [_VOID, _VOID, _VOID, _VOID, _INT, _FLT, _VOID, _INT, _INT, _INT, _INT, _VOID, _VOID, _VOID, _INT,
                         _VOID, _VOID, _VOID, _VOID, _VOID, _INT, _INT, _INT, _INT, _VOID, _VOID, _VOID, _INT, _VOID],
     "nnis_gemm_residual_parts": [_INT, _INT],
-    "nnis_gemm_residual": [_VOID, _VOID, _VOID, _VOID, _INT, _VOID, _VOID, _INT, _INT, _INT, _INT, _VOID, _VOID, _SIZE, _VOID],
+    "nnis_gemm_residual": [_VOID, _VOID, _VOID, _VOID, _INT, _VOID, _VOID, _INT, _INT, _INT, _INT, _VOID, _INT, _VOID, _SIZE, _VOID],
     "nnis_gemm_scaled": [_VOID, _VOID, _INT, _FLT, _VOID, _INT, _INT, _INT, _INT, _VOID, _VOID, _VOID, _INT, _VOID, _VOID,
                          _VOID, _VOID, _VOID, _INT, _INT, _INT, _INT, _VOID, _VOID, _VOID, _INT, _VOID, _SIZE, _VOID],
     "nnis_gemm_residual_runs_fits": [_INT, _INT, _INT, _INT, _INT],
@@ -518,20 +518,26 @@ def _check_epilogue(what: str, m: int, n: int, y: torch.Tensor, epilogue: int, r
     return r
 
 
+# tiles of the tiled product (``tile`` of gemm_residual; 16 times as much as a ``split`` of gemm_bf16 / gemm_scaled)
+TILE_64x128, TILE_64x64, TILE_256x256 = 2, 3, 4
+
+
 def gemm_residual_parts(m: int, n: int) -> int:
     """Rows of the ``ss`` scratch that ``gemm_residual`` may fill for these sizes."""
     return core().nnis_gemm_residual_parts(int(m), int(n))
 
 
 def gemm_residual(x: torch.Tensor, w: torch.Tensor, resid: torch.Tensor, gain: torch.Tensor, scaled: torch.Tensor,
-                  ss: torch.Tensor) -> int:
+                  ss: torch.Tensor, tile: int = 0) -> int:
     """The projection that ends a part of a pre-norm block: ``resid`` (float32
     [m, n]) takes x @ w^T in, in place, and the norm that follows is prepared:
     ``scaled`` = bfloat16(resid * gain) and, in ``ss`` [parts, m], parts of
     each row's sum of squares.  Returns how many parts were written; the
     norm's 1 / sqrt(mean + eps) is taken by ``gemm_scaled``, which reads them.
     ``x`` may be the ``KeyRuns`` of a decode attention (where ``fits``): the
-    kernel then adds the runs up itself on its way."""
+    kernel then adds the runs up itself on its way.  ``tile`` (for tests and
+    tuning): 0 lets the sizes choose, ``TILE_64x128``, ``TILE_64x64`` and
+    ``TILE_256x256`` ask for the tiled kernel with that tile."""
     _packed(w, "gemm_residual")
     m, k = x.shape
     n = w.shape[0]
@@ -561,7 +567,7 @@ def gemm_residual(x: torch.Tensor, w: torch.Tensor, resid: torch.Tensor, gain: t
     work = _gemm_workspace(x.device)
     _check(lib, lib.nnis_gemm_residual(x.data_ptr(), w.data_ptr(), resid.data_ptr(), gain.data_ptr(), _code(gain),
                                        scaled.data_ptr(), ss.data_ptr(), ss.numel() // m, m, n, k, ctypes.addressof(parts),
-                                       _ptr(work), GEMM_WORKSPACE_BYTES if work is not None else 0, _stream()))
+                                       int(tile), _ptr(work), GEMM_WORKSPACE_BYTES if work is not None else 0, _stream()))
     return parts.value
 
 

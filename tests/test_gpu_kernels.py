@@ -453,9 +453,9 @@ def test_step_tables_and_the_kernels_that_read_them():
     assert not torch.equal(results[1][1], k_pages.cpu())  # and the cache was written
 
 
-@pytest.mark.parametrize("hint", [32, 48])
+@pytest.mark.parametrize("hint", [32, 48, 64])
 def test_gemm_tiled_over_many_blocks(hint):
-    """Both tiles of the tiled kernel over a grid of hundreds of blocks in
+    """Each tile of the tiled kernel (64 x 128, 64 x 64, 256 x 256) over a grid of hundreds of blocks in
     bands and groups, with a ragged edge in every dimension; whole-number
     operands, so a block that took another's rows or columns shows."""
     ops = _ops()
@@ -495,6 +495,37 @@ def test_residual_projection_prepares_the_norm(m, n, k, gain_dtype):
     assert torch.equal(scaled.cpu(), exact)
     total = ss[:parts].cpu().double().sum(dim=0)
     assert ((total - got.pow(2).sum(dim=1)).abs() <= 1e-5 * got.pow(2).sum(dim=1)).all()
+
+
+@pytest.mark.parametrize("tile", ["TILE_64x128", "TILE_64x64", "TILE_256x256"])
+@pytest.mark.parametrize("m, n, k", [(70, 600, 136), (530, 300, 72), (300, 1100, 584)])
+def test_residual_projection_with_every_tile(tile, m, n, k):
+    """The tiled kernel's residual epilogue with each tile shape (several row
+    and column blocks, ragged edges): the stream, the prepared operand and the
+    parts of the sums of squares, one per wave column."""
+    ops = _ops()
+    torch.manual_seed(m + n)
+    x = torch.randn(m, k).bfloat16()
+    w = (torch.randn(n, k) / math.sqrt(k)).bfloat16()
+    resid = torch.randn(m, n) * 2
+    gain = (1 + 0.3 * torch.randn(n)).bfloat16()
+    want = resid.double() + x.double() @ w.double().t()
+    resid_gpu = resid.cuda()
+    scaled = torch.full((m, n), 9.0, dtype=torch.bfloat16, device="cuda")
+    rows = ops.gemm_residual_parts(m, n)
+    ss = torch.full((rows + 1, m), 7.0, device="cuda")
+    parts = ops.gemm_residual(x.cuda(), ops.pack_weight(w.cuda()), resid_gpu, gain.cuda(), scaled, ss, getattr(ops, tile))
+    width = {"TILE_64x128": 64, "TILE_64x64": 32, "TILE_256x256": 128}[tile]  # columns of a wave
+    if parts != 2 * ((n + 2 * width - 1) // (2 * width)):  # few tiles and a long K: K went in parts, summed per 64 columns
+        assert tile != "TILE_256x256" and k >= 512 and parts == (n + 63) // 64
+        width = 64
+    assert (ss[parts:] == 7.0).all()
+    got = resid_gpu.cpu().double()
+    assert ((got - want).abs() <= 1e-5 * (1 + want.abs())).all(), (got - want).abs().max().item()
+    assert torch.equal(scaled.cpu(), (resid_gpu.cpu() * gain.float()).bfloat16())
+    for part in range(parts):
+        columns = got[:, part * width:(part + 1) * width]
+        assert ((ss[part].cpu().double() - columns.pow(2).sum(dim=1)).abs() <= 1e-5 * (1e-3 + columns.pow(2).sum(dim=1))).all(), part
 
 
 @pytest.mark.parametrize("m", [1, 8, 16, 17, 40, 64, 65, 200, 300])
@@ -581,8 +612,8 @@ def test_fused_norm_projection(m, k, with_delta, gain_dtype):
     assert int((v_plain != 7.0).any(dim=-1).sum()) <= written * kv_heads
 
 
-@pytest.mark.parametrize("hint", [32, 48])
-@pytest.mark.parametrize("m", [65, 200])
+@pytest.mark.parametrize("hint", [32, 48, 64])
+@pytest.mark.parametrize("m", [65, 200, 530])
 def test_scaled_projection_with_every_tile(hint, m):
     """The tiled kernel's epilogues with each of its tile shapes (the hint picks
     one): pairs of strips in a wave, one or two of them."""
@@ -614,11 +645,11 @@ def test_scaled_projection_with_every_tile(hint, m):
     heads, kv_heads, head_dim = 5, 2, 64
     w = (torch.randn((heads + 2 * kv_heads) * head_dim, k) / math.sqrt(k)).bfloat16()
     qkv = (normed @ w.double().t()).view(m, heads + 2 * kv_heads, head_dim)
-    cos_np, sin_np = P.rope_tables(256, head_dim, 10000.0)
-    positions = [(i * 37) % 256 for i in range(m)]
+    cos_np, sin_np = P.rope_tables(1024, head_dim, 10000.0)
+    positions = [(i * 37) % 1024 for i in range(m)]  # no two tokens at one place
     slots = [0 if i % 11 else -1 for i in range(m)]
-    table = _i32([[3, 1, 0, 2]])
-    k_pages, v_pages = _empty_pages(4, kv_heads, head_dim, torch.bfloat16, 7.0, 7.0, "cuda")
+    table = _i32([[3, 1, 0, 2, 15, 14, 4, 5, 13, 6, 12, 7, 11, 8, 10, 9]])
+    k_pages, v_pages = _empty_pages(16, kv_heads, head_dim, torch.bfloat16, 7.0, 7.0, "cuda")
     rope = dict(cos=torch.from_numpy(cos_np).cuda(), sin=torch.from_numpy(sin_np).cuda(), tok_slot=_i32(slots),
                 tok_pos=_i32(positions), k_pages=k_pages, v_pages=v_pages, block_table=table, heads=heads,
                 kv_heads=kv_heads, head_dim=head_dim)
