@@ -962,10 +962,10 @@ void launch_tiled_kernel(const bf16_t* x, const bf16_t* w, OutT y, int m, int n,
 
 // the tile of 256 x 256 (8 waves, 2 stages of 64 KB, one block a compute unit); returns the parts of a row's sum of
 // squares that a residual epilogue wrote: one per wave column
-template <typename OutT>
+template <int BN, typename OutT>
 int launch_tiled_large(const bf16_t* x, const bf16_t* w, OutT y, int m, int n, int k, int columns, hipStream_t stream) {
-  const int col_blocks = (columns + 255) / 256, row_blocks = (m + 255) / 256;
-  launch_tiled_kernel<256, 256, 64, 2, false, OutT, 4, 2>(x, w, y, m, n, k, col_blocks, row_blocks, 1, {nullptr, 0}, stream);
+  const int col_blocks = (columns + BN - 1) / BN, row_blocks = (m + 255) / 256;
+  launch_tiled_kernel<256, BN, 64, 2, false, OutT, 4, 2>(x, w, y, m, n, k, col_blocks, row_blocks, 1, {nullptr, 0}, stream);
   return 2 * col_blocks;
 }
 
@@ -1003,7 +1003,7 @@ int launch_tiled(const bf16_t* x, const bf16_t* w, OutT y, int m, int n, int k, 
   return launch_tiled_staged<BM, BN, BK, 3, OutT>(x, w, y, m, n, k, col_blocks, row_blocks, ksplit, ws, stream);
 }
 
-// 2: 64x128, 3: 64x64, 4: 256x256 -- the larger tile when it still gives (nearly) every compute unit a block.
+// 2: 64x128, 3: 64x64, 4: 256x256, 5: 256x192 -- the larger tile when it still gives (nearly) every compute unit a block.
 // (A tile of 128x128 was measured slower than 64x128 on every product from 2048 x 576 x 576 to 2048 x 6144 x 2048;
 // the tile of 256x256 against 64x128, microseconds: 2048 x 6144 x 2048, 192 blocks, 57 against 68; 2048 x 11264 x
 // 2048, 352 blocks, 108 against 119; but 2048 x 2560 x 2048, 80 blocks, 48 against 34, and 2048 x 2048 x 8192, 64
@@ -1013,17 +1013,24 @@ int launch_tiled(const bf16_t* x, const bf16_t* w, OutT y, int m, int n, int k, 
 #endif
 int pick_tile(int m, int columns, int k, int tile_hint) {
   const long long blocks_64_128 = (long long)((m + 63) / 64) * ((columns + 127) / 128);
-  const long long blocks_256_256 = (long long)((m + 255) / 256) * ((columns + 255) / 256);
+  const long long rows_256 = (m + 255) / 256;
+  const long long blocks_256_256 = rows_256 * ((columns + 255) / 256), blocks_256_192 = rows_256 * ((columns + 191) / 192);
   int tile = blocks_64_128 >= 256 ? 2 : 3;
-  if (blocks_256_256 >= NNIS_LARGE_TILE_BLOCKS && k >= 256) tile = 4;
-  if (tile_hint >= 2 && tile_hint <= 4) tile = tile_hint;  // for tuning runs
+  if (blocks_256_256 >= NNIS_LARGE_TILE_BLOCKS && k >= 256) {
+    // a compute unit runs one large tile at a time: of the two widths, the one whose rounds of blocks come to
+    // fewer columns a compute unit (2048 x 6144: 192 blocks of 256 columns or 256 of 192, a round either way)
+    const long long units = 256;
+    const long long cost_256 = ((blocks_256_256 + units - 1) / units) * 256, cost_192 = ((blocks_256_192 + units - 1) / units) * 192;
+    tile = cost_192 < cost_256 ? 5 : 4;
+  }
+  if (tile_hint >= 2 && tile_hint <= 5) tile = tile_hint;  // for tuning runs
   return tile;
 }
 
 // the most parts of a row's sum of squares that a residual epilogue of the tiled kernel writes for these sizes
 int tiled_parts(int m, int columns, int k, int tile_hint) {
   const int tile = pick_tile(m, columns, k, tile_hint);
-  const int width = tile == 4 ? 256 : (tile == 2 ? 128 : 64);
+  const int width = tile == 4 ? 256 : (tile == 5 ? 192 : (tile == 2 ? 128 : 64));
   return 2 * ((columns + width - 1) / width);  // with K in parts: one per 64 columns, which is no more
 }
 
@@ -1033,7 +1040,8 @@ int dispatch_tiled(const bf16_t* x, const bf16_t* w, OutT y, int m, int n, int k
                    int columns = 0) {
   if (columns <= 0) columns = n;
   const int tile = pick_tile(m, columns, k, tile_hint);
-  if (tile == 4) return launch_tiled_large<OutT>(x, w, y, m, n, k, columns, stream);
+  if (tile == 4) return launch_tiled_large<256, OutT>(x, w, y, m, n, k, columns, stream);
+  if (tile == 5) return launch_tiled_large<192, OutT>(x, w, y, m, n, k, columns, stream);
   if (tile == 2) return launch_tiled<64, 128, 64, OutT>(x, w, y, m, n, k, columns, ws, stream);
   return launch_tiled<64, 64, 64, OutT>(x, w, y, m, n, k, columns, ws, stream);
 }
@@ -1125,7 +1133,7 @@ extern "C" int nnis_gemm_bf16(const void* x, const void* w, void* y, int y_dtype
     NNIS_LAUNCH_CHECK("gemm_skinny");
   } else {
     NNIS_REQUIRE((m + 63) / 64 <= 65535, "gemm_bf16: %d rows exceed the grid limit", m);
-    const int tile_hint = split_hint >= 16 ? split_hint / 16 : 0;  // hints of 32, 48 and 64 pick the tile: 64x128, 64x64, 256x256
+    const int tile_hint = split_hint >= 16 ? split_hint / 16 : 0;  // hints of 32, 48, 64 and 80 pick the tile: 64x128, 64x64, 256x256, 256x192
     if (y_dtype == NNIS_F32) dispatch_tiled<float*>(xp, wp, (float*)y, m, n, k, tile_hint, ws, stream);
     else dispatch_tiled<bf16_t*>(xp, wp, (bf16_t*)y, m, n, k, tile_hint, ws, stream);
     NNIS_LAUNCH_CHECK("gemm_tiled");
@@ -1156,7 +1164,7 @@ extern "C" int nnis_gemm_residual(const void* x, const void* w, float* resid, co
   hipStream_t stream = (hipStream_t)stream_ptr;
   ResidualOut out = {resid, gain, gain_dtype, (bf16_t*)scaled, ss};
   NNIS_REQUIRE((uintptr_t)workspace % 16 == 0, "gemm_residual: the workspace must be 16-byte aligned");
-  NNIS_REQUIRE(tile_hint == 0 || (tile_hint >= 2 && tile_hint <= 4), "gemm_residual: unknown tile %d", tile_hint);
+  NNIS_REQUIRE(tile_hint == 0 || (tile_hint >= 2 && tile_hint <= 5), "gemm_residual: unknown tile %d", tile_hint);
   const bool few = tile_hint == 0 && takes_few_tokens_with_parts(m, n, k, workspace != nullptr);  // a tile hint asks for the tiled kernel
   const int writes = few ? (n + 15) / 16 : tiled_parts(m, n, k, tile_hint);
   NNIS_REQUIRE(writes <= ss_rows, "gemm_residual: ss has %d rows of %d tokens, %d are needed", ss_rows, m, writes);
