@@ -1016,7 +1016,8 @@ int pick_tile(int m, int columns, int k, int tile_hint) {
   const long long rows_256 = (m + 255) / 256;
   const long long blocks_256_256 = rows_256 * ((columns + 255) / 256), blocks_256_192 = rows_256 * ((columns + 191) / 192);
   int tile = blocks_64_128 >= 256 ? 2 : 3;
-  if (blocks_256_256 >= NNIS_LARGE_TILE_BLOCKS && k >= 256) {
+  // (rows that fill three quarters of their tiles of 256 at least: 300 rows would be multiplied as 512)
+  if (blocks_256_256 >= NNIS_LARGE_TILE_BLOCKS && k >= 256 && 4LL * m >= 3 * 256 * rows_256) {
     // a compute unit runs one large tile at a time: of the two widths, the one whose rounds of blocks come to
     // fewer columns a compute unit (2048 x 6144: 192 blocks of 256 columns or 256 of 192, a round either way)
     const long long units = 256;
