@@ -343,46 +343,57 @@ __device__ __forceinline__ const bf16_t* v_page_ptr(const MfmaArgs& a, int page,
   return a.v_pages + ((size_t)page * a.kv_heads + kv_head) * nnis_v_page_elems(HD);
 }
 
+// A wave's state in LDS, for another wave to take in: per column the output tiles as 16 bytes a lane
+// ([tile][lane][4]: one store or load a tile), then the reference and the sum ([lane] each);
+// kStateFloats floats a column.
+constexpr int kStateFloats = (kTilesD * 4 + 2) * kWave;
+
+template <int C>
+__device__ __forceinline__ void leave_state(const AttnState<C>& st, float* slot, int lane) {
+#pragma unroll
+  for (int c = 0; c < C; ++c) {
+    float* col = slot + (size_t)c * kStateFloats;
+#pragma unroll
+    for (int t = 0; t < kTilesD; ++t) *(f32x4*)(col + (t * kWave + lane) * 4) = st.o[c][t];
+    col[kTilesD * 4 * kWave + lane] = st.m[c];
+    col[(kTilesD * 4 + 1) * kWave + lane] = st.l[c];
+  }
+}
+
+// st becomes the softmax state of its keys and the other wave's together
+template <int C>
+__device__ __forceinline__ void take_state(AttnState<C>& st, const float* slot, int lane) {
+#pragma unroll
+  for (int c = 0; c < C; ++c) {
+    const float* col = slot + (size_t)c * kStateFloats;
+    const float m_other = col[kTilesD * 4 * kWave + lane];
+    const float l_other = col[(kTilesD * 4 + 1) * kWave + lane];
+    f32x4 theirs[kTilesD];
+#pragma unroll
+    for (int t = 0; t < kTilesD; ++t) theirs[t] = *(const f32x4*)(col + (t * kWave + lane) * 4);
+    const float m_new = fmaxf(st.m[c], m_other);
+    const float m_safe = m_new == -INFINITY ? 0.0f : m_new;
+    const float mine_w = __builtin_amdgcn_exp2f(st.m[c] - m_safe);
+    const float their_w = __builtin_amdgcn_exp2f(m_other - m_safe);
+    st.l[c] = st.l[c] * mine_w + l_other * their_w;
+    st.m[c] = m_new;
+#pragma unroll
+    for (int t = 0; t < kTilesD; ++t)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) st.o[c][t][e] = st.o[c][t][e] * mine_w + theirs[t][e] * their_w;
+  }
+}
+
 // Waves of a block (a power of two) that dealt a run of key blocks among themselves fold their states
 // into wave 0's, in halving rounds: the upper half of the waves still in play leave their states in LDS,
 // the lower half take one each.  Returns false for the waves that are done.  `merge` holds
 // [waves / 2][C][kTilesD * 4 + 2][64] floats.
 template <int C>
 __device__ __forceinline__ bool merge_waves(AttnState<C>& st, float* merge, int wave, int waves, int lane) {
-  constexpr int kValues = kTilesD * 4 + 2;
   for (int half = waves >> 1; half >= 1; half >>= 1) {
-    if (wave >= half && wave < 2 * half) {
-      float* mine = merge + (size_t)(wave - half) * C * kValues * kWave;
-#pragma unroll
-      for (int c = 0; c < C; ++c) {
-        float* col = mine + (size_t)c * kValues * kWave + lane;
-#pragma unroll
-        for (int t = 0; t < kTilesD; ++t)
-#pragma unroll
-          for (int e = 0; e < 4; ++e) col[(4 * t + e) * kWave] = st.o[c][t][e];
-        col[(kTilesD * 4) * kWave] = st.m[c];
-        col[(kTilesD * 4 + 1) * kWave] = st.l[c];
-      }
-    }
+    if (wave >= half && wave < 2 * half) leave_state<C>(st, merge + (size_t)(wave - half) * C * kStateFloats, lane);
     __syncthreads();
-    if (wave < half) {
-      const float* theirs = merge + (size_t)wave * C * kValues * kWave;
-#pragma unroll
-      for (int c = 0; c < C; ++c) {
-        const float* col = theirs + (size_t)c * kValues * kWave + lane;
-        const float m_other = col[(kTilesD * 4) * kWave];
-        const float m_new = fmaxf(st.m[c], m_other);
-        const float m_safe = m_new == -INFINITY ? 0.0f : m_new;
-        const float mine_w = __builtin_amdgcn_exp2f(st.m[c] - m_safe);
-        const float their_w = __builtin_amdgcn_exp2f(m_other - m_safe);
-        st.l[c] = st.l[c] * mine_w + col[(kTilesD * 4 + 1) * kWave] * their_w;
-        st.m[c] = m_new;
-#pragma unroll
-        for (int t = 0; t < kTilesD; ++t)
-#pragma unroll
-          for (int e = 0; e < 4; ++e) st.o[c][t][e] = st.o[c][t][e] * mine_w + col[(4 * t + e) * kWave] * their_w;
-      }
-    }
+    if (wave < half) take_state<C>(st, merge + (size_t)wave * C * kStateFloats, lane);
     if (half > 1) __syncthreads();  // the next round writes where this one read
   }
   return wave == 0;
@@ -394,42 +405,12 @@ __device__ __forceinline__ bool merge_waves(AttnState<C>& st, float* merge, int 
 // meet at the same barriers; a group that is done early only waits.  Returns true for the member that is left.
 template <int C>
 __device__ __forceinline__ bool merge_group(AttnState<C>& st, float* slots, int index, int size, int rounds, int lane) {
-  constexpr int kValues = kTilesD * 4 + 2;
   int n = size;
   for (int round = 0; round < rounds; ++round) {
     const int keep = (n + 1) / 2;  // members [keep, n) hand over to members [0, n - keep)
-    if (index >= keep && index < n) {
-      float* mine = slots + (size_t)(index - keep) * C * kValues * kWave;
-#pragma unroll
-      for (int c = 0; c < C; ++c) {
-        float* col = mine + (size_t)c * kValues * kWave + lane;
-#pragma unroll
-        for (int t = 0; t < kTilesD; ++t)
-#pragma unroll
-          for (int e = 0; e < 4; ++e) col[(4 * t + e) * kWave] = st.o[c][t][e];
-        col[(kTilesD * 4) * kWave] = st.m[c];
-        col[(kTilesD * 4 + 1) * kWave] = st.l[c];
-      }
-    }
+    if (index >= keep && index < n) leave_state<C>(st, slots + (size_t)(index - keep) * C * kStateFloats, lane);
     __syncthreads();
-    if (index < n - keep) {
-      const float* theirs = slots + (size_t)index * C * kValues * kWave;
-#pragma unroll
-      for (int c = 0; c < C; ++c) {
-        const float* col = theirs + (size_t)c * kValues * kWave + lane;
-        const float m_other = col[(kTilesD * 4) * kWave];
-        const float m_new = fmaxf(st.m[c], m_other);
-        const float m_safe = m_new == -INFINITY ? 0.0f : m_new;
-        const float mine_w = __builtin_amdgcn_exp2f(st.m[c] - m_safe);
-        const float their_w = __builtin_amdgcn_exp2f(m_other - m_safe);
-        st.l[c] = st.l[c] * mine_w + col[(kTilesD * 4 + 1) * kWave] * their_w;
-        st.m[c] = m_new;
-#pragma unroll
-        for (int t = 0; t < kTilesD; ++t)
-#pragma unroll
-          for (int e = 0; e < 4; ++e) st.o[c][t][e] = st.o[c][t][e] * mine_w + col[(4 * t + e) * kWave] * their_w;
-      }
-    }
+    if (index < n - keep) take_state<C>(st, slots + (size_t)index * C * kStateFloats, lane);
     if (round + 1 < rounds) __syncthreads();  // the next round writes where this one read
     n = keep;
   }
@@ -517,7 +498,7 @@ constexpr int kPrefillRing = HD > 64 ? 2 : (C <= 2 ? NNIS_PREFILL_RING_NARROW : 
 template <int QT, int GH>
 __global__ __launch_bounds__(64 * kBlockWaves) void attention_prefill_kernel(MfmaArgs a, int waves, int items, int singles,
                                                                             int per_tile) {
-  extern __shared__ float merge[];
+  extern __shared__ __attribute__((aligned(16))) float merge[];
   constexpr int C = QT * GH;
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave, r = lane % 16, g = lane / 16;
   const int group = a.heads / a.kv_heads;
@@ -624,9 +605,8 @@ __global__ __launch_bounds__(64 * kBlockWaves) void attention_prefill_kernel(Mfm
       first_share = 2 * ((waves * pages_of[0] + pages_of[0] + pages_of[1]) / (2 * (pages_of[0] + pages_of[1])));
       first_share = first_share < 2 ? 2 : (first_share > waves - 2 ? waves - 2 : first_share);
     }
-    constexpr int kValues = kTilesD * 4 + 2;
     if (wave < first_share) run_item(0, wave, first_share, merge, rounds);
-    else run_item(1, wave - first_share, waves - first_share, merge + (size_t)(first_share / 2) * C * kValues * kWave, rounds);
+    else run_item(1, wave - first_share, waves - first_share, merge + (size_t)(first_share / 2) * C * kStateFloats, rounds);
   }
 }
 
@@ -679,7 +659,7 @@ __device__ __forceinline__ void finish_decode(AttnState<C>& st, const bool (&liv
 // more than one split every block leaves its state in `partial` for the combine kernel.
 template <int C>
 __global__ __launch_bounds__(64 * kBlockWaves) void attention_decode_kernel(MfmaArgs a, int waves) {
-  extern __shared__ float merge[];  // [waves / 2][C][kTilesD * 4 + 2][64]
+  extern __shared__ __attribute__((aligned(16))) float merge[];  // [waves / 2][C][kTilesD * 4 + 2][64]
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave, r = lane % 16, g = lane / 16;
   const int token = blockIdx.x, kv_head = blockIdx.y, split = blockIdx.z;
   // With the step's tables a token's pages are a row of its own and nothing is asked of its slot: the first
@@ -751,7 +731,7 @@ __device__ __forceinline__ bf16x4 low4(bf16x8 v) { return __builtin_shufflevecto
 __device__ __forceinline__ bf16x4 high4(bf16x8 v) { return __builtin_shufflevector(v, v, 4, 5, 6, 7); }
 
 __global__ __launch_bounds__(64 * kKeysWaves) void attention_decode_keys_kernel(MfmaArgs a, int waves) {
-  extern __shared__ float merge[];  // [waves / 2][kTilesD * 4 + 2][64]
+  extern __shared__ __attribute__((aligned(16))) float merge[];  // [waves / 2][kTilesD * 4 + 2][64]
   constexpr int kStageRow = kPageTokens + 8;  // bfloat16 per head: a page's probabilities, rows apart in the banks
   __shared__ __attribute__((aligned(16))) bf16_t stage[kKeysWaves][4][kStageRow];
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave, r = lane % 16, g = lane / 16;
