@@ -620,7 +620,11 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_tiled_kernel(const bf16_t
   asm volatile("" ::: "memory");
   int stage = 0;
   for (int step = step0; step < step1; ++step) {
-    ask(step + NS - 1, stage == 0 ? NS - 1 : stage - 1);
+    // The tile of 256 x 256 asks for the next step between its two halves, under the first half's products
+    // (2048 x 16384 x 2048 137 us against 141, 6224 x 11264 x 2048 277 against 294); the tile of 256 x 192, whose
+    // steps are shorter, loses by the later start of its loads (2048 x 11264 x 2048 105 against 95).
+    constexpr bool kAskBetween = TM * TN > 16 && BN >= 256;
+    if constexpr (!kAskBetween) ask(step + NS - 1, stage == 0 ? NS - 1 : stage - 1);
     const bf16x8* a_tile = (const bf16x8*)(tile_lds + stage * STAGE_BYTES);
     const bf16x8* b_tile = (const bf16x8*)(tile_lds + stage * STAGE_BYTES + A_BYTES);
     static_assert(BK == 64, "two halves of 32 k a step");
@@ -663,6 +667,9 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_tiled_kernel(const bf16_t
         for (int jj = 0; jj < TN; ++jj)
 #pragma unroll
           for (int i = 0; i < TM; ++i) acc[i][jj] = mfma(b_frag[jj], a_frag[i], acc[i][jj]);
+        if constexpr (kAskBetween) {
+          if (half == 0) ask(step + NS - 1, stage == 0 ? NS - 1 : stage - 1);
+        }
       }
     }
     // what this wave read of its stage has arrived too: the stage is the next step's to fill
