@@ -12,10 +12,11 @@
 //    registers; a wave owns a strip of 16 weight rows; X (small, shared by all
 //    waves) comes through the caches.  Waves of a block may split K and add
 //    their parts through LDS.
-//  * gemm_tiled_kernel: any M (prefill).  64x128 or 64x64 output tiles, K in
-//    steps of 64 that go from memory straight into LDS, a ring of stages
-//    deep, with an XOR swizzle of the 16-byte chunks so that operand reads
-//    are free of bank conflicts.
+//  * gemm_tiled_kernel: any M (prefill).  64x128 or 64x64 output tiles of 4
+//    waves, or, where a product still fills the chip with them, 256x256 or
+//    256x192 tiles of 8 waves; K in steps of 64 that go from memory straight
+//    into LDS, a ring of stages deep, with an XOR swizzle of the 16-byte
+//    chunks so that operand reads are free of bank conflicts.
 //
 // Both need K % 8 == 0 and 16-byte aligned operands (the host checks) and take
 // any M and N.
