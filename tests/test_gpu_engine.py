@@ -571,3 +571,88 @@ def test_a_sequence_cut_back_goes_on_from_there(model_dirs, dtype):
     engine.reset(slot)
     rows = engine.step([StepEntry(slot, first[:5], [4])])
     _close(rows.cpu(), plain.logits(first[:5])[4:5], dtype, "reset and used again", yard)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name, seed", [("A", 1), ("B", 2), ("C", 3), ("B", 4)])
+def test_schedules_drawn_from_a_seed(model_dirs, name, seed, dtype):
+    """Sequences are started, fed in pieces of a length drawn at random (whole
+    prompts, a few tokens, one token; sequences that start, go on with several
+    tokens and go on with one token side by side in a step), cut back, reset
+    and ended in an order drawn from the seed, in a cache of ten pages, so
+    that slots and pages change hands all the time.  Every wanted row is the
+    plain model's row for the sequence as it then is; a step that does not
+    fit is refused and leaves everything as it was."""
+    from nnis_amd.engine.batch import StepEntry
+    from nnis_amd.errors import CacheFull
+
+    config, _ = TINY_CONFIGS[name]
+    rng = np.random.default_rng(1000 + seed)
+    plain = P.PlainLlama(model_dirs[name])
+    yard = _yard(model_dirs, name) if dtype == "bfloat16" else None
+    engine = _engine(model_dirs, name, dtype, max_tokens=10 * 64)
+    longest = min(300, config["max_position_embeddings"])
+    live = {}  # slot -> [ids, their logits, tokens fed]
+
+    def start():
+        ids = rng.integers(0, config["vocab_size"], size=int(rng.integers(1, longest + 1))).tolist()
+        live[engine.start_sequence()] = [ids, plain.logits(ids), 0]
+
+    checked = 0
+    for turn in range(150):
+        action = rng.random()
+        if len(live) < 2 or (action < 0.15 and len(live) < 5):
+            start()
+            continue
+        slot = int(rng.choice(sorted(live)))
+        ids, want, fed = live[slot]
+        if action < 0.25:
+            engine.end_sequence(slot)
+            del live[slot]
+            continue
+        if action < 0.35 and fed > 1:  # cut back: other tokens follow from there
+            keep = int(rng.integers(1, fed))
+            engine.truncate(slot, keep)
+            room = min(40, config["max_position_embeddings"] - keep)
+            ids = ids[:keep] + rng.integers(0, config["vocab_size"], size=int(rng.integers(1, room + 1))).tolist()
+            live[slot] = [ids, plain.logits(ids), keep]
+            continue
+        if action < 0.4:
+            engine.reset(slot)
+            live[slot][2] = 0
+            continue
+        # a step of some of the live sequences that still have tokens to feed
+        some = [s for s in sorted(live) if live[s][2] < len(live[s][0]) and rng.random() < 0.7]
+        if not some:
+            continue
+        one_each = rng.random() < 0.4  # a step of single tokens (replayed from a graph), else pieces of any length
+        entries, places = [], []
+        for s in some:
+            ids, want, fed = live[s]
+            left = len(ids) - fed
+            count = 1 if one_each else int(min(left, rng.choice([1, 2, 7, 64, 65, left])))
+            wanted = sorted(set(rng.integers(0, count, size=int(rng.integers(0, 4))).tolist()))
+            entries.append(StepEntry(s, ids[fed:fed + count], wanted))
+            places.append((s, fed, count, wanted))
+        lengths = {s: engine.length(s) for s in live}
+        free = engine.free_pages()
+        try:
+            rows = engine.step(entries)
+        except CacheFull:  # more pages than the cache has left: nothing has changed, and a sequence makes room
+            assert {s: engine.length(s) for s in live} == lengths and engine.free_pages() == free
+            victim = max(live, key=lambda s: engine.length(s))
+            engine.end_sequence(victim)
+            del live[victim]
+            continue
+        expect = [live[s][1][fed + p] for s, fed, _, wanted in places for p in wanted]
+        assert rows.shape[0] == len(expect)
+        if expect:
+            _close(rows.cpu(), torch.stack(expect), dtype, f"tiny {name} {dtype} seed {seed} turn {turn}", yard)
+            checked += len(expect)
+        for s, fed, count, _ in places:
+            live[s][2] = fed + count
+            assert engine.length(s) == fed + count
+    assert checked >= 60
+    for slot in list(live):
+        engine.end_sequence(slot)
+    assert engine.free_pages() == 10
