@@ -72,9 +72,9 @@ class DecodeGraph:
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
         self.graph = torch.cuda.CUDAGraph()
-        # A graph that the cycle collector destroys while another is being captured aborts the process:
-        # collect now, and keep the collector off until the capture ends.
-        gc.collect()
+        # A graph that the cycle collector destroys while another is being captured aborts the process: the
+        # collector stays off until the capture ends.  (Graphs hold their engine weakly, so an engine that is
+        # dropped takes its graphs with it at once; a full collection here cost 30 ms a capture, most of it.)
         collecting = gc.isenabled()
         gc.disable()
         try:
@@ -216,8 +216,7 @@ class PrefillGraph:
             return None  # (a work list that the shape's record does not name: the caller runs the step as any step)
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
-        gc.collect()  # (as for the decode graphs: no graph may be destroyed while one is captured)
-        collecting = gc.isenabled()
+        collecting = gc.isenabled()  # (as for the decode graphs: no graph may be destroyed while one is captured)
         gc.disable()
         try:
             with torch.cuda.graph(graph):
