@@ -140,12 +140,14 @@ class DecodeGraphs:
 # Prompt steps whose shape comes again
 # ---------------------------------------------------------------------------------------------
 # A step over a few thousand tokens launches 150 kernels and more; where the model is small the host
-# needs as long to launch them as the GPU to run them.  A step's *shape* -- how many new tokens each of
-# its sequences brings, how many logit rows are wanted, and the class of its longest sequence (which
-# picks the attention kernels' plan) -- fixes every launch; tokens, slots, positions and the order of the
-# attention's work items are data.  The second time a shape comes it is captured into a graph whose
-# kernels read that data from fixed buffers; from the third time on the step is a copy into the buffers
-# and a replay.  Only shapes of up to PREFILL_GRAPH_MOST_TOKENS tokens are kept, the most recently used
+# needs as long to launch them as the GPU to run them.  A step's *shape* -- how many sequences it has, how
+# many tokens in all (rounded up: ``prefill_rows``), how many logit rows are wanted, and the class of its
+# longest sequence (which picks the attention kernels' plan) -- fixes every launch; tokens, slots,
+# positions, how the tokens divide among the sequences and the attention's work items are data.  The rows
+# beyond a step's tokens belong to no sequence (slot -1): every kernel computes them like any row and writes
+# nothing of them into the cache, and the attention's work lists are filled up with items that have no rows.
+# The second time a shape comes it is captured into a graph whose kernels read that data from fixed
+# buffers; from the third time on the step is a copy into the buffers and a replay.  Only shapes of up to PREFILL_GRAPH_MOST_TOKENS tokens are kept, the most recently used
 # PREFILL_GRAPHS_KEPT of them (a graph keeps its activations' memory), and only where the step's kernels are
 # short enough for the host to matter: tokens x width^2 up to PREFILL_GRAPH_MOST_WORK.  Measured, one prompt a
 # step, launched against replayed, milliseconds: width 576, 30 layers: 64 tokens 2.27 / 0.83, 256 2.33 / 1.33,
@@ -153,20 +155,32 @@ class DecodeGraphs:
 # 2.77 / 2.75, from 1,024 on equal (4.24, 7.28): there the kernels bound the step and a graph would only hold memory.
 PREFILL_GRAPH_MOST_TOKENS = 4096
 PREFILL_GRAPH_MOST_WORK = 1.5e9
-PREFILL_GRAPHS_KEPT = 4
+PREFILL_GRAPHS_KEPT = 16
+
+
+def prefill_rows(total: int) -> int:
+    """Rows of the replayed prompt step that takes ``total`` tokens: the next multiple of 64 up to 1,024
+    tokens, of 128 up to 2,048, of 256 beyond."""
+    unit = 64 if total <= 1024 else (128 if total <= 2048 else 256)
+    return ((total + unit - 1) // unit) * unit
+
+
+# a work item of the attention that has no rows: its first row lies beyond any sequence's tokens
+_NO_ROWS = 1 << 24
 
 
 class PrefillGraph:
-    def __init__(self, engine, counts: Sequence[int], wanted: int, plan_class: int, tile_rows: Sequence[int]):
+    def __init__(self, engine, batch: int, total: int, wanted: int, plan_class: int, tile_rows: Sequence[int]):
+        """``total``: the rows of the step (``prefill_rows`` of its tokens), ``batch``: its sequences."""
         self.engine = engine if isinstance(engine, weakref.ProxyTypes) else weakref.proxy(engine)
         ops = engine.rt.ops
         device = engine.rt.device
-        self.counts = list(counts)
-        total, batch = sum(counts), len(counts)
+        self.total = total
         # the step's arrays in one buffer, in the order the step function stages them
         self.sizes = [total, total, total, batch, batch + 1, batch, wanted]
         self.tile_rows = list(tile_rows)
-        self.tile_counts = [sum((n + rows - 1) // rows for n in counts) for rows in self.tile_rows]
+        # the most tiles of `rows` rows that `batch` sequences with `total` tokens between them can have
+        self.tile_counts = [total // rows + batch for rows in self.tile_rows]
         sizes = self.sizes + [2 * n for n in self.tile_counts]
         self.spans, offset = [], 0
         for size in sizes:
@@ -181,23 +195,32 @@ class PrefillGraph:
         self.ids, self.want_rows = views[0], views[6]
         self.ctx = StepContext(
             tokens=total, batch=batch, tok_slot=views[1], tok_pos=views[2], seq_slot=views[3], seq_start=views[4],
-            seq_pos0=views[5], decode=False, max_new=max(counts), max_len=ops.PREFILL_CLASS_LENGTH[plan_class],
+            seq_pos0=views[5], decode=False, max_new=total, max_len=ops.PREFILL_CLASS_LENGTH[plan_class],
             host_new=None, host_pos0=None, tiles=tiles)  # (no host lists: a work list that is not in `tiles` is an error)
         self.graph = None
         self.logits = None
 
-    def fill(self, arrays, first_positions: Sequence[int]) -> None:
+    def fill(self, arrays, counts: Sequence[int], first_positions: Sequence[int]) -> None:
         """The step's data into the buffers: ``arrays`` as the step function stages them (ids, slot and position
-        of each token, slot, first row and first position of each sequence, wanted rows)."""
+        of each token, slot, first row and first position of each sequence, wanted rows); ``counts``: the
+        tokens each sequence brings.  Rows beyond the tokens get id 0, slot -1, position 0."""
         ops = self.engine.rt.ops
         self.copied.synchronize()  # the previous copy has left the pinned buffer
         host = self.host.numpy()
-        for (offset, size), array in zip(self.spans, arrays):
-            host[offset:offset + size] = array
+        tokens = sum(counts)
+        for index, ((offset, size), array) in enumerate(zip(self.spans, arrays)):
+            if index < 3:
+                host[offset:offset + tokens] = array
+                host[offset + tokens:offset + size] = -1 if index == 1 else 0
+            else:
+                host[offset:offset + size] = array
         for (offset, _), rows, n in zip(self.spans[7:], self.tile_rows, self.tile_counts):
-            seqs, row0s = ops.prefill_tile_items(self.counts, first_positions, rows)
-            host[offset:offset + n] = seqs
-            host[offset + n:offset + 2 * n] = row0s
+            seqs, row0s = ops.prefill_tile_items(counts, first_positions, rows)
+            have = len(seqs)
+            host[offset:offset + have] = seqs
+            host[offset + have:offset + n] = 0
+            host[offset + n:offset + n + have] = row0s
+            host[offset + n + have:offset + 2 * n] = _NO_ROWS
         self.meta.copy_(self.host, non_blocking=True)
         self.copied.record()
 
@@ -245,13 +268,14 @@ class PrefillGraphs:
         self.refused = set()  # shapes whose capture failed
         self.graphs: Dict[tuple, PrefillGraph] = {}  # in the order of their last use
 
-    def step(self, key: tuple, arrays, first_positions: Sequence[int], tile_rows):
+    def step(self, key: tuple, arrays, counts: Sequence[int], first_positions: Sequence[int], tile_rows):
         """(logits, borrowed) if this step is replayed or captured; None if it is to run as any step.
-        ``tile_rows``: called for the row counts of the attention's work lists the shape's eager run made."""
+        ``key``: (sequences, rows, wanted logit rows, plan class); ``tile_rows``: called for the row counts of
+        the attention's work lists that the shape's eager run made."""
         graph = self.graphs.pop(key, None)
         if graph is not None:
             self.graphs[key] = graph  # the most recently used is last
-            graph.fill(arrays, first_positions)
+            graph.fill(arrays, counts, first_positions)
             return graph.run(), True
         if key in self.refused:
             return None
@@ -262,9 +286,9 @@ class PrefillGraphs:
         rows = tile_rows()
         if times < 2 or rows is None:
             return None
-        counts, wanted, plan_class = key
-        graph = PrefillGraph(self.engine, counts, wanted, plan_class, rows)
-        graph.fill(arrays, first_positions)
+        batch, total, wanted, plan_class = key
+        graph = PrefillGraph(self.engine, batch, total, wanted, plan_class, rows)
+        graph.fill(arrays, counts, first_positions)
         logits = graph.first_run()
         if graph.graph is None:
             self.refused.add(key)

@@ -256,10 +256,11 @@ def test_selector_refuses_a_row_that_is_not_finite(model_dirs):
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_prompt_steps_whose_shape_comes_again(model_dirs, dtype):
-    """The second time a step's shape comes (new tokens per sequence, wanted rows, class of the longest
-    sequence) it is captured, from the third time on replayed: with other tokens, other slots, other first
-    positions (a prompt's second run of tokens) and other wanted places each time, the logits are the plain
-    model's; shapes beyond the kept few push the oldest out, and a shape that comes back is captured again."""
+    """The second time a step's shape comes (sequences, tokens in all rounded up to a multiple of 64, wanted
+    rows, class of the longest sequence) it is captured, from the third time on replayed: with other tokens,
+    other slots, other first positions (a prompt's second run of tokens), other wanted places and the tokens
+    divided otherwise among the sequences each time, the logits are the plain model's; shapes beyond the
+    kept few push the oldest out, and a shape that comes back is captured again."""
     from nnis_amd.engine import graph as G
     from nnis_amd.engine.batch import StepEntry
 
@@ -297,36 +298,43 @@ def test_prompt_steps_whose_shape_comes_again(model_dirs, dtype):
     run([37, 5, 70], [0, 0, 0], [[0, 36], None, [69]])
     run([37, 5, 70], [0, 0, 0], [[1, 2], None, [3]])
     graphs = engine._prefill_graphs.graphs
-    assert len(graphs) == 1
+    of_three = lambda: [key for key in graphs if key[0] == 3]  # noqa: E731  (single prompts here share a graph of their own)
+    assert of_three() == [(3, 128, 4, 0)]
     other = engine.start_sequence()
     engine.step([StepEntry(other, [4, 5], None)])
     run([37, 5, 70], [3, 20, 0], [[36, 0], None, [10]])
     run([37, 5, 70], [0, 9, 30], [None, [4], [0, 69]])
     engine.end_sequence(keeper)
     run([37, 5, 70], [11, 0, 1], [[5], [0, 4], None])
-    assert len(graphs) == 1
+    assert len(of_three()) == 1
+    # the same rows (128), divided otherwise and not filled: the same graph, whose last rows belong to no sequence
+    run([40, 2, 70], [0, 0, 0], [[0, 39], None, [69]])
+    run([30, 30, 30], [5, 0, 64], [None, [0, 29], [7]])
+    run([1, 64, 1], [0, 0, 0], [[0], [0, 63], None])
+    run([64, 63, 1], [0, 1, 2], [[63], [0, 62], None])
+    assert len(of_three()) == 1
     # a longer first position puts the step into another class of the attention's plan: a shape of its own
     run([37, 5, 70], [0, 0, 100], [[0, 36], None, [69]])
     run([37, 5, 70], [0, 0, 100], [[0, 36], None, [69]])
-    assert len(graphs) == 2
+    assert len(of_three()) == 2
     # more shapes than are kept: the oldest goes, and comes back through a new capture
-    first = next(iter(graphs))
+    first = of_three()[0]
     for n in range(G.PREFILL_GRAPHS_KEPT):
         for _ in range(3):
-            run([3 + n], [0], [None])
+            run([3] * (n + 5), [0] * (n + 5), [None] * (n + 5))
     assert len(graphs) == G.PREFILL_GRAPHS_KEPT and first not in graphs
     for _ in range(3):
         run([37, 5, 70], [0, 0, 0], [[0, 36], None, [69]])
     assert first in graphs
     # a step that cannot be captured (here: a work list that the record of the shape's first run does not name)
     # is launched as any step, this time and from then on
-    run([21, 40], [0, 0], [None, None])
-    (shape,) = [key for key in engine._tile_rows if key[0] == (21, 40)]
+    run([21, 40], [0, 0], [[0, 1, 2], [3, 4, 5]])
+    (shape,) = [key for key in engine._tile_rows if key[:3] == (2, 64, 6)]
     if engine._tile_rows[shape]:  # (the 32-bit attention has no work lists)
         engine._tile_rows[shape] = []
         kept = list(graphs)
         for _ in range(3):
-            run([21, 40], [0, 0], [[0], [5]])
+            run([21, 40], [0, 0], [[0, 7, 8], [5, 6, 9]])
         assert shape in engine._prefill_graphs.refused and list(graphs) == kept
     engine.end_sequence(other)
     assert engine.free_slots() == engine.cache.max_slots
