@@ -664,3 +664,27 @@ def test_schedules_drawn_from_a_seed(model_dirs, name, seed, dtype):
     for slot in list(live):
         engine.end_sequence(slot)
     assert engine.free_pages() == 10
+
+
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_greedy_requests_drawn_from_a_seed(model_dirs, name):
+    """Batches of one to eight requests with prompts, limits, stop sets and
+    a batch size drawn from a seed, through the generation loop in 32-bit, in
+    a cache of twelve pages: the tokens are the plain model's greedy ones (a
+    stop token is kept, as the reference keeps it), and every page comes back."""
+    from nnis_amd.engine.generate import GenerationRequest, generate
+
+    config, _ = TINY_CONFIGS[name]
+    plain = P.PlainLlama(model_dirs[name])
+    engine = _engine(model_dirs, name, "float32", max_tokens=12 * 64)
+    for trial in range(5):
+        rng = np.random.default_rng(5000 + trial)
+        count = int(rng.integers(1, 9))
+        prompts = [rng.integers(0, config["vocab_size"], size=int(rng.integers(1, 90))).tolist() for _ in range(count)]
+        limits = [int(rng.integers(1, 25)) for _ in range(count)]
+        stops = [sorted(set(rng.integers(0, config["vocab_size"], size=int(rng.integers(0, 40))).tolist())) for _ in range(count)]
+        want = [plain.greedy(p, n, s) for p, n, s in zip(prompts, limits, stops)]
+        out = generate(engine, [GenerationRequest(p, max_new_tokens=n, stop_token_ids=s) for p, n, s in zip(prompts, limits, stops)],
+                       max_batch=int(rng.integers(1, 7)))
+        assert [r.tokens for r in out] == want, f"tiny {name} trial {trial}"
+        assert engine.free_pages() == 12 and engine.free_slots() == engine.cache.max_slots
