@@ -141,7 +141,7 @@ class DecodeGraphs:
 # ---------------------------------------------------------------------------------------------
 # A step over a few thousand tokens launches 150 kernels and more; where the model is small the host
 # needs as long to launch them as the GPU to run them.  A step's *shape* -- how many sequences it has, how
-# many tokens in all (rounded up: ``prefill_rows``), how many logit rows are wanted, and the class of its
+# many tokens in all (rounded up: ``ops.prefill_rows``), how many logit rows are wanted, and the class of its
 # longest sequence (which picks the attention kernels' plan) -- fixes every launch; tokens, slots,
 # positions, how the tokens divide among the sequences and the attention's work items are data.  The rows
 # beyond a step's tokens belong to no sequence (slot -1): every kernel computes them like any row and writes
@@ -158,20 +158,13 @@ PREFILL_GRAPH_MOST_WORK = 1.5e9
 PREFILL_GRAPHS_KEPT = 16
 
 
-def prefill_rows(total: int) -> int:
-    """Rows of the replayed prompt step that takes ``total`` tokens: the next multiple of 64 up to 1,024
-    tokens, of 128 up to 2,048, of 256 beyond."""
-    unit = 64 if total <= 1024 else (128 if total <= 2048 else 256)
-    return ((total + unit - 1) // unit) * unit
-
-
 # a work item of the attention that has no rows: its first row lies beyond any sequence's tokens
 _NO_ROWS = 1 << 24
 
 
 class PrefillGraph:
     def __init__(self, engine, batch: int, total: int, wanted: int, plan_class: int, tile_rows: Sequence[int]):
-        """``total``: the rows of the step (``prefill_rows`` of its tokens), ``batch``: its sequences."""
+        """``total``: the rows of the step (``ops.prefill_rows`` of its tokens), ``batch``: its sequences."""
         self.engine = engine if isinstance(engine, weakref.ProxyTypes) else weakref.proxy(engine)
         ops = engine.rt.ops
         device = engine.rt.device

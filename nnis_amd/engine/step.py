@@ -17,7 +17,7 @@ import torch
 from ..cache import SequenceCache
 from ..errors import InvalidInput
 from .batch import StepContext, StepEntry
-from .graph import PREFILL_GRAPH_MOST_TOKENS, PREFILL_GRAPH_MOST_WORK, PrefillGraphs, prefill_rows
+from .graph import PREFILL_GRAPH_MOST_TOKENS, PREFILL_GRAPH_MOST_WORK, PrefillGraphs
 
 
 class Engine:
@@ -166,7 +166,7 @@ class Engine:
         if (self.use_graphs and total <= PREFILL_GRAPH_MOST_TOKENS and want_rows
                 and total * float(self.model.spec.width) ** 2 <= PREFILL_GRAPH_MOST_WORK):
             # a shape that comes again is replayed from a graph (engine/graph.py)
-            shape = (len(counts), prefill_rows(total), len(want_rows), self.rt.ops.prefill_plan_class(longest))
+            shape = (len(counts), self.rt.ops.prefill_rows(total), len(want_rows), self.rt.ops.prefill_plan_class(longest))
             if self._prefill_graphs is None:
                 self._prefill_graphs = PrefillGraphs(self)
             done = self._prefill_graphs.step(shape, arrays, counts, pos0, lambda: self._tile_rows.get(shape))

@@ -799,11 +799,38 @@ def decode_plan(batch: int, kv_heads: int, longest: int, max_waves: int = 4, wid
     return splits, waves
 
 
-# One column tile a wave (and so up to 8 waves a block) for long sequences was measured slower than the full
-# group a wave with 4 waves (2,048 tokens, 9/3 heads of 64: 5.5 ms a step against 4.6): keys and values are read
-# once per query head then.  The switch (for steps whose longest sequence has 1,024 tokens and more) stays for other
-# shapes; 0 is off.
-PREFILL_COLUMNS = 0
+# The prefill attention's plan: the waves of a block, and the most column tiles (query tiles x heads of a group) a
+# wave carries, 0 for as many as the head size allows.  Fewer columns make more and lighter work items, which a step
+# of few tokens needs to fill the chip, and read keys and values more often, which a long one pays for.  Measured on
+# one sequence, microseconds a layer, as it was (2, 4, 8 waves from 128, 512, 1,024 tokens on, always the widest
+# tiles) against these plans: 9/3 heads of 64 at 128 / 512 / 768 tokens 16.9 / 11.7 / 11.0 against 9.8 / 9.7 / 10.1;
+# 32/32 heads at 128 / 512 / 1,024 10.9 / 12.9 / 22.5 against 9.4 / 11.1 / 16.7; 32/4 heads 10.3 / 12.1 / 22.3
+# against 9.6 / 10.8 / 17.3.  From 1,024 tokens on 9/3 heads are fastest with the widest tiles and 8 waves (12.9
+# against 13.3), from 1,536 on all three are (9/3: 14.9 against 22.9 with two columns).  Whole prompt steps, ms:
+# TinyLlama shape 128 / 1,024 tokens 1.68 / 4.31 -> 1.60 / 4.19, 135M shape 128 / 256 1.04 / 1.32 -> 0.99 / 1.23.
+PREFILL_MANY_ROWS = 65536  # rows x query heads from which a step has work items enough for the widest tiles
+PREFILL_SOME_ROWS = 16384  # ... from which a step of 1,024 to 1,279 tokens still gains by two columns
+
+
+def prefill_rows(total: int) -> int:
+    """Rows of the replayed prompt step that takes ``total`` tokens: the next multiple of 64 up to 1,024
+    tokens, of 128 up to 2,048, of 256 beyond.  (Plans that look at a step's size look at this, so that a step
+    launched and the same step replayed from a graph's rows take the same kernels.)"""
+    unit = 64 if total <= 1024 else (128 if total <= 2048 else 256)
+    return ((total + unit - 1) // unit) * unit
+
+
+def prefill_plan(longest: int, rows: int, heads: int):
+    """(waves of a block, column option) of the prefill attention for a step of ``rows`` tokens whose longest
+    sequence has ``longest``."""
+    plan_class = prefill_plan_class(longest)
+    size = prefill_rows(rows) * heads
+    waves = (1, 2, 4, 8, 8)[plan_class]
+    if plan_class == 0 or plan_class == 4 or size >= PREFILL_MANY_ROWS:
+        return waves, 0
+    if plan_class == 3:
+        return (4, 2) if size >= PREFILL_SOME_ROWS else (8, 0)
+    return waves, plan_class  # 2 waves and one column from 128 tokens on, 4 waves and two columns from 512 on
 
 
 # The work list of a prefill step goes to the device through pinned memory, so that the copy does not make the
@@ -815,10 +842,10 @@ _tile_staging = {}
 def prefill_plan_class(longest: int) -> int:
     """Steps whose longest sequence falls into the same class launch the same prefill attention kernels
     (``attention`` picks the waves of a block, and the column option, by these thresholds)."""
-    return 3 if longest >= 1024 else (2 if longest >= 512 else (1 if longest >= 128 else 0))
+    return 4 if longest >= 1280 else (3 if longest >= 1024 else (2 if longest >= 512 else (1 if longest >= 128 else 0)))
 
 
-PREFILL_CLASS_LENGTH = (1, 128, 512, 1024)  # a length of each class
+PREFILL_CLASS_LENGTH = (1, 128, 512, 1024, 1280)  # a length of each class
 
 
 def prefill_tile_items(new_tokens, first_positions, rows: int):
@@ -882,10 +909,8 @@ def attention(q: torch.Tensor, out: torch.Tensor, view, ctx, heads: int, kv_head
     if fast and not ctx.decode:
         # A tile's keys are a chain of dependent loads: the longest tile sets the kernel's time.  The waves of
         # a block deal the keys among themselves (their merge lives in LDS).
-        plan_class = prefill_plan_class(ctx.max_len)
-        columns = PREFILL_COLUMNS if plan_class == 3 else 0
-        most = prefill_max_waves(heads, kv_heads, head_dim, columns)
-        waves = min(most, (1, 2, 4, 8)[plan_class])
+        waves, columns = prefill_plan(ctx.max_len, ctx.tokens, heads)
+        waves = min(waves, prefill_max_waves(heads, kv_heads, head_dim, columns))
         tile_seq, tile_row0 = _prefill_tiles(ctx, prefill_tile_rows(heads, kv_heads, head_dim, columns), q.device)
         return attention_prefill_bf16(q, out, view.k_pages, view.v_pages, view.block_table, tile_seq, tile_row0,
                                       ctx.seq_slot, ctx.seq_start, ctx.seq_pos0, heads, kv_heads, head_dim, scale, window,

@@ -34,7 +34,7 @@ def test_decode_plan_measured_cases():
 
 
 def test_prefill_plan_class_and_work_lists():
-    assert [prefill_plan_class(n) for n in (1, 127, 128, 511, 512, 1023, 1024, 5000)] == [0, 0, 1, 1, 2, 2, 3, 3]
+    assert [prefill_plan_class(n) for n in (1, 127, 128, 511, 512, 1023, 1024, 1279, 1280, 5000)] == [0, 0, 1, 1, 2, 2, 3, 3, 4, 4]
     for plan_class, least in enumerate(PREFILL_CLASS_LENGTH):
         assert prefill_plan_class(least) == plan_class
     # every row of every sequence lies in exactly one tile; longest tiles (by the keys they read) first
@@ -45,3 +45,18 @@ def test_prefill_plan_class_and_work_lists():
         assert seen == sorted((s, r) for s, n in enumerate(counts) for r in range(0, n, rows))
         ends = [first[s] + min(r + rows, counts[s]) for s, r in zip(seqs, row0s)]
         assert ends == sorted(ends, reverse=True)
+
+
+def test_prefill_plan_by_class_and_size():
+    from nnis_amd.kernels.ops import prefill_plan, prefill_rows
+
+    assert [prefill_rows(n) for n in (1, 64, 65, 1024, 1025, 2048, 2049, 4000)] == [64, 64, 128, 1024, 1152, 2048, 2304, 4096]
+    for n in (1, 64, 100, 1000, 1100, 2000, 3000):
+        assert prefill_rows(prefill_rows(n)) == prefill_rows(n)  # a step replayed from a graph's rows plans as the step launched
+    assert prefill_plan(100, 100, 9) == (1, 0)
+    assert prefill_plan(300, 300, 9) == (2, 1)
+    assert prefill_plan(700, 700, 9) == (4, 2)
+    assert prefill_plan(1024, 1024, 32) == (4, 2) and prefill_plan(1024, 1024, 9) == (8, 0)
+    assert prefill_plan(1024, 1900, 32) == (4, 2) and prefill_plan(1024, 2000, 32) == (8, 0)  # items enough: the widest tiles
+    assert prefill_plan(600, 4000, 32) == (4, 0)
+    assert prefill_plan(2048, 2048, 9) == (8, 0) and prefill_plan(1300, 1300, 32) == (8, 0)
