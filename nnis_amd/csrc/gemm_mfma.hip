@@ -1017,20 +1017,30 @@ int launch_tiled(const bf16_t* x, const bf16_t* w, OutT y, int m, int n, int k, 
 // 2048, 352 blocks, 108 against 119; but 2048 x 2560 x 2048, 80 blocks, 48 against 34, and 2048 x 2048 x 8192, 64
 // blocks, 152 against 89.)
 #ifndef NNIS_LARGE_TILE_BLOCKS
-#define NNIS_LARGE_TILE_BLOCKS 192
+#define NNIS_LARGE_TILE_BLOCKS 160
 #endif
 int pick_tile(int m, int columns, int k, int tile_hint) {
   const long long blocks_64_128 = (long long)((m + 63) / 64) * ((columns + 127) / 128);
   const long long rows_256 = (m + 255) / 256;
-  const long long blocks_256_256 = rows_256 * ((columns + 255) / 256), blocks_256_192 = rows_256 * ((columns + 191) / 192);
   int tile = blocks_64_128 >= 256 ? 2 : 3;
-  // (rows that fill three quarters of their tiles of 256 at least: 300 rows would be multiplied as 512)
-  if (blocks_256_256 >= NNIS_LARGE_TILE_BLOCKS && k >= 256 && 4LL * m >= 3 * 256 * rows_256) {
-    // a compute unit runs one large tile at a time: of the two widths, the one whose rounds of blocks come to
-    // fewer columns a compute unit (2048 x 6144: 192 blocks of 256 columns or 256 of 192, a round either way)
+  // The large tiles: rows that fill three quarters of their tiles of 256 at least (300 rows would be multiplied as
+  // 512), and of the two widths one that makes NNIS_LARGE_TILE_BLOCKS blocks and more -- a compute unit runs one large
+  // tile at a time, and fewer leave too many idle: 512 x 16384 x 2048 in 172 tiles of 256 x 192 takes 46 us against 52,
+  // 768 x 11264 x 2048 in 177 47 against 54, but 1024 x 6144 x 2048 in 128 44 against 34.  Where both widths do, the
+  // one whose rounds of blocks come to fewer columns a compute unit (2048 x 6144: 192 blocks of 256 columns or 256
+  // of 192, a round either way; 1024 x 11264: 176 or 236, 60 us against 49).
+  if (k >= 256 && 4LL * m >= 3 * 256 * rows_256) {
     const long long units = 256;
-    const long long cost_256 = ((blocks_256_256 + units - 1) / units) * 256, cost_192 = ((blocks_256_192 + units - 1) / units) * 192;
-    tile = cost_192 < cost_256 ? 5 : 4;
+    long long best = 0;
+    for (int width : {256, 192}) {
+      const long long blocks = rows_256 * ((columns + width - 1) / width);
+      if (blocks < NNIS_LARGE_TILE_BLOCKS) continue;
+      const long long cost = ((blocks + units - 1) / units) * width;
+      if (best == 0 || cost < best) {
+        best = cost;
+        tile = width == 256 ? 4 : 5;
+      }
+    }
   }
   if (tile_hint >= 2 && tile_hint <= 5) tile = tile_hint;  // for tuning runs
   return tile;
