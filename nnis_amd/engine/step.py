@@ -198,6 +198,20 @@ class Engine:
                 self._tile_rows.clear()
         return logits
 
+    def prepare_decode(self, batch: int, longest: int) -> None:
+        """Makes the graph that a step of one token for each of ``batch``
+        sequences replays when the longest of them has ``longest`` tokens
+        after it, if it is not there yet: a caller that knows what is coming
+        (a measurement, a server before it opens) pays for the capture then
+        and not in the step.  Nothing of the cache changes."""
+        if not self.use_graphs:
+            return
+        from .graph import DecodeGraphs
+
+        if self._graphs is None:
+            self._graphs = DecodeGraphs(self)
+        self._graphs.get(batch, longest)
+
     def step_from_device(self, slots: Sequence[int], ids_device: torch.Tensor) -> torch.Tensor:
         """A step of one token per sequence whose ids are on the device already
         (int32, row j for ``slots[j]``; what a selection kernel wrote, so in

@@ -688,3 +688,23 @@ def test_greedy_requests_drawn_from_a_seed(model_dirs, name):
                        max_batch=int(rng.integers(1, 7)))
         assert [r.tokens for r in out] == want, f"tiny {name} trial {trial}"
         assert engine.free_pages() == 12 and engine.free_slots() == engine.cache.max_slots
+
+
+def test_decode_graphs_made_ahead(model_dirs):
+    """``prepare_decode`` captures the graph of a coming step and changes
+    nothing else: the step then replays it and gives the plain model's logits."""
+    from nnis_amd.engine.batch import StepEntry
+
+    config, seed = TINY_CONFIGS["A"]
+    ids = np.random.default_rng(seed).integers(0, config["vocab_size"], size=40).tolist()
+    engine = _engine(model_dirs, "A", "bfloat16", max_tokens=4 * 64)
+    slot = engine.start_sequence()
+    engine.step([StepEntry(slot, ids[:30], [])])
+    free, length = engine.free_pages(), engine.length(slot)
+    for longest in range(31, 41):
+        engine.prepare_decode(1, longest)
+    graphs = dict(engine._graphs.graphs)
+    assert graphs and engine.free_pages() == free and engine.length(slot) == length
+    rows = torch.cat([engine.step([StepEntry(slot, [token], [0])]) for token in ids[30:]])
+    assert dict(engine._graphs.graphs) == graphs  # nothing was captured on the way
+    _close(rows.cpu(), P.PlainLlama(model_dirs["A"]).logits(ids)[30:], "bfloat16", "steps on graphs made ahead", _yard(model_dirs, "A"))
