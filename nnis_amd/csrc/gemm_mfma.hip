@@ -936,7 +936,7 @@ void dispatch_skinny(const bf16_t* x, const bf16_t* w, OutT y, int m, int n, int
 #endif
 constexpr int kDeepRingBlocks = NNIS_DEEP_RING_BLOCKS;  // grids up to this many blocks take the ring of 6 stages
 #ifndef NNIS_SHALLOW_RING_BLOCKS
-#define NNIS_SHALLOW_RING_BLOCKS 640
+#define NNIS_SHALLOW_RING_BLOCKS 513
 #endif
 constexpr int kShallowRingBlocks = NNIS_SHALLOW_RING_BLOCKS;  // grids of 64 x 128 tiles from this many blocks on: 2 stages
 
@@ -1022,14 +1022,18 @@ int launch_tiled(const bf16_t* x, const bf16_t* w, OutT y, int m, int n, int k, 
 int pick_tile(int m, int columns, int k, int tile_hint) {
   const long long blocks_64_128 = (long long)((m + 63) / 64) * ((columns + 127) / 128);
   const long long rows_256 = (m + 255) / 256;
-  int tile = blocks_64_128 >= 256 ? 2 : 3;
+  // The narrow tile up to one wide block a compute unit: 1024 x 2048 x 2048 in 256 wide blocks takes 19.1 us, in 512
+  // narrow ones 16.0 (x 8192: 59.5 against 53.5); with 320 wide blocks (1024 x 2560) the wide tile is ahead, 20.9 to 22.3.
+  int tile = blocks_64_128 > 256 ? 2 : 3;
   // The large tiles: rows that fill three quarters of their tiles of 256 at least (300 rows would be multiplied as
-  // 512), and of the two widths one that makes NNIS_LARGE_TILE_BLOCKS blocks and more -- a compute unit runs one large
+  // 512; up to 768 rows the large tile is only a tenth ahead when full, so it has to be: 384 x 16384 x 2048 took 44.5 us
+  // as 512 rows against 34.2 in tiles of 64), and of the two widths one that makes NNIS_LARGE_TILE_BLOCKS blocks and more -- a compute unit runs one large
   // tile at a time, and fewer leave too many idle: 512 x 16384 x 2048 in 172 tiles of 256 x 192 takes 46 us against 52,
   // 768 x 11264 x 2048 in 177 47 against 54, but 1024 x 6144 x 2048 in 128 44 against 34.  Where both widths do, the
   // one whose rounds of blocks come to fewer columns a compute unit (2048 x 6144: 192 blocks of 256 columns or 256
   // of 192, a round either way; 1024 x 11264: 176 or 236, 60 us against 49).
-  if (k >= 256 && 4LL * m >= 3 * 256 * rows_256) {
+  const bool filled = rows_256 >= 4 ? 4LL * m >= 3 * 256 * rows_256 : 16LL * m >= 15 * 256 * rows_256;
+  if (k >= 256 && filled) {
     const long long units = 256;
     long long best = 0;
     for (int width : {256, 192}) {
