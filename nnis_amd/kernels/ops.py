@@ -380,9 +380,6 @@ class PackedWeight:
     def is_contiguous(self) -> bool:
         return True
 
-    def storage_bytes(self) -> int:
-        return self.data.numel() * self.data.element_size()
-
 
 def packed_weight_elems(n: int, k: int) -> int:
     """Strips of 16 rows, each an odd number of chunks of 64 k (1024 elements) long."""
