@@ -1055,13 +1055,14 @@ int pick_tile(int m, int columns, int k, int tile_hint) {
       }
     }
   }
-  // The tile of 128 x 128, a block of 8 waves a compute unit: where its blocks fill one or two rounds of the chip (nine
-  // tenths at least) over a long K and no large tile fills three quarters of its rounds.  Microseconds, into the
-  // stream, against what was taken before: 2048 x 2048 x 8192 (256 blocks) 79 to 85 against 88 to 102 in tiles of
-  // 64 x 128, x 5632 57.5 against 62, x 2048 28.1 against 28.9; 4096 x 2048 x 8192 (512) 160 against 195 in 176 tiles of
-  // 256 x 192, x 5632 and x 2048 the same; slower where a round is left partly empty (2048 x 2560: 46 against 37) or
-  // half the chip is (1024 x 2048 x 8192: 65 against 58).
-  if (k >= 2048 && 8LL * m >= 7 * 128 * ((m + 127) / 128)) {
+  // The tile of 128 x 128, a block of 8 waves a compute unit: where its blocks fill one or two rounds of the chip
+  // (seven eighths at least) over a K of 1,024 and more and no large tile fills three quarters of its rounds.
+  // Microseconds, into the stream, against what was taken before: 2048 x 2048 x 8192 (256 blocks) 79 to 85 against 88
+  // to 102 in tiles of 64 x 128, x 5632 57.5 against 62, x 2048 28.1 against 28.9, x 1024 20.4 against 20.9; 4096 x
+  // 2048 x 8192 (512) 160 against 195 in 176 tiles of 256 x 192, x 5632 and x 2048 the same; 2048 x 1792 x 4096 (224)
+  // 45 against 48; slower where a round is left partly empty (2048 x 2560: 46 against 37; 3072 x 2048 x 4096, a round
+  // and a half: 81 against 69) or half the chip is (1024 x 2048 x 8192: 65 against 58).
+  if (k >= 1024 && 8LL * m >= 7 * 128 * ((m + 127) / 128)) {
     const long long blocks = (long long)((m + 127) / 128) * ((columns + 127) / 128);
     const long long rounds = (blocks + 255) / 256;
     bool large_fills = false;
@@ -1069,7 +1070,7 @@ int pick_tile(int m, int columns, int k, int tile_hint) {
       const long long large = rows_256 * ((columns + (tile == 4 ? 255 : 191)) / (tile == 4 ? 256 : 192));
       large_fills = 4 * large >= 3 * 256 * ((large + 255) / 256);
     }
-    if (rounds <= 2 && 10 * blocks >= 9 * 256 * rounds && !large_fills) tile = 6;
+    if (rounds <= 2 && 8 * blocks >= 7 * 256 * rounds && !large_fills) tile = 6;
   }
   if (tile_hint >= 2 && tile_hint <= 6) tile = tile_hint;  // for tuning runs
   return tile;
