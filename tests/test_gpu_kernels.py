@@ -321,7 +321,7 @@ def test_prefill_attention_with_more_items_than_compute_units(heads, kv_heads, h
                     for row0 in range(0, n, tile)), reverse=True)  # longest first, as the engine hands them over
     group_chunks = kv_heads * -(-(heads // kv_heads) // max(1, min(heads // kv_heads, 4)))
     assert len(items) * group_chunks > 256 + 32  # more than the compute units of the chip: the grid folds
-    for waves in (8, 2):
+    for waves in (8, 2, 1):  # (one wave: each item whole, a block's two one after the other)
         waves = min(waves, ops.prefill_max_waves(heads, kv_heads, head_dim))
         out = torch.full((sum(lengths), heads * head_dim), 3.0, dtype=torch.bfloat16, device="cuda")
         ops.attention_prefill_bf16(q, out, k_pages, v_pages, table, _i32([s for _, s, _ in items]), _i32([r for _, _, r in items]),

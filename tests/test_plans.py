@@ -60,3 +60,7 @@ def test_prefill_plan_by_class_and_size():
     assert prefill_plan(1024, 1900, 32) == (4, 2) and prefill_plan(1024, 2000, 32) == (8, 0)  # items enough: the widest tiles
     assert prefill_plan(600, 4000, 32) == (4, 0)
     assert prefill_plan(2048, 2048, 9) == (8, 0) and prefill_plan(1300, 1300, 32) == (8, 0)
+    # items for twice the chip's waves: one wave an item (64 rows x heads an item up to 64 channels, 32 up to 128)
+    assert prefill_plan(8192, 8192, 32) == (1, 0) and prefill_plan(4096, 4096, 32) == (8, 0) and prefill_plan(8192, 8192, 9) == (8, 0)
+    assert prefill_plan(2048, 2048, 32, 128) == (1, 0) and prefill_plan(2048, 2048, 16, 128) == (8, 0)
+    assert prefill_plan(600, 34000, 32) == (1, 0) and prefill_plan(1024, 1024, 32, 256) == (1, 0)
