@@ -228,7 +228,7 @@ def test_prefill_attention_on_the_matrix_cores(heads, kv_heads, head_dim):
     items = [(seq, row0) for seq, (_, _, n) in enumerate(sequences) for row0 in range(0, n, tile)]
     starts = [0, 130, 167, 168]
     starts = [0, 130, 167, 168]
-    for window, waves, columns in ((0, 1, 0), (40, 1, 0), (0, 8, 0), (40, 2, 0), (0, 8, 1), (40, 4, 2)):
+    for window, waves, columns in ((0, 1, 0), (40, 1, 0), (0, 8, 0), (40, 2, 0), (0, 8, 1), (40, 4, 2), (0, 1, 2)):
         waves = min(waves, ops.prefill_max_waves(heads, kv_heads, head_dim, columns))
         tile = ops.prefill_tile_rows(heads, kv_heads, head_dim, columns)
         items = [(seq, row0) for seq, (_, _, n) in enumerate(sequences) for row0 in range(0, n, tile)]
