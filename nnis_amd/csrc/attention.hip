@@ -483,9 +483,13 @@ __device__ __forceinline__ void attend_run(AttnState<C>& st, const QFrag (&q)[C]
   }
 }
 
-// key blocks a prefilling wave has in flight: as many as its registers hold beside C columns' states
+// key blocks a prefilling wave has in flight: as many as its registers hold beside C columns' states.  Beyond 96
+// channels two columns and two blocks need more than 256 registers, which leaves a SIMD one wave: with one block
+// in flight two waves fit, and the other wave's work fills the wait (32/8 heads of 128, one wave an item, at 8,192
+// tokens 833 -> 687 us a layer, 24/8 heads of 112 922 -> 652; at 80 and 96 channels, where two waves fit either
+// way, the second block in flight is worth 5 to 8%).
 template <int C>
-constexpr int kPrefillRing = HD > 64 ? 2 : (C <= 2 ? NNIS_PREFILL_RING_NARROW : NNIS_PREFILL_RING_WIDE);
+constexpr int kPrefillRing = HD > 96 ? (C <= 1 ? 2 : 1) : (HD > 64 ? 2 : (C <= 2 ? NNIS_PREFILL_RING_NARROW : NNIS_PREFILL_RING_WIDE));
 
 // ---- prefill: a wave = (query tile, kv head, chunk of GH query heads); C = QT * GH column tiles --------
 // An item is a (tile, kv head, chunk of heads); the tiles come longest first, and item i = tile i / per_tile.
