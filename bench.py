@@ -41,7 +41,8 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
 FLOP_PEAK = {"bfloat16": 2.5e15, "float32": 157.3e12}
-NAMES = {"smollm2-135m": "SmolLM2-135M", "smollm2-1.7b": "SmolLM2-1.7B", "tinyllama-1.1b": "TinyLlama-1.1B"}
+NAMES = {"smollm2-135m": "SmolLM2-135M", "smollm2-1.7b": "SmolLM2-1.7B", "tinyllama-1.1b": "TinyLlama-1.1B", "llama-8b": "Llama-8B"}
+POINT_SHAPES = ("smollm2-135m", "smollm2-1.7b", "tinyllama-1.1b")  # the shapes whose figures go into `points` beside the headline's
 
 
 def step_flops(config, tokens_per_sequence, wanted_rows):
@@ -301,7 +302,7 @@ def main() -> int:
     if not args.no_points and not args.no_other_shapes:
         import torch
 
-        for other in sorted(NAMES):
+        for other in POINT_SHAPES:
             if other == args.shape:
                 continue
             torch.cuda.empty_cache()

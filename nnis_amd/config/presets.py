@@ -3,7 +3,8 @@ two tiny ones its smoke runs use, as the config.json each would carry.
 
 SmolLM2-135M and TinyLlama-1.1B are the reference's pinned checkpoints
 (/root/reference/crates/nnis-model/src/exact_checkpoint_spec.rs:219-259);
-SmolLM2-1.7B has the same architecture at 24 layers of width 2048.  A preset
+SmolLM2-1.7B has the same architecture at 24 layers of width 2048; "llama-8b"
+is a fourth shape for measurements only.  A preset
 gives sizes only: weights come from a checkpoint of that shape or from the
 random-weights mode (``write_random_model(folder, preset("smollm2-135m"),
 seed)``).
@@ -35,6 +36,12 @@ _PRESETS: Dict[str, Dict[str, Any]] = {
         num_hidden_layers=22, hidden_size=2048, num_attention_heads=32, num_key_value_heads=4, head_dim=64,
         intermediate_size=5632, vocab_size=32000, rope_theta=10000.0, rms_norm_eps=1e-5, tie_word_embeddings=False,
         max_position_embeddings=2048, eos_token_id=2),
+    # beyond the reference's checkpoints: the sizes of an 8B Llama, grouped heads of 128 channels (for measurements
+    # at a head size and widths that the three above do not have; usually run with fewer layers)
+    "llama-8b": _llama(
+        num_hidden_layers=32, hidden_size=4096, num_attention_heads=32, num_key_value_heads=8, head_dim=128,
+        intermediate_size=14336, vocab_size=128256, rope_theta=500000.0, rms_norm_eps=1e-5, tie_word_embeddings=False,
+        max_position_embeddings=8192),
     # two tiny models that differ in every size and option
     "tiny-a": _llama(
         num_hidden_layers=2, hidden_size=64, num_attention_heads=4, num_key_value_heads=2, intermediate_size=176,

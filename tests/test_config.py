@@ -111,7 +111,9 @@ def test_presets_and_the_capability_record():
     (/root/reference/crates/nnis-model/src/exact_checkpoint_spec.rs:10-30,219-259)."""
     from nnis_amd.config import preset, preset_names
 
-    assert {"smollm2-135m", "smollm2-1.7b", "tinyllama-1.1b", "tiny-a", "tiny-b"} <= set(preset_names())
+    assert {"smollm2-135m", "smollm2-1.7b", "tinyllama-1.1b", "llama-8b", "tiny-a", "tiny-b"} <= set(preset_names())
+    big = LlamaConfig.from_dict(preset("llama-8b"))
+    assert (big.head_dim, big.num_attention_heads // big.num_key_value_heads) == (128, 4)
     small = LlamaConfig.from_dict(preset("smollm2-135m"))
     assert small.capability_record() == ("NNIS-DECODER-CAPABILITY-V1\nattention=grouped_query\nrope=llama_rotate_half_unscaled\n"
                                          "mlp=swiglu_silu\nweight_dtype=bf16\nq_heads=9\nkv_heads=3\nhead_dim=64\n")
