@@ -43,8 +43,9 @@ FLAGS = [
 ]
 # Per source: the matrix instructions keep their sums in the ordinary vector registers.  Left to itself the
 # compiler puts them into the accumulation registers and moves them to and fro: in the tiled product's loop 48
-# moves a step for 16 matrix instructions, in the decode attention with keys on lanes 336 for 144 (no kernel
-# of either file spills with the sums in vector registers, at any head size).
+# moves a step for 16 matrix instructions, in the decode attention with keys on lanes 336 for 144.  (With the
+# sums in vector registers the prefill attention's four-column kernels at 64 channels keep 17 to 26 registers
+# in scratch memory, all outside their loops over the keys; no other kernel of either file spills.)
 _VECTOR_SUMS = ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]
 SOURCE_FLAGS = {"gemm_mfma.hip": _VECTOR_SUMS, "attention.hip": _VECTOR_SUMS}
 HEADERS = {"core": ["common.h", "epilogue.h", "nnis_noalloc.h"], "attention": ["common.h"]}  # what a module's sources include
