@@ -16,8 +16,8 @@ from __future__ import annotations
 import json
 import math
 import os
-from dataclasses import dataclass, field, asdict
-from typing import Any, Dict, Optional, Tuple
+from dataclasses import dataclass, field
+from typing import Any, Dict, Tuple
 
 from ..errors import InvalidInput, Unsupported
 

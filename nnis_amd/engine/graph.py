@@ -16,9 +16,8 @@ from __future__ import annotations
 
 import gc
 import weakref
-from typing import Dict, List, Sequence, Tuple
+from typing import Dict, Sequence
 
-import numpy as np
 import torch
 
 from ..errors import KernelError

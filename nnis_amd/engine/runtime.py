@@ -6,9 +6,6 @@ with 32-bit accumulation, statistics, residual stream and logits.
 
 from __future__ import annotations
 
-from dataclasses import dataclass
-from typing import Any
-
 import torch
 
 from ..errors import InvalidInput, KernelError

@@ -4,7 +4,7 @@ kernel is checked against it; the generation loop's CPU tests use it."""
 
 from __future__ import annotations
 
-from typing import List, Sequence
+from typing import Sequence
 
 import numpy as np
 
