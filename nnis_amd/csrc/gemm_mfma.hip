@@ -620,6 +620,58 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_tiled_kernel(const bf16_t
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
   int stage = 0;
+  // One block of 8 waves a compute unit (the tiles of 128 and 256 x 128): the two waves of a SIMD leave a step's barrier
+  // together, and with reads first and products after, the matrix unit would wait at the head of every step.  So a
+  // step's second half is multiplied after the barrier, while the next step's first half is read, and its first
+  // half before it, while the second is read: the operands of a half are in registers one barrier ahead.  Every
+  // read of a stage is still waited for before the barrier that lets the stage be filled again, and a sum takes
+  // its halves in the same order as before.
+  constexpr bool kCarry = TM * TN <= 16 && W == 8;
+  if constexpr (kCarry) {
+    static_assert(BK == 64, "two halves of 32 k a step");
+    bf16x8 a0[TM], b0[TN], a1[TM], b1[TN];
+    auto read_half = [&](int from, int half, bf16x8 (&a)[TM], bf16x8 (&b)[TN]) {
+      const bf16x8* a_tile = (const bf16x8*)(tile_lds + from * STAGE_BYTES);
+      const bf16x8* b_tile = (const bf16x8*)(tile_lds + from * STAGE_BYTES + A_BYTES);
+#pragma unroll
+      for (int i = 0; i < TM; ++i) a[i] = a_tile[swizzled<CH>(wave_m * WM + i * 16 + r, g * 2 + half)];
+#pragma unroll
+      for (int jj = 0; jj < TN; ++jj) b[jj] = b_tile[((wave_n * TN + jj) * 2 + half) * kWave + lane];
+    };
+    auto multiply = [&](const bf16x8 (&a)[TM], const bf16x8 (&b)[TN]) {
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int jj = 0; jj < TN; ++jj) acc[i][jj] = mfma(b[jj], a[i], acc[i][jj]);
+    };
+    // for the scheduler: a read behind each of the first products, then the rest of the products
+    auto interleave = [&]() {
+#pragma unroll
+      for (int n = 0; n < TM + TN; ++n) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - (TM + TN), 0);
+    };
+    static_assert(TM * TN >= TM + TN, "a product for every read");
+    if (step0 < step1) read_half(0, 0, a0, b0);
+    for (int step = step0; step < step1; ++step) {
+      ask(step + NS - 1, stage == 0 ? NS - 1 : stage - 1);
+      read_half(stage, 1, a1, b1);
+      multiply(a0, b0);
+      interleave();
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      wait_loads_but<(NS - 2) * LOADS>();
+      __builtin_amdgcn_sched_barrier(0);
+      __builtin_amdgcn_s_barrier();
+      __builtin_amdgcn_sched_barrier(0);
+      asm volatile("" ::: "memory");
+      stage = stage + 1 == NS ? 0 : stage + 1;
+      read_half(stage, 0, a0, b0);  // (after the last step: of a stage that nobody multiplies; no branch in the loop's body)
+      multiply(a1, b1);
+      interleave();
+    }
+  } else {
   for (int step = step0; step < step1; ++step) {
     // The tile of 256 x 256 asks for the next step between its two halves, under the first half's products
     // (2048 x 16384 x 2048 137 us against 141, 6224 x 11264 x 2048 277 against 294); the tile of 256 x 192, whose
@@ -679,6 +731,7 @@ __global__ __launch_bounds__(64 * WGM * WGN) void gemm_tiled_kernel(const bf16_t
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
     stage = stage + 1 == NS ? 0 : stage + 1;
+  }
   }
   wait_loads_but<0>();  // the steps asked for beyond the end: nothing of this block is in flight when it ends
 
