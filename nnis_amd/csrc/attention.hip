@@ -1029,13 +1029,17 @@ extern "C" int nnis_attention_prefill_tile_rows(int heads, int kv_heads, int col
   return 16 * qt;
 }
 
+// the most LDS a block's merge takes: half its waves leave a state at a time (eight waves of four columns at 64
+// channels: 72 KB)
+constexpr size_t kMergeLdsMost = 96 * 1024;
+
 // waves a block of the prefill kernel may have for these sizes (LDS of the merge)
 extern "C" int nnis_attention_prefill_max_waves(int heads, int kv_heads, int columns) {
   int qt, gh;
   prefill_shape(heads, kv_heads, columns, &qt, &gh);
   const size_t per_wave = (size_t)qt * gh * (kTilesD * 4 + 2) * kWave * sizeof(float);
   int waves = 1;  // a power of two; half of them leave a state in LDS at a time
-  while (waves * 2 <= kBlockWaves && waves * per_wave <= 65536) waves *= 2;
+  while (waves * 2 <= kBlockWaves && waves * per_wave <= kMergeLdsMost) waves *= 2;
   return waves;
 }
 
@@ -1062,13 +1066,19 @@ extern "C" int nnis_attention_prefill_bf16(const void* q, void* out, const void*
   const int singles = 2 * blocks - items;
   const dim3 grid(blocks);
   const size_t per_wave = (size_t)qt * gh * (kTilesD * 4 + 2) * kWave * sizeof(float);
-  NNIS_REQUIRE(waves >= 1 && waves <= kBlockWaves && (waves & (waves - 1)) == 0 && (waves / 2) * per_wave <= 65536,
+  NNIS_REQUIRE(waves >= 1 && waves <= kBlockWaves && (waves & (waves - 1)) == 0 && (waves / 2) * per_wave <= kMergeLdsMost,
                "attention: %d waves a block: a power of two that fits this head size (LDS) is needed", waves);
   const size_t lds = (waves / 2) * per_wave;
   const dim3 block(kWave * waves);
   hipStream_t s = (hipStream_t)stream;
-#define NNIS_PREFILL(QT_, GH_) \
-  hipLaunchKernelGGL((attention_prefill_kernel<QT_, GH_>), grid, block, lds, s, a, waves, items, singles, per_tile)
+  // (beyond 64 KB a kernel has to be told once; a refusal shows as the launch's failure)
+#define NNIS_PREFILL(QT_, GH_)                                                                                          \
+  do {                                                                                                                  \
+    static const hipError_t allowed = hipFuncSetAttribute((const void*)attention_prefill_kernel<QT_, GH_>,              \
+                                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMergeLdsMost); \
+    (void)allowed;                                                                                                      \
+    hipLaunchKernelGGL((attention_prefill_kernel<QT_, GH_>), grid, block, lds, s, a, waves, items, singles, per_tile); \
+  } while (0)
   bool launched = true;
   if constexpr (kMaxColumns >= 4) {
     if (qt == 4 && gh == 1) NNIS_PREFILL(4, 1);

@@ -808,6 +808,11 @@ def decode_plan(batch: int, kv_heads: int, longest: int, max_waves: int = 4, wid
 # TinyLlama shape 128 / 1,024 tokens 1.68 / 4.31 -> 1.60 / 4.19, 135M shape 128 / 256 1.04 / 1.32 -> 0.99 / 1.23.
 PREFILL_MANY_ROWS = 65536  # rows x query heads from which a step has work items enough for the widest tiles
 PREFILL_SOME_ROWS = 16384  # ... from which a step of 1,024 to 1,279 tokens still gains by two columns
+# Items of four columns (up to 64 channels, any group but 3) merge the states of 8 waves through 72 KB of LDS: worth it
+# while a step's items are few (16 heads of 64 at 2,048 tokens 26 us a layer against 37 with 4 waves, 16/4 heads of 48
+# 25 against 39; 32 heads at 1,024 tokens 21 against 25), not beyond (32 heads at 1,536 tokens 41 against 35, 64/8 heads
+# at 2,048 83 against 73).
+PREFILL_EIGHT_WAVES_MOST = 40960
 
 
 def prefill_rows(total: int) -> int:
@@ -842,6 +847,8 @@ def prefill_plan(longest: int, rows: int, heads: int, head_dim: int = 64, kv_hea
     if head_dim <= 64 and 2 * size >= many and (group == 1 or group % 2 == 0):
         return 1, 2
     waves = (1, 2, 4, 8, 8)[plan_class]
+    if waves == 8 and head_dim <= 64 and group != 3 and size > PREFILL_EIGHT_WAVES_MOST:
+        waves = 4
     if plan_class == 0 or plan_class == 4 or size >= PREFILL_MANY_ROWS:
         return waves, 0
     if plan_class == 3:

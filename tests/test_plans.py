@@ -59,11 +59,12 @@ def test_prefill_plan_by_class_and_size():
     assert prefill_plan(1024, 1024, 32) == (4, 2) and prefill_plan(1024, 1024, 9) == (8, 0)
     assert prefill_plan(1024, 1900, 32) == (4, 2) and prefill_plan(1024, 2000, 33, 64, 11) == (8, 0)  # items enough: the widest tiles
     assert prefill_plan(600, 4000, 36, 64, 12) == (4, 0)
-    assert prefill_plan(2048, 2048, 9) == (8, 0) and prefill_plan(1300, 1300, 32) == (8, 0)
+    assert prefill_plan(2048, 2048, 9) == (8, 0) and prefill_plan(1300, 1300, 32) == (4, 0)
+    assert prefill_plan(2048, 2048, 16) == (8, 0)  # few items of four columns: 8 waves deal an item's keys
     # items for twice the chip's waves: one wave an item (64 rows x heads an item up to 64 channels, 32 up to 128)
     assert prefill_plan(8192, 8192, 32) == (1, 0) and prefill_plan(8192, 8192, 9, 64, 3) == (8, 0)
     # half of that: one wave an item of two columns, where two divide the group
     assert prefill_plan(4096, 4096, 32) == (1, 2) and prefill_plan(2048, 2048, 64, 64, 8) == (1, 2) and prefill_plan(4096, 4096, 36, 64, 12) == (8, 0)
-    assert prefill_plan(2048, 2048, 32) == (8, 0)
+    assert prefill_plan(2048, 2048, 32) == (4, 0)
     assert prefill_plan(2048, 2048, 32, 128) == (1, 0) and prefill_plan(2048, 2048, 16, 128) == (8, 0)
     assert prefill_plan(600, 34000, 32) == (1, 0) and prefill_plan(1024, 1024, 32, 256) == (1, 0) and prefill_plan(1024, 1024, 32, 128) == (4, 2)
