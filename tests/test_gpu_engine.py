@@ -708,3 +708,36 @@ def test_decode_graphs_made_ahead(model_dirs):
     rows = torch.cat([engine.step([StepEntry(slot, [token], [0])]) for token in ids[30:]])
     assert dict(engine._graphs.graphs) == graphs  # nothing was captured on the way
     _close(rows.cpu(), P.PlainLlama(model_dirs["A"]).logits(ids)[30:], "bfloat16", "steps on graphs made ahead", _yard(model_dirs, "A"))
+
+
+@pytest.mark.parametrize("heads, head_dim, inner, tokens, plan", [
+    (64, 16, 512, 2048, (1, 2)), (64, 16, 512, 4096, (1, 0)),  # width 1024
+    (32, 64, 1024, 2048, (4, 0)), (32, 64, 1024, 4096, (1, 2))])  # width 2048: products in tiles of 128 and 256 x 128, 256 x 192
+def test_long_prompts_on_many_heads(tmp_path, heads, head_dim, inner, tokens, plan):
+    """A prompt whose rows x heads give the prefill attention items for all the chip's waves: each item goes to
+    one wave (of two columns at half the size, of four beyond); and at a width of 2,048 its products take the
+    tiles that a step of thousands of rows is given.  One layer in bfloat16, the logits at places all along
+    the prompt and of eight tokens decoded after it, against the plain model with the yardstick of its
+    bfloat16 twin."""
+    import nnis_amd
+    from configs import llama
+    from nnis_amd.api import load_engine
+    from nnis_amd.engine.batch import StepEntry
+    from nnis_amd.kernels import ops
+
+    config = llama(num_hidden_layers=1, hidden_size=heads * head_dim, num_attention_heads=heads, num_key_value_heads=heads,
+                   intermediate_size=inner, vocab_size=300, rope_theta=10000.0, rms_norm_eps=1e-5, tie_word_embeddings=True,
+                   max_position_embeddings=4096 + 64, torch_dtype="bfloat16")
+    assert ops.prefill_plan(tokens, tokens, heads, head_dim, heads) == plan
+    folder = str(tmp_path / "model")
+    os.makedirs(folder)
+    nnis_amd.write_random_model(folder, config, 5)
+    ids = np.random.default_rng(tokens).integers(0, config["vocab_size"], size=tokens + 8).tolist()
+    engine = load_engine(folder, dtype="bfloat16", max_tokens=tokens + 128)
+    slot = engine.start_sequence()
+    places = list(range(0, tokens, 193)) + list(range(tokens - 33, tokens))
+    got = torch.cat([engine.step([StepEntry(slot, ids[:tokens], places)])] +
+                    [engine.step([StepEntry(slot, [token], [0])]) for token in ids[tokens:]]).cpu()
+    plain = P.PlainLlama(folder)
+    rows = places + list(range(tokens, tokens + 8))
+    Bf16Yardstick(plain, [ids[:600]]).check(got, plain.logits(ids)[rows], f"a prompt of {tokens} tokens on {heads} heads")
