@@ -1120,7 +1120,9 @@ int pick_tile(int m, int columns, int k, int tile_hint) {
   // 2048 x 8192 in 256 blocks 121 us plain and 131 into the stream (1.12 PFLOP/s) against 146 to 161 and 158 to 165
   // in 512 tiles of 128 x 128, x 2048 37 and 46 against 43 and 54; 2048 x 4096 x 14336 214 and 226 against 258 and
   // 267; 3840 x 2048 x 5632 (240 blocks) 82 and 92 against 100 and 108.  Where a large tile fills its rounds it stays
-  // (4096 x 4096 x 4096: 112 plain in 256 tiles of 256 x 256 against 126 in 512 of 256 x 128, into the stream alike).
+  // (4096 x 4096 x 4096: 112 plain in 256 tiles of 256 x 256 against 126 in 512 of 256 x 128, into the stream alike);
+  // where it fills less than three quarters this tile is ahead of it too: 512 x 16384 x 2048 in 256 blocks 38 us over
+  // weights from memory, in 172 tiles of 256 x 192 57 to 69; 3072 x 2560 x 2048 (240 blocks) 35 against 46.
   bool large_fills = false;
   if (tile == 4 || tile == 5) {
     const long long large = rows_256 * ((columns + (tile == 4 ? 255 : 191)) / (tile == 4 ? 256 : 192));
@@ -1257,6 +1259,10 @@ extern "C" int nnis_gemm_bf16(const void* x, const void* w, void* y, int y_dtype
   }
   return 0;
 }
+
+// The tile that the tiled kernel takes for m rows, `columns` weight rows and a depth of k (2: 64 x 128, 3: 64 x 64,
+// 4: 256 x 256, 5: 256 x 192, 6: 128 x 128, 7: 256 x 128): for tests and tuning.
+extern "C" int nnis_gemm_tile(int m, int columns, int k) { return pick_tile(m, columns, k, 0); }
 
 // The projection that ends a part of a pre-norm block: resid += x . w^T in 32-bit, in place, and the norm
 // that follows prepared -- scaled = bf16(resid * gain) and parts of each row's sum of squares in ss

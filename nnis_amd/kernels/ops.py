@@ -38,6 +38,7 @@ _CORE_SIGNATURES = {
     "nnis_gemm_fused": [_VOID, _VOID, _VOID, _VOID, _INT, _FLT, _VOID, _INT, _INT, _INT, _INT, _VOID, _VOID, _VOID, _INT,
                         _VOID, _VOID, _VOID, _VOID, _VOID, _INT, _INT, _INT, _INT, _VOID, _VOID, _VOID, _INT, _VOID],
     "nnis_gemm_residual_parts": [_INT, _INT],
+    "nnis_gemm_tile": [_INT, _INT, _INT],
     "nnis_gemm_residual": [_VOID, _VOID, _VOID, _VOID, _INT, _VOID, _VOID, _INT, _INT, _INT, _INT, _VOID, _INT, _VOID, _SIZE, _VOID],
     "nnis_gemm_scaled": [_VOID, _VOID, _INT, _FLT, _VOID, _INT, _INT, _INT, _INT, _VOID, _VOID, _VOID, _INT, _VOID, _VOID,
                          _VOID, _VOID, _VOID, _INT, _INT, _INT, _INT, _VOID, _VOID, _VOID, _INT, _VOID, _SIZE, _VOID],
@@ -517,6 +518,11 @@ def _check_epilogue(what: str, m: int, n: int, y: torch.Tensor, epilogue: int, r
 
 # tiles of the tiled product (``tile`` of gemm_residual; 16 times as much as a ``split`` of gemm_bf16 / gemm_scaled)
 TILE_64x128, TILE_64x64, TILE_256x256, TILE_256x192, TILE_128x128, TILE_256x128 = 2, 3, 4, 5, 6, 7
+
+
+def gemm_tile(m: int, n: int, k: int) -> int:
+    """The tile (``TILE_*``) that the tiled kernel takes for a product of m rows with n weight rows of k."""
+    return core().nnis_gemm_tile(int(m), int(n), int(k))
 
 
 def gemm_residual_parts(m: int, n: int) -> int:

@@ -881,3 +881,27 @@ def test_refusals():
         ops.silu_mul(f(4, 11), f(4, 5))
     with pytest.raises(KernelError):
         ops.argmax(f(4, 11), torch.zeros(4, dtype=torch.int64, device="cuda"))
+
+
+def test_the_tiles_that_products_are_given():
+    """The tiled kernel's choice of tile by the product's sizes, at the sizes its rules were measured on (the
+    library's own host code: no launch)."""
+    ops = _ops()
+    T = ops
+    for (m, n, k), tile in {
+        (2048, 16384, 2048): T.TILE_256x256,  # two full rounds of large tiles
+        (2048, 6144, 2048): T.TILE_256x192,   # 256 blocks of 192 columns, where 256 columns make 192
+        (1024, 11264, 2048): T.TILE_256x192,  # 236 blocks
+        (512, 16384, 2048): T.TILE_256x128,   # 256 blocks where tiles of 256 x 192 make 172
+        (384, 16384, 2048): T.TILE_64x128,    # ... rows that do not
+        (4096, 4096, 4096): T.TILE_256x256,   # a large tile that fills its round stays
+        (4096, 2048, 8192): T.TILE_256x128,   # 256 blocks, one a compute unit, where large tiles would be 176
+        (2048, 4096, 14336): T.TILE_256x128,
+        (2048, 2048, 8192): T.TILE_128x128,   # 256 blocks of 128 rows where 256 rows make 128
+        (2048, 2048, 512): T.TILE_64x128,     # ... over a short K the small tiles
+        (2048, 2560, 2048): T.TILE_64x128,    # a round and a quarter of 128 x 128: not taken
+        (1024, 2048, 2048): T.TILE_64x64,     # no more than one wide block a compute unit: the narrow tile
+        (2048, 576, 1536): T.TILE_64x64,
+        (2048, 3072, 576): T.TILE_64x128,
+    }.items():
+        assert ops.gemm_tile(m, n, k) == tile, (m, n, k, ops.gemm_tile(m, n, k))
