@@ -1110,7 +1110,7 @@ int pick_tile(int m, int columns, int k, int tile_hint) {
     }
   }
   // The tile of 128 x 128, a block of 8 waves a compute unit: where its blocks fill one or two rounds of the chip
-  // (seven eighths at least) over a K of 1,024 and more and no large tile fills three quarters of its rounds.
+  // (see below how far) over a K of 1,024 and more and no large tile fills three quarters of its rounds.
   // Microseconds, into the stream, against what was taken before: 2048 x 2048 x 8192 (256 blocks) 79 to 85 against 88
   // to 102 in tiles of 64 x 128, x 5632 57.5 against 62, x 2048 28.1 against 28.9, x 1024 20.4 against 20.9; 4096 x
   // 2048 x 8192 (512) 160 against 195 in 176 tiles of 256 x 192, x 5632 and x 2048 the same; 2048 x 1792 x 4096 (224)
@@ -1123,6 +1123,11 @@ int pick_tile(int m, int columns, int k, int tile_hint) {
   // (4096 x 4096 x 4096: 112 plain in 256 tiles of 256 x 256 against 126 in 512 of 256 x 128, into the stream alike);
   // where it fills less than three quarters this tile is ahead of it too: 512 x 16384 x 2048 in 256 blocks 38 us over
   // weights from memory, in 172 tiles of 256 x 192 57 to 69; 3072 x 2560 x 2048 (240 blocks) 35 against 46.
+  // A single round may be eleven sixteenths full (2304 x 2560 x 2048 in 180 tiles of 256 x 128 29.4 us against 32.3;
+  // 2048 x 3072 x 2048 in 192 tiles of 256 x 128 32 us against 34.5 in
+  // tiles of 64 x 128, 1536 x 4096 x 4096 55 against 60; 2048 x 1536 x 2048 in 192 of 128 x 128 19.7 against 21.4; at
+  // five eighths, 2048 x 2560 x 2048, 31.7 against 32.4: not taken), two rounds seven eighths (3072 x 2048 x 4096 in
+  // 384 tiles of 128 x 128: 81 against 69).
   bool large_fills = false;
   if (tile == 4 || tile == 5) {
     const long long large = rows_256 * ((columns + (tile == 4 ? 255 : 191)) / (tile == 4 ? 256 : 192));
@@ -1134,7 +1139,7 @@ int pick_tile(int m, int columns, int k, int tile_hint) {
       if (8LL * m < 7 * rows * row_blocks) continue;
       const long long blocks = row_blocks * ((columns + 127) / 128);
       const long long rounds = (blocks + 255) / 256;
-      if (rounds <= 2 && 8 * blocks >= 7 * 256 * rounds) {
+      if (rounds == 1 ? 16 * blocks >= 11 * 256 : (rounds == 2 && 8 * blocks >= 7 * 256 * rounds)) {
         tile = rows == 256 ? 7 : 6;
         break;
       }

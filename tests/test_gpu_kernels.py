@@ -899,7 +899,10 @@ def test_the_tiles_that_products_are_given():
         (2048, 4096, 14336): T.TILE_256x128,
         (2048, 2048, 8192): T.TILE_128x128,   # 256 blocks of 128 rows where 256 rows make 128
         (2048, 2048, 512): T.TILE_64x128,     # ... over a short K the small tiles
-        (2048, 2560, 2048): T.TILE_64x128,    # a round and a quarter of 128 x 128: not taken
+        (2048, 2560, 2048): T.TILE_64x128,    # a round and a quarter of 128 x 128, five eighths of one of 256 x 128: not taken
+        (2048, 3072, 2048): T.TILE_256x128,   # three quarters of a round (eleven sixteenths are enough)
+        (2048, 1536, 2048): T.TILE_128x128,
+        (3072, 2048, 4096): T.TILE_256x128,   # (192 blocks, where 128 x 128 would make a round and a half)
         (1024, 2048, 2048): T.TILE_64x64,     # no more than one wide block a compute unit: the narrow tile
         (2048, 576, 1536): T.TILE_64x64,
         (2048, 3072, 576): T.TILE_64x128,
