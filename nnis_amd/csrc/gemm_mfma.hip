@@ -1030,13 +1030,14 @@ int launch_tiled_large(const bf16_t* x, const bf16_t* w, OutT y, int m, int n, i
   return 2 * col_blocks;
 }
 
-// the tiles of 128 x 128 and 256 x 128 (8 waves as 4 x 2, a wave tile of 32 x 64 or 64 x 64; 3 stages of 32 or 48 KB:
+// the tiles of 128 x 128, 128 x 192 and 256 x 128 (8 waves as 4 x 2, a wave tile of 32 x 64, 32 x 96 or 64 x 64; 3 stages
+// of 32, 40 or 48 KB:
 // one block a compute unit, whose row blocks share each column block's weights); returns the parts of a row's
 // sum of squares written
-template <int BM, typename OutT>
+template <int BM, int BN, typename OutT>
 int launch_tiled_medium(const bf16_t* x, const bf16_t* w, OutT y, int m, int n, int k, int columns, hipStream_t stream) {
-  const int col_blocks = (columns + 127) / 128, row_blocks = (m + BM - 1) / BM;
-  launch_tiled_kernel<BM, 128, 64, 3, false, OutT, 4, 2>(x, w, y, m, n, k, col_blocks, row_blocks, 1, {nullptr, 0}, stream);
+  const int col_blocks = (columns + BN - 1) / BN, row_blocks = (m + BM - 1) / BM;
+  launch_tiled_kernel<BM, BN, 64, 3, false, OutT, 4, 2>(x, w, y, m, n, k, col_blocks, row_blocks, 1, {nullptr, 0}, stream);
   return 2 * col_blocks;
 }
 
@@ -1074,7 +1075,7 @@ int launch_tiled(const bf16_t* x, const bf16_t* w, OutT y, int m, int n, int k, 
   return launch_tiled_staged<BM, BN, BK, 3, OutT>(x, w, y, m, n, k, col_blocks, row_blocks, ksplit, ws, stream);
 }
 
-// 2: 64x128, 3: 64x64, 4: 256x256, 5: 256x192, 6: 128x128, 7: 256x128 -- the larger tile when it still gives (nearly) every compute unit a block.
+// 2: 64x128, 3: 64x64, 4: 256x256, 5: 256x192, 6: 128x128, 7: 256x128, 8: 128x192 -- the larger tile when it still gives (nearly) every compute unit a block.
 // (A tile of 128x128 was measured slower than 64x128 on every product from 2048 x 576 x 576 to 2048 x 6144 x 2048;
 // the tile of 256x256 against 64x128, microseconds: 2048 x 6144 x 2048, 192 blocks, 57 against 68; 2048 x 11264 x
 // 2048, 352 blocks, 108 against 119; but 2048 x 2560 x 2048, 80 blocks, 48 against 34, and 2048 x 2048 x 8192, 64
@@ -1133,26 +1134,35 @@ int pick_tile(int m, int columns, int k, int tile_hint) {
     const long long large = rows_256 * ((columns + (tile == 4 ? 255 : 191)) / (tile == 4 ? 256 : 192));
     large_fills = 4 * large >= 3 * 256 * ((large + 255) / 256);
   }
+  // Of the three the one whose rounds come to the least area over its rate: a compute unit multiplies a tile of 128
+  // x 192 (a wave tile of 32 x 96) at about 0.85 and one of 128 x 128 at about 0.8 of the rate of 256 x 128.  2048 x 3072
+  // x 2048 with the gate's epilogue in 256 tiles of 128 x 192 27.7 us against 31 in 192 of 256 x 128; 1024 x 6144 x
+  // 2048 with the rotation 33 against 37.6; 2048 x 2560 x 2048 (224 tiles, where 256 x 128 makes 160) 33 to 34.5
+  // against 36 in tiles of 64 x 128.
   if (k >= 1024 && !large_fills) {
-    for (int rows : {256, 128}) {
-      const long long row_blocks = (m + rows - 1) / rows;
-      if (8LL * m < 7 * rows * row_blocks) continue;
-      const long long blocks = row_blocks * ((columns + 127) / 128);
+    struct Candidate { int tile, rows, width, rate; };
+    long long best = 0;
+    for (const Candidate c : {Candidate{7, 256, 128, 100}, Candidate{8, 128, 192, 85}, Candidate{6, 128, 128, 80}}) {
+      const long long row_blocks = (m + c.rows - 1) / c.rows;
+      if (8LL * m < 7LL * c.rows * row_blocks) continue;
+      const long long blocks = row_blocks * ((columns + c.width - 1) / c.width);
       const long long rounds = (blocks + 255) / 256;
-      if (rounds == 1 ? 16 * blocks >= 11 * 256 : (rounds == 2 && 8 * blocks >= 7 * 256 * rounds)) {
-        tile = rows == 256 ? 7 : 6;
-        break;
+      if (!(rounds == 1 ? 16 * blocks >= 11 * 256 : (rounds == 2 && 8 * blocks >= 7 * 256 * rounds))) continue;
+      const long long cost = rounds * c.rows * c.width * 100 / c.rate;
+      if (best == 0 || cost < best) {
+        best = cost;
+        tile = c.tile;
       }
     }
   }
-  if (tile_hint >= 2 && tile_hint <= 7) tile = tile_hint;  // for tuning runs
+  if (tile_hint >= 2 && tile_hint <= 8) tile = tile_hint;  // for tuning runs
   return tile;
 }
 
 // the most parts of a row's sum of squares that a residual epilogue of the tiled kernel writes for these sizes
 int tiled_parts(int m, int columns, int k, int tile_hint) {
   const int tile = pick_tile(m, columns, k, tile_hint);
-  const int width = tile == 4 ? 256 : (tile == 5 ? 192 : (tile == 2 || tile == 6 || tile == 7 ? 128 : 64));
+  const int width = tile == 4 ? 256 : (tile == 5 || tile == 8 ? 192 : (tile == 2 || tile == 6 || tile == 7 ? 128 : 64));
   return 2 * ((columns + width - 1) / width);  // with K in parts: one per 64 columns, which is no more
 }
 
@@ -1164,8 +1174,9 @@ int dispatch_tiled(const bf16_t* x, const bf16_t* w, OutT y, int m, int n, int k
   const int tile = pick_tile(m, columns, k, tile_hint);
   if (tile == 4) return launch_tiled_large<256, OutT>(x, w, y, m, n, k, columns, stream);
   if (tile == 5) return launch_tiled_large<192, OutT>(x, w, y, m, n, k, columns, stream);
-  if (tile == 6) return launch_tiled_medium<128, OutT>(x, w, y, m, n, k, columns, stream);
-  if (tile == 7) return launch_tiled_medium<256, OutT>(x, w, y, m, n, k, columns, stream);
+  if (tile == 6) return launch_tiled_medium<128, 128, OutT>(x, w, y, m, n, k, columns, stream);
+  if (tile == 7) return launch_tiled_medium<256, 128, OutT>(x, w, y, m, n, k, columns, stream);
+  if (tile == 8) return launch_tiled_medium<128, 192, OutT>(x, w, y, m, n, k, columns, stream);
   if (tile == 2) return launch_tiled<64, 128, 64, OutT>(x, w, y, m, n, k, columns, ws, stream);
   return launch_tiled<64, 64, 64, OutT>(x, w, y, m, n, k, columns, ws, stream);
 }
@@ -1257,7 +1268,7 @@ extern "C" int nnis_gemm_bf16(const void* x, const void* w, void* y, int y_dtype
     NNIS_LAUNCH_CHECK("gemm_skinny");
   } else {
     NNIS_REQUIRE((m + 63) / 64 <= 65535, "gemm_bf16: %d rows exceed the grid limit", m);
-    const int tile_hint = split_hint >= 16 ? split_hint / 16 : 0;  // hints of 32, 48, .. 112 pick the tile: 64x128, 64x64, 256x256, 256x192, 128x128, 256x128
+    const int tile_hint = split_hint >= 16 ? split_hint / 16 : 0;  // hints of 32, 48, .. 128 pick the tile: 64x128, 64x64, 256x256, 256x192, 128x128, 256x128, 128x192
     if (y_dtype == NNIS_F32) dispatch_tiled<float*>(xp, wp, (float*)y, m, n, k, tile_hint, ws, stream);
     else dispatch_tiled<bf16_t*>(xp, wp, (bf16_t*)y, m, n, k, tile_hint, ws, stream);
     NNIS_LAUNCH_CHECK("gemm_tiled");
@@ -1266,7 +1277,7 @@ extern "C" int nnis_gemm_bf16(const void* x, const void* w, void* y, int y_dtype
 }
 
 // The tile that the tiled kernel takes for m rows, `columns` weight rows and a depth of k (2: 64 x 128, 3: 64 x 64,
-// 4: 256 x 256, 5: 256 x 192, 6: 128 x 128, 7: 256 x 128): for tests and tuning.
+// 4: 256 x 256, 5: 256 x 192, 6: 128 x 128, 7: 256 x 128, 8: 128 x 192): for tests and tuning.
 extern "C" int nnis_gemm_tile(int m, int columns, int k) { return pick_tile(m, columns, k, 0); }
 
 // The projection that ends a part of a pre-norm block: resid += x . w^T in 32-bit, in place, and the norm
@@ -1292,7 +1303,7 @@ extern "C" int nnis_gemm_residual(const void* x, const void* w, float* resid, co
   hipStream_t stream = (hipStream_t)stream_ptr;
   ResidualOut out = {resid, gain, gain_dtype, (bf16_t*)scaled, ss};
   NNIS_REQUIRE((uintptr_t)workspace % 16 == 0, "gemm_residual: the workspace must be 16-byte aligned");
-  NNIS_REQUIRE(tile_hint == 0 || (tile_hint >= 2 && tile_hint <= 7), "gemm_residual: unknown tile %d", tile_hint);
+  NNIS_REQUIRE(tile_hint == 0 || (tile_hint >= 2 && tile_hint <= 8), "gemm_residual: unknown tile %d", tile_hint);
   const bool few = tile_hint == 0 && takes_few_tokens_with_parts(m, n, k, workspace != nullptr);  // a tile hint asks for the tiled kernel
   const int writes = few ? (n + 15) / 16 : tiled_parts(m, n, k, tile_hint);
   NNIS_REQUIRE(writes <= ss_rows, "gemm_residual: ss has %d rows of %d tokens, %d are needed", ss_rows, m, writes);

@@ -517,7 +517,7 @@ def _check_epilogue(what: str, m: int, n: int, y: torch.Tensor, epilogue: int, r
 
 
 # tiles of the tiled product (``tile`` of gemm_residual; 16 times as much as a ``split`` of gemm_bf16 / gemm_scaled)
-TILE_64x128, TILE_64x64, TILE_256x256, TILE_256x192, TILE_128x128, TILE_256x128 = 2, 3, 4, 5, 6, 7
+TILE_64x128, TILE_64x64, TILE_256x256, TILE_256x192, TILE_128x128, TILE_256x128, TILE_128x192 = 2, 3, 4, 5, 6, 7, 8
 
 
 def gemm_tile(m: int, n: int, k: int) -> int:
@@ -540,8 +540,8 @@ def gemm_residual(x: torch.Tensor, w: torch.Tensor, resid: torch.Tensor, gain: t
     ``x`` may be the ``KeyRuns`` of a decode attention (where ``fits``): the
     kernel then adds the runs up itself on its way.  ``tile`` (for tests and
     tuning): 0 lets the sizes choose, ``TILE_64x128``, ``TILE_64x64``,
-    ``TILE_256x256``, ``TILE_256x192``, ``TILE_128x128`` and ``TILE_256x128`` ask for
-    the tiled kernel with that tile."""
+    ``TILE_256x256``, ``TILE_256x192``, ``TILE_128x128``, ``TILE_256x128`` and
+    ``TILE_128x192`` ask for the tiled kernel with that tile."""
     _packed(w, "gemm_residual")
     m, k = x.shape
     n = w.shape[0]

@@ -453,9 +453,9 @@ def test_step_tables_and_the_kernels_that_read_them():
     assert not torch.equal(results[1][1], k_pages.cpu())  # and the cache was written
 
 
-@pytest.mark.parametrize("hint", [32, 48, 64, 80, 96, 112])
+@pytest.mark.parametrize("hint", [32, 48, 64, 80, 96, 112, 128])
 def test_gemm_tiled_over_many_blocks(hint):
-    """Each tile of the tiled kernel (64 x 128, 64 x 64, 256 x 256, 256 x 192, 128 x 128, 256 x 128) over a grid of hundreds of blocks in
+    """Each tile of the tiled kernel (64 x 128, 64 x 64, 256 x 256, 256 x 192, 128 x 128, 256 x 128, 128 x 192) over a grid of hundreds of blocks in
     bands and groups, with a ragged edge in every dimension; whole-number
     operands, so a block that took another's rows or columns shows."""
     ops = _ops()
@@ -497,7 +497,7 @@ def test_residual_projection_prepares_the_norm(m, n, k, gain_dtype):
     assert ((total - got.pow(2).sum(dim=1)).abs() <= 1e-5 * got.pow(2).sum(dim=1)).all()
 
 
-@pytest.mark.parametrize("tile", ["TILE_64x128", "TILE_64x64", "TILE_256x256", "TILE_256x192", "TILE_128x128", "TILE_256x128"])
+@pytest.mark.parametrize("tile", ["TILE_64x128", "TILE_64x64", "TILE_256x256", "TILE_256x192", "TILE_128x128", "TILE_256x128", "TILE_128x192"])
 @pytest.mark.parametrize("m, n, k", [(70, 600, 136), (530, 300, 72), (300, 1100, 584)])
 def test_residual_projection_with_every_tile(tile, m, n, k):
     """The tiled kernel's residual epilogue with each tile shape (several row
@@ -515,7 +515,7 @@ def test_residual_projection_with_every_tile(tile, m, n, k):
     rows = ops.gemm_residual_parts(m, n)
     ss = torch.full((rows + 1, m), 7.0, device="cuda")
     parts = ops.gemm_residual(x.cuda(), ops.pack_weight(w.cuda()), resid_gpu, gain.cuda(), scaled, ss, getattr(ops, tile))
-    width = {"TILE_64x128": 64, "TILE_64x64": 32, "TILE_256x256": 128, "TILE_256x192": 96, "TILE_128x128": 64, "TILE_256x128": 64}[tile]  # columns of a wave
+    width = {"TILE_64x128": 64, "TILE_64x64": 32, "TILE_256x256": 128, "TILE_256x192": 96, "TILE_128x128": 64, "TILE_256x128": 64, "TILE_128x192": 96}[tile]  # columns of a wave
     if parts != 2 * ((n + 2 * width - 1) // (2 * width)):  # few tiles and a long K: K went in parts, summed per 64 columns
         assert tile in ("TILE_64x128", "TILE_64x64") and k >= 512 and parts == (n + 63) // 64
         width = 64
@@ -612,7 +612,7 @@ def test_fused_norm_projection(m, k, with_delta, gain_dtype):
     assert int((v_plain != 7.0).any(dim=-1).sum()) <= written * kv_heads
 
 
-@pytest.mark.parametrize("hint", [32, 48, 64, 80, 96, 112])
+@pytest.mark.parametrize("hint", [32, 48, 64, 80, 96, 112, 128])
 @pytest.mark.parametrize("m", [65, 200, 530])
 def test_scaled_projection_with_every_tile(hint, m):
     """The tiled kernel's epilogues with each of its tile shapes (the hint picks
@@ -899,8 +899,11 @@ def test_the_tiles_that_products_are_given():
         (2048, 4096, 14336): T.TILE_256x128,
         (2048, 2048, 8192): T.TILE_128x128,   # 256 blocks of 128 rows where 256 rows make 128
         (2048, 2048, 512): T.TILE_64x128,     # ... over a short K the small tiles
-        (2048, 2560, 2048): T.TILE_64x128,    # a round and a quarter of 128 x 128, five eighths of one of 256 x 128: not taken
-        (2048, 3072, 2048): T.TILE_256x128,   # three quarters of a round (eleven sixteenths are enough)
+        (2048, 2560, 2048): T.TILE_128x192,   # 224 tiles, where 256 x 128 makes 160 and 128 x 128 a round and a quarter
+        (1536, 2560, 2048): T.TILE_128x128,
+        (2048, 3072, 2048): T.TILE_128x192,   # a full round of 128 x 192 before three quarters of one of 256 x 128
+        (1536, 4096, 4096): T.TILE_256x128,   # three quarters of a round (eleven sixteenths are enough)
+        (1024, 6144, 2048): T.TILE_128x192,
         (2048, 1536, 2048): T.TILE_128x128,
         (3072, 2048, 4096): T.TILE_256x128,   # (192 blocks, where 128 x 128 would make a round and a half)
         (1024, 2048, 2048): T.TILE_64x64,     # no more than one wide block a compute unit: the narrow tile
