@@ -1075,84 +1075,63 @@ int launch_tiled(const bf16_t* x, const bf16_t* w, OutT y, int m, int n, int k, 
   return launch_tiled_staged<BM, BN, BK, 3, OutT>(x, w, y, m, n, k, col_blocks, row_blocks, ksplit, ws, stream);
 }
 
-// 2: 64x128, 3: 64x64, 4: 256x256, 5: 256x192, 6: 128x128, 7: 256x128, 8: 128x192 -- the larger tile when it still gives (nearly) every compute unit a block.
-// (A tile of 128x128 was measured slower than 64x128 on every product from 2048 x 576 x 576 to 2048 x 6144 x 2048;
-// the tile of 256x256 against 64x128, microseconds: 2048 x 6144 x 2048, 192 blocks, 57 against 68; 2048 x 11264 x
-// 2048, 352 blocks, 108 against 119; but 2048 x 2560 x 2048, 80 blocks, 48 against 34, and 2048 x 2048 x 8192, 64
-// blocks, 152 against 89.)
+// The tile of a product: 2: 64x128, 3: 64x64 (4 waves, several blocks a compute unit), and five tiles of 8 waves that
+// a compute unit runs one at a time -- 4: 256x256, 5: 256x192 (two stages), 7: 256x128, 8: 128x192, 6: 128x128 (three
+// stages, a step's second half multiplied behind the barrier).
+//
+// Among the five the one whose rounds of blocks (blocks / 256 compute units, rounded up) come to the least tile area
+// over the tile's rate.  Rates, from full rounds at K = 2048 over weights from memory, relative to 256x128 (32768
+// outputs in 35.5 us): 256x256 1.10, 256x192 1.08, 128x192 0.91, 128x128 0.82.  The rule names the fastest tile, or
+// one within a few per cent of it, on all of 77 products of 256 to 4,096 rows with 2,048 to 16,384 columns (auto
+// against each tile asked for); a few of them, microseconds: 2048 x 16384 in 512 tiles of 256x256 128 (256x128: 141);
+// 2048 x 6144 in 256 of 256x192 49 (256x256, 192 tiles: 56); 3072 x 6144 in 768 of 128x192 80 (384 of 256x192: 92);
+// 1536 x 16384 in 768 of 256x128 99 (384 of 256x256: 113); 4096 x 2048 in 256 of 256x128 35.5 (512 of 128x128: 43);
+// 2048 x 2560 in 224 of 128x192 26.5 (64x128: 29); 2048 x 2048 in 256 of 128x128 21.6 (64x128: 23.6).  At a K of
+// 8,192 the three-stage tiles gain on the others (4096 x 2048 x 8192 in 256 of 256x128: 117 us, 1.18 PFLOP/s): from
+// a K of 8,192 on the rates are 256x256 0.97, 256x192 0.93, 128x192 0.90, 128x128 0.80 of 256x128, from 4,096 on
+// the same but 256x256 1.03 (4096 x 6144 x 8192 in 768 tiles of 256x128 347 us against 383 in 512 of 256x192; 2048 x 28672 x
+// 4096 in 1792 of them 438 against 473 in 896 of 256x256); there the rule is within a tenth of the fastest tile on
+// the same 77 products but one (1536 x 6144 x 8192: 190 in 192 tiles of 256x192, 162 in 384 of 128x192, a round and
+// a half that the rule below keeps out).
+//
+// What keeps a tile out:
+//  * rows that do not fill its row blocks: 300 rows would be multiplied as 512.  Three quarters for the three-stage
+//    tiles (384 x 16384 x 4096 as 512 rows in 256 tiles of 256x128: 61 us against 75 in tiles of 64x128); for the two-stage ones three quarters from 1,024 rows on and fifteen sixteenths below (384 x 16384 x
+//    2048 as 512 rows of 256x192 took 44.5 us against 34.2 in tiles of 64x128);
+//  * blocks too few for the chip, against the 4-wave tiles, which several of fit a compute unit: the two-stage tiles
+//    want 160 blocks (1024 x 6144 x 2048 in 128 tiles: 44 us against 34), a single round of the others five eighths
+//    of the compute units (1024 x 2560 x 2048 in 160 tiles of 128x128: 20.0 against 21.6; 1024 x 2048 x 8192 in 128:
+//    58 against 51; in 144, 768 x 3072 60 against 67 but 384 x 6144 77 against 68), two rounds seven eighths of them (3072 x 2048 x 4096 in 384 tiles of 128x128: 81 against 69),
+//    more rounds a last one that is half full (1280 x 16384 x 8192 in 640 tiles of 256x128: 334 against 372);
+//  * a short K: the three-stage tiles from 1,024 on, the others from 256.
+// Of the 4-wave tiles the narrow one up to one wide block a compute unit: 1024 x 2048 x 2048 in 256 wide blocks takes
+// 19.1 us, in 512 narrow ones 16.0; with 320 wide blocks (1024 x 2560) the wide tile is ahead, 20.9 to 22.3.
 #ifndef NNIS_LARGE_TILE_BLOCKS
 #define NNIS_LARGE_TILE_BLOCKS 160
 #endif
 int pick_tile(int m, int columns, int k, int tile_hint) {
   const long long blocks_64_128 = (long long)((m + 63) / 64) * ((columns + 127) / 128);
-  const long long rows_256 = (m + 255) / 256;
-  // The narrow tile up to one wide block a compute unit: 1024 x 2048 x 2048 in 256 wide blocks takes 19.1 us, in 512
-  // narrow ones 16.0 (x 8192: 59.5 against 53.5); with 320 wide blocks (1024 x 2560) the wide tile is ahead, 20.9 to 22.3.
   int tile = blocks_64_128 > 256 ? 2 : 3;
-  // The large tiles: rows that fill three quarters of their tiles of 256 at least (300 rows would be multiplied as
-  // 512; up to 768 rows the large tile is only a tenth ahead when full, so it has to be: 384 x 16384 x 2048 took 44.5 us
-  // as 512 rows against 34.2 in tiles of 64), and of the two widths one that makes NNIS_LARGE_TILE_BLOCKS blocks and more -- a compute unit runs one large
-  // tile at a time, and fewer leave too many idle: 512 x 16384 x 2048 in 172 tiles of 256 x 192 takes 46 us against 52,
-  // 768 x 11264 x 2048 in 177 47 against 54, but 1024 x 6144 x 2048 in 128 44 against 34.  Where both widths do, the
-  // one whose rounds of blocks come to fewer columns a compute unit (2048 x 6144: 192 blocks of 256 columns or 256
-  // of 192, a round either way; 1024 x 11264: 176 or 236, 60 us against 49).
-  const bool filled = rows_256 >= 4 ? 4LL * m >= 3 * 256 * rows_256 : 16LL * m >= 15 * 256 * rows_256;
-  if (k >= 256 && filled) {
-    const long long units = 256;
-    long long best = 0;
-    for (int width : {256, 192}) {
-      const long long blocks = rows_256 * ((columns + width - 1) / width);
-      if (blocks < NNIS_LARGE_TILE_BLOCKS) continue;
-      const long long cost = ((blocks + units - 1) / units) * width;
-      if (best == 0 || cost < best) {
-        best = cost;
-        tile = width == 256 ? 4 : 5;
-      }
+  struct Candidate { int tile, rows, width, rate[3], stages; };  // rates for a K below 4,096, below 8,192, and beyond
+  const int depth = k >= 8192 ? 2 : (k >= 4096 ? 1 : 0);
+  long long best = 0;
+  for (const Candidate c : {Candidate{4, 256, 256, {110, 103, 97}, 2}, Candidate{5, 256, 192, {108, 93, 93}, 2},
+                            Candidate{7, 256, 128, {100, 100, 100}, 3}, Candidate{8, 128, 192, {91, 90, 90}, 3},
+                            Candidate{6, 128, 128, {82, 80, 80}, 3}}) {
+    const long long row_blocks = (m + c.rows - 1) / c.rows;
+    const long long blocks = row_blocks * ((columns + c.width - 1) / c.width);
+    const long long rounds = (blocks + 255) / 256;
+    if (c.stages == 2) {
+      const bool filled = row_blocks >= 4 ? 4LL * m >= 3LL * c.rows * row_blocks : 16LL * m >= 15LL * c.rows * row_blocks;
+      if (k < 256 || !filled || blocks < NNIS_LARGE_TILE_BLOCKS) continue;
+    } else {
+      if (k < 1024 || 4LL * m < 3LL * c.rows * row_blocks) continue;
+      if (rounds == 1 ? 8 * blocks < 5 * 256 : (rounds == 2 ? 8 * blocks < 7 * 256 * 2 : 2 * blocks < (2 * rounds - 1) * 256)) continue;
     }
-  }
-  // The tile of 128 x 128, a block of 8 waves a compute unit: where its blocks fill one or two rounds of the chip
-  // (see below how far) over a K of 1,024 and more and no large tile fills three quarters of its rounds.
-  // Microseconds, into the stream, against what was taken before: 2048 x 2048 x 8192 (256 blocks) 79 to 85 against 88
-  // to 102 in tiles of 64 x 128, x 5632 57.5 against 62, x 2048 28.1 against 28.9, x 1024 20.4 against 20.9; 4096 x
-  // 2048 x 8192 (512) 160 against 195 in 176 tiles of 256 x 192, x 5632 and x 2048 the same; 2048 x 1792 x 4096 (224)
-  // 45 against 48; slower where a round is left partly empty (2048 x 2560: 46 against 37; 3072 x 2048 x 4096, a round
-  // and a half: 81 against 69) or half the chip is (1024 x 2048 x 8192: 65 against 58).
-  // The tile of 256 x 128 (three stages, a wave tile of 64 x 64) by the same rule, before that of 128 x 128: 4096 x
-  // 2048 x 8192 in 256 blocks 121 us plain and 131 into the stream (1.12 PFLOP/s) against 146 to 161 and 158 to 165
-  // in 512 tiles of 128 x 128, x 2048 37 and 46 against 43 and 54; 2048 x 4096 x 14336 214 and 226 against 258 and
-  // 267; 3840 x 2048 x 5632 (240 blocks) 82 and 92 against 100 and 108.  Where a large tile fills its rounds it stays
-  // (4096 x 4096 x 4096: 112 plain in 256 tiles of 256 x 256 against 126 in 512 of 256 x 128, into the stream alike);
-  // where it fills less than three quarters this tile is ahead of it too: 512 x 16384 x 2048 in 256 blocks 38 us over
-  // weights from memory, in 172 tiles of 256 x 192 57 to 69; 3072 x 2560 x 2048 (240 blocks) 35 against 46.
-  // A single round may be eleven sixteenths full (2304 x 2560 x 2048 in 180 tiles of 256 x 128 29.4 us against 32.3;
-  // 2048 x 3072 x 2048 in 192 tiles of 256 x 128 32 us against 34.5 in
-  // tiles of 64 x 128, 1536 x 4096 x 4096 55 against 60; 2048 x 1536 x 2048 in 192 of 128 x 128 19.7 against 21.4; at
-  // five eighths, 2048 x 2560 x 2048, 31.7 against 32.4: not taken), two rounds seven eighths (3072 x 2048 x 4096 in
-  // 384 tiles of 128 x 128: 81 against 69).
-  bool large_fills = false;
-  if (tile == 4 || tile == 5) {
-    const long long large = rows_256 * ((columns + (tile == 4 ? 255 : 191)) / (tile == 4 ? 256 : 192));
-    large_fills = 4 * large >= 3 * 256 * ((large + 255) / 256);
-  }
-  // Of the three the one whose rounds come to the least area over its rate: a compute unit multiplies a tile of 128
-  // x 192 (a wave tile of 32 x 96) at about 0.85 and one of 128 x 128 at about 0.8 of the rate of 256 x 128.  2048 x 3072
-  // x 2048 with the gate's epilogue in 256 tiles of 128 x 192 27.7 us against 31 in 192 of 256 x 128; 1024 x 6144 x
-  // 2048 with the rotation 33 against 37.6; 2048 x 2560 x 2048 (224 tiles, where 256 x 128 makes 160) 33 to 34.5
-  // against 36 in tiles of 64 x 128.
-  if (k >= 1024 && !large_fills) {
-    struct Candidate { int tile, rows, width, rate; };
-    long long best = 0;
-    for (const Candidate c : {Candidate{7, 256, 128, 100}, Candidate{8, 128, 192, 85}, Candidate{6, 128, 128, 80}}) {
-      const long long row_blocks = (m + c.rows - 1) / c.rows;
-      if (8LL * m < 7LL * c.rows * row_blocks) continue;
-      const long long blocks = row_blocks * ((columns + c.width - 1) / c.width);
-      const long long rounds = (blocks + 255) / 256;
-      if (!(rounds == 1 ? 16 * blocks >= 11 * 256 : (rounds == 2 && 8 * blocks >= 7 * 256 * rounds))) continue;
-      const long long cost = rounds * c.rows * c.width * 100 / c.rate;
-      if (best == 0 || cost < best) {
-        best = cost;
-        tile = c.tile;
-      }
+    const long long cost = rounds * c.rows * c.width * 100 / c.rate[depth];
+    if (best == 0 || cost < best) {
+      best = cost;
+      tile = c.tile;
     }
   }
   if (tile_hint >= 2 && tile_hint <= 8) tile = tile_hint;  // for tuning runs

@@ -893,7 +893,8 @@ def test_the_tiles_that_products_are_given():
         (2048, 6144, 2048): T.TILE_256x192,   # 256 blocks of 192 columns, where 256 columns make 192
         (1024, 11264, 2048): T.TILE_256x192,  # 236 blocks
         (512, 16384, 2048): T.TILE_256x128,   # 256 blocks where tiles of 256 x 192 make 172
-        (384, 16384, 2048): T.TILE_64x128,    # ... rows that do not
+        (384, 16384, 2048): T.TILE_256x128,   # rows that fill three quarters of their blocks: enough for a three-stage tile
+        (320, 16384, 2048): T.TILE_64x128,    # ... and rows that do not (the blocks of 128 rows would be 384: a round and a half)
         (4096, 4096, 4096): T.TILE_256x256,   # a large tile that fills its round stays
         (4096, 2048, 8192): T.TILE_256x128,   # 256 blocks, one a compute unit, where large tiles would be 176
         (2048, 4096, 14336): T.TILE_256x128,
