@@ -840,17 +840,19 @@ def prefill_plan(longest: int, rows: int, heads: int, head_dim: int = 64, kv_hea
     # heads of 64 at 8,192 tokens 349 against 467; 64/8 heads of 64 at 4,096 180 against 243; 32/8 heads of 128 at
     # 2,048 66 against 102, at 8,192 833 against 1,306; 16 heads of 96 at 8,192 259 against 349.  Up to 64 channels a
     # step of half that size has the items with two columns: 32 heads at 4,096 tokens 119 against 137, 64/8 heads at
-    # 2,048 64 against 74, 16 heads at 8,192 213 against 243 -- where two columns divide a group's heads (of 9/3
-    # heads they would leave a quarter of the columns empty: 227 against 145 at 8,192).  At a quarter (32 heads at
-    # 2,048 tokens) the kernel alone took 49 against 47 to 56 and whole prompts 2 to 3% longer: not taken there.
+    # 2,048 64 against 74, 16 heads at 8,192 213 against 243, and from three eighths on 32 heads at 3,072 83 against
+    # 93 -- where two columns divide a group's heads (of 9/3 heads they would leave a quarter of the columns empty:
+    # 227 against 145 at 8,192; 24/8 heads of 64 at 8,192 tokens have items of three columns for twice the chip's
+    # waves: 276 with one wave an item against 345).  At a quarter (32 heads at 2,048 tokens) the kernel alone took 49
+    # against 47 to 56 and whole prompts 2 to 3% longer: not taken there.
     # With fewer items the waves of a block deal an item's keys: 9/3 heads of 64 at 8,192 tokens 141 with 8 waves,
     # 193 with one.
-    wide = 4 if head_dim <= 64 else (2 if head_dim <= 128 else 1)
+    group = heads // kv_heads if kv_heads else 1
+    wide = (3 if group == 3 else 4) if head_dim <= 64 else (2 if head_dim <= 128 else 1)  # (a group of 3 heads fills 3 columns)
     many = 2 * (2048 if head_dim <= 64 else 1024) * 16 * wide
     if size >= many:
         return 1, 0
-    group = heads // kv_heads if kv_heads else 1
-    if head_dim <= 64 and 2 * size >= many and (group == 1 or group % 2 == 0):
+    if head_dim <= 64 and 8 * size >= 3 * many and (group == 1 or group % 2 == 0):
         return 1, 2
     waves = (1, 2, 4, 8, 8)[plan_class]
     if waves == 8 and head_dim <= 64 and group != 3 and size > PREFILL_EIGHT_WAVES_MOST:
@@ -858,7 +860,9 @@ def prefill_plan(longest: int, rows: int, heads: int, head_dim: int = 64, kv_hea
     if plan_class == 0 or plan_class == 4 or size >= PREFILL_MANY_ROWS:
         return waves, 0
     if plan_class == 3:
-        return (4, 2) if size >= PREFILL_SOME_ROWS else (8, 0)
+        if size < PREFILL_SOME_ROWS:
+            return 8, 0
+        return (4, 0) if group == 3 else (4, 2)  # (two columns would leave a group of 3 heads a quarter of them empty)
     return waves, plan_class  # 2 waves and one column from 128 tokens on, 4 waves and two columns from 512 on
 
 
