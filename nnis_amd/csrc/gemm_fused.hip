@@ -493,9 +493,16 @@ int run_fused(FusedArgs& a, int epilogue, int table_positions, int split_hint, f
   const int chunks = (k + 63) / 64;
   const int per_wave = (size_t)n * k * sizeof(bf16_t) <= kRereadWeightBytes ? 1 : (a.m + 15) / 16;  // token tiles a wave takes
   const int depth = a.scaled ? (per_wave <= 2 ? 4 : 2) : (per_wave == 1 ? 2 : 1);  // the kernel's steps in flight
+  // On a prepared operand no more waves than take 4,096 strips of 16 weight rows between them (two waves a SIMD at
+  // pairs of strips): every wave begins with the row's scale, and beyond that number the beginnings cost more than
+  // the shorter shares save.  Measured at 1 and 8 tokens over cold weights, microseconds with 8 / 4 / 2 waves a unit:
+  // gate/up of 2 x 5632 x 2048 14.1 / 12.5 / 13.3, 2 x 8192 x 2048 16.2 / 15.3 / 15.5, 2 x 14336 x 4096 49.0 / 46.1 /
+  // 45.3; plain rows 11264 x 2048 14.2 / 11.7 / 14.5, 28672 x 2048 30.5 / 25.6 / 25.9; up to 512 strips 8 waves
+  // are the fastest (8192 x 2048 9.4 / 9.9 / 11.3).
+  const int strips = epilogue == EPI_STORE ? units : (epilogue == EPI_SILU ? 2 * units : 0);  // (the rotating epilogue gains nothing: 96 x 128 x 4096 25.1 / 25.7 / 26.0)
   int split = 1;
   if (units < 2048) {
-    while (split < 8 && chunks > split * depth) split *= 2;
+    while (split < 8 && chunks > split * depth && (!a.scaled || strips * split * 2 <= 4096)) split *= 2;
   }
   if (split_hint == 1 || split_hint == 2 || split_hint == 4 || split_hint == 8) split = split_hint;  // for tuning runs
   if (epilogue == EPI_STORE) dispatch_fused<EPI_STORE>(a, units, split, stream);
