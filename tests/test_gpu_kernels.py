@@ -670,6 +670,35 @@ def test_scaled_projection_with_every_tile(hint, m):
     assert int((k_plain != 7.0).any(dim=-1).sum()) <= written * kv_heads  # padding rows wrote nothing
 
 
+@pytest.mark.parametrize("m", [1, 8, 16, 30])
+@pytest.mark.parametrize("n, paired", [(8192, False), (11264, False), (32000, False), (2 * 4096, True), (2 * 5632, True), (2 * 14336, True)])
+def test_prepared_projection_on_wide_weights(n, paired, m):
+    """Few tokens on a prepared operand over hundreds to thousands of strips of 16 weight rows, where the
+    number of waves that share a strip's K goes from 8 to 4, 2 and 1 with the width: every width the rule
+    tells apart, with the sizes' own choice."""
+    ops = _ops()
+    torch.manual_seed(n + m)
+    k, eps = 2048, 1e-5
+    v = torch.randn(m, k) * 2
+    gain = (1 + 0.3 * torch.randn(k)).bfloat16()
+    normed = P.rms_norm(v.double(), gain.double(), eps)
+    scaled = torch.empty(m, k, dtype=torch.bfloat16, device="cuda")
+    ss = torch.empty(ops.gemm_residual_parts(m, k), m, device="cuda")
+    parts = ops.gemm_residual(torch.zeros(m, 8, dtype=torch.bfloat16, device="cuda"), ops.pack_weight(torch.zeros(k, 8, dtype=torch.bfloat16, device="cuda")),
+                              v.cuda(), gain.cuda(), scaled, ss)
+    w = (torch.randn(n, k) / math.sqrt(k)).bfloat16()
+    both = normed @ w.double().t()
+    if paired:
+        want = P.silu(both[:, :n // 2]) * both[:, n // 2:]
+        y = torch.empty(m, n // 2, dtype=torch.bfloat16, device="cuda")
+        got = ops.gemm_scaled(scaled, ss, parts, eps, ops.pack_weight(w.cuda()), y, ops.EPILOGUE_SILU).cpu().double()
+    else:
+        want = both
+        y = torch.empty(m, n, dtype=torch.bfloat16, device="cuda")
+        got = ops.gemm_scaled(scaled, ss, parts, eps, ops.pack_weight(w.cuda()), y, ops.EPILOGUE_STORE).cpu().double()
+    assert ((got - want).abs() <= 2e-2 * (1 + want.abs())).all(), (got - want).abs().max().item()
+
+
 def _k_index(head_dim):
     """[64 tokens, head_dim] -> offset of each (token, channel) in a page's keys of one head."""
     t = torch.arange(64).view(64, 1)
