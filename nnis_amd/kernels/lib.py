@@ -51,7 +51,7 @@ SOURCE_FLAGS = {"gemm_mfma.hip": _VECTOR_SUMS, "attention.hip": _VECTOR_SUMS}
 HEADERS = {"core": ["common.h", "epilogue.h", "nnis_noalloc.h"], "attention": ["common.h"]}  # what a module's sources include
 CORE_SOURCES = ["elementwise.hip", "gemm.hip", "gemm_mfma.hip", "gemm_fused.hip", "sampling.hip"]
 ATTENTION_SOURCES = ["attention.hip"]
-PREBUILT_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 112, 128)
+PREBUILT_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 112, 128, 192, 256)
 
 _loaded: Dict[str, ctypes.CDLL] = {}
 _lock = threading.Lock()

@@ -142,7 +142,7 @@ def test_gemm_bf16_refuses_what_it_cannot_load():
 
 
 MFMA_SHAPES = [(4, 2, 16), (3, 3, 16), (3, 1, 32), (6, 2, 48), (6, 6, 48), (4, 2, 48), (9, 3, 64), (2, 2, 64), (5, 5, 80),
-               (4, 1, 112), (8, 2, 128), (32, 1, 64), (40, 2, 16), (8, 1, 64), (12, 2, 32)]
+               (4, 1, 112), (8, 2, 128), (32, 1, 64), (40, 2, 16), (8, 1, 64), (12, 2, 32), (2, 1, 192), (3, 3, 256)]
 
 
 def _small_decode_call(heads, kv_heads, head_dim):
@@ -168,7 +168,7 @@ def _plain_rows(q_rows, ks, vs, scale, window=0):
 @pytest.mark.parametrize("kernel", ["columns", "keys"])
 def test_decode_attention_on_the_matrix_cores(heads, kv_heads, head_dim, splits, waves, kernel):
     ops = _ops()
-    if kernel == "keys" and heads // kv_heads > 4:
+    if kernel == "keys" and (heads // kv_heads > 4 or head_dim > 128):  # refused, in words
         with pytest.raises(Exception, match="keys on lanes"):
             ops.attention_decode_bf16(*_small_decode_call(heads, kv_heads, head_dim), kernel="keys")
         return
@@ -745,7 +745,7 @@ def _paged(k_seqs, v_seqs, dtype, kv_heads, head_dim, page_order=None, pages=32,
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("heads, kv_heads, head_dim", [(4, 2, 16), (3, 1, 32), (9, 3, 64), (5, 5, 80), (8, 2, 128)])
+@pytest.mark.parametrize("heads, kv_heads, head_dim", [(4, 2, 16), (3, 1, 32), (9, 3, 64), (5, 5, 80), (8, 2, 128), (2, 1, 192), (3, 3, 256)])
 def test_attention_over_pages(dtype, heads, kv_heads, head_dim):
     """Queries at the end of three sequences of unequal length (and one in the
     middle of a sequence), pages handed out in reverse order."""

@@ -62,7 +62,7 @@ def test_rotary_tables_equal_the_plain_ones():
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("heads, kv_heads, head_dim, width", [(4, 2, 16, 64), (3, 1, 32, 80), (6, 6, 48, 100)])
+@pytest.mark.parametrize("heads, kv_heads, head_dim, width", [(4, 2, 16, 64), (3, 1, 32, 80), (6, 6, 48, 100), (2, 1, 192, 96), (3, 3, 256, 96)])
 def test_attention_part(dtype, heads, kv_heads, head_dim, width):
     """Two sequences of unequal length, whole and then continued by single
     tokens, against the plain functions on each whole sequence."""
