@@ -741,3 +741,53 @@ def test_long_prompts_on_many_heads(tmp_path, heads, head_dim, inner, tokens, pl
     plain = P.PlainLlama(folder)
     rows = places + list(range(tokens, tokens + 8))
     Bf16Yardstick(plain, [ids[:600]]).check(got, plain.logits(ids)[rows], f"a prompt of {tokens} tokens on {heads} heads")
+
+
+AWKWARD = {
+    # widths and an inner size that are no multiple of 8 (no 16-byte rows: the ordered product), five heads of 16
+    "width 100": dict(num_hidden_layers=2, hidden_size=100, num_attention_heads=5, num_key_value_heads=5, head_dim=16, intermediate_size=130,
+                      vocab_size=777, tie_word_embeddings=True),
+    # seven query heads on one key/value head, an inner size below the width, a vocabulary that is odd
+    "seven on one": dict(num_hidden_layers=2, hidden_size=104, num_attention_heads=7, num_key_value_heads=1, head_dim=32, intermediate_size=100,
+                         vocab_size=1003, tie_word_embeddings=False),
+    # a width of 36 and a vocabulary of 61: smaller than any tile
+    "width 36": dict(num_hidden_layers=1, hidden_size=36, num_attention_heads=3, num_key_value_heads=3, head_dim=16, intermediate_size=52,
+                     vocab_size=61, tie_word_embeddings=True),
+    # heads of 192 channels: beyond what the decode kernel with keys on lanes takes
+    "heads of 192": dict(num_hidden_layers=2, hidden_size=192, num_attention_heads=2, num_key_value_heads=1, head_dim=192, intermediate_size=264,
+                         vocab_size=333, tie_word_embeddings=True),
+}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("case", sorted(AWKWARD))
+def test_awkward_sizes(tmp_path, case, dtype):
+    """Sizes that no kernel's tiles divide: three prompts of unequal length in one step and six tokens each one by
+    one, every logit against the plain model."""
+    import nnis_amd
+    from configs import llama
+    from nnis_amd.api import load_engine
+    from nnis_amd.engine.batch import StepEntry
+
+    config = llama(rope_theta=10000.0, rms_norm_eps=1e-5, max_position_embeddings=256, torch_dtype="bfloat16", **AWKWARD[case])
+    folder = str(tmp_path / "model")
+    os.makedirs(folder)
+    nnis_amd.write_random_model(folder, config, 3)
+    plain = P.PlainLlama(folder)
+    rng = np.random.default_rng(len(case))
+    sequences = [rng.integers(0, config["vocab_size"], size=n + 6).tolist() for n in (70, 9, 1)]
+    yard = Bf16Yardstick(plain, sequences) if dtype == "bfloat16" else None
+    engine = load_engine(folder, dtype=dtype, max_tokens=8 * 64)
+    slots = [engine.start_sequence() for _ in sequences]
+    got = [[] for _ in sequences]
+    rows = engine.step([StepEntry(slot, ids[:-6], list(range(len(ids) - 6))) for slot, ids in zip(slots, sequences)])
+    at = 0
+    for i, ids in enumerate(sequences):
+        got[i].append(rows[at:at + len(ids) - 6])
+        at += len(ids) - 6
+    for step in range(6):
+        rows = engine.step([StepEntry(slot, [ids[len(ids) - 6 + step]], [0]) for slot, ids in zip(slots, sequences)])
+        for i in range(len(sequences)):
+            got[i].append(rows[i:i + 1])
+    for i, ids in enumerate(sequences):
+        _close(torch.cat(got[i]).cpu(), plain.logits(ids), dtype, f"{case}, sequence {i}", yard)
