@@ -261,22 +261,40 @@ __device__ __forceinline__ void make_activations(const RunsIn& runs, bf16_t* x_t
 
 // RUNS: x is not read but made, by the block for its 16 * MT tokens, from `runs` into LDS (every block makes
 // the same few KB again: cheaper than a kernel of its own between the attention and this projection).
-template <int MT, int KSPLIT, bool RUNS, typename OutT>
+// PAIR: two blocks share a strip's K (block 2 s takes the even shares, 2 s + 1 the odd ones).  Each leaves its sums
+// in `pair.sums`; the one that finds the other's already there (a count per strip in `pair.count`, which it sets
+// back to zero) adds them to its own and ends the strip.  Nobody waits for anybody.  For strips so few that they
+// leave half the chip without a block, on a K long enough that a compute unit's own rate of reading bounds the kernel.
+struct PairScratch {
+  float* sums;  // [strips][2][MT][64 lanes][4]
+  int* count;   // [strips], zero between calls
+};
+
+template <int MT, int KSPLIT, bool RUNS, typename OutT, bool PAIR = false>
 __global__ __launch_bounds__(KSPLIT > 4 ? 64 * KSPLIT : 256) void gemm_skinny_kernel(const bf16_t* __restrict__ x,
                                                                                    const bf16_t* __restrict__ w,
                                                                                    OutT y, int m, int n, int k, int tiles,
-                                                                                   int stream_weights, RunsIn runs) {
+                                                                                   int stream_weights, RunsIn runs,
+                                                                                   PairScratch pair) {
   constexpr int kWaves = KSPLIT > 4 ? KSPLIT : 4;
   constexpr int kStrips = kWaves / KSPLIT;  // strips of 16 weight rows per block
+  constexpr int kShares = PAIR ? 2 * KSPLIT : KSPLIT;  // waves that share a strip's K
+  static_assert(!PAIR || (!RUNS && kStrips == 1), "paired blocks: one strip a block, activations from memory");
   constexpr int DEPTH = MT <= 2 ? 4 : 2;
   __shared__ float partial[KSPLIT > 1 ? kWaves : 1][MT][kWave][4];
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
   int strip_block, tile;
-  nnis_deal_tiles(blockIdx.x, tiles, strip_block, tile);
+  if constexpr (PAIR) {
+    strip_block = blockIdx.x / 2;  // (one tile of tokens)
+    tile = 0;
+  } else {
+    nnis_deal_tiles(blockIdx.x, tiles, strip_block, tile);
+  }
   const int strip = strip_block * kStrips + wave / KSPLIT;
   const int token0 = tile * 16 * MT;  // this block's tokens: token0 + (0 .. 16 * MT - 1)
   const int x_row = k + 8;  // elements of a row of the activations in LDS: 16 rows apart fall into different banks
   const int part = wave % KSPLIT;
+  const int share = PAIR ? 2 * part + (int)(blockIdx.x % 2) : part;  // this wave's place among those that share the strip's K
   const int r = lane % 16, g = lane / 16;
   const int strips = (n + 15) / 16;
   const bool active = strip < strips;
@@ -304,19 +322,19 @@ __global__ __launch_bounds__(KSPLIT > 4 ? 64 * KSPLIT : 256) void gemm_skinny_ke
   const int chunks = nnis_packed_chunks(k);
   // packed weights: the strip's padding rows and the last chunk's padding are zeros that are there to read
   const bf16_t* w_ptr = w + nnis_packed_lane(active ? strip * 16 + r : 0, g, k);
-  // a round: DEPTH steps of 64 k of this wave (base, base + KSPLIT, ..): their weights ...
+  // a round: DEPTH steps of 64 k of this wave (base, base + kShares, ..): their weights ...
   auto ask_weights = [&](int base, bf16x8 (&wa)[DEPTH], bf16x8 (&wb)[DEPTH]) {
     if (stream_weights) {
 #pragma unroll
       for (int d = 0; d < DEPTH; ++d) {
-        const int c = base + d * KSPLIT;
+        const int c = base + d * kShares;
         wa[d] = c < chunks ? load_stream(w_ptr + (size_t)c * kPackedChunkElems) : zero_chunk();  // zeros for steps beyond the last
         wb[d] = c < chunks ? load_stream(w_ptr + (size_t)c * kPackedChunkElems + kPackedHalfElems) : zero_chunk();
       }
     } else {
 #pragma unroll
       for (int d = 0; d < DEPTH; ++d) {
-        const int c = base + d * KSPLIT;
+        const int c = base + d * kShares;
         wa[d] = c < chunks ? load_chunk(w_ptr + (size_t)c * kPackedChunkElems) : zero_chunk();
         wb[d] = c < chunks ? load_chunk(w_ptr + (size_t)c * kPackedChunkElems + kPackedHalfElems) : zero_chunk();
       }
@@ -338,7 +356,7 @@ __global__ __launch_bounds__(KSPLIT > 4 ? 64 * KSPLIT : 256) void gemm_skinny_ke
     bf16x8 xa[DEPTH][MT], xb[DEPTH][MT];
 #pragma unroll
     for (int d = 0; d < DEPTH; ++d) {
-      const int ka = (base + d * KSPLIT) * 64 + g * 16, kb = ka + 8;
+      const int ka = (base + d * kShares) * 64 + g * 16, kb = ka + 8;
 #pragma unroll
       for (int t = 0; t < MT; ++t) {
         xa[d][t] = ka + 8 <= k ? load_x(t, ka) : zero_chunk();
@@ -353,7 +371,7 @@ __global__ __launch_bounds__(KSPLIT > 4 ? 64 * KSPLIT : 256) void gemm_skinny_ke
         acc[t] = mfma(wb[d], xb[d][t], acc[t]);
       }
   };
-  int base = part;
+  int base = share;
   if constexpr (RUNS) {
     // the first round's weights are asked for before the block makes its activations: the two latencies overlap
     bf16x8 wa[DEPTH], wb[DEPTH];
@@ -364,11 +382,11 @@ __global__ __launch_bounds__(KSPLIT > 4 ? 64 * KSPLIT : 256) void gemm_skinny_ke
     __syncthreads();
     if (active && base < chunks) {
       multiply(base, wa, wb);
-      base += KSPLIT * DEPTH;
+      base += kShares * DEPTH;
     }
   }
   if (active) {
-    for (; base < chunks; base += KSPLIT * DEPTH) {
+    for (; base < chunks; base += kShares * DEPTH) {
       bf16x8 wa[DEPTH], wb[DEPTH];
       ask_weights(base, wa, wb);
       multiply(base, wa, wb);
@@ -392,6 +410,29 @@ __global__ __launch_bounds__(KSPLIT > 4 ? 64 * KSPLIT : 256) void gemm_skinny_ke
         for (int e = 0; e < 4; ++e) acc[t][e] += partial[wave + other][t][lane][e];
   }
   if (!active) return;
+  if constexpr (PAIR) {
+    // (one wave of the block is left.)  The sums go out past the caches, are waited for, and then the count:
+    // who finds it at one has the other block's sums in memory.
+    float* mine = pair.sums + ((size_t)strip * 2 + blockIdx.x % 2) * (MT * kWave * 4);
+    const float* theirs = pair.sums + ((size_t)strip * 2 + 1 - blockIdx.x % 2) * (MT * kWave * 4);
+#pragma unroll
+    for (int t = 0; t < MT; ++t)
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        __hip_atomic_store(mine + (t * kWave + lane) * 4 + e, acc[t][e], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    int before = 0;
+    if (lane == 0) before = __hip_atomic_fetch_add(pair.count + strip, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    before = __builtin_amdgcn_readfirstlane(before);
+    asm volatile("" ::: "memory");
+    if (before == 0) return;  // the first of the two: the other ends the strip
+#pragma unroll
+    for (int t = 0; t < MT; ++t)
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        acc[t][e] += __hip_atomic_load(theirs + (t * kWave + lane) * 4 + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (lane == 0) __hip_atomic_store(pair.count + strip, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
 
 #pragma unroll
   for (int t = 0; t < MT; ++t) {
@@ -950,12 +991,30 @@ void launch_skinny(const bf16_t* x, const bf16_t* w, OutT y, int m, int n, int k
   if constexpr (std::is_same<OutT, ResidualOut>::value) {
     if (runs) {
       hipLaunchKernelGGL((gemm_skinny_kernel<MT, KSPLIT, true, OutT>), grid, block, skinny_runs_lds(MT, k), stream, x, w, y, m, n, k,
-                         tiles, stream_weights, *runs);
+                         tiles, stream_weights, *runs, PairScratch{});
       return;
     }
   }
   hipLaunchKernelGGL((gemm_skinny_kernel<MT, KSPLIT, false, OutT>), grid, block, 0, stream, x, w, y, m, n, k, tiles, stream_weights,
-                     RunsIn{});
+                     RunsIn{}, PairScratch{});
+}
+
+// Two blocks a strip (see PairScratch), for up to 16 tokens into the stream: where the strips leave half the chip
+// without a block and each block's share of the weights is long -- a compute unit reads about 30 GB/s whatever its
+// waves, so 128 blocks read 2048 x 8192 no faster than 3.7 TB/s.
+constexpr int kPairStripsMost = 128, kPairChunksLeast = 80;
+bool takes_paired_blocks(int m, int n, int k, const float* workspace, size_t workspace_bytes, const int* pair_count) {
+  const int strips = (n + 15) / 16;
+  return pair_count && workspace && m <= 16 && strips <= kPairStripsMost && nnis_packed_chunks(k) >= kPairChunksLeast &&
+         (size_t)strips * 2 * kWave * 4 * sizeof(float) <= workspace_bytes;
+}
+
+void launch_skinny_paired(const bf16_t* x, const bf16_t* w, ResidualOut y, int m, int n, int k, float* workspace, int* pair_count,
+                          hipStream_t stream) {
+  const int strips = (n + 15) / 16;
+  const int stream_weights = (size_t)n * k * sizeof(bf16_t) > kStreamWeightBytes;
+  hipLaunchKernelGGL((gemm_skinny_kernel<1, 8, false, ResidualOut, true>), dim3(2 * strips), dim3(64 * 8), 0, stream, x, w, y, m, n, k, 1,
+                     stream_weights, RunsIn{}, PairScratch{workspace, pair_count});
 }
 
 template <int MT, typename OutT>
@@ -1270,7 +1329,7 @@ extern "C" int nnis_gemm_residual_parts(int m, int n) {
 
 extern "C" int nnis_gemm_residual(const void* x, const void* w, float* resid, const void* gain, int gain_dtype, void* scaled,
                                   float* ss, int ss_rows, int m, int n, int k, int* parts, int tile_hint, float* workspace,
-                                  size_t workspace_bytes, void* stream_ptr) {
+                                  size_t workspace_bytes, int* pair_count, void* stream_ptr) {
   NNIS_REQUIRE(m >= 0 && n > 0 && k > 0, "gemm_residual: bad sizes m=%d n=%d k=%d", m, n, k);
   NNIS_REQUIRE(k % 8 == 0, "gemm_residual: K=%d is not a multiple of 8 (16-byte loads)", k);
   NNIS_REQUIRE(nnis_dtype_ok(gain_dtype), "gemm_residual: unknown norm weight dtype %d", gain_dtype);
@@ -1288,7 +1347,10 @@ extern "C" int nnis_gemm_residual(const void* x, const void* w, float* resid, co
   NNIS_REQUIRE(writes <= ss_rows, "gemm_residual: ss has %d rows of %d tokens, %d are needed", ss_rows, m, writes);
   if (few) {
     *parts = (n + 15) / 16;
-    dispatch_skinny<ResidualOut>((const bf16_t*)x, (const bf16_t*)w, out, m, n, k, skinny_split(m, n, k, 0), stream);
+    if (takes_paired_blocks(m, n, k, workspace, workspace_bytes, pair_count))
+      launch_skinny_paired((const bf16_t*)x, (const bf16_t*)w, out, m, n, k, workspace, pair_count, stream);
+    else
+      dispatch_skinny<ResidualOut>((const bf16_t*)x, (const bf16_t*)w, out, m, n, k, skinny_split(m, n, k, 0), stream);
     NNIS_LAUNCH_CHECK("gemm_residual");
   } else {
     NNIS_REQUIRE((m + 63) / 64 <= 65535, "gemm_residual: %d rows exceed the grid limit", m);

@@ -39,7 +39,7 @@ _CORE_SIGNATURES = {
                         _VOID, _VOID, _VOID, _VOID, _VOID, _INT, _INT, _INT, _INT, _VOID, _VOID, _VOID, _INT, _VOID],
     "nnis_gemm_residual_parts": [_INT, _INT],
     "nnis_gemm_tile": [_INT, _INT, _INT],
-    "nnis_gemm_residual": [_VOID, _VOID, _VOID, _VOID, _INT, _VOID, _VOID, _INT, _INT, _INT, _INT, _VOID, _INT, _VOID, _SIZE, _VOID],
+    "nnis_gemm_residual": [_VOID, _VOID, _VOID, _VOID, _INT, _VOID, _VOID, _INT, _INT, _INT, _INT, _VOID, _INT, _VOID, _SIZE, _VOID, _VOID],
     "nnis_gemm_scaled": [_VOID, _VOID, _INT, _FLT, _VOID, _INT, _INT, _INT, _INT, _VOID, _VOID, _VOID, _INT, _VOID, _VOID,
                          _VOID, _VOID, _VOID, _INT, _INT, _INT, _INT, _VOID, _VOID, _VOID, _INT, _VOID, _SIZE, _VOID],
     "nnis_gemm_residual_runs_fits": [_INT, _INT, _INT, _INT, _INT],
@@ -415,13 +415,15 @@ def _packed(w, what: str) -> None:
 # stream.  It is made outside a graph capture only: a capture that finds none goes without the cut.
 GEMM_WORKSPACE_BYTES = 4 << 20
 _gemm_workspaces = {}
+PAIR_COUNTS = 1024  # 32-bit words kept behind the workspace for the strips' counts
 
 
 def _gemm_workspace(device) -> Optional[torch.Tensor]:
     key = (device.type, device.index)
     held = _gemm_workspaces.get(key)
     if held is None and not torch.cuda.is_current_stream_capturing():
-        held = _gemm_workspaces[key] = torch.empty(GEMM_WORKSPACE_BYTES // 4, dtype=torch.float32, device=device)
+        # behind the workspace proper: the counts of the strips that two blocks share (`gemm_residual`), zero between calls
+        held = _gemm_workspaces[key] = torch.zeros(GEMM_WORKSPACE_BYTES // 4 + PAIR_COUNTS, dtype=torch.float32, device=device)
     return held
 
 
@@ -571,7 +573,8 @@ def gemm_residual(x: torch.Tensor, w: torch.Tensor, resid: torch.Tensor, gain: t
     work = _gemm_workspace(x.device)
     _check(lib, lib.nnis_gemm_residual(x.data_ptr(), w.data_ptr(), resid.data_ptr(), gain.data_ptr(), _code(gain),
                                        scaled.data_ptr(), ss.data_ptr(), ss.numel() // m, m, n, k, ctypes.addressof(parts),
-                                       int(tile), _ptr(work), GEMM_WORKSPACE_BYTES if work is not None else 0, _stream()))
+                                       int(tile), _ptr(work), GEMM_WORKSPACE_BYTES if work is not None else 0,
+                                       work.data_ptr() + GEMM_WORKSPACE_BYTES if work is not None else None, _stream()))
     return parts.value
 
 

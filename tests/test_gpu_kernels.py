@@ -497,6 +497,40 @@ def test_residual_projection_prepares_the_norm(m, n, k, gain_dtype):
     assert ((total - got.pow(2).sum(dim=1)).abs() <= 1e-5 * got.pow(2).sum(dim=1)).all()
 
 
+@pytest.mark.parametrize("m", [1, 5, 16])
+@pytest.mark.parametrize("n, k", [(2048, 5632), (1990, 5128), (48, 8192), (2048, 5120)])
+def test_residual_projection_with_two_blocks_a_strip(m, n, k):
+    """Up to 16 tokens on few strips and a long K (from 5,120 on): two blocks share each strip, and the second
+    to be done adds the sums of the first to its own.  Three calls in a row on the same stream, with a tiled
+    product that cuts its K into parts (and fills the workspace they share) between them: each is right, and
+    the strips' counts are back at zero."""
+    ops = _ops()
+    torch.manual_seed(m + n + k)
+    gain = (1 + 0.3 * torch.randn(n)).bfloat16()
+    other_x = torch.randn(64, 4096).bfloat16().cuda()
+    other_w = ops.pack_weight((torch.randn(2048, 4096) / 64).bfloat16().cuda())
+    other_y = torch.empty(64, 2048, dtype=torch.bfloat16, device="cuda")
+    rows = ops.gemm_residual_parts(m, n)
+    for call in range(3):
+        x = torch.randn(m, k).bfloat16()
+        w = (torch.randn(n, k) / math.sqrt(k)).bfloat16()
+        resid = torch.randn(m, n) * 2
+        want = resid.double() + x.double() @ w.double().t()
+        resid_gpu = resid.cuda()
+        scaled = torch.full((m, n), 9.0, dtype=torch.bfloat16, device="cuda")
+        ss = torch.full((rows + 1, m), 7.0, device="cuda")
+        parts = ops.gemm_residual(x.cuda(), ops.pack_weight(w.cuda()), resid_gpu, gain.cuda(), scaled, ss)
+        ops.gemm_bf16(other_x, other_w, other_y)  # 64 tokens on 2048 x 4096: K in parts, through the workspace
+        assert 0 < parts <= rows and (ss[parts:] == 7.0).all()
+        got = resid_gpu.cpu().double()
+        assert ((got - want).abs() <= 1e-5 * (1 + want.abs())).all(), (call, (got - want).abs().max().item())
+        assert torch.equal(scaled.cpu(), (resid_gpu.cpu() * gain.float()).bfloat16())
+        total = ss[:parts].cpu().double().sum(dim=0)
+        assert ((total - got.pow(2).sum(dim=1)).abs() <= 1e-5 * got.pow(2).sum(dim=1)).all()
+        counts = ops._gemm_workspace(resid_gpu.device)[ops.GEMM_WORKSPACE_BYTES // 4:].view(torch.int32)
+        assert int(counts.abs().sum()) == 0
+
+
 @pytest.mark.parametrize("tile", ["TILE_64x128", "TILE_64x64", "TILE_256x256", "TILE_256x192", "TILE_128x128", "TILE_256x128", "TILE_128x192"])
 @pytest.mark.parametrize("m, n, k", [(70, 600, 136), (530, 300, 72), (300, 1100, 584)])
 def test_residual_projection_with_every_tile(tile, m, n, k):
