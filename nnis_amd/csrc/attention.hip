@@ -332,7 +332,7 @@ struct MfmaArgs {
   // decode: one token per sequence
   const int* tok_slot;    // [tokens]
   const int* tok_pos;     // [tokens]
-  int splits;
+  int splits, heads_first;
   float* partial;         // [tokens, heads, splits, kPartial] when splits > 1: HD outputs, maximum, sum
 };
 
@@ -665,7 +665,7 @@ template <int C>
 __global__ __launch_bounds__(64 * kBlockWaves) void attention_decode_kernel(MfmaArgs a, int waves) {
   extern __shared__ __attribute__((aligned(16))) float merge[];  // [waves / 2][C][kTilesD * 4 + 2][64]
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave, r = lane % 16, g = lane / 16;
-  const int token = blockIdx.x, kv_head = blockIdx.y, split = blockIdx.z;
+  const int token = a.heads_first ? blockIdx.y : blockIdx.x, kv_head = a.heads_first ? blockIdx.x : blockIdx.y, split = blockIdx.z;
   // With the step's tables a token's pages are a row of its own and nothing is asked of its slot: the first
   // pages' numbers are one round trip away, not two.  (A padding row then reads the page its row names, 0,
   // and leaves a result that nobody reads.)
@@ -740,7 +740,7 @@ __global__ __launch_bounds__(64 * kKeysWaves) void attention_decode_keys_kernel(
   __shared__ __attribute__((aligned(16))) bf16_t stage[kKeysWaves][4][kStageRow];
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave, r = lane % 16, g = lane / 16;
   const int blk = lane / 4, j = lane % 4;  // the scores' layout: keys 4 blk .. 4 blk + 3 of a page, head j of the group
-  const int token = blockIdx.x, kv_head = blockIdx.y, split = blockIdx.z;
+  const int token = a.heads_first ? blockIdx.y : blockIdx.x, kv_head = a.heads_first ? blockIdx.x : blockIdx.y, split = blockIdx.z;
   int slot = 0;
   if (!a.rows_by_token) {  // (see attention_decode_kernel)
     slot = a.tok_slot[token];
@@ -994,7 +994,7 @@ int fill_common(MfmaArgs& a, const void* q, void* out, const void* k_pages, cons
   a.block_table = block_table; a.max_pages = max_pages; a.heads = heads; a.kv_heads = kv_heads; a.window = window;
   a.scale_log2 = scale * kLog2e;
   a.tile_seq = a.tile_row0 = a.seq_slot = a.seq_start = a.seq_pos0 = a.tok_slot = a.tok_pos = nullptr;
-  a.splits = 1; a.partial = nullptr; a.rows_by_token = 0;
+  a.splits = 1; a.heads_first = 0; a.partial = nullptr; a.rows_by_token = 0;
   return 0;
 }
 }  // namespace
@@ -1148,7 +1148,15 @@ extern "C" int nnis_attention_decode_bf16(const void* q, void* out, const void* 
   NNIS_REQUIRE(kind != 2 || keys_fit, "attention: the kernel with keys on lanes takes groups of up to 4 heads of up to %d channels",
                kKeysMaxHD);
   a.tok_slot = tok_slot; a.tok_pos = tok_pos; a.splits = splits; a.partial = partial;
-  const dim3 grid(tokens, kv_heads, splits);
+  // Blocks go to the chip's 8 dies in turn.  With the tokens as the grid's fastest index a die runs all heads of its
+  // tokens: its L2 holds a token's query, pages' numbers and tables once (8 tokens on 9/3 heads: 9,470 tokens/s
+  // against 9,200 with a token's blocks spread), but a long sequence's keys all come through one die.  Where the
+  // key/value heads deal evenly to the dies (a multiple of 8) they are the fastest index: every die then reads an
+  // eighth of every sequence (32/32 heads of 64, unequal lengths up to 2k keys: 64 tokens 15,330 -> 16,860 tokens/s in
+  // whole steps, 8 tokens 5,430 -> 5,515; 32/8 heads of 128: 60,700 -> 62,150 and 11,950 -> 12,020).
+  // (4 and 3 key/value heads as the fastest index at 16 to 64 tokens: 0.3% slower in whole steps.)
+  a.heads_first = kv_heads % 8 == 0 && tokens <= 65535;
+  const dim3 grid(a.heads_first ? kv_heads : tokens, a.heads_first ? tokens : kv_heads, splits);
   hipStream_t s = (hipStream_t)stream;
   const int tiles = (group + 15) / 16;
   const size_t lds = (size_t)(waves / 2) * tiles * (kTilesD * 4 + 2) * kWave * sizeof(float);
