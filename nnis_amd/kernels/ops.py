@@ -799,9 +799,10 @@ def decode_plan(batch: int, kv_heads: int, longest: int, max_waves: int = 4, wid
         room = max(1, 1024 // max(1, batch * kv_heads * waves))
         while splits * 2 <= room and splits < wanted:
             splits *= 2
-    if splits == 1 and batch * kv_heads >= 1024:
-        # four and more blocks a compute unit: two waves a block read faster than four (batch 64 on 32 key-value
-        # heads of 64, microseconds a layer: 1,100 keys each 104 against 116, 128 to 2k 114 against 121, 2k 180 against 187)
+    if splits == 1 and batch * kv_heads >= 2048:
+        # eight and more blocks a compute unit: two waves a block read as fast as four or faster (batch 64 on 32
+        # key-value heads of 64, whole steps: 1,000 to 1,100 keys each 16,230 tokens/s against 15,900, 128 to 2k
+        # 15,620 either way); at four blocks a unit four waves are faster (batch 32: 12,010 against 11,600)
         waves = min(waves, 2)
     return splits, waves
 
