@@ -21,7 +21,11 @@ four measurements at the SmolLM2-1.7B and TinyLlama-1.1B layer sizes (all
 layers), each with the fraction of its roofline, and the TinyLlama workload
 of 64 unequal prompts (16 to 1,024 tokens, prefilled in one step, decoded
 until every sequence holds 2,048 tokens) run through ``nnis_amd.generate``.
-A decode point is the better of two windows of K steps over the same prompts.
+For the SmolLM2 shapes there are further points at long contexts: decode at
+batch 8 and 64 over prompts of 7,800 to 8,000 tokens (``*_ctx8k``) and a prompt
+of 8,192 tokens in one step (``*_prefill_8192``).  A decode point is the
+median of three windows of K steps, one after the other on the same batch; a
+prefill figure is the median of three runs of a shape seen before.
 ``--workload tinyllama-ragged`` runs that workload alone.
 
 Peaks used for the fractions are the published MI355X ones: HBM 8 TB/s; dense
@@ -84,21 +88,34 @@ class Shape:
         return Engine(self.model, self.rt, max_tokens=max_tokens, max_slots=max_slots)
 
 
-def decode_run(shape, rng, batch, steps, warmup, prompt_min, prompt_max):
-    """Prefills ``batch`` prompts in one step, then times ``steps`` decode steps.  Returns a dict."""
+PROMPT_STEP_MOST_TOKENS = 16384  # a batch's prompts go in one step up to this many tokens, in several beyond
+
+
+def decode_run(shape, rng, batch, steps, warmup, prompt_min, prompt_max, windows=1):
+    """Prefills ``batch`` prompts (in one step where they are 16k tokens or fewer between them), then times
+    ``windows`` windows of ``steps`` decode steps each, one after the other, and reports the median window.
+    Returns a dict."""
     import torch
 
     from nnis_amd.engine.batch import StepEntry
     from nnis_amd.sampling.device import DeviceSelector
 
-    longest = min(prompt_max, shape.context - 2 * steps - warmup - 1)
+    longest = min(prompt_max, shape.context - (windows + 1) * steps - warmup - 1)
     shortest = max(1, min(prompt_min, longest))
     lengths = rng.integers(shortest, longest + 1, size=batch).tolist()
     engine = shape.engine(batch * shape.context, max_slots=batch)  # every sequence may grow to the model's context
     selector = DeviceSelector(engine)
     slots = [engine.start_sequence() for _ in range(batch)]
     prompts = [rng.integers(0, shape.vocab, size=n).tolist() for n in lengths]
-    logits = engine.step([StepEntry(s, p, None) for s, p in zip(slots, prompts)])
+    rows, group, held = [], [], 0
+    for slot, prompt in zip(slots, prompts):
+        if group and held + len(prompt) > PROMPT_STEP_MOST_TOKENS:
+            rows.append(engine.step([StepEntry(s, p, None) for s, p in group]))
+            group, held = [], 0
+        group.append((slot, prompt))
+        held += len(prompt)
+    rows.append(engine.step([StepEntry(s, p, None) for s, p in group]))
+    logits = rows[0] if len(rows) == 1 else torch.cat(rows)
     greedy = [None] * batch
     sync = torch.cuda.synchronize
     if engine.use_graphs:
@@ -129,16 +146,20 @@ def decode_run(shape, rng, batch, steps, warmup, prompt_min, prompt_max):
     # the graphs of the lengths that the timed steps (and the pass with events) reach are captured before the clock
     # starts: as the sequences grow a step may cross into another plan of the attention, whose first use costs 8 ms
     reached = max(engine.length(s) for s in slots)
-    for ahead in range(1, min(2 * steps + 1, shape.context - reached) + 1):
+    for ahead in range(1, min((windows + 1) * steps + 1, shape.context - reached) + 1):
         engine.prepare_decode(batch, reached + ahead)
-    sync()
-    start = time.perf_counter()
-    for _ in range(steps):
-        pending = one_step(pending)
-    finish(pending)
-    sync()
-    seconds = time.perf_counter() - start
-    context_tokens = sum(engine.length(s) for s in slots) - batch * steps / 2.0  # mean over the timed steps
+    timed = []
+    for _ in range(windows):
+        sync()
+        start = time.perf_counter()
+        for _ in range(steps):
+            pending = one_step(pending)
+        finish(pending)
+        sync()
+        seconds = time.perf_counter() - start
+        # (seconds, tokens held on average over the window's steps)
+        timed.append((seconds, sum(engine.length(s) for s in slots) - batch * steps / 2.0))
+    seconds, context_tokens = sorted(timed)[len(timed) // 2]
     # the steps' own times, in a pass of its own (an event on the stream after every step costs the step a little)
     spread = min(steps, shape.context - max(engine.length(s) for s in slots) - 1)
     marks = [torch.cuda.Event(enable_timing=True) for _ in range(spread + 1)]
@@ -175,7 +196,7 @@ def prefill_run(shape, rng, tokens=2048):
     engine.step([StepEntry(slot, warm, None)])  # another shape: kernels loaded, buffers made
     engine.end_sequence(slot)
     times = []
-    for _ in range(5):
+    for _ in range(6):
         slot = engine.start_sequence()
         torch.cuda.synchronize()
         start = time.perf_counter()
@@ -185,7 +206,7 @@ def prefill_run(shape, rng, tokens=2048):
         engine.end_sequence(slot)
     del engine
     torch.cuda.empty_cache()
-    seconds = min(times[2:])
+    seconds = sorted(times[3:])[1]  # the median of three runs of a shape that has come before (and is captured, where it is)
     flops = step_flops(shape.config, [tokens], 1)
     return {"value": round(tokens / seconds, 1), "tokens": tokens, "ms": round(1000.0 * seconds, 3),
             "frac": round(flops / seconds / FLOP_PEAK[shape.dtype], 5), "first_ms": round(1000.0 * times[0], 3)}
@@ -238,6 +259,8 @@ def environment():
                                        timeout=10).stdout.strip() or None
     except (OSError, subprocess.SubprocessError):
         env["commit"] = None
+    if not env["commit"]:
+        env["commit"] = os.environ.get("NNIS_COMMIT") or None  # a copy of the tree without its history: whoever made it may say
     return env
 
 
@@ -283,20 +306,28 @@ def main() -> int:
         prefill = prefill_run(shape, rng)
         points = {}
 
-        def point_run(shape, batch):
-            """A point beside the headline: the better of two windows over the same prompts (the box is shared, and
-            a window of a few dozen milliseconds shows every stall of the host)."""
-            state = rng.bit_generator.state
-            first = decode_run(shape, rng, batch, args.steps, args.warmup, args.prompt_min, args.prompt_max)
-            rng.bit_generator.state = state
-            second = decode_run(shape, rng, batch, args.steps, args.warmup, args.prompt_min, args.prompt_max)
-            return first if first["tokens_per_second"] >= second["tokens_per_second"] else second
+        def point_run(shape, batch, prompt_min=args.prompt_min, prompt_max=args.prompt_max):
+            """A point beside the headline: the median of three windows on one batch."""
+            return decode_run(shape, rng, batch, args.steps, args.warmup, prompt_min, prompt_max, windows=3)
+
+        def long_points(shape, prefix):
+            """Contexts near the model's end: decode over prompts of 7,800 to 8,000 tokens, and a prompt of 8,192."""
+            if shape.context < 8192:
+                return
+            for batch in (8, 64):
+                run = point_run(shape, batch, 7800, 8000)
+                points[f"{prefix}decode_b{batch}_ctx8k"] = round(run["tokens_per_second"], 1)
+                points[f"{prefix}decode_b{batch}_ctx8k_hbm_frac"] = round(run["gbs"] / HBM_PEAK_GBS, 4)
+            long_prefill = prefill_run(shape, rng, tokens=8192)
+            points[f"{prefix}prefill_8192"] = long_prefill["value"]
+            points[f"{prefix}prefill_8192_frac"] = long_prefill["frac"]
 
         if not args.no_points:
             for batch in (1, 64):
                 run = point_run(shape, batch)
                 points[f"decode_b{batch}"] = round(run["tokens_per_second"], 1)
                 points[f"decode_b{batch}_hbm_frac"] = round(run["gbs"] / HBM_PEAK_GBS, 4)
+            long_points(shape, "")
         config, layers, layers_of_model = shape.config, shape.config["num_hidden_layers"], shape.layers_of_model
         del shape
     if not args.no_points and not args.no_other_shapes:
@@ -315,6 +346,7 @@ def main() -> int:
                 other_prefill = prefill_run(shape, rng)
                 points[f"{other}_prefill_{other_prefill['tokens']}"] = other_prefill["value"]
                 points[f"{other}_prefill_{other_prefill['tokens']}_frac"] = other_prefill["frac"]
+                long_points(shape, f"{other}_")
                 if other == "tinyllama-1.1b":
                     ragged = ragged_run(shape, rng)
                     points["tinyllama-1.1b_ragged64_prefill"] = ragged["prefill_tokens_per_second"]

@@ -23,8 +23,10 @@ def load_model(model_dir: str, dtype="bfloat16", device="cuda:0", narrow_to_bflo
     _, spec = spec_from_config(raw)
     rt = Runtime(device=device, dtype=dtype)
     model = DecoderModel(spec)
+    model.check(rt)  # a size that the kernels do not take is refused here, before a byte of the weights is read
     weights = load_weights(model_dir, model.tensors(), rt.device, widen_to_float32=rt.is_fp32,
-                           declared_dtype=spec.stored_dtype, narrow_to_bfloat16=narrow_to_bfloat16)
+                           declared_dtype=spec.stored_dtype, narrow_to_bfloat16=narrow_to_bfloat16,
+                           ignored_suffixes=spec.ignored_tensor_suffixes)
     model.bind(weights, rt)
     return model, rt
 

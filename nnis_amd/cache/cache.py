@@ -64,6 +64,12 @@ class KVGroup:
         self.block_table = torch.zeros((slots, per_slot), dtype=torch.int32, device=device)
         self._table_rows = self.block_table_host.numpy()  # the same memory: an entry is written without a tensor operation
         self._dirty = set()
+        # The rows go to the device by copies that do not wait (``flush``); such a copy reads the pinned row when
+        # the stream gets to it, which may be long after.  Whoever writes into a row again (a slot that grows,
+        # or that another sequence has taken over) first waits for the last flush to have left the pinned
+        # memory: otherwise an earlier step's copy would carry the new owner's pages.
+        self._flushed = torch.cuda.Event() if pinned else None
+        self._flush_pending = False
 
     def bytes_per_token(self) -> int:
         return (len(self.entries) * self.request.kv_heads * (self.request.head_dim + self.request.value_head_dim)
@@ -72,15 +78,27 @@ class KVGroup:
     def grow(self, slot: int, new_length: int) -> None:
         changed = self.table.grow(slot, new_length)
         if changed:
+            self._settle()
             row = self.table.rows[slot]
             self._table_rows[slot, changed[0]:changed[-1] + 1] = row[changed[0]:changed[-1] + 1]  # (the new pages follow one another)
             self._dirty.add(slot)
 
+    def _settle(self) -> None:
+        """Waits until the last flush's copies have read the pinned rows."""
+        if self._flush_pending:
+            self._flushed.synchronize()
+            self._flush_pending = False
+
     def flush(self) -> None:
         """Copies the block-table rows that changed to the device."""
+        if not self._dirty:
+            return
         for slot in sorted(self._dirty):
             self.block_table[slot].copy_(self.block_table_host[slot], non_blocking=True)
         self._dirty.clear()
+        if self._flushed is not None:
+            self._flushed.record()
+            self._flush_pending = True
 
 
 class SequenceCache:
@@ -185,28 +203,45 @@ class SequenceCache:
         self.lengths[slot] = int(length)
 
     def reset(self, slot: int) -> None:
-        """The slot as it was when acquired: no tokens, no pages, state zero
-        (kv_cache.rs:170-172).  The slot stays held."""
+        """The sequence as it was before its first token: no tokens, no pages,
+        and the state that the model's layers keep for it zero
+        (kv_cache.rs:170-172 sets the lengths to 0).  The slot stays held,
+        and so does what others keep in the slot's state regions for the
+        sequence (a sampler's generator state and options): the sequence goes
+        on drawing where it was."""
         self.length(slot)  # raises if the slot is not held
         for group in self.kv_groups:
             group.table.shrink(slot, 0)
         self.lengths[slot] = 0
-        for region in self.state_regions.values():
-            region[slot].zero_()
+        for name in self._layer_state:
+            self.state_regions[name][slot].zero_()
+
+    def roll_back(self, lengths: Dict[int, int]) -> None:
+        """Undoes a ``grow`` whose step was not launched: each slot back to
+        the length it had (never longer than it is), its pages beyond that
+        back to the pools.  Unlike ``truncate`` it is not refused for fixed-size
+        state, which a failed step may have touched and nothing can wind back."""
+        for slot, length in lengths.items():
+            if slot in self.lengths and 0 <= int(length) < self.lengths[slot]:
+                for group in self.kv_groups:
+                    group.table.shrink(slot, int(length))
+                self.lengths[slot] = int(length)
 
     def check_room(self, growth: Dict[int, int]) -> None:
         """Raises before anything changes if the slots cannot grow by the given
         token counts (all or nothing, as the reference's append:
         /root/reference/crates/nnis-rt/src/kv_cache.rs:223-228)."""
+        # (the end of the positions holds for every model, also for one that keeps no keys at all)
+        for slot, extra in growth.items():
+            new_length = self.length(slot) + extra
+            if new_length > self.max_positions:
+                raise CacheFull(
+                    f"slot {slot} would hold {new_length} tokens; the model's positions end at {self.max_positions}"
+                )
         for group in self.kv_groups:
             need = 0
             for slot, extra in growth.items():
-                new_length = self.length(slot) + extra
-                if new_length > self.max_positions:
-                    raise CacheFull(
-                        f"slot {slot} would hold {new_length} tokens; the model's positions end at {self.max_positions}"
-                    )
-                need += group.table.pages_needed(slot, new_length)
+                need += group.table.pages_needed(slot, self.lengths[slot] + extra)
             if need > group.table.pool.free:
                 raise CacheFull(
                     f"the cache has {group.table.pool.free} free pages of {PAGE_TOKENS} tokens; this step needs {need}"
@@ -223,10 +258,8 @@ class SequenceCache:
         for group in self.kv_groups:
             group.flush()
 
-    def grow_by_one(self, slots: Sequence[int]) -> List[int]:
-        """One more token for each of the slots (a decode step): returns their
-        lengths before.  Only a sequence that starts a new page takes the long
-        way; all or nothing as ``grow``."""
+    def _one_more(self, slots: Sequence[int]):
+        """(lengths before, slots that start a new page) of one more token for each slot; raises as ``check_room``."""
         lengths = self.lengths
         try:
             before = [lengths[slot] for slot in slots]
@@ -237,6 +270,21 @@ class SequenceCache:
             self.check_room({slot: 1 for slot in slots})  # raises, naming the slot
         if crossing:
             self.check_room(crossing)
+        return before, crossing
+
+    def check_one_more(self, slots: Sequence[int]):
+        """Raises if ``grow_by_one`` would; changes nothing.  Returns what it
+        found (the lengths now, first), which ``grow_by_one`` takes as
+        ``checked`` if nothing of the cache has changed in between."""
+        return self._one_more(slots)
+
+    def grow_by_one(self, slots: Sequence[int], checked=None) -> List[int]:
+        """One more token for each of the slots (a decode step): returns their
+        lengths before.  Only a sequence that starts a new page takes the long
+        way; all or nothing as ``grow``."""
+        lengths = self.lengths
+        before, crossing = checked if checked is not None else self._one_more(slots)
+        if crossing:
             for slot in crossing:
                 for group in self.kv_groups:
                     group.grow(slot, lengths[slot] + 1)

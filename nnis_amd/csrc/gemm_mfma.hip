@@ -412,7 +412,16 @@ __global__ __launch_bounds__(KSPLIT > 4 ? 64 * KSPLIT : 256) void gemm_skinny_ke
   if (!active) return;
   if constexpr (PAIR) {
     // (one wave of the block is left.)  The sums go out past the caches, are waited for, and then the count:
-    // who finds it at one has the other block's sums in memory.
+    // who finds it at one has the other block's sums in memory.  All of it with relaxed order at agent scope,
+    // which rests on three facts of this chip and not on the language's memory model: (1) a wave's stores are
+    // counted by vmcnt, and `s_waitcnt vmcnt(0)` below ends only when they have been written where agent-scope
+    // accesses see them; (2) atomic loads and stores at agent scope go past the dies' own L2 (each die has
+    // one), so the second block reads what the first wrote and not a line its die had kept; (3) a wave issues
+    // no load before the branch it stands behind is decided, so the sums are not read before the count.  The
+    // same with a release on the count and an acquire fence for the second block (the compiler then writes
+    // back and invalidates the L2 around them) was measured: 2048 x 5632 at 1 / 8 / 16 tokens 7.8 / 8.3 / 9.7
+    // -> 10.1 / 10.4 / 12.0 us, 2048 x 8192 9.7 / 10.2 / 11.7 -> 12.4 / 13.3 / 15.2: more than the second
+    // block gains.  The asm statements keep the compiler from moving memory accesses across them.
     float* mine = pair.sums + ((size_t)strip * 2 + blockIdx.x % 2) * (MT * kWave * 4);
     const float* theirs = pair.sums + ((size_t)strip * 2 + 1 - blockIdx.x % 2) * (MT * kWave * 4);
 #pragma unroll
@@ -1317,6 +1326,14 @@ extern "C" int nnis_gemm_bf16(const void* x, const void* w, void* y, int y_dtype
 // The tile that the tiled kernel takes for m rows, `columns` weight rows and a depth of k (2: 64 x 128, 3: 64 x 64,
 // 4: 256 x 256, 5: 256 x 192, 6: 128 x 128, 7: 256 x 128, 8: 128 x 192): for tests and tuning.
 extern "C" int nnis_gemm_tile(int m, int columns, int k) { return pick_tile(m, columns, k, 0); }
+
+// 1 if nnis_gemm_residual gives these sizes to two blocks a strip (with a workspace of `workspace_bytes` and counts
+// behind it), 0 if to another kernel: for callers and tests that have to know which kernel ran.
+extern "C" int nnis_gemm_takes_pair(int m, int n, int k, size_t workspace_bytes) {
+  static const int some_counts = 0;
+  static const float some_workspace = 0.0f;
+  return takes_few_tokens_with_parts(m, n, k, true) && takes_paired_blocks(m, n, k, &some_workspace, workspace_bytes, &some_counts) ? 1 : 0;
+}
 
 // The projection that ends a part of a pre-norm block: resid += x . w^T in 32-bit, in place, and the norm
 // that follows prepared -- scaled = bf16(resid * gain) and parts of each row's sum of squares in ss

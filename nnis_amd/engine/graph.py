@@ -20,8 +20,10 @@ from typing import Dict, Sequence
 
 import torch
 
+import numpy as np
+
 from ..errors import KernelError
-from .batch import StepContext
+from .batch import RecordedLists, StepContext
 
 BUCKETS = (1, 2, 4, 8, 12, 16, 24, 32, 48, 64)
 
@@ -52,10 +54,11 @@ class DecodeGraph:
         self.copied.record()
         self.ctx = StepContext(
             tokens=padded, batch=padded, tok_slot=self.meta[1], tok_pos=self.meta[2], seq_slot=self.meta[1],
-            seq_start=self.rows, seq_pos0=self.meta[2], decode=True, max_new=1, max_len=0, plan_len=plan_len)
+            seq_start=self.rows, seq_pos0=self.meta[2], decode=True, max_new=1, max_len=0, host_new=None, host_pos0=None,
+            plan_len=plan_len)
         self.graph = None
         self.logits = None
-        self.scratch = None  # the kernels' shared scratch whose address the capture baked in: held as long as the graph
+        self.held = []  # memory the parts' kernels keep between calls, whose addresses the capture baked in: held as long as the graph
 
     def _forward(self) -> torch.Tensor:
         engine = self.engine
@@ -82,10 +85,11 @@ class DecodeGraph:
         finally:
             if collecting:
                 gc.enable()
-        # The split attention's partial sums go through a scratch tensor that the kernels' wrapper keeps per
-        # device.  The eager run above sized it and the capture baked its address in, so the graph holds it:
-        # whatever the wrapper does later, a replay never writes into memory that has gone back to the allocator.
-        self.scratch = self.engine.rt.ops.decode_scratch_held(self.engine.rt.device)
+        # A part's kernels may go through scratch that is kept between calls (the runs of a decode attention's
+        # keys meet in one).  The eager run above sized it and the capture baked its address in, so the graph
+        # holds what the parts name (``Part.held_buffers``): whatever its keeper does later, a replay never writes
+        # into memory that has gone back to the allocator.
+        self.held = list(self.engine.model.held_buffers(self.engine.rt))
 
     def run(self, ids, slots: Sequence[int], positions: Sequence[int], ids_device: torch.Tensor = None) -> torch.Tensor:
         """``ids``: the step's token ids, or None when they are on the device
@@ -140,13 +144,15 @@ class DecodeGraphs:
 # ---------------------------------------------------------------------------------------------
 # A step over a few thousand tokens launches 150 kernels and more; where the model is small the host
 # needs as long to launch them as the GPU to run them.  A step's *shape* -- how many sequences it has, how
-# many tokens in all (rounded up: ``ops.prefill_rows``), how many logit rows are wanted, and the class of its
-# longest sequence (which picks the attention kernels' plan) -- fixes every launch; tokens, slots,
-# positions, how the tokens divide among the sequences and the attention's work items are data.  The rows
+# many tokens in all (rounded up: ``prompt_rows``), how many logit rows are wanted, and how the model's parts
+# plan their launches for it (``DecoderModel.prompt_plan``) -- fixes every launch; tokens, slots,
+# positions, how the tokens divide among the sequences and the parts' work lists are data.  The rows
 # beyond a step's tokens belong to no sequence (slot -1): every kernel computes them like any row and writes
-# nothing of them into the cache, and the attention's work lists are filled up with items that have no rows.
-# The second time a shape comes it is captured into a graph whose kernels read that data from fixed
-# buffers; from the third time on the step is a copy into the buffers and a replay.  Only shapes of up to PREFILL_GRAPH_MOST_TOKENS tokens are kept, the most recently used
+# nothing of them into the cache, and the parts fill their work lists up with items that do nothing
+# (``StepLists``).  The second time a shape comes it runs once from fixed buffers as any step runs, which
+# shows which lists its parts ask for, and is then captured into a graph whose kernels read all that data
+# from the buffers; from the third time on the step is a copy into the buffers and a replay.  Only shapes of
+# up to PREFILL_GRAPH_MOST_TOKENS tokens are kept, the most recently used
 # PREFILL_GRAPHS_KEPT of them (a graph keeps its activations' memory), and only where the step's kernels are
 # short enough for the host to matter: tokens x width^2 up to PREFILL_GRAPH_MOST_WORK.  Measured, one prompt a
 # step, launched against replayed, milliseconds: width 576, 30 layers: 64 tokens 2.27 / 0.83, 256 2.33 / 1.33,
@@ -157,46 +163,57 @@ PREFILL_GRAPH_MOST_WORK = 1.5e9
 PREFILL_GRAPHS_KEPT = 16
 
 
-# a work item of the attention that has no rows: its first row lies beyond any sequence's tokens
-_NO_ROWS = 1 << 24
+def prompt_rows(total: int) -> int:
+    """Rows of the replayed prompt step that takes ``total`` tokens: the next multiple of 64 up to 1,024
+    tokens, of 128 up to 2,048, of 256 beyond.  (Parts that plan by a step's size are given this, so that a
+    step launched and the same step replayed from a graph's rows take the same kernels.)"""
+    unit = 64 if total <= 1024 else (128 if total <= 2048 else 256)
+    return ((total + unit - 1) // unit) * unit
 
 
 class PrefillGraph:
-    def __init__(self, engine, batch: int, total: int, wanted: int, plan_class: int, tile_rows: Sequence[int]):
-        """``total``: the rows of the step (``ops.prefill_rows`` of its tokens), ``batch``: its sequences."""
+    def __init__(self, engine, batch: int, total: int, wanted: int, plan_len: int):
+        """``total``: the rows of the step (``prompt_rows`` of its tokens), ``batch``: its sequences,
+        ``plan_len``: a longest sequence for which the parts plan as they do for this shape."""
         self.engine = engine if isinstance(engine, weakref.ProxyTypes) else weakref.proxy(engine)
-        ops = engine.rt.ops
-        device = engine.rt.device
-        self.total = total
+        self.batch, self.total, self.plan_len = batch, total, plan_len
         # the step's arrays in one buffer, in the order the step function stages them
         self.sizes = [total, total, total, batch, batch + 1, batch, wanted]
-        self.tile_rows = list(tile_rows)
-        # the most tiles of `rows` rows that `batch` sequences with `total` tokens between them can have
-        self.tile_counts = [total // rows + batch for rows in self.tile_rows]
-        sizes = self.sizes + [2 * n for n in self.tile_counts]
+        self.lists = None  # the parts' work lists: who makes which, as the first run found them
+        self.copied = torch.cuda.Event()
+        self.copied.record()
+        self.graph = None
+        self.logits = None
+        self.held = []
+        self._lay_out({})
+
+    def _lay_out(self, list_shapes) -> None:
+        """One device buffer and one pinned one for the step's arrays and the lists of ``list_shapes``."""
+        device = self.engine.rt.device
+        self.list_keys = list(list_shapes)
+        sizes = self.sizes + [int(np.prod(list_shapes[key])) for key in self.list_keys]
         self.spans, offset = [], 0
         for size in sizes:
             self.spans.append((offset, size))
             offset += size
         self.meta = torch.zeros(offset, dtype=torch.int32, device=device)
         self.host = torch.empty(offset, dtype=torch.int32, pin_memory=True)
-        self.copied = torch.cuda.Event()
-        self.copied.record()
         views = [self.meta[o:o + n] for o, n in self.spans]
-        tiles = {rows: (views[7 + i][:n], views[7 + i][n:]) for i, (rows, n) in enumerate(zip(self.tile_rows, self.tile_counts))}
         self.ids, self.want_rows = views[0], views[6]
+        fixed = {key: view.view(list_shapes[key]) for key, view in zip(self.list_keys, views[7:])}
+        if self.lists is not None:
+            self.lists.fixed = fixed
+        # (no host lists: a work list that the first run did not ask for is an error)
         self.ctx = StepContext(
-            tokens=total, batch=batch, tok_slot=views[1], tok_pos=views[2], seq_slot=views[3], seq_start=views[4],
-            seq_pos0=views[5], decode=False, max_new=total, max_len=ops.PREFILL_CLASS_LENGTH[plan_class],
-            host_new=None, host_pos0=None, tiles=tiles)  # (no host lists: a work list that is not in `tiles` is an error)
-        self.graph = None
-        self.logits = None
+            tokens=self.total, batch=self.batch, tok_slot=views[1], tok_pos=views[2], seq_slot=views[3], seq_start=views[4],
+            seq_pos0=views[5], decode=False, max_new=self.total, max_len=self.plan_len, host_new=None, host_pos0=None,
+            plan_len=self.plan_len, plan_rows=self.total, lists=self.lists)
 
     def fill(self, arrays, counts: Sequence[int], first_positions: Sequence[int]) -> None:
         """The step's data into the buffers: ``arrays`` as the step function stages them (ids, slot and position
         of each token, slot, first row and first position of each sequence, wanted rows); ``counts``: the
-        tokens each sequence brings.  Rows beyond the tokens get id 0, slot -1, position 0."""
-        ops = self.engine.rt.ops
+        tokens each sequence brings.  Rows beyond the tokens get id 0, slot -1, position 0; the parts' lists
+        are made anew by those who made them in the first run."""
         self.copied.synchronize()  # the previous copy has left the pinned buffer
         host = self.host.numpy()
         tokens = sum(counts)
@@ -206,13 +223,11 @@ class PrefillGraph:
                 host[offset + tokens:offset + size] = -1 if index == 1 else 0
             else:
                 host[offset:offset + size] = array
-        for (offset, _), rows, n in zip(self.spans[7:], self.tile_rows, self.tile_counts):
-            seqs, row0s = ops.prefill_tile_items(counts, first_positions, rows)
-            have = len(seqs)
-            host[offset:offset + have] = seqs
-            host[offset + have:offset + n] = 0
-            host[offset + n:offset + n + have] = row0s
-            host[offset + n + have:offset + 2 * n] = _NO_ROWS
+        for (offset, size), key in zip(self.spans[7:], self.list_keys):
+            made = np.asarray(self.lists.makers[key](counts, first_positions, (self.batch, self.total)), dtype=np.int32)
+            if made.shape != self.lists.shapes[key]:
+                raise KernelError(f"work list {key!r} has shape {made.shape} now, {self.lists.shapes[key]} when the step was captured")
+            host[offset:offset + size] = made.reshape(-1)
         self.meta.copy_(self.host, non_blocking=True)
         self.copied.record()
 
@@ -221,14 +236,20 @@ class PrefillGraph:
         self.ctx.tables = {}  # (as for the decode graphs)
         return engine.model.forward(self.ids, self.ctx, engine.cache, self.want_rows, engine.rt)
 
-    def first_run(self):
-        """Runs the step that the buffers hold as any step runs, then captures its launches.  Returns that
-        run's logits (the caller's to keep), or None if the step cannot run from these buffers; ``graph`` is
-        None afterwards if it could not be captured."""
+    def first_run(self, arrays, counts: Sequence[int], first_positions: Sequence[int]):
+        """Runs the step from the buffers as any step runs (its parts make their lists, padded to the shape,
+        and are recorded), lays the buffers out again with room for those lists, and captures the step's
+        launches.  Returns the first run's logits (the caller's to keep), or None if the step cannot run from
+        fixed buffers; ``graph`` is None afterwards if it could not be captured."""
+        self.fill(arrays, counts, first_positions)
+        self.lists = RecordedLists(counts, first_positions, self.engine.rt.device, (self.batch, self.total))
+        self.ctx.lists = self.lists
         try:
             logits = self._forward()
         except KernelError:
-            return None  # (a work list that the shape's record does not name: the caller runs the step as any step)
+            return None  # (a part that needs the host's view of the step: the caller runs the step as any step)
+        self._lay_out(dict(self.lists.shapes))
+        self.fill(arrays, counts, first_positions)
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
         collecting = gc.isenabled()  # (as for the decode graphs: no graph may be destroyed while one is captured)
@@ -237,6 +258,7 @@ class PrefillGraph:
             with torch.cuda.graph(graph):
                 self.logits = self._forward()
             self.graph = graph
+            self.held = list(self.engine.model.held_buffers(self.engine.rt))
         except KernelError:
             # a part that cannot run under capture: the shape goes on being launched
             self.graph = self.logits = None
@@ -260,10 +282,10 @@ class PrefillGraphs:
         self.refused = set()  # shapes whose capture failed
         self.graphs: Dict[tuple, PrefillGraph] = {}  # in the order of their last use
 
-    def step(self, key: tuple, arrays, counts: Sequence[int], first_positions: Sequence[int], tile_rows):
+    def step(self, key: tuple, arrays, counts: Sequence[int], first_positions: Sequence[int], longest: int):
         """(logits, borrowed) if this step is replayed or captured; None if it is to run as any step.
-        ``key``: (sequences, rows, wanted logit rows, plan class); ``tile_rows``: called for the row counts of
-        the attention's work lists that the shape's eager run made."""
+        ``key``: (sequences, rows, wanted logit rows, the parts' plans); ``longest``: the step's longest
+        sequence (one for which the parts plan as the key says)."""
         graph = self.graphs.pop(key, None)
         if graph is not None:
             self.graphs[key] = graph  # the most recently used is last
@@ -275,17 +297,17 @@ class PrefillGraphs:
         self.seen[key] = times
         if len(self.seen) > 1024:
             self.seen.clear()
-        rows = tile_rows()
-        if times < 2 or rows is None:
+        if times < 2:
             return None
-        batch, total, wanted, plan_class = key
-        graph = PrefillGraph(self.engine, batch, total, wanted, plan_class, rows)
-        graph.fill(arrays, counts, first_positions)
-        logits = graph.first_run()
+        batch, total, wanted, _ = key
+        graph = PrefillGraph(self.engine, batch, total, wanted, longest)
+        logits = graph.first_run(arrays, counts, first_positions)
         if graph.graph is None:
             self.refused.add(key)
             return None if logits is None else (logits, False)
         while len(self.graphs) >= PREFILL_GRAPHS_KEPT:
+            # (the stream may still replay the oldest: it is destroyed only when the GPU has left it)
+            torch.cuda.synchronize()
             self.graphs.pop(next(iter(self.graphs)))
         self.graphs[key] = graph
         return logits, False

@@ -31,6 +31,10 @@ def parse_dtype(name) -> torch.dtype:
 
 
 class Runtime:
+    """One runtime drives one GPU: it makes its device the current one, and
+    every kernel is launched on that device's current stream.  A process that
+    has bound its kernels to one GPU refuses a runtime on another."""
+
     def __init__(self, device="cuda:0", dtype="bfloat16"):
         self.device = torch.device(device)
         self.dtype = parse_dtype(dtype)
@@ -40,10 +44,26 @@ class Runtime:
             )
         if not torch.cuda.is_available():
             raise KernelError("no GPU is visible to this process; the engine has no host path")
+        index = torch.cuda.current_device() if self.device.index is None else self.device.index
+        count = torch.cuda.device_count()
+        if not 0 <= index < count:
+            raise InvalidInput(f"device ordinal {index} names no GPU of this process (it sees {count})")
+        self.device = torch.device("cuda", index)
         from ..kernels import ops
 
         self.ops = ops
+        ops.bind_device(index)  # refuses a second GPU in one process
+        torch.cuda.set_device(index)  # launches, symbol addresses and new streams are the current device's
         ops.core()  # fails loudly here if the extension is neither built nor buildable
+
+    def check_current(self) -> None:
+        """Raises if the caller has made another GPU current since: a launch
+        would then go to a stream of the wrong device."""
+        current = torch.cuda.current_device()
+        if current != self.device.index:
+            raise InvalidInput(
+                f"this engine runs on {self.device}, but the process's current device is cuda:{current}; "
+                f"make it current again (torch.cuda.set_device({self.device.index})) before a step")
 
     @property
     def is_fp32(self) -> bool:

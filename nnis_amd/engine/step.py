@@ -17,7 +17,7 @@ import torch
 from ..cache import SequenceCache
 from ..errors import InvalidInput
 from .batch import StepContext, StepEntry
-from .graph import PREFILL_GRAPH_MOST_TOKENS, PREFILL_GRAPH_MOST_WORK, PrefillGraphs
+from .graph import PREFILL_GRAPH_MOST_TOKENS, PREFILL_GRAPH_MOST_WORK, PrefillGraphs, prompt_rows
 
 
 class Engine:
@@ -26,6 +26,7 @@ class Engine:
             raise InvalidInput("the model has no weights bound; load it first")
         self.model = model
         self.rt = rt
+        model.check(rt)  # (a model that was not loaded through ``load_model``: sizes the kernels refuse stop here)
         self.vocab_size = model.spec.vocab_size
         self.max_positions = model.spec.max_positions
         requests, shared = model.cache_requests()
@@ -39,7 +40,13 @@ class Engine:
         self.use_graphs = model.graph_safe() if use_graphs is None else (use_graphs and model.graph_safe())
         self._graphs = None
         self._prefill_graphs = None  # prompt steps whose shape comes again
-        self._tile_rows = {}  # per shape: rows a tile of the attention's work lists, as the eager run made them
+        # A step's positions index the rotation tables on the device, where nothing can refuse them: the tables
+        # reach as far as the cache lets a sequence grow, so the check of the lengths before a step covers both.
+        for name, position in model.positions.items():
+            tables = position.rotary()
+            if tables is not None and tables.cos.shape[0] < self.max_positions:
+                raise InvalidInput(f"position encoding {name!r} has tables for {tables.cos.shape[0]} positions; "
+                                   f"the model's sequences may reach {self.max_positions}")
 
     # ---- sequences -----------------------------------------------------------
     def start_sequence(self) -> int:
@@ -133,6 +140,7 @@ class Engine:
         """As ``step``, but the rows may view a buffer that the next step
         overwrites: for callers that read them at once (the generation loop)."""
         self._borrowed = False
+        self.rt.check_current()
         if self.use_graphs and entries and all(len(e.tokens) == 1 for e in entries):
             return self._decode_step(entries)
         growth, token_arrays = self._validate(entries)
@@ -155,27 +163,33 @@ class Engine:
             row += n
             seq_start[index + 1] = row
         self.cache.grow(growth)
+        try:
+            return self._run_prompts(entries, counts, pos0, total, want_rows, [
+                ids, tok_slot, tok_pos,
+                np.asarray([e.slot for e in entries], dtype=np.int32), seq_start,
+                np.asarray(pos0, dtype=np.int32), np.asarray(want_rows, dtype=np.int32),
+            ])
+        except BaseException:
+            # A step that could not be launched (a kernel refused a size, a part raised) leaves the sequences
+            # as long as they were: the pages it took go back.  What it wrote into pages it keeps lies beyond
+            # the lengths and is never read.  (Fixed-size state that a part had already advanced stays advanced.)
+            self.cache.roll_back(dict(zip((e.slot for e in entries), pos0)))
+            raise
 
-        arrays = [
-            ids, tok_slot, tok_pos,
-            np.asarray([e.slot for e in entries], dtype=np.int32), seq_start,
-            np.asarray(pos0, dtype=np.int32), np.asarray(want_rows, dtype=np.int32),
-        ]
+    def _run_prompts(self, entries, counts, pos0, total, want_rows, arrays) -> torch.Tensor:
         longest = max(p + n for p, n in zip(pos0, counts))
-        shape = None
+        rows = prompt_rows(total)
         if (self.use_graphs and total <= PREFILL_GRAPH_MOST_TOKENS and want_rows
                 and total * float(self.model.spec.width) ** 2 <= PREFILL_GRAPH_MOST_WORK):
             # a shape that comes again is replayed from a graph (engine/graph.py)
-            shape = (len(counts), self.rt.ops.prefill_rows(total), len(want_rows), self.rt.ops.prefill_plan_class(longest))
+            shape = (len(counts), rows, len(want_rows), self.model.prompt_plan(len(counts), rows, longest, self.rt))
             if self._prefill_graphs is None:
                 self._prefill_graphs = PrefillGraphs(self)
-            done = self._prefill_graphs.step(shape, arrays, counts, pos0, lambda: self._tile_rows.get(shape))
+            done = self._prefill_graphs.step(shape, arrays, counts, pos0, longest)
             if done is not None:
                 logits, self._borrowed = done
                 return logits
-        dev = self._stage([
-            *arrays,
-        ])
+        dev = self._stage(arrays)
         ctx = StepContext(
             tokens=total,
             batch=len(entries),
@@ -190,13 +204,9 @@ class Engine:
             host_slots=[e.slot for e in entries],
             host_new=counts,
             host_pos0=pos0,
+            plan_rows=rows,
         )
-        logits = self.model.forward(dev[0], ctx, self.cache, dev[6], self.rt)
-        if shape is not None:
-            self._tile_rows[shape] = sorted(ctx.tiles)  # the attention's work lists this shape needs
-            if len(self._tile_rows) > 1024:
-                self._tile_rows.clear()
-        return logits
+        return self.model.forward(dev[0], ctx, self.cache, dev[6], self.rt)
 
     def prepare_decode(self, batch: int, longest: int) -> None:
         """Makes the graph that a step of one token for each of ``batch``
@@ -224,6 +234,7 @@ class Engine:
         if ids_device.dtype != torch.int32 or ids_device.dim() != 1 or ids_device.numel() < len(slots) or not slots:
             raise InvalidInput("step_from_device: one int32 id per slot is needed")
         self._borrowed = False
+        self.rt.check_current()
         return self._decode_step([StepEntry(s, (), None) for s in slots], ids_device)
 
     def _decode_step(self, entries: Sequence[StepEntry], ids_device: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -247,11 +258,17 @@ class Engine:
                         raise InvalidInput(f"slot {entry.slot}: wanted place {place} is not among its 1 tokens")
         if self._graphs is None:
             self._graphs = DecodeGraphs(self)
-        # the graph first (its capture may fail), the cache's growth after it: a refused step changes nothing
-        longest = max(self.cache.length(slot) for slot in slots) + 1
-        graph = self._graphs.get(len(entries), longest)
-        pos0 = self.cache.grow_by_one(slots)
-        logits = graph.run(ids, slots, pos0, ids_device)
+        # What only reads comes first (room in the cache, the positions' end: a step that is refused has then
+        # cost no capture), then the graph (its capture may fail), the cache's growth after it: a refused
+        # step changes nothing.
+        checked = self.cache.check_one_more(slots)
+        graph = self._graphs.get(len(entries), max(checked[0]) + 1)
+        pos0 = self.cache.grow_by_one(slots, checked)
+        try:
+            logits = graph.run(ids, slots, pos0, ids_device)
+        except BaseException:
+            self.cache.roll_back(dict(zip(slots, pos0)))
+            raise
         wanted = [i for i, e in enumerate(entries) if e.want is None or len(e.want) > 0]
         if len(wanted) == len(entries):
             self._borrowed = True

@@ -22,7 +22,8 @@ import sys
 import tempfile
 import threading
 import time
-from typing import Dict, List, Optional, Tuple
+from dataclasses import dataclass
+from typing import Callable, Dict, List, Optional, Sequence, Tuple
 
 from ..errors import KernelError
 
@@ -47,46 +48,98 @@ FLAGS = [
 # sums in vector registers the prefill attention's four-column kernels at 64 channels keep 17 to 26 registers
 # in scratch memory, all outside their loops over the keys; no other kernel of either file spills.)
 _VECTOR_SUMS = ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]
-SOURCE_FLAGS = {"gemm_mfma.hip": _VECTOR_SUMS, "attention.hip": _VECTOR_SUMS}
-HEADERS = {"core": ["common.h", "epilogue.h", "nnis_noalloc.h"], "attention": ["common.h"]}  # what a module's sources include
-CORE_SOURCES = ["elementwise.hip", "gemm.hip", "gemm_mfma.hip", "gemm_fused.hip", "sampling.hip"]
-ATTENTION_SOURCES = ["attention.hip"]
 PREBUILT_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 112, 128, 192, 256)
 
 _loaded: Dict[str, ctypes.CDLL] = {}
 _lock = threading.Lock()
 
 
+@dataclass(frozen=True)
+class ModuleRecipe:
+    """What a module is made from: source files and the headers they include (names inside ``directory``),
+    preprocessor definitions, and extra compiler flags per source."""
+
+    sources: Tuple[str, ...]
+    headers: Tuple[str, ...] = ()
+    defines: Tuple[Tuple[str, str], ...] = ()
+    source_flags: Tuple[Tuple[str, Tuple[str, ...]], ...] = ()
+    directory: str = CSRC
+
+    def flags_of(self, source: str) -> List[str]:
+        return [flag for name, flags in self.source_flags if name == source for flag in flags]
+
+
+_modules: Dict[str, ModuleRecipe] = {}
+_families: Dict[str, Callable[[str], ModuleRecipe]] = {}  # by prefix: the rest of a module's name -> its recipe
+
+
+def register_module(name: str, sources: Sequence[str], headers: Sequence[str] = (), defines: Optional[Dict[str, str]] = None,
+                    source_flags: Optional[Dict[str, Sequence[str]]] = None, directory: str = CSRC, replace: bool = False) -> None:
+    """Makes ``load_module(name)`` build and load a library from ``sources``
+    under ``directory`` (every flag of the library's own kernels applies; the
+    library's headers are on the include path).  A part that brings kernels
+    of its own registers them here and declares their entry points with
+    ``ops.bind``; nothing else in the library has to know the module.  The
+    module exports ``const char* nnis_last_error()`` (``common.h`` has the
+    helpers that fill it), and its entry points return 0 or an error."""
+    if name in _modules and not replace:
+        raise KernelError(f"kernel module {name!r} is registered already")
+    _modules[name] = ModuleRecipe(tuple(sources), tuple(headers), tuple(sorted((defines or {}).items())),
+                                  tuple(sorted((k, tuple(v)) for k, v in (source_flags or {}).items())), directory)
+
+
+def register_module_family(prefix: str, recipe: Callable[[str], ModuleRecipe], replace: bool = False) -> None:
+    """Modules compiled per size: ``load_module(prefix + rest)`` builds what ``recipe(rest)`` describes."""
+    if prefix in _families and not replace:
+        raise KernelError(f"kernel module family {prefix!r} is registered already")
+    _families[prefix] = recipe
+
+
+def _attention_recipe(rest: str) -> ModuleRecipe:
+    try:
+        head_dim = int(rest)
+    except ValueError:
+        raise KernelError(f"unknown kernel module 'attn_hd{rest}'") from None
+    return ModuleRecipe(("attention.hip",), ("common.h",), (("NNIS_HEAD_DIM", str(head_dim)),), (("attention.hip", tuple(_VECTOR_SUMS)),))
+
+
+# the library's own modules: ``core`` holds the kernels whose sizes are run-time arguments; attention is compiled per head size
+register_module("core", ["elementwise.hip", "gemm.hip", "gemm_mfma.hip", "gemm_fused.hip", "sampling.hip"],
+                headers=["common.h", "epilogue.h", "nnis_noalloc.h"], source_flags={"gemm_mfma.hip": _VECTOR_SUMS})
+register_module_family("attn_hd", _attention_recipe)
+
+
 def _say(message: str) -> None:
     print(f"[nnis_amd] {message}", file=sys.stderr, flush=True)
 
 
-def module_recipe(module: str) -> Tuple[List[str], Dict[str, str]]:
-    """Sources and preprocessor definitions of a module name."""
-    if module == "core":
-        return [s for s in CORE_SOURCES if os.path.exists(os.path.join(CSRC, s))], {}
-    if module.startswith("attn_hd"):
-        head_dim = int(module[len("attn_hd"):])
-        return list(ATTENTION_SOURCES), {"NNIS_HEAD_DIM": str(head_dim)}
+def module_recipe(module: str) -> ModuleRecipe:
+    """What a module name is made from."""
+    if module in _modules:
+        return _modules[module]
+    for prefix, recipe in _families.items():
+        if module.startswith(prefix):
+            return recipe(module[len(prefix):])
     raise KernelError(f"unknown kernel module {module!r}")
 
 
-def _module_hash(sources: List[str], defines: Dict[str, str]) -> str:
+def _module_hash(recipe: ModuleRecipe) -> str:
     digest = hashlib.sha256()
-    headers = HEADERS["attention" if sources == ATTENTION_SOURCES else "core"]
-    for name in headers + sources:
-        with open(os.path.join(CSRC, name), "rb") as handle:
+    for name in recipe.headers + recipe.sources:
+        path = os.path.join(recipe.directory, name)
+        if not os.path.exists(path):
+            path = os.path.join(CSRC, name)  # (a module from elsewhere may include the library's headers)
+        with open(path, "rb") as handle:
             digest.update(name.encode())
             digest.update(handle.read())
     digest.update(" ".join(FLAGS).encode())
-    digest.update(repr(sorted((name, flags) for name, flags in SOURCE_FLAGS.items() if name in sources)).encode())
-    digest.update(repr(sorted(defines.items())).encode())
+    digest.update(repr(sorted((name, list(flags)) for name, flags in recipe.source_flags if name in recipe.sources)).encode())
+    digest.update(repr(sorted(recipe.defines)).encode())
     return digest.hexdigest()[:12]
 
 
 def module_filename(module: str) -> str:
-    sources, defines = module_recipe(module)
-    return f"libnnis_{module}-{_module_hash(sources, defines)}.so"
+    return f"libnnis_{module}-{_module_hash(module_recipe(module))}.so"
 
 
 def _fallback_dir() -> str:
@@ -146,7 +199,8 @@ def _run_with_heartbeat(commands: List[Tuple[str, List[str]]], env: Dict[str, st
 
 def build_module(module: str, force: bool = False) -> str:
     """Compiles one module and returns the library's path."""
-    sources, defines = module_recipe(module)
+    recipe = module_recipe(module)
+    sources, defines = list(recipe.sources), dict(recipe.defines)
     name = module_filename(module)
     if not force:
         found = find_built(module)
@@ -172,7 +226,8 @@ def build_module(module: str, force: bool = False) -> str:
             obj = os.path.join(work, source + ".o")
             objects.append(obj)
             commands.append(
-                (f"{source} [{module}]", [hipcc] + FLAGS + SOURCE_FLAGS.get(source, []) + define_flags + ["-I", CSRC, "-c", os.path.join(CSRC, source), "-o", obj])
+                (f"{source} [{module}]", [hipcc] + FLAGS + recipe.flags_of(source) + define_flags
+                 + ["-I", recipe.directory, "-I", CSRC, "-c", os.path.join(recipe.directory, source), "-o", obj])
             )
         _run_with_heartbeat(commands, env)
         tmp_out = os.path.join(work, name)

@@ -11,7 +11,7 @@ from typing import Optional
 import torch
 
 from ..cache.layout import k_page_shape, v_page_shape
-from ..errors import KernelError
+from ..errors import KernelError, Unsupported
 from . import lib as _lib
 
 PAGE_TOKENS = 64
@@ -39,6 +39,7 @@ _CORE_SIGNATURES = {
                         _VOID, _VOID, _VOID, _VOID, _VOID, _INT, _INT, _INT, _INT, _VOID, _VOID, _VOID, _INT, _VOID],
     "nnis_gemm_residual_parts": [_INT, _INT],
     "nnis_gemm_tile": [_INT, _INT, _INT],
+    "nnis_gemm_takes_pair": [_INT, _INT, _INT, _SIZE],
     "nnis_gemm_residual": [_VOID, _VOID, _VOID, _VOID, _INT, _VOID, _VOID, _INT, _INT, _INT, _INT, _VOID, _INT, _VOID, _SIZE, _VOID, _VOID],
     "nnis_gemm_scaled": [_VOID, _VOID, _INT, _FLT, _VOID, _INT, _INT, _INT, _INT, _VOID, _VOID, _VOID, _INT, _VOID, _VOID,
                          _VOID, _VOID, _VOID, _INT, _INT, _INT, _INT, _VOID, _VOID, _VOID, _INT, _VOID, _SIZE, _VOID],
@@ -77,6 +78,22 @@ def _code(t: torch.Tensor) -> int:
         raise KernelError(f"kernels take float32 or bfloat16 tensors, got {t.dtype}") from None
 
 
+def bind(module: str, signatures):
+    """Loads a kernel module (one that ``kernels.lib`` has built in, or one that a part registered there with
+    ``register_module``) and declares its entry points: ``signatures`` maps a name to its argument types; every
+    entry point returns an int, 0 or an error whose text ``nnis_last_error()`` holds (``check`` raises it)."""
+    return _bind(module, signatures)
+
+
+def stream() -> int:
+    """The raw handle of the stream that launches go to (the last argument of every entry point)."""
+    return _stream()
+
+
+def check(lib, status: int) -> None:
+    _check(lib, status)
+
+
 def _bind(module: str, signatures):
     lib = _lib.load_module(module)
     if not getattr(lib, "_nnis_bound", False):
@@ -101,10 +118,18 @@ def core():
     return _core
 
 
+ATTENTION_MOST_CHANNELS = 256
+
+
+def attention_check(head_dim: int) -> None:
+    """Raises ``Unsupported`` for a head size that no attention kernel here takes."""
+    if head_dim <= 0 or head_dim % 2 != 0 or head_dim > ATTENTION_MOST_CHANNELS:
+        raise Unsupported(f"the attention kernels take an even head_dim up to {ATTENTION_MOST_CHANNELS}, got {head_dim}")
+
+
 def attention_module(head_dim: int):
     if head_dim not in _attn:
-        if head_dim <= 0 or head_dim % 2 != 0 or head_dim > 256:
-            raise KernelError(f"attention kernels take an even head_dim up to 256, got {head_dim}")
+        attention_check(head_dim)
         _attn[head_dim] = _bind(f"attn_hd{head_dim}", _ATTN_SIGNATURES)
     return _attn[head_dim]
 
@@ -117,13 +142,29 @@ def _check(lib, status: int) -> None:
 _device_index: Optional[int] = None
 
 
-def _stream() -> int:
-    """The current stream's handle.  (``torch.cuda.current_stream().cuda_stream``
-    builds a Python stream object on every call, which cost a third of an
-    operation's time on the host; the raw query does not.)"""
+def bind_device(index: int) -> None:
+    """Names the one GPU whose streams this process's launches go to.  The
+    runtime calls it when it is made (and makes that device current); a
+    second runtime on another GPU is refused, because every launch below
+    takes the bound device's current stream and the per-device arrays
+    (``argmax_no_alloc``, the products' workspace) are looked up for it."""
     global _device_index
+    if _device_index is not None and _device_index != int(index):
+        raise KernelError(f"this process already runs its kernels on cuda:{_device_index}; a process drives one GPU "
+                          f"(cuda:{int(index)} was asked for)")
+    _device_index = int(index)
+
+
+def bound_device() -> Optional[int]:
+    return _device_index
+
+
+def _stream() -> int:
+    """The bound device's current stream (a raw handle:
+    ``torch.cuda.current_stream().cuda_stream`` builds a Python stream object
+    on every call, which cost a third of an operation's time on the host)."""
     if _device_index is None:
-        _device_index = torch.cuda.current_device()  # the library runs on one GPU
+        bind_device(torch.cuda.current_device())  # kernels called without a runtime (tests of one kernel)
     return torch._C._cuda_getCurrentRawStream(_device_index)
 
 
@@ -239,6 +280,9 @@ def silu_mul(gate_up: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     return out
 
 
+STATIC_SCRATCH_WORDS = 65536  # NNIS_STATIC_SCRATCH_WORDS of csrc/nnis_noalloc.h
+
+
 def argmax(logits: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     _dev(logits, "logits"), _dev(out, "out")
     rows, vocab = logits.shape
@@ -247,12 +291,14 @@ def argmax(logits: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     if not logits.is_contiguous():
         raise KernelError("argmax: logits must be contiguous")
     lib = core()
-    scratch = torch.empty(max(1, lib.nnis_argmax_scratch(rows, vocab)), dtype=torch.float32, device=logits.device)
+    need = lib.nnis_argmax_scratch(rows, vocab)
+    if need <= STATIC_SCRATCH_WORDS:
+        # the array that the library holds on the GPU: nothing to allocate (calls follow one another on one stream)
+        _check(lib, lib.nnis_argmax_static(logits.data_ptr(), out.data_ptr(), rows, vocab, _stream()))
+        return out
+    scratch = torch.empty(max(1, need), dtype=torch.float32, device=logits.device)
     _check(lib, lib.nnis_argmax(logits.data_ptr(), out.data_ptr(), rows, vocab, scratch.data_ptr(), _stream()))
     return out
-
-
-STATIC_SCRATCH_WORDS = 65536  # NNIS_STATIC_SCRATCH_WORDS of csrc/nnis_noalloc.h
 
 
 def argmax_no_alloc(logits: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
@@ -425,6 +471,19 @@ def _gemm_workspace(device) -> Optional[torch.Tensor]:
         # behind the workspace proper: the counts of the strips that two blocks share (`gemm_residual`), zero between calls
         held = _gemm_workspaces[key] = torch.zeros(GEMM_WORKSPACE_BYTES // 4 + PAIR_COUNTS, dtype=torch.float32, device=device)
     return held
+
+
+def gemm_takes_pair(m: int, n: int, k: int) -> bool:
+    """Whether ``gemm_residual`` gives a product of these sizes to two blocks a strip (the kernel whose blocks
+    meet in the workspace and count in the words behind it)."""
+    return bool(core().nnis_gemm_takes_pair(int(m), int(n), int(k), GEMM_WORKSPACE_BYTES))
+
+
+def gemm_pair_counts(device) -> Optional[torch.Tensor]:
+    """The strips' counts of the products with two blocks a strip on ``device`` (int32 [PAIR_COUNTS]; None
+    before the first product there): every word is zero whenever no such product is running."""
+    work = _gemm_workspace(torch.device(device))
+    return None if work is None else work[GEMM_WORKSPACE_BYTES // 4:].view(torch.int32)
 
 
 def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, split: int = 0) -> torch.Tensor:
@@ -825,19 +884,12 @@ PREFILL_SOME_ROWS = 16384  # ... from which a step of 1,024 to 1,279 tokens stil
 PREFILL_EIGHT_WAVES_MOST = 40960
 
 
-def prefill_rows(total: int) -> int:
-    """Rows of the replayed prompt step that takes ``total`` tokens: the next multiple of 64 up to 1,024
-    tokens, of 128 up to 2,048, of 256 beyond.  (Plans that look at a step's size look at this, so that a step
-    launched and the same step replayed from a graph's rows take the same kernels.)"""
-    unit = 64 if total <= 1024 else (128 if total <= 2048 else 256)
-    return ((total + unit - 1) // unit) * unit
-
-
 def prefill_plan(longest: int, rows: int, heads: int, head_dim: int = 64, kv_heads: int = 0):
-    """(waves of a block, column option) of the prefill attention for a step of ``rows`` tokens whose longest
-    sequence has ``longest`` (``kv_heads``: 0 for as many as ``heads``)."""
+    """(waves of a block, column option) of the prefill attention for a step of ``rows`` rows (what the engine
+    plans for: a step's tokens rounded up as a replayed step's are) whose longest sequence has ``longest``
+    (``kv_heads``: 0 for as many as ``heads``)."""
     plan_class = prefill_plan_class(longest)
-    size = prefill_rows(rows) * heads
+    size = rows * heads
     # A step with work items for about twice the waves that the chip holds (two a SIMD up to 64 channels, one
     # beyond; an item is 16 rows x 4, 2 or 1 columns) gives each item to one wave, which needs no merge and pays an
     # item's first loads once.  One sequence, microseconds a layer with one wave against the plan by length: 32
@@ -870,12 +922,6 @@ def prefill_plan(longest: int, rows: int, heads: int, head_dim: int = 64, kv_hea
     return waves, plan_class  # 2 waves and one column from 128 tokens on, 4 waves and two columns from 512 on
 
 
-# The work list of a prefill step goes to the device through pinned memory, so that the copy does not make the
-# host wait for the kernels already on the stream (a copy from ordinary memory does: 70 to 100 us a step).  One
-# buffer per device, grown when a step needs more; the event says when the last copy has left it.
-_tile_staging = {}
-
-
 def prefill_plan_class(longest: int) -> int:
     """Steps whose longest sequence falls into the same class launch the same prefill attention kernels
     (``attention`` picks the waves of a block, and the column option, by these thresholds)."""
@@ -894,47 +940,41 @@ def prefill_tile_items(new_tokens, first_positions, rows: int):
     return [seq for _, seq, _ in items], [row0 for _, _, row0 in items]
 
 
-def _prefill_tiles(ctx, rows: int, device):
-    """Work items of a prefill step for tiles of ``rows`` query rows, longest first."""
-    cached = ctx.tiles.get(rows)
-    if cached is None:
-        if ctx.host_new is None or torch.cuda.is_current_stream_capturing():
-            # (a step that runs from fixed buffers brings its lists; a copy recorded under capture would bring
-            # this step's list to every replay)
-            raise KernelError(f"a prompt step from fixed buffers has no work list for tiles of {rows} rows")
-        seqs, row0s = prefill_tile_items(ctx.host_new, ctx.host_pos0, rows)
-        count = len(seqs)
-        key = (device.type, device.index)
-        held = _tile_staging.get(key)
-        if held is None or held[0].shape[1] < count:
-            size = max(256, 1 << (count - 1).bit_length())
-            held = _tile_staging[key] = (torch.empty((2, size), dtype=torch.int32, pin_memory=True), torch.cuda.Event())
-        else:
-            held[1].synchronize()
-        host, copied = held
-        view = host.numpy()
-        view[0, :count] = seqs
-        view[1, :count] = row0s
-        packed = torch.empty((2, count), dtype=torch.int32, device=device)
-        packed.copy_(host[:, :count], non_blocking=True)
-        copied.record()
-        cached = ctx.tiles[rows] = (packed[0], packed[1])
-    return cached
+NO_ROWS = 1 << 24  # first row of a work item that has none: it lies beyond any sequence's tokens
+
+
+def prefill_tile_list(new_tokens, first_positions, padded, rows: int):
+    """``prefill_tile_items`` as one int32 array [2, items] (row 0 the sequences, row 1 the first rows), the form in
+    which a step keeps its work lists (``StepContext.lists``).  ``padded``: None, or (sequences, rows of the step)
+    of a step that runs from fixed buffers: the list then has as many items as any step of that shape can have
+    (rows of the step / rows of a tile + sequences), those beyond the step's own with no rows."""
+    import numpy as np
+
+    seqs, row0s = prefill_tile_items(new_tokens, first_positions, rows)
+    count = len(seqs)
+    if padded is not None:
+        count = padded[1] // rows + padded[0]
+        if len(seqs) > count:
+            raise KernelError(f"{len(seqs)} work items for a step of {padded[0]} sequences and {padded[1]} rows")
+    out = np.empty((2, count), dtype=np.int32)
+    out[0, :len(seqs)], out[0, len(seqs):] = seqs, 0
+    out[1, :len(seqs)], out[1, len(seqs):] = row0s, NO_ROWS
+    return out
 
 
 def attention(q: torch.Tensor, out: torch.Tensor, view, ctx, heads: int, kv_heads: int, head_dim: int, scale: float,
-              window: int = 0, keep_runs: bool = False, tables: Optional[StepTables] = None):
+              window: int = 0, keep_runs: bool = False, tables: Optional[StepTables] = None, plan=None):
     """Attention of the step's tokens over the cache ``view``: bfloat16 with a
     head size in steps of 16 runs on the matrix cores (one kernel for single
     tokens, one for runs of tokens); anything else takes the 32-bit kernel.
     ``keep_runs``: a decode step whose keys are cut into runs may return them
-    as ``KeyRuns`` instead of the output (see ``attention_decode_bf16``)."""
+    as ``KeyRuns`` instead of the output (see ``attention_decode_bf16``).
+    ``plan``: (runs, waves) of a step of single tokens (``decode_plan``), or
+    (waves, columns) of a step of prompts (``prefill_plan``); None: as those
+    functions choose for the step's planned sizes."""
     fast = (q.dtype == torch.bfloat16 and view.k_pages.dtype == torch.bfloat16 and head_dim % 16 == 0)
     if fast and ctx.decode and heads // kv_heads <= 16 * (4 if head_dim <= 64 else (2 if head_dim <= 128 else 1)):
-        if ctx.splits:
-            splits, waves = ctx.splits, ctx.waves
-        else:
-            splits, waves = decode_plan(ctx.batch, kv_heads, ctx.plan_len or ctx.max_len, width=heads * head_dim)
+        splits, waves = plan or decode_plan(ctx.batch, kv_heads, ctx.planned_len, width=heads * head_dim)
         waves = min(waves, decode_max_waves(heads, kv_heads, head_dim))
         partial = None
         if splits > 1:
@@ -946,10 +986,11 @@ def attention(q: torch.Tensor, out: torch.Tensor, view, ctx, heads: int, kv_head
     if fast and not ctx.decode:
         # A tile's keys are a chain of dependent loads: the longest tile sets the kernel's time.  The waves of
         # a block deal the keys among themselves (their merge lives in LDS).
-        waves, columns = prefill_plan(ctx.max_len, ctx.tokens, heads, head_dim, kv_heads)
+        waves, columns = plan or prefill_plan(ctx.planned_len, ctx.planned_rows, heads, head_dim, kv_heads)
         waves = min(waves, prefill_max_waves(heads, kv_heads, head_dim, columns))
-        tile_seq, tile_row0 = _prefill_tiles(ctx, prefill_tile_rows(heads, kv_heads, head_dim, columns), q.device)
-        return attention_prefill_bf16(q, out, view.k_pages, view.v_pages, view.block_table, tile_seq, tile_row0,
+        rows = prefill_tile_rows(heads, kv_heads, head_dim, columns)
+        tiles = ctx.lists.device_list(("attention_tiles", rows), lambda new, first, padded: prefill_tile_list(new, first, padded, rows))
+        return attention_prefill_bf16(q, out, view.k_pages, view.v_pages, view.block_table, tiles[0], tiles[1],
                                       ctx.seq_slot, ctx.seq_start, ctx.seq_pos0, heads, kv_heads, head_dim, scale, window,
                                       waves, columns)
     return attention_rows(q, out, view.k_pages, view.v_pages, view.block_table, ctx.tok_slot, ctx.tok_pos, heads,

@@ -25,6 +25,7 @@ class DecoderModel:
         self.head = build_part("head", spec.head)
         self.bound = False
         self._plans = {}
+        self._prompt_plans = {}
 
     # ---- weights -------------------------------------------------------------
     def parts(self):
@@ -61,6 +62,26 @@ class DecoderModel:
         """True when a step's kernels read tokens, slots and positions from
         device memory only, so that a captured step can be replayed."""
         return all(getattr(part, "graph_safe", False) for part in self.parts())
+
+    def check(self, rt) -> None:
+        """Every part's own check of its sizes against the kernels (``Part.check``): raises ``Unsupported``."""
+        for part in self.parts():
+            part.check(rt)
+
+    def held_buffers(self, rt):
+        """What the parts' kernels keep between calls and a captured step has baked in (``Part.held_buffers``)."""
+        return [buffer for part in self.parts() for buffer in part.held_buffers(rt)]
+
+    def prompt_plan(self, batch: int, rows: int, longest: int, rt):
+        """The plans of every run of the schedule for a step of prompts (``Part.prompt_plan``)."""
+        key = (batch, rows, longest)
+        plans = self._prompt_plans.get(key)
+        if plans is None:
+            if len(self._prompt_plans) > 4096:
+                self._prompt_plans.clear()
+            plans = self._prompt_plans[key] = tuple(
+                self.layers[entry.layer].prompt_plan(batch, rows, longest, rt) for entry in self.spec.schedule)
+        return plans
 
     def decode_plan(self, batch: int, longest: int, rt):
         """The plans of every run of the schedule for a step of one token

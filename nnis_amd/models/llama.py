@@ -92,6 +92,8 @@ def llama_spec(cfg: LlamaConfig) -> ModelSpec:
             "tied_to": "model.embed_tokens.weight" if cfg.tie_word_embeddings else None,
         },
         stop_token_ids=cfg.eos_token_ids,
+        # a buffer that older Llama checkpoints carry beside the weights (the tables are made from theta here)
+        ignored_tensor_suffixes=("rotary_emb.inv_freq",),
         config_json=cfg.to_dict(),
     )
     spec.validate()

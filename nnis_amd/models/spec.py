@@ -39,6 +39,8 @@ class ModelSpec:
     final_norm: Dict[str, Any]
     head: Dict[str, Any]
     stop_token_ids: Tuple[int, ...] = ()
+    # endings of tensor names that a folder may hold beside the weights without being an error
+    ignored_tensor_suffixes: Tuple[str, ...] = ()
     config_json: Dict[str, Any] = field(default_factory=dict)  # what a model folder's config.json holds
 
     def validate(self) -> None:

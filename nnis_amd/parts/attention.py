@@ -55,9 +55,26 @@ class CausalSelfAttention(Mixer):
     def cache_request(self):
         return KVRequest(self.kv_heads, self.head_dim, self.window)
 
+    def check(self, rt):
+        rt.ops.attention_check(self.head_dim)
+
+    def _matrix_cores(self, rt) -> bool:
+        return rt.dtype == torch.bfloat16 and self.head_dim % 16 == 0
+
     def decode_plan(self, batch, longest, rt):
-        # what ``ops.attention`` picks for a step of single tokens with these sizes
+        # (runs of the keys, waves of a block) of a step of single tokens with these sizes
         return rt.ops.decode_plan(batch, self.kv_heads, longest, width=self.heads * self.head_dim)
+
+    def prompt_plan(self, batch, rows, longest, rt):
+        # (waves of a block, columns a wave carries) of the matrix-core kernel; the 32-bit kernel has no plan
+        if not self._matrix_cores(rt):
+            return None
+        return rt.ops.prefill_plan(longest, rows, self.heads, self.head_dim, self.kv_heads)
+
+    def held_buffers(self, rt):
+        # the runs of a decode step's keys meet in a scratch that the kernels' wrapper keeps per device
+        held = rt.ops.decode_scratch_held(rt.device)
+        return [] if held is None else [held]
 
     takes_pending_norm = True
     adds_to_residual = True
@@ -100,8 +117,12 @@ class CausalSelfAttention(Mixer):
         step = None
         if ctx.decode and q.dtype == torch.bfloat16:
             step = ctx.step_tables(rt, self.position.rotary() if self.position is not None else None, view.block_table)
+        plan = ctx.options.get("causal_attention")  # (a test or a sweep names the launch; else the sizes choose)
+        if plan is None:
+            plan = (self.decode_plan(ctx.batch, ctx.planned_len, rt) if ctx.decode
+                    else self.prompt_plan(ctx.batch, ctx.planned_rows, ctx.planned_len, rt))
         attn = rt.ops.attention(q, attn, view, ctx, self.heads, self.kv_heads, self.head_dim, self.scale, self.window or 0,
-                                keep_runs=into is not None, tables=step)
+                                keep_runs=into is not None, tables=step, plan=plan)
         if isinstance(attn, rt.ops.KeyRuns) and not (into.can_take(attn, self.out.weight) and attn.fits(self.out.weight.shape[0])):
             attn = attn.combine()
         if into is not None and into.can_take(attn, self.out.weight):

@@ -23,7 +23,10 @@ The interfaces:
     in the schedule (``KVRequest``, ``StateRequest`` or ``None``);
     ``forward(x, ctx, view, rt)`` -> y, where ``x`` is ``[tokens, width]`` in
     the activation type, ``ctx`` is the step's ``StepContext`` and ``view``
-    is the cache's view for this schedule entry.  A mixer that sets
+    is the cache's view for this schedule entry.  A mixer whose launches
+    depend on the step's lengths says how (``decode_plan``, ``prompt_plan``);
+    lists that it makes on the host for a step of prompts go through
+    ``ctx.lists`` (``StepLists``), which is what lets the step be replayed.  A mixer that sets
     ``takes_pending_norm = True`` is handed a ``PendingNorm`` instead of ``x``
     and must consume it (``materialize()`` or ``fused(...)``).
 ``FeedForward``
@@ -110,6 +113,33 @@ class Part:
         """Bytes of weights one step has to read through this part."""
         return 0
 
+    def check(self, rt) -> None:
+        """Raises ``Unsupported`` if the kernels this part would launch under
+        ``rt`` do not take its sizes.  Asked when a model is put together,
+        before any weight is read or any cache made, so that a size nobody
+        runs is refused at load and not at the first step."""
+
+    def decode_plan(self, batch: int, longest: int, rt):
+        """How this part would launch a step of one token for each of
+        ``batch`` sequences, the longest of ``longest`` tokens: anything that
+        can be hashed and compared, or None if its launches do not depend on
+        the lengths.  A captured step is replayed only for steps whose plans
+        equal those it was captured with."""
+        return None
+
+    def prompt_plan(self, batch: int, rows: int, longest: int, rt):
+        """The same for a step of prompts: ``batch`` sequences that bring
+        ``rows`` tokens between them (rounded up as the engine rounds a
+        replayed step's rows), the longest of ``longest`` tokens after it."""
+        return None
+
+    def held_buffers(self, rt):
+        """Device memory beyond a step's own tensors that this part's kernels
+        go through and that a captured step therefore has baked in (scratch
+        that the part, or the kernels' wrapper for it, keeps between calls):
+        a graph holds what this returns for as long as it lives."""
+        return []
+
     def packed_sources(self):
         """[((address, shape) of a loaded tensor, its packed copy)] for the
         tensors this part packed when it was bound and no longer keeps in the
@@ -157,14 +187,6 @@ class Mixer(Part):
     def cache_request(self):
         return None
 
-    def decode_plan(self, batch: int, longest: int, rt):
-        """How this mixer would launch a step of one token for each of
-        ``batch`` sequences, the longest of ``longest`` tokens: anything that
-        can be hashed and compared, or None if its launches do not depend on
-        the lengths.  A captured step is replayed only for steps whose plans
-        equal those it was captured with."""
-        return None
-
     def forward(self, x, ctx, view, rt):
         raise NotImplementedError
 
@@ -176,9 +198,6 @@ class FeedForward(Part):
 
 class Block(Part):
     def cache_request(self):
-        return None
-
-    def decode_plan(self, batch: int, longest: int, rt):
         return None
 
     def forward(self, stream, ctx, view, rt):

@@ -19,6 +19,13 @@ from .base import Block, build_part, register_part
 from .lazy import PendingNorm, ResidualInto
 
 
+def _joined(plans):
+    """The parts' plans as one: None where none of them plans anything, the
+    plan itself where one part does (the mixer, as a rule)."""
+    plans = tuple(plan for plan in plans if plan is not None)
+    return None if not plans else (plans[0] if len(plans) == 1 else plans)
+
+
 class PreNormBlock(Block):
     def __init__(self, width, norm1, mixer, norm2, feed_forward, positions=None):
         self.width = int(width)
@@ -42,8 +49,18 @@ class PreNormBlock(Block):
     def cache_request(self):
         return self.mixer.cache_request()
 
+    def check(self, rt):
+        for part in self._parts:
+            part.check(rt)
+
     def decode_plan(self, batch, longest, rt):
-        return self.mixer.decode_plan(batch, longest, rt)
+        return _joined(part.decode_plan(batch, longest, rt) for part in self._parts)
+
+    def prompt_plan(self, batch, rows, longest, rt):
+        return _joined(part.prompt_plan(batch, rows, longest, rt) for part in self._parts)
+
+    def held_buffers(self, rt):
+        return [buffer for part in self._parts for buffer in part.held_buffers(rt)]
 
     @property
     def entry_norm(self):

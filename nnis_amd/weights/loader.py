@@ -36,8 +36,6 @@ SINGLE = "model.safetensors"
 INDEX = "model.safetensors.index.json"
 _STORED = {"F32": torch.float32, "BF16": torch.bfloat16}
 _STORED_INTEGERS = {"I32": torch.int32, "I64": torch.int64}  # what a table of integers may be stored as
-# buffers that older checkpoints carry beside the weights
-_IGNORED_SUFFIXES = ("rotary_emb.inv_freq",)
 
 
 def _confined(model_dir: str, relative: str) -> str:
@@ -82,11 +80,14 @@ _DECLARED = {"float32": "F32", "bfloat16": "BF16"}
 
 
 def load_weights(model_dir: str, specs: Sequence[TensorSpec], device, widen_to_float32: bool,
-                 declared_dtype: Optional[str] = None, narrow_to_bfloat16: bool = False) -> Dict[str, torch.Tensor]:
+                 declared_dtype: Optional[str] = None, narrow_to_bfloat16: bool = False,
+                 ignored_suffixes: Sequence[str] = ()) -> Dict[str, torch.Tensor]:
     """``declared_dtype``: config.json's ``torch_dtype`` ("float32" or
     "bfloat16"; None skips the check, for callers without a config.json).
     ``narrow_to_bfloat16``: round tensors stored in 32-bit to bfloat16 at load
-    (not with ``widen_to_float32``)."""
+    (not with ``widen_to_float32``).  ``ignored_suffixes``: endings of names
+    that a folder of this architecture may hold beside its weights without
+    being an error (the model's description names them)."""
     if narrow_to_bfloat16 and widen_to_float32:
         raise WeightError("narrow_to_bfloat16 is for a bfloat16 runtime; the 32-bit path keeps 32-bit weights")
     if declared_dtype is not None and declared_dtype not in _DECLARED:
@@ -135,7 +136,7 @@ def load_weights(model_dir: str, specs: Sequence[TensorSpec], device, widen_to_f
             continue
         plan.append((spec.name, source))
     unexpected = sorted(
-        name for name in where if name not in consumed and not name.endswith(_IGNORED_SUFFIXES)
+        name for name in where if name not in consumed and not name.endswith(tuple(ignored_suffixes))
     )
 
     if missing or unexpected or wrong_shape or wrong_type or duplicates:

@@ -37,7 +37,9 @@ TINY_CONFIGS = {"A": (TINY_A, 0), "B": (TINY_B, 1), "C": (TINY_C, 2)}
 
 # The layer sizes of the models the library is measured on, with two layers and a
 # small vocabulary so that the plain implementation stays quick: grouped heads 3:1
-# with a width that is no power of two; one key/value head per query head; groups of 8.
+# with a width that is no power of two; one key/value head per query head; groups of 8;
+# and a fourth shape that is measured beside BASELINE's three: groups of 4 heads of 128
+# channels, a width of 4,096 and an inner size of 14,336.
 SHAPE_CONFIGS = {
     "smollm2-135m": (llama(
         num_hidden_layers=2, hidden_size=576, num_attention_heads=9, num_key_value_heads=3, intermediate_size=1536,
@@ -51,4 +53,8 @@ SHAPE_CONFIGS = {
         num_hidden_layers=2, hidden_size=2048, num_attention_heads=32, num_key_value_heads=4, intermediate_size=5632,
         vocab_size=3001, rope_theta=10000.0, rms_norm_eps=1e-5, tie_word_embeddings=False,
         max_position_embeddings=2048, torch_dtype="bfloat16"), 13),
+    "llama-8b": (llama(
+        num_hidden_layers=2, hidden_size=4096, num_attention_heads=32, num_key_value_heads=8, head_dim=128, intermediate_size=14336,
+        vocab_size=3001, rope_theta=500000.0, rms_norm_eps=1e-5, tie_word_embeddings=False,
+        max_position_embeddings=2048, torch_dtype="bfloat16"), 14),
 }

@@ -219,15 +219,23 @@ def test_truncate_gives_pages_back_and_keeps_the_rest():
 
 
 def test_reset_empties_a_slot_that_stays_held():
-    cache = _cache(max_tokens=256)
+    """Lengths, pages and the layers' own state go; what somebody else keeps
+    for the sequence in the slot's state regions (a sampler's generator and
+    options) stays: a sampled sequence goes on after a reset
+    (kv_cache.rs:170-172 only sets lengths to 0)."""
+    cache = _cache(max_tokens=256, extra=[(4, StateRequest((3,)))])
     region = cache.add_state_region("extra", (2,), torch.float32)
     a = cache.acquire()
     cache.grow({a: 130})
     region[a] = 3.0
+    cache.view(4).state[a] = 5.0
     cache.reset(a)
     assert cache.length(a) == 0 and a in cache.slots.held
     assert all(g.table.pool.free == 4 for g in cache.kv_groups)
-    assert region[a].abs().sum() == 0
+    assert cache.view(4).state[a].abs().sum() == 0  # the mixer's state starts over
+    assert bool((region[a] == 3.0).all())  # the sampler's does not
+    cache.release(a)
+    assert cache.acquire() == a and region[a].abs().sum() == 0  # a new sequence in the slot starts from zero everywhere
     cache.grow({a: 256})  # the whole cache again
     assert cache.length(a) == 256
     cache.release(a)
@@ -271,3 +279,85 @@ def test_values_may_be_narrower_than_keys():
     narrow = cache.kv_groups[0]
     assert narrow.k.shape[2:] == (2, 4, 64, 8) and narrow.v.shape[2:] == (2, 1, 2, 4, 16, 8)
     assert narrow.bytes_per_token() == 2 * (32 + 16) * 4 and cache.kv_groups[1].bytes_per_token() == 2 * 64 * 4
+
+
+def test_roll_back_returns_what_a_failed_step_took():
+    """A step whose launch failed after the cache grew: lengths and pages as
+    before, also where fixed-size state makes ``truncate`` refuse; a slot that
+    is not held, or a length not below the present one, is left alone."""
+    cache = _cache(max_tokens=512, extra=[(4, StateRequest((3,)))])
+    a, b = cache.acquire(), cache.acquire()
+    cache.grow({a: 70, b: 10})
+    free = [g.table.pool.free for g in cache.kv_groups]
+    before = {a: cache.length(a), b: cache.length(b)}
+    cache.grow({a: 200, b: 1})
+    cache.roll_back(before)
+    assert {a: cache.length(a), b: cache.length(b)} == before
+    assert [g.table.pool.free for g in cache.kv_groups] == free
+    cache.roll_back({a: 500, 99: 0})  # nothing to undo
+    assert cache.length(a) == 70
+    cache.grow({a: 1})
+    assert cache.length(a) == 71  # and the sequence goes on where it was
+
+
+def test_one_more_is_checked_without_a_change():
+    cache = _cache(max_tokens=192)
+    a, b = cache.acquire(), cache.acquire()
+    cache.grow({a: 64, b: 64})
+    cache.check_one_more([a])  # one page is free
+    with pytest.raises(CacheFull):
+        cache.check_one_more([a, b])  # both start a page, one is left
+    assert cache.length(a) == 64 and cache.length(b) == 64
+    checked = cache.check_one_more([a])
+    assert cache.grow_by_one([a], checked) == [64] and cache.length(a) == 65
+    with pytest.raises(InvalidInput, match="not held"):
+        cache.check_one_more([7])
+
+
+def test_positions_end_for_a_model_without_keys():
+    """A model that keeps only fixed-size state is stopped at its last position too."""
+    cache = SequenceCache([(0, StateRequest((2,)))], {}, max_tokens=1024, max_positions=100, dtype=torch.float32, device="cpu")
+    a = cache.acquire()
+    cache.grow({a: 99})
+    cache.grow_by_one([a])
+    with pytest.raises(CacheFull, match="positions end at 100"):
+        cache.grow({a: 1})
+    with pytest.raises(CacheFull, match="positions end at 100"):
+        cache.grow_by_one([a])
+    assert cache.length(a) == 100
+
+
+class _Event:
+    """Stands in for the event behind a flush: counts who waits for it."""
+
+    def __init__(self):
+        self.recorded = self.waited = 0
+
+    def record(self):
+        self.recorded += 1
+
+    def synchronize(self):
+        self.waited += 1
+
+
+def test_a_row_is_not_rewritten_before_its_copy_has_left():
+    """The block table's rows go to the device by copies that do not wait;
+    whoever writes into the pinned rows again waits for the last flush first,
+    and only then (no wait where nothing is pending)."""
+    cache = _cache(max_tokens=512)
+    group = cache.kv_groups[0]
+    group._flushed = event = _Event()
+    a = cache.acquire()
+    cache.grow({a: 10})  # first pages: nothing pending yet
+    assert (event.recorded, event.waited) == (1, 0)
+    cache.grow({a: 20})  # no new page: no flush, no wait
+    assert (event.recorded, event.waited) == (1, 0)
+    cache.grow({a: 60})  # a new page: the row is written again, after the first flush has left
+    assert (event.recorded, event.waited) == (2, 1)
+    cache.release(a)
+    b = cache.acquire()  # the same slot, another sequence
+    assert b == a
+    cache.grow({b: 1})
+    assert (event.recorded, event.waited) == (3, 2)
+    cache.grow_by_one([b])  # inside its page
+    assert (event.recorded, event.waited) == (3, 2)

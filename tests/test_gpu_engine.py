@@ -112,6 +112,100 @@ def test_refused_steps_change_nothing(model_dirs):
         big.step([StepEntry(s, [1] * 257, None)])  # the model has 256 positions
 
 
+def test_a_size_the_kernels_refuse_is_refused_at_load(tmp_path):
+    """A head size that the attention kernels do not take: said when the
+    model is put together, before a weight is read (the folder holds none)
+    or a cache made (session_batch.rs:86-101: fails before any session is
+    touched)."""
+    import json
+
+    from configs import llama
+    from nnis_amd.api import load_engine
+    from nnis_amd.errors import Unsupported
+
+    config = llama(num_hidden_layers=1, hidden_size=64, num_attention_heads=2, num_key_value_heads=1, head_dim=258,
+                   intermediate_size=96, vocab_size=100, rope_theta=10000.0, rms_norm_eps=1e-5, tie_word_embeddings=True,
+                   max_position_embeddings=128, torch_dtype="bfloat16")
+    folder = tmp_path / "model"
+    folder.mkdir()
+    (folder / "config.json").write_text(json.dumps(config))
+    for dtype in ("bfloat16", "float32"):
+        with pytest.raises(Unsupported, match="head_dim up to 256, got 258"):
+            load_engine(str(folder), dtype=dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_step_that_fails_in_flight_gives_back_what_it_took(model_dirs, dtype):
+    """A kernel that refuses in the middle of a step (here: the second
+    layer's mixer raises) after the cache has grown: lengths and pages are as
+    before, for a step of prompts and for a step of single tokens, and the
+    same step then runs and is right."""
+    from nnis_amd.engine.batch import StepEntry
+    from nnis_amd.errors import KernelError
+
+    engine = _engine(model_dirs, "A", dtype, max_tokens=512)
+    plain = P.PlainLlama(model_dirs["A"])
+    yard = _yard(model_dirs, "A") if dtype == "bfloat16" else None
+    rng = np.random.default_rng(3)
+    a, b = rng.integers(0, 512, size=140).tolist(), rng.integers(0, 512, size=30).tolist()
+    sa, sb = engine.start_sequence(), engine.start_sequence()
+    engine.step([StepEntry(sa, a[:60], None)])
+    mixer = engine.model.layers[1].mixer
+    forward = mixer.forward
+    failing = [True]
+
+    def sometimes(*args, **more):
+        if failing[0]:
+            raise KernelError("refused in flight")
+        return forward(*args, **more)
+
+    mixer.forward = sometimes
+    try:
+        free = engine.free_pages()
+        with pytest.raises(KernelError, match="in flight"):
+            engine.step([StepEntry(sa, a[60:130], None), StepEntry(sb, b[:20], None)])  # two new pages and one
+        assert (engine.length(sa), engine.length(sb), engine.free_pages()) == (60, 0, free)
+        failing[0] = False
+        rows = engine.step([StepEntry(sa, a[60:130], None), StepEntry(sb, b[:20], None)])
+        _close(rows.cpu(), torch.stack([plain.logits(a)[129], plain.logits(b)[19]]), dtype, "the step again", yard)
+        # single tokens: a graph that is there already replays and cannot fail; one that has to be captured can
+        engine._graphs = None
+        failing[0] = True
+        free = engine.free_pages()
+        with pytest.raises(KernelError, match="in flight"):
+            engine.step([StepEntry(sa, [a[130]], None), StepEntry(sb, [b[20]], None)])
+        assert (engine.length(sa), engine.length(sb), engine.free_pages()) == (130, 20, free)
+        failing[0] = False
+        rows = engine.step([StepEntry(sa, [a[130]], None), StepEntry(sb, [b[20]], None)])
+        _close(rows.cpu(), torch.stack([plain.logits(a)[130], plain.logits(b)[20]]), dtype, "single tokens again", yard)
+    finally:
+        mixer.forward = forward
+
+
+def test_a_sampled_sequence_goes_on_after_a_reset(model_dirs):
+    """``Engine.reset`` empties the sequence, not what the sampler keeps for
+    it in the slot: temperature, top-k, top-p and the generator's state stay,
+    and the draws go on (a temperature of zero left behind by a reset would
+    divide the logits by zero)."""
+    from nnis_amd.engine.batch import StepEntry
+    from nnis_amd.sampling.device import DeviceSelector
+    from nnis_amd.sampling.host import HostSampler
+    from nnis_amd.sampling.params import SamplingParams
+
+    engine = _engine(model_dirs, "B", "float32")
+    params = SamplingParams(seed=11, temperature=0.7, top_k=50, top_p=0.9)
+    selector = DeviceSelector(engine)
+    host = HostSampler(params, engine.vocab_size)
+    slot = engine.start_sequence()
+    selector.start(slot, params)
+    for prompt in ([5, 6, 7, 8], [9, 10], [11]):  # the second and third after a reset
+        logits = engine.step([StepEntry(slot, prompt, None)])
+        token = selector.select(logits, [slot], [params])[0]
+        assert token == host.sample(logits[0].cpu().numpy())  # the same generator, three draws on
+        engine.reset(slot)
+        assert engine.length(slot) == 0
+
+
 @pytest.mark.parametrize("name", ["A", "B", "C"])
 def test_greedy_generation_through_the_entry_point(model_dirs, name):
     import nnis_amd
@@ -299,7 +393,7 @@ def test_prompt_steps_whose_shape_comes_again(model_dirs, dtype):
     run([37, 5, 70], [0, 0, 0], [[1, 2], None, [3]])
     graphs = engine._prefill_graphs.graphs
     of_three = lambda: [key for key in graphs if key[0] == 3]  # noqa: E731  (single prompts here share a graph of their own)
-    assert of_three() == [(3, 128, 4, 0)]
+    assert [key[:3] for key in of_three()] == [(3, 128, 4)]
     other = engine.start_sequence()
     engine.step([StepEntry(other, [4, 5], None)])
     run([37, 5, 70], [3, 20, 0], [[36, 0], None, [10]])
@@ -313,10 +407,11 @@ def test_prompt_steps_whose_shape_comes_again(model_dirs, dtype):
     run([1, 64, 1], [0, 0, 0], [[0], [0, 63], None])
     run([64, 63, 1], [0, 1, 2], [[63], [0, 62], None])
     assert len(of_three()) == 1
-    # a longer first position puts the step into another class of the attention's plan: a shape of its own
+    # a longer first position makes the matrix-core attention plan its launch otherwise: a shape of its own
+    # (the 32-bit attention launches one way whatever the lengths: the same graph)
     run([37, 5, 70], [0, 0, 100], [[0, 36], None, [69]])
     run([37, 5, 70], [0, 0, 100], [[0, 36], None, [69]])
-    assert len(of_three()) == 2
+    assert len(of_three()) == (2 if dtype == "bfloat16" else 1)
     # more shapes than are kept: the oldest goes, and comes back through a new capture
     first = of_three()[0]
     for n in range(G.PREFILL_GRAPHS_KEPT):
@@ -326,16 +421,28 @@ def test_prompt_steps_whose_shape_comes_again(model_dirs, dtype):
     for _ in range(3):
         run([37, 5, 70], [0, 0, 0], [[0, 36], None, [69]])
     assert first in graphs
-    # a step that cannot be captured (here: a work list that the record of the shape's first run does not name)
+    # a step that cannot run from fixed buffers (here: a part that refuses while the step is tried from them)
     # is launched as any step, this time and from then on
     run([21, 40], [0, 0], [[0, 1, 2], [3, 4, 5]])
-    (shape,) = [key for key in engine._tile_rows if key[:3] == (2, 64, 6)]
-    if engine._tile_rows[shape]:  # (the 32-bit attention has no work lists)
-        engine._tile_rows[shape] = []
+    from nnis_amd.errors import KernelError
+
+    mixer = engine.model.layers[0].mixer
+    forward = mixer.forward
+
+    def refusing(x, ctx, view, rt, **more):
+        if ctx.host_new is None and not ctx.decode:  # (a prompt step from a graph's buffers brings no host lists)
+            raise KernelError("this part wants the host's view of the step")
+        return forward(x, ctx, view, rt, **more)
+
+    mixer.forward = refusing
+    try:
         kept = list(graphs)
         for _ in range(3):
             run([21, 40], [0, 0], [[0, 7, 8], [5, 6, 9]])
-        assert shape in engine._prefill_graphs.refused and list(graphs) == kept
+        (shape,) = [key for key in engine._prefill_graphs.refused if key[:3] == (2, 64, 6)]
+        assert list(graphs) == kept
+    finally:
+        mixer.forward = forward
     engine.end_sequence(other)
     assert engine.free_slots() == engine.cache.max_slots
 
@@ -501,7 +608,7 @@ def test_a_captured_step_keeps_the_scratch_it_was_captured_with(tmp_path):
     small = ops.decode_scratch_held(engine.rt.device)
     assert small is not None and small.numel() == 1 << 16
     graph = next(iter(engine._graphs.graphs.values()))
-    assert graph.scratch.data_ptr() == small.data_ptr()
+    assert [held.data_ptr() for held in graph.held] == [small.data_ptr()] * len(graph.held) and graph.held
 
     others = [engine.start_sequence() for _ in range(7)]
     engine.step([StepEntry(s, t[:1100], []) for s, t in zip(others, sequences[1:])])
@@ -512,7 +619,7 @@ def test_a_captured_step_keeps_the_scratch_it_was_captured_with(tmp_path):
     del small
     torch.cuda.synchronize()
     sentinels = [torch.full((1 << 16,), 7.0, device="cuda") for _ in range(6)]  # what would take a freed block of that size
-    assert all(s.data_ptr() != graph.scratch.data_ptr() for s in sentinels)
+    assert all(s.data_ptr() != graph.held[0].data_ptr() for s in sentinels)
 
     for slot in others[1:]:
         engine.end_sequence(slot)

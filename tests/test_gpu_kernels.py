@@ -505,6 +505,8 @@ def test_residual_projection_with_two_blocks_a_strip(m, n, k):
     product that cuts its K into parts (and fills the workspace they share) between them: each is right, and
     the strips' counts are back at zero."""
     ops = _ops()
+    assert ops.gemm_takes_pair(m, n, k)  # the kernel under test is the one that runs (and not at sizes beside its rule)
+    assert not ops.gemm_takes_pair(17, n, k) and not ops.gemm_takes_pair(m, n, 5056) and not ops.gemm_takes_pair(m, 2064, k)
     torch.manual_seed(m + n + k)
     gain = (1 + 0.3 * torch.randn(n)).bfloat16()
     other_x = torch.randn(64, 4096).bfloat16().cuda()
@@ -527,8 +529,8 @@ def test_residual_projection_with_two_blocks_a_strip(m, n, k):
         assert torch.equal(scaled.cpu(), (resid_gpu.cpu() * gain.float()).bfloat16())
         total = ss[:parts].cpu().double().sum(dim=0)
         assert ((total - got.pow(2).sum(dim=1)).abs() <= 1e-5 * got.pow(2).sum(dim=1)).all()
-        counts = ops._gemm_workspace(resid_gpu.device)[ops.GEMM_WORKSPACE_BYTES // 4:].view(torch.int32)
-        assert int(counts.abs().sum()) == 0
+        counts = ops.gemm_pair_counts(resid_gpu.device)
+        assert counts.numel() == ops.PAIR_COUNTS and int(counts.abs().sum()) == 0
 
 
 @pytest.mark.parametrize("tile", ["TILE_64x128", "TILE_64x64", "TILE_256x256", "TILE_256x192", "TILE_128x128", "TILE_256x128", "TILE_128x192"])
@@ -938,8 +940,11 @@ def test_refusals():
         ops.gemm_ordered(torch.zeros(3, 8), f(5, 8), f(3, 5))
     with pytest.raises(KernelError, match="float32 or bfloat16"):
         ops.gemm_ordered(f(3, 8, dtype=torch.float16), f(5, 8), f(3, 5))
-    with pytest.raises(KernelError, match="head_dim"):
-        ops.attention_module(7)
+    from nnis_amd.errors import Unsupported
+
+    for head_dim in (7, 258, 0):  # a size nobody runs: said as such (the model's check at load raises the same)
+        with pytest.raises(Unsupported, match="head_dim"):
+            ops.attention_module(head_dim)
     with pytest.raises(KernelError):
         ops.silu_mul(f(4, 11), f(4, 5))
     with pytest.raises(KernelError):

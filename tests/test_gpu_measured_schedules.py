@@ -86,7 +86,7 @@ def test_long_contexts(tmp_path_factory, shape, positions, length, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("shape, longest", [("smollm2-135m", 1024), ("tinyllama-1.1b", 1024), ("smollm2-1.7b", 256)])
+@pytest.mark.parametrize("shape, longest", [("smollm2-135m", 1024), ("tinyllama-1.1b", 1024), ("smollm2-1.7b", 256), ("llama-8b", 96)])
 def test_batches_of_64_unequal_prompts(tmp_path_factory, shape, longest, dtype):
     """64 prompts of 16 to ``longest`` tokens in one step, then 4 steps of one
     token each during which 8 sequences end; then a second batch of 64 in a
@@ -132,7 +132,7 @@ def test_batches_of_64_unequal_prompts(tmp_path_factory, shape, longest, dtype):
 
 
 @pytest.mark.parametrize("m", [1, 8, 64, 300])
-@pytest.mark.parametrize("n, k", [(49152, 576), (49152, 2048), (32000, 2048)])
+@pytest.mark.parametrize("n, k", [(49152, 576), (49152, 2048), (32000, 2048), (128256, 4096)])
 def test_the_head_at_real_vocabularies(m, n, k):
     """The head's product as every measured run launches it: whole-number
     operands, so a block that took another's rows or columns, or a strip of
@@ -142,7 +142,7 @@ def test_the_head_at_real_vocabularies(m, n, k):
     torch.manual_seed(m + k)
     x = torch.randint(-3, 4, (m, k)).to(torch.bfloat16)
     w = torch.randint(-3, 4, (n, k)).to(torch.bfloat16)
-    want = x.double() @ w.double().t()
+    want = (x.cuda().double() @ w.cuda().double().t()).cpu()  # whole numbers: exact in any order
     packed = ops.pack_weight(w.cuda())
     for dtype in (torch.float32, torch.bfloat16):
         y = torch.full((m, n), 7.0, dtype=dtype, device="cuda")

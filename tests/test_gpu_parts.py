@@ -141,7 +141,7 @@ def test_feed_forward_embedding_and_head_parts(dtype):
 # sequence, next to attention blocks; one layer runs twice, one reads another's cache
 # ---------------------------------------------------------------------------
 
-def _register_toy():
+def _register_toy(mixer_kind="running_mean", architecture="ToyForCausalLM"):
     from nnis_amd.config import register_architecture
     from nnis_amd.models import ModelSpec, ScheduleEntry
     from nnis_amd.parts import Mixer, StateRequest, TensorSpec, register_part
@@ -199,7 +199,7 @@ def _register_toy():
         for index in range(cfg.layers):
             p = f"blocks.{index}."
             if index % 2 == 0:
-                mixer = {"kind": "running_mean", "width": w, "weight": p + "mix"}
+                mixer = {"kind": mixer_kind, "width": w, "weight": p + "mix"}
             else:
                 mixer = {"kind": "causal_attention", "width": w, "heads": 2, "kv_heads": 1, "head_dim": 16,
                          "position": "rope", "q": p + "q", "k": p + "k", "v": p + "v", "o": p + "o"}
@@ -208,7 +208,7 @@ def _register_toy():
         # entry runs layer 1 again on the cache that entry 1 filled
         schedule = [ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(2), ScheduleEntry(0), ScheduleEntry(1, reads_cache_of=1)]
         return ModelSpec(
-            architecture="ToyForCausalLM", width=w, vocab_size=cfg.vocab_size, max_positions=256, stored_dtype="bfloat16",
+            architecture=architecture, width=w, vocab_size=cfg.vocab_size, max_positions=256, stored_dtype="bfloat16",
             embedding={"kind": "table", "vocab_size": cfg.vocab_size, "width": w, "weight": "emb"},
             positions={"rope": {"kind": "rotary_half", "rot_dim": 16, "theta": 1000.0, "max_positions": 256}},
             layers=layers, schedule=schedule,
@@ -217,7 +217,7 @@ def _register_toy():
             config_json=cfg.raw)
 
     register_part("mixer", "running_mean", RunningMean, replace=True)
-    register_architecture("ToyForCausalLM", ToyConfig, toy_spec, replace=True)
+    register_architecture(architecture, ToyConfig, toy_spec, replace=True)
 
 
 def _plain_toy(folder, ids):
@@ -286,6 +286,121 @@ def test_toy_architecture_with_a_stateful_mixer(tmp_path, dtype):
     assert again == sa
     rows = engine.step([StepEntry(again, b, list(range(13)))]).cpu()
     assert_close(rows, want_b, dtype, "toy reused slot")
+
+
+# ---------------------------------------------------------------------------
+# the same architecture with the running mean as a kernel of the test's own
+# (tests/toy_running_mean.hip, a kernel module that the test registers) that
+# reads the step from device memory and a work list that the mixer makes on
+# the host: steps of prompts and of single tokens are replayed from graphs,
+# with no word about this mixer, its list or its module in the library
+# ---------------------------------------------------------------------------
+
+def _register_kernel_toy():
+    import ctypes
+    import os
+
+    from nnis_amd.kernels import lib, ops
+    from nnis_amd.parts import Mixer, StateRequest, TensorSpec, register_part
+    from nnis_amd.parts.linear import Projection
+
+    lib.register_module("toy_mean", ["toy_running_mean.hip"], headers=["common.h"], directory=os.path.dirname(os.path.abspath(__file__)),
+                        replace=True)
+    # (common.h is the library's: found on the include path, hashed from the test's folder if a copy lay there)
+    void, integer = ctypes.c_void_p, ctypes.c_int
+    signatures = {"toy_running_mean": [void, void, void, void, void, void, void, integer, integer, integer, void]}
+
+    def rows_of_sequences(counts, first_positions, padded):
+        """The sequence of each row of a step of prompts; rows that belong to none name a sequence beyond the last."""
+        rows = padded[1] if padded is not None else sum(counts)
+        out = np.full(rows, len(counts) if padded is None else padded[0], dtype=np.int32)
+        at = 0
+        for index, count in enumerate(counts):
+            out[at:at + count] = index
+            at += count
+        return out
+
+    class RunningMeanKernel(Mixer):
+        graph_safe = True  # the kernel reads slots and positions from the step's device arrays
+        asked = []  # the plans the engine asked for
+
+        def __init__(self, width, weight):
+            self.width, self.weight_name, self.proj = width, weight, None
+
+        def tensors(self):
+            return [TensorSpec(self.weight_name, (self.width, self.width))]
+
+        def bind(self, weights, rt):
+            self.proj = Projection(weights[self.weight_name], rt)
+            self.lib = ops.bind("toy_mean", signatures)
+
+        def cache_request(self):
+            return StateRequest((self.width,), "float32")
+
+        def prompt_plan(self, batch, rows, longest, rt):
+            type(self).asked.append((batch, rows, longest))
+            return ("toy", rows > 64)  # (it launches the same way always; the plan only shows that it is asked and kept)
+
+        def forward(self, x, ctx, view, rt):
+            assert not view.read_only
+            x = x.float().contiguous()
+            y = torch.empty_like(x)
+            row_seq = None if ctx.decode else ctx.lists.device_list(("toy_rows",), rows_of_sequences)
+            ops.check(self.lib, self.lib.toy_running_mean(
+                x.data_ptr(), None if row_seq is None else row_seq.data_ptr(), ctx.seq_start.data_ptr(), ctx.seq_slot.data_ptr(),
+                ctx.tok_pos.data_ptr(), view.state.data_ptr(), y.data_ptr(), ctx.tokens, ctx.batch, self.width, ops.stream()))
+            return self.proj(y.to(rt.dtype), rt)
+
+    register_part("mixer", "running_mean_kernel", RunningMeanKernel, replace=True)
+    _register_toy("running_mean_kernel", "ToyKernelForCausalLM")
+    return RunningMeanKernel
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_toy_mixer_with_a_kernel_and_a_list_of_its_own_is_replayed_from_graphs(tmp_path, dtype):
+    import nnis_amd
+    from nnis_amd.api import load_engine
+    from nnis_amd.engine.batch import StepEntry
+
+    mixer_class = _register_kernel_toy()
+    folder = str(tmp_path / "toy")
+    raw = {"architectures": ["ToyKernelForCausalLM"], "model_type": "toy", "width": 48, "vocab_size": 211, "layers": 3}
+    nnis_amd.write_random_model(folder, raw, seed=4)
+    engine = load_engine(folder, dtype=dtype, max_tokens=2048)
+    assert engine.use_graphs
+    rng = np.random.default_rng(2)
+
+    def run(lengths, decode):
+        """Prompts of these lengths in one step (all their logits), then ``decode`` steps of one token each."""
+        sequences = [rng.integers(0, 211, size=n + decode).tolist() for n in lengths]
+        want = [_plain_toy(folder, ids) for ids in sequences]
+        slots = [engine.start_sequence() for _ in sequences]
+        rows = engine.step([StepEntry(s, ids[:n], list(range(n))) for s, ids, n in zip(slots, sequences, lengths)]).cpu()
+        at = 0
+        for w, n in zip(want, lengths):
+            assert_close(rows[at:at + n], w[:n], dtype, f"prompts of {lengths}")
+            at += n
+        for step in range(decode):
+            rows = engine.step([StepEntry(s, [ids[n + step]], [0]) for s, ids, n in zip(slots, sequences, lengths)]).cpu()
+            for j, (w, n) in enumerate(zip(want, lengths)):
+                assert_close(rows[j], w[n + step], dtype, f"decode step {step} after prompts of {lengths}")
+        for slot in slots:
+            engine.end_sequence(slot)
+
+    run([37, 5, 70], 3)  # launched
+    run([37, 5, 70], 0)  # from fixed buffers, captured
+    graphs = engine._prefill_graphs.graphs
+    (key,) = list(graphs)
+    assert key[:3] == (3, 128, 112) and "'toy', True" in repr(key[3])  # the toy's plan is part of the shape
+    graph = graphs[key]
+    assert ("toy_rows",) in graph.list_keys  # the toy's list lies in the graph's buffers, beside the attention's own
+    if dtype == "bfloat16":
+        assert any(k[0] == "attention_tiles" for k in graph.list_keys)
+    assert mixer_class.asked and mixer_class.asked[-1][:2] == (3, 128)
+    run([37, 5, 70], 2)  # replayed, in other slots' state rows than before
+    run([30, 42, 40], 2)  # the same shape, divided otherwise: the lists are made anew for it
+    run([70, 1, 41], 0)
+    assert list(graphs) == [key] and engine._graphs is not None and engine._graphs.graphs  # single tokens from graphs too
 
 
 # ---------------------------------------------------------------------------

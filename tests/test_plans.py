@@ -48,7 +48,11 @@ def test_prefill_plan_class_and_work_lists():
 
 
 def test_prefill_plan_by_class_and_size():
-    from nnis_amd.kernels.ops import prefill_plan, prefill_rows
+    from nnis_amd.engine.graph import prompt_rows as prefill_rows
+    from nnis_amd.kernels import ops
+
+    def prefill_plan(longest, rows, *sizes):
+        return ops.prefill_plan(longest, prefill_rows(rows), *sizes)  # (the engine plans for a step's rows rounded up)
 
     assert [prefill_rows(n) for n in (1, 64, 65, 1024, 1025, 2048, 2049, 4000)] == [64, 64, 128, 1024, 1152, 2048, 2304, 4096]
     for n in (1, 64, 100, 1000, 1100, 2000, 3000):

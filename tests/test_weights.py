@@ -91,14 +91,18 @@ def test_one_error_lists_everything(model_dirs, tmp_path):
     tensors.append(("model.layers.7.extra.weight", torch.zeros(2)))  # unexpected
     tensors.append(("model.layers.0.self_attn.rotary_emb.inv_freq", torch.zeros(16)))  # a known buffer: ignored
     write_safetensors(os.path.join(folder, "model.safetensors"), tensors)
+    spec = spec_from_config(TINY_B)[1]
+    assert spec.ignored_tensor_suffixes == ("rotary_emb.inv_freq",)  # the Llama description names it, not the loader
     with pytest.raises(WeightError) as info:
-        load_weights(folder, _specs(TINY_B), "cpu", widen_to_float32=False)
+        load_weights(folder, _specs(TINY_B), "cpu", widen_to_float32=False, ignored_suffixes=spec.ignored_tensor_suffixes)
     text = str(info.value)
     assert "missing tensors (1)" in text and "model.layers.1.mlp.up_proj.weight [256, 96]" in text
     assert "unexpected tensors (1)" in text and "model.layers.7.extra.weight" in text
     assert "wrong shapes (1)" in text and "expected [32, 96], file has [32, 95]" in text
     assert "wrong stored types (1)" in text and "F16" in text
     assert "inv_freq" not in text
+    with pytest.raises(WeightError, match=r"unexpected tensors \(2\)"):  # a model that does not name the buffer does not know it
+        load_weights(folder, _specs(TINY_B), "cpu", widen_to_float32=False)
 
 
 def test_untied_model_without_head_is_an_error(model_dirs, tmp_path):
