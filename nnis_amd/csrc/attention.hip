@@ -297,6 +297,94 @@ __device__ __forceinline__ void attend_block(AttnState<C>& st, const QFrag (&q)[
   }
 }
 
+// The same work with the matrix unit and the vector unit side by side.  A unit is one block's 32 keys for one
+// column tile: 2 * (HD / 32) matrix instructions for its scores, then the softmax's vector work on them (eight
+// maxima, eight exponentials, sums and conversions a lane: more cycles than the matrix instructions of the unit
+// take), then HD / 16 matrix instructions for the outputs.  One after the other the two units of the SIMD take
+// turns idling.  Here the scores of the unit that follows are asked for before the softmax of this one: `s` comes
+// in holding the scores of (f, column 0) and goes out holding those of (`next`, column 0), where AHEAD says that
+// `next` holds the block that follows.  The compiler's scheduler is told the order inside each stretch of
+// straight-line code (from one unit's exponentials to the next unit's test of its maximum): a score instruction
+// of the unit after next between every few of this unit's exponentials, then this unit's output instructions
+// between the next unit's maxima.  MASKED: keys are looked at one by one for the columns' lower and upper ends
+// (a block on the diagonal, at a window's edge, or a tile with rows or heads beyond the last); without it every
+// key of the block counts for every column.
+constexpr int kScoreMfmas = 2 * (kFullD + (kTailD ? 1 : 0));
+template <int C, bool MASKED, bool AHEAD>
+__device__ __forceinline__ void attend_block_ahead(AttnState<C>& st, const QFrag (&q)[C], const BlockFrags& f, const BlockFrags& next,
+                                                   f32x4 (&s)[2], int key0, const int (&lo)[C], const int (&hi)[C],
+                                                   float scale_log2, int g) {
+#pragma unroll
+  for (int c = 0; c < C; ++c) {
+    f32x4 ahead[2];
+    if (c + 1 < C) {
+#pragma unroll
+      for (int t = 0; t < 2; ++t) ahead[t] = score_tile(f.keys[t], q[c + 1]);
+    } else if (AHEAD) {
+#pragma unroll
+      for (int t = 0; t < 2; ++t) ahead[t] = score_tile(next.keys[t], q[0]);
+    }
+    if (MASKED) {
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int key = key0 + 8 * g + 4 * t + e;
+          s[t][e] = (key >= lo[c] && key <= hi[c]) ? s[t][e] : -INFINITY;
+        }
+    }
+    float block_max = -INFINITY;
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) block_max = fmaxf(block_max, s[t][e]);
+    block_max *= scale_log2;
+    // the stretch that ends here began behind the test of the unit before: its exponentials and output
+    // instructions, then this unit's score instructions for the next and its maxima
+    if (c + 1 < C || AHEAD) {
+#pragma unroll
+      for (int n = 0; n < kScoreMfmas; ++n) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, (36 + kScoreMfmas - 1) / kScoreMfmas, 0);
+      }
+    }
+#pragma unroll
+    for (int n = 0; n < kTilesD; ++n) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, kTilesD <= 4 ? 3 : 2, 0);
+    }
+    if (__any(block_max > st.m[c] + kLazyRise)) {  // (see attend_block)
+      float moved = fmaxf(st.m[c], block_max);
+      moved = fmaxf(moved, __shfl_xor(moved, 16, kWave));
+      moved = fmaxf(moved, __shfl_xor(moved, 32, kWave));
+      const float shrink = st.m[c] == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(st.m[c] - moved);
+      st.l[c] *= shrink;
+#pragma unroll
+      for (int t = 0; t < kTilesD; ++t) st.o[c][t] = st.o[c][t] * shrink;
+      st.m[c] = moved;
+    }
+    const float base = st.m[c] == -INFINITY ? 0.0f : st.m[c];
+    bf16x8 p;
+    float sum = 0.0f;
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float w = __builtin_amdgcn_exp2f(fmaf(s[t][e], scale_log2, -base));
+        sum += w;
+        p[4 * t + e] = (__bf16)w;
+      }
+    st.l[c] += sum;
+#pragma unroll
+    for (int t = 0; t < kTilesD; ++t)
+      st.o[c][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.values[t], p, st.o[c][t], 0, 0, 0);
+    if (c + 1 < C || AHEAD) {
+      s[0] = ahead[0];
+      s[1] = ahead[1];
+    }
+  }
+}
+
 // The pages of a run of key blocks, 64 at a time in the lanes of the wave: a
 // block's page is a lane broadcast, not a dependent load in front of every block.
 struct PageRun {
@@ -459,11 +547,38 @@ __device__ __forceinline__ void attend_run(AttnState<C>& st, const QFrag (&q)[C]
   if (blocks >= 2 * RING) {
 #pragma unroll
     for (int i = 0; i < RING; ++i) ask(ring[i], i);
+    // the ends between which every key counts for every column of every lane (a dead column has hi = -1: none)
+    int every_lo = lo[0], every_hi = hi[0];
+#pragma unroll
+    for (int c = 1; c < C; ++c) {
+      every_lo = max(every_lo, lo[c]);
+      every_hi = min(every_hi, hi[c]);
+    }
+#pragma unroll
+    for (int offset = kWave / 2; offset > 0; offset >>= 1) {
+      every_lo = max(every_lo, __shfl_xor(every_lo, offset, kWave));
+      every_hi = min(every_hi, __shfl_xor(every_hi, offset, kWave));
+    }
+    constexpr bool kAhead = RING > 1;  // (with one block in flight the next is asked for only when this one is done)
+    f32x4 s[2];
+    if (kAhead) {
+#pragma unroll
+      for (int t = 0; t < 2; ++t) s[t] = score_tile(ring[0].keys[t], q[0]);
+    }
     for (; b0 + 2 * RING <= blocks; b0 += RING) {
 #pragma unroll
       for (int i = 0; i < RING; ++i) {
-        work(ring[i], b0 + i);
-        ask(ring[i], b0 + i + RING);
+        const int b = b0 + i;
+        const int key0 = (first + (b >> 1) * stride) * kPageTokens + (b & 1) * 32;
+        if (!kAhead) {
+#pragma unroll
+          for (int t = 0; t < 2; ++t) s[t] = score_tile(ring[i].keys[t], q[0]);
+        }
+        if (key0 >= every_lo && key0 + 31 <= every_hi)
+          attend_block_ahead<C, false, kAhead>(st, q, ring[i], ring[(i + 1) % RING], s, key0, lo, hi, a.scale_log2, g);
+        else
+          attend_block_ahead<C, true, kAhead>(st, q, ring[i], ring[(i + 1) % RING], s, key0, lo, hi, a.scale_log2, g);
+        ask(ring[i], b + RING);
       }
     }
   } else {

@@ -72,6 +72,35 @@ class Bf16Yardstick:
         return 4.0 * self.worst
 
 
+class Fp32Yardstick:
+    """What 32-bit sums alone do to a wide model's logits: the plain model in
+    32-bit against the plain model in 64-bit.  The engine's 32-bit path sums
+    as the reference does, one ascending chain of fused multiply-adds per
+    output, where the plain model's library sums in blocks; a chain's
+    rounding grows with its length, so the engine is off by more than the
+    plain 32-bit model, by a factor that was measured at 2.0 for sums of up
+    to 1,536 terms (width 576), 3.2 up to 8,192 (width 2,048) and 3.8 up to
+    14,336 (width 4,096: worst logit 4.0e-5 against 1.0e-5, logits of 1.3 in
+    root mean square).  Up to a width of 2,048 the flat bound of the other
+    tests (2e-5 + 2e-5 |x|) is the tighter one and stays; beyond it the
+    engine may be off by ``FACTOR`` times the 32-bit twin, in the worst logit
+    and in root mean square.  A fault moves logits by their own size, four
+    orders of magnitude more."""
+
+    FACTOR = 6.0
+
+    def __init__(self, plain64, plain32, sequences):
+        error = torch.cat([(plain32.logits(list(ids)).double() - plain64.logits(list(ids)).double()).flatten() for ids in sequences])
+        self.rms, self.worst = float(error.pow(2).mean().sqrt()), float(error.abs().max())
+        assert 0 < self.worst < 1e-4, self.worst
+
+    def check(self, got, want, what=""):
+        error = (torch.as_tensor(np.asarray(got)).double() - torch.as_tensor(np.asarray(want)).double()).flatten()
+        worst, rms = float(error.abs().max()), float(error.pow(2).mean().sqrt())
+        assert worst <= self.FACTOR * self.worst, f"{what}: worst logit off by {worst:.3g}; the 32-bit twin's worst is {self.worst:.3g}"
+        assert rms <= self.FACTOR * self.rms, f"{what}: rms error {rms:.3g}; the 32-bit twin's is {self.rms:.3g}"
+
+
 def _bf16_round(x):
     return x.to(torch.bfloat16).to(x.dtype)
 

@@ -16,7 +16,7 @@ import torch
 
 import plain_llama as P
 from configs import SHAPE_CONFIGS
-from gpu_helpers import Bf16Yardstick
+from gpu_helpers import Bf16Yardstick, Fp32Yardstick
 
 pytestmark = pytest.mark.gpu
 
@@ -39,7 +39,7 @@ def _model(tmp_path_factory, shape, max_positions):
 
 def _check(got, want, dtype, yard, what):
     got, want = got.double().cpu(), want.double()
-    if dtype == "float32":
+    if dtype == "float32" and yard is None:
         error = (got - want).abs()
         bound = 2e-5 + 2e-5 * want.abs()
         assert bool((error <= bound).all()), f"{what}: max error {error.max().item():.3g}"
@@ -100,6 +100,8 @@ def test_batches_of_64_unequal_prompts(tmp_path_factory, shape, longest, dtype):
     first = [rng.integers(0, vocab, size=int(n) + 4).tolist() for n in rng.integers(16, longest + 1, size=64)]
     second = [rng.integers(0, vocab, size=int(n) + 2).tolist() for n in rng.integers(1, 130, size=64)]
     yard = Bf16Yardstick(plain, first[:3]) if dtype == "bfloat16" else None
+    if dtype == "float32" and SHAPE_CONFIGS[shape][0]["hidden_size"] > 2048:
+        yard = Fp32Yardstick(plain, P.PlainLlama(folder, torch.float32), first[:3])  # sums of 14,336 terms: see the yardstick
     pages = sum((len(t) + 63) // 64 for t in first)
     assert sum((len(t) + 63) // 64 for t in second) <= pages
     engine = load_engine(folder, dtype=dtype, max_tokens=pages * 64, max_slots=64)
