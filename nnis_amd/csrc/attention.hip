@@ -21,6 +21,9 @@
 #ifndef NNIS_PREFILL_RING_NARROW
 #define NNIS_PREFILL_RING_NARROW 3
 #endif
+#ifndef NNIS_AHEAD_VALU
+#define NNIS_AHEAD_VALU 36  // vector instructions of a unit's exponentials, between which the next unit's score instructions go
+#endif
 #ifndef NNIS_PREFILL_RING_WIDE
 #define NNIS_PREFILL_RING_WIDE 2
 #endif
@@ -297,92 +300,104 @@ __device__ __forceinline__ void attend_block(AttnState<C>& st, const QFrag (&q)[
   }
 }
 
-// The same work with the matrix unit and the vector unit side by side.  A unit is one block's 32 keys for one
-// column tile: 2 * (HD / 32) matrix instructions for its scores, then the softmax's vector work on them (eight
-// maxima, eight exponentials, sums and conversions a lane: more cycles than the matrix instructions of the unit
-// take), then HD / 16 matrix instructions for the outputs.  One after the other the two units of the SIMD take
-// turns idling.  Here the scores of the unit that follows are asked for before the softmax of this one: `s` comes
-// in holding the scores of (f, column 0) and goes out holding those of (`next`, column 0), where AHEAD says that
-// `next` holds the block that follows.  The compiler's scheduler is told the order inside each stretch of
-// straight-line code (from one unit's exponentials to the next unit's test of its maximum): a score instruction
-// of the unit after next between every few of this unit's exponentials, then this unit's output instructions
-// between the next unit's maxima.  MASKED: keys are looked at one by one for the columns' lower and upper ends
-// (a block on the diagonal, at a window's edge, or a tile with rows or heads beyond the last); without it every
-// key of the block counts for every column.
-constexpr int kScoreMfmas = 2 * (kFullD + (kTailD ? 1 : 0));
-template <int C, bool MASKED, bool AHEAD>
-__device__ __forceinline__ void attend_block_ahead(AttnState<C>& st, const QFrag (&q)[C], const BlockFrags& f, const BlockFrags& next,
-                                                   f32x4 (&s)[2], int key0, const int (&lo)[C], const int (&hi)[C],
-                                                   float scale_log2, int g) {
+// The same work with the matrix unit and the vector unit side by side, for blocks all of whose keys count for
+// every column (no key is looked at).  A unit is one block's 32 keys for one column tile: 2 * (HD / 32) matrix
+// instructions for its scores, then the softmax's vector work on them (eight exponentials of 16 cycles a wave
+// and some thirty other vector instructions of 4: about 250 cycles, where the unit's matrix instructions take
+// 16 each), then HD / 16 matrix instructions for the outputs.  A SIMD runs vector instructions while its
+// matrix unit works (a matrix instruction with eight independent multiply-adds behind it takes as long as
+// the eight alone), but a wave that meets a matrix instruction while the unit is busy stands there: left to
+// the compiler the matrix instructions come in runs of six and more and a unit takes about 360 cycles of a
+// SIMD with two waves on it.  So every matrix instruction here is one that needs nothing of the vector work
+// around it: the scores of the unit that follows (of the next column, or of the next block's first column: `s`
+// comes in holding the scores of (f, column 0) and goes out holding those of (`next`, column 0), where AHEAD
+// says that `next` holds the block that follows), and the outputs of the unit before, whose probabilities are
+// kept for that long; only a block's last column multiplies its own outputs at once (the values' registers are
+// asked for again behind the block).  The compiler's scheduler is told the order inside each stretch of
+// straight-line code, from behind one unit's test of its maximum to the next unit's: one of those matrix
+// instructions, a few vector instructions, and so on.
+template <int C, bool AHEAD, int c>
+__device__ __forceinline__ void attend_unit_ahead(AttnState<C>& st, const QFrag (&q)[C], const BlockFrags& f, const BlockFrags& next,
+                                                  f32x4 (&s)[2], bf16x8& before, float scale_log2) {
+  constexpr int kScores = 2 * (kFullD + (kTailD ? 1 : 0));
+  float block_max = -INFINITY;
 #pragma unroll
-  for (int c = 0; c < C; ++c) {
-    f32x4 ahead[2];
-    if (c + 1 < C) {
+  for (int t = 0; t < 2; ++t)
 #pragma unroll
-      for (int t = 0; t < 2; ++t) ahead[t] = score_tile(f.keys[t], q[c + 1]);
-    } else if (AHEAD) {
+    for (int e = 0; e < 4; ++e) block_max = fmaxf(block_max, s[t][e]);
+  block_max *= scale_log2;
+  {
+    // the stretch that ends here: the unit before this one (the block before's last column, for column 0)
+    constexpr int unit = c == 0 ? C - 1 : c - 1;
+    constexpr int free_ones = ((unit + 1 < C || AHEAD) ? kScores : 0) + (unit > 0 ? kTilesD : 0);
+    if constexpr (free_ones > 0) {
 #pragma unroll
-      for (int t = 0; t < 2; ++t) ahead[t] = score_tile(next.keys[t], q[0]);
-    }
-    if (MASKED) {
-#pragma unroll
-      for (int t = 0; t < 2; ++t)
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int key = key0 + 8 * g + 4 * t + e;
-          s[t][e] = (key >= lo[c] && key <= hi[c]) ? s[t][e] : -INFINITY;
-        }
-    }
-    float block_max = -INFINITY;
-#pragma unroll
-    for (int t = 0; t < 2; ++t)
-#pragma unroll
-      for (int e = 0; e < 4; ++e) block_max = fmaxf(block_max, s[t][e]);
-    block_max *= scale_log2;
-    // the stretch that ends here began behind the test of the unit before: its exponentials and output
-    // instructions, then this unit's score instructions for the next and its maxima
-    if (c + 1 < C || AHEAD) {
-#pragma unroll
-      for (int n = 0; n < kScoreMfmas; ++n) {
+      for (int n = 0; n < free_ones; ++n) {
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x002, (36 + kScoreMfmas - 1) / kScoreMfmas, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, (NNIS_AHEAD_VALU + free_ones - 1) / free_ones, 0);
       }
     }
+    if constexpr (unit == C - 1) {
 #pragma unroll
-    for (int n = 0; n < kTilesD; ++n) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x002, kTilesD <= 4 ? 3 : 2, 0);
-    }
-    if (__any(block_max > st.m[c] + kLazyRise)) {  // (see attend_block)
-      float moved = fmaxf(st.m[c], block_max);
-      moved = fmaxf(moved, __shfl_xor(moved, 16, kWave));
-      moved = fmaxf(moved, __shfl_xor(moved, 32, kWave));
-      const float shrink = st.m[c] == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(st.m[c] - moved);
-      st.l[c] *= shrink;
-#pragma unroll
-      for (int t = 0; t < kTilesD; ++t) st.o[c][t] = st.o[c][t] * shrink;
-      st.m[c] = moved;
-    }
-    const float base = st.m[c] == -INFINITY ? 0.0f : st.m[c];
-    bf16x8 p;
-    float sum = 0.0f;
-#pragma unroll
-    for (int t = 0; t < 2; ++t)
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const float w = __builtin_amdgcn_exp2f(fmaf(s[t][e], scale_log2, -base));
-        sum += w;
-        p[4 * t + e] = (__bf16)w;
+      for (int n = 0; n < kTilesD; ++n) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
       }
-    st.l[c] += sum;
-#pragma unroll
-    for (int t = 0; t < kTilesD; ++t)
-      st.o[c][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.values[t], p, st.o[c][t], 0, 0, 0);
-    if (c + 1 < C || AHEAD) {
-      s[0] = ahead[0];
-      s[1] = ahead[1];
     }
   }
+  if (__any(block_max > st.m[c] + kLazyRise)) {  // (see attend_block)
+    float moved = fmaxf(st.m[c], block_max);
+    moved = fmaxf(moved, __shfl_xor(moved, 16, kWave));
+    moved = fmaxf(moved, __shfl_xor(moved, 32, kWave));
+    const float shrink = st.m[c] == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(st.m[c] - moved);
+    st.l[c] *= shrink;
+#pragma unroll
+    for (int t = 0; t < kTilesD; ++t) st.o[c][t] = st.o[c][t] * shrink;
+    st.m[c] = moved;
+  }
+  f32x4 ahead[2];
+  if constexpr (c + 1 < C) {
+#pragma unroll
+    for (int t = 0; t < 2; ++t) ahead[t] = score_tile(f.keys[t], q[c + 1]);
+  } else if constexpr (AHEAD) {
+#pragma unroll
+    for (int t = 0; t < 2; ++t) ahead[t] = score_tile(next.keys[t], q[0]);
+  }
+  if constexpr (c > 0) {
+#pragma unroll
+    for (int t = 0; t < kTilesD; ++t)
+      st.o[c - 1][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.values[t], before, st.o[c - 1][t], 0, 0, 0);
+  }
+  const float base = st.m[c] == -INFINITY ? 0.0f : st.m[c];
+  bf16x8 p;
+  float sum = 0.0f;
+#pragma unroll
+  for (int t = 0; t < 2; ++t)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const float w = __builtin_amdgcn_exp2f(fmaf(s[t][e], scale_log2, -base));
+      sum += w;
+      p[4 * t + e] = (__bf16)w;
+    }
+  st.l[c] += sum;
+  if constexpr (c + 1 < C) {
+    before = p;
+  } else {
+#pragma unroll
+    for (int t = 0; t < kTilesD; ++t) st.o[c][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.values[t], p, st.o[c][t], 0, 0, 0);
+  }
+  if constexpr (c + 1 < C || AHEAD) {
+    s[0] = ahead[0];
+    s[1] = ahead[1];
+  }
+  if constexpr (c + 1 < C) attend_unit_ahead<C, AHEAD, c + 1>(st, q, f, next, s, before, scale_log2);
+}
+
+template <int C, bool AHEAD>
+__device__ __forceinline__ void attend_block_ahead(AttnState<C>& st, const QFrag (&q)[C], const BlockFrags& f, const BlockFrags& next,
+                                                   f32x4 (&s)[2], float scale_log2) {
+  bf16x8 before;  // the probabilities of the column before, whose outputs are still to be multiplied
+  attend_unit_ahead<C, AHEAD, 0>(st, q, f, next, s, before, scale_log2);
 }
 
 // The pages of a run of key blocks, 64 at a time in the lanes of the wave: a
@@ -547,45 +562,62 @@ __device__ __forceinline__ void attend_run(AttnState<C>& st, const QFrag (&q)[C]
   if (blocks >= 2 * RING) {
 #pragma unroll
     for (int i = 0; i < RING; ++i) ask(ring[i], i);
-    // the ends between which every key counts for every column of every lane (a dead column has hi = -1: none)
-    int every_lo = lo[0], every_hi = hi[0];
+  } else {
 #pragma unroll
-    for (int c = 1; c < C; ++c) {
-      every_lo = max(every_lo, lo[c]);
-      every_hi = min(every_hi, hi[c]);
-    }
+    for (int i = 0; i < RING; ++i)
+      if (i < blocks) ask(ring[i], i);
+  }
+  // The blocks all of whose keys count for every column of every lane lie together in the middle of the run (in
+  // a causal step without a window: at its start): pages n of the run with every_lo <= their keys <= every_hi.
+  // (A dead column has hi = -1: then there are none.)
+  int every_lo = lo[0], every_hi = hi[0];
 #pragma unroll
-    for (int offset = kWave / 2; offset > 0; offset >>= 1) {
-      every_lo = max(every_lo, __shfl_xor(every_lo, offset, kWave));
-      every_hi = min(every_hi, __shfl_xor(every_hi, offset, kWave));
+  for (int c = 1; c < C; ++c) {
+    every_lo = max(every_lo, lo[c]);
+    every_hi = min(every_hi, hi[c]);
+  }
+#pragma unroll
+  for (int offset = kWave / 2; offset > 0; offset >>= 1) {
+    every_lo = max(every_lo, __shfl_xor(every_lo, offset, kWave));
+    every_hi = min(every_hi, __shfl_xor(every_hi, offset, kWave));
+  }
+  const int whole_pages = (every_hi + 1) / kPageTokens;  // pages 0 .. whole_pages - 1 of the sequence end at or below every_hi
+  const int inner_end = whole_pages > first ? 2 * min(mine, (whole_pages - first + stride - 1) / stride) : 0;  // in blocks of the run
+  const int low_page = (every_lo + kPageTokens - 1) / kPageTokens;
+  int inner_begin = low_page > first ? 2 * ((low_page - first + stride - 1) / stride) : 0;
+  inner_begin = (inner_begin + RING - 1) / RING * RING;  // whole rounds of the ring
+  // blocks before them (a window's edge) one by one
+  for (; b0 < inner_begin && b0 < blocks; b0 += RING) {
+#pragma unroll
+    for (int i = 0; i < RING; ++i) {
+      const int b = b0 + i;
+      if (b < blocks) {
+        work(ring[i], b);
+        if (b + RING < blocks) ask(ring[i], b + RING);
+      }
     }
+  }
+  // whole rounds of them whose every block has a successor RING on: one straight line, nothing behind a branch
+  if (b0 + 2 * RING <= blocks && b0 + RING <= inner_end) {
     constexpr bool kAhead = RING > 1;  // (with one block in flight the next is asked for only when this one is done)
     f32x4 s[2];
     if (kAhead) {
 #pragma unroll
       for (int t = 0; t < 2; ++t) s[t] = score_tile(ring[0].keys[t], q[0]);
     }
-    for (; b0 + 2 * RING <= blocks; b0 += RING) {
+    for (; b0 + 2 * RING <= blocks && b0 + RING <= inner_end; b0 += RING) {
 #pragma unroll
       for (int i = 0; i < RING; ++i) {
-        const int b = b0 + i;
-        const int key0 = (first + (b >> 1) * stride) * kPageTokens + (b & 1) * 32;
         if (!kAhead) {
 #pragma unroll
           for (int t = 0; t < 2; ++t) s[t] = score_tile(ring[i].keys[t], q[0]);
         }
-        if (key0 >= every_lo && key0 + 31 <= every_hi)
-          attend_block_ahead<C, false, kAhead>(st, q, ring[i], ring[(i + 1) % RING], s, key0, lo, hi, a.scale_log2, g);
-        else
-          attend_block_ahead<C, true, kAhead>(st, q, ring[i], ring[(i + 1) % RING], s, key0, lo, hi, a.scale_log2, g);
-        ask(ring[i], b + RING);
+        attend_block_ahead<C, kAhead>(st, q, ring[i], ring[(i + 1) % RING], s, a.scale_log2);
+        ask(ring[i], b0 + i + RING);
       }
     }
-  } else {
-#pragma unroll
-    for (int i = 0; i < RING; ++i)
-      if (i < blocks) ask(ring[i], i);
   }
+  // what is left (the diagonal, a short run) one by one
   for (; b0 < blocks; b0 += RING) {
 #pragma unroll
     for (int i = 0; i < RING; ++i) {
@@ -718,12 +750,12 @@ __global__ __launch_bounds__(64 * kBlockWaves) void attention_prefill_kernel(Mfm
       const int rows_here = min(row0_of[which] + 16 * QT, rows_of[which]);
       pages_of[which] = (pos0_of[which] + rows_here - 1) / kPageTokens + 1;
     }
-    // even shares (their merges then need waves / 2 states of room together), at least 2 waves each; of 2 waves, 1 each
-    int first_share = 1;
-    if (waves >= 4) {
-      first_share = 2 * ((waves * pages_of[0] + pages_of[0] + pages_of[1]) / (2 * (pages_of[0] + pages_of[1])));
-      first_share = first_share < 2 ? 2 : (first_share > waves - 2 ? waves - 2 : first_share);
-    }
+    // shares in proportion to the pages, at least one wave each (a group of n waves needs n / 2 states of room, rounded
+    // down, for its merge: the two groups' rooms lie behind one another and come to at most waves / 2 together).  With
+    // even shares only, four waves went 2 + 2 whatever the pages: 30 pages beside 3 were 15 a wave where 3 + 1 give 10.
+    const int all_pages = pages_of[0] + pages_of[1];
+    int first_share = (2 * waves * pages_of[0] + all_pages) / (2 * all_pages);
+    first_share = first_share < 1 ? 1 : (first_share > waves - 1 ? waves - 1 : first_share);
     if (wave < first_share) run_item(0, wave, first_share, merge, rounds);
     else run_item(1, wave - first_share, waves - first_share, merge + (size_t)(first_share / 2) * C * kStateFloats, rounds);
   }

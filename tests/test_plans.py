@@ -70,8 +70,8 @@ def test_prefill_plan_by_class_and_size():
     # half of that: one wave an item of two columns, where two divide the group
     assert prefill_plan(4096, 4096, 32) == (1, 2) and prefill_plan(2048, 2048, 64, 64, 8) == (1, 2) and prefill_plan(4096, 4096, 36, 64, 12) == (8, 0)
     assert prefill_plan(2048, 2048, 32) == (4, 0)
-    assert prefill_plan(2048, 2048, 32, 128) == (1, 0) and prefill_plan(2048, 2048, 16, 128) == (8, 0)
+    assert prefill_plan(4096, 4096, 32, 128) == (1, 0) and prefill_plan(2048, 2048, 32, 128) == (8, 0) and prefill_plan(2048, 2048, 16, 128) == (8, 0)
     assert prefill_plan(600, 34000, 32) == (1, 0) and prefill_plan(1024, 1024, 32, 256) == (1, 0) and prefill_plan(1024, 1024, 32, 128) == (4, 2)
     # a group of 3 heads: items of three columns (no two-column plans), one wave an item from twice the chip's waves of them
     assert prefill_plan(8192, 8192, 24, 64, 8) == (1, 0) and prefill_plan(1216, 1216, 24, 64, 8) == (4, 0)
-    assert prefill_plan(3072, 3072, 32, 64, 32) == (1, 2)
+    assert prefill_plan(3072, 3072, 32, 64, 32) == (4, 0)
