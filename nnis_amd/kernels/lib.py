@@ -64,6 +64,7 @@ class ModuleRecipe:
     defines: Tuple[Tuple[str, str], ...] = ()
     source_flags: Tuple[Tuple[str, Tuple[str, ...]], ...] = ()
     directory: str = CSRC
+    host_only: bool = False  # plain C++ for the host compiler: no device code, no GPU needed to run it
 
     def flags_of(self, source: str) -> List[str]:
         return [flag for name, flags in self.source_flags if name == source for flag in flags]
@@ -74,7 +75,8 @@ _families: Dict[str, Callable[[str], ModuleRecipe]] = {}  # by prefix: the rest 
 
 
 def register_module(name: str, sources: Sequence[str], headers: Sequence[str] = (), defines: Optional[Dict[str, str]] = None,
-                    source_flags: Optional[Dict[str, Sequence[str]]] = None, directory: str = CSRC, replace: bool = False) -> None:
+                    source_flags: Optional[Dict[str, Sequence[str]]] = None, directory: str = CSRC, replace: bool = False,
+                    host_only: bool = False) -> None:
     """Makes ``load_module(name)`` build and load a library from ``sources``
     under ``directory`` (every flag of the library's own kernels applies; the
     library's headers are on the include path).  A part that brings kernels
@@ -85,7 +87,7 @@ def register_module(name: str, sources: Sequence[str], headers: Sequence[str] = 
     if name in _modules and not replace:
         raise KernelError(f"kernel module {name!r} is registered already")
     _modules[name] = ModuleRecipe(tuple(sources), tuple(headers), tuple(sorted((defines or {}).items())),
-                                  tuple(sorted((k, tuple(v)) for k, v in (source_flags or {}).items())), directory)
+                                  tuple(sorted((k, tuple(v)) for k, v in (source_flags or {}).items())), directory, host_only)
 
 
 def register_module_family(prefix: str, recipe: Callable[[str], ModuleRecipe], replace: bool = False) -> None:
@@ -107,6 +109,9 @@ def _attention_recipe(rest: str) -> ModuleRecipe:
 register_module("core", ["elementwise.hip", "gemm.hip", "gemm_mfma.hip", "gemm_fused.hip", "sampling.hip"],
                 headers=["common.h", "epilogue.h", "nnis_noalloc.h"], source_flags={"gemm_mfma.hip": _VECTOR_SUMS})
 register_module_family("attn_hd", _attention_recipe)
+# plain host references of the kernels' operations, for the tests (no device code: the host compiler builds them)
+register_module("reference", ["reference.cpp"], host_only=True)
+HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-ffp-contract=off"]  # a multiply-add is fused only where the source says fmaf
 
 
 def _say(message: str) -> None:
@@ -132,7 +137,7 @@ def _module_hash(recipe: ModuleRecipe) -> str:
         with open(path, "rb") as handle:
             digest.update(name.encode())
             digest.update(handle.read())
-    digest.update(" ".join(FLAGS).encode())
+    digest.update(" ".join(HOST_FLAGS if recipe.host_only else FLAGS).encode())
     digest.update(repr(sorted((name, list(flags)) for name, flags in recipe.source_flags if name in recipe.sources)).encode())
     digest.update(repr(sorted(recipe.defines)).encode())
     return digest.hexdigest()[:12]
@@ -165,12 +170,19 @@ def _hipcc() -> str:
     raise KernelError("hipcc was not found (PATH, $HIPCC, /opt/rocm/bin): the HIP kernels cannot be built")
 
 
+def _host_compiler() -> str:
+    for candidate in (os.environ.get("CXX"), shutil.which("g++"), shutil.which("c++"), shutil.which("clang++")):
+        if candidate and (os.path.isabs(candidate) and os.path.exists(candidate) or shutil.which(candidate)):
+            return shutil.which(candidate) or candidate
+    raise KernelError("no host C++ compiler was found (CXX, g++, c++, clang++): the plain references cannot be built")
+
+
 def _run_with_heartbeat(commands: List[Tuple[str, List[str]]], env: Dict[str, str]) -> None:
     """Runs the commands in parallel, printing a line when each starts and
     ends and one every 20 s in between."""
     running = []
     for label, command in commands:
-        _say(f"compiling {label} for {ARCH} ...")
+        _say(f"compiling {label} ...")
         running.append((label, subprocess.Popen(command, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, env=env)))
     started = time.time()
     last = started
@@ -206,7 +218,8 @@ def build_module(module: str, force: bool = False) -> str:
         found = find_built(module)
         if found:
             return found
-    hipcc = _hipcc()
+    hipcc = _host_compiler() if recipe.host_only else _hipcc()
+    base_flags = HOST_FLAGS if recipe.host_only else FLAGS
     try:
         os.makedirs(LIB_DIR, exist_ok=True)
         probe = tempfile.NamedTemporaryFile(dir=LIB_DIR, delete=True)
@@ -226,12 +239,13 @@ def build_module(module: str, force: bool = False) -> str:
             obj = os.path.join(work, source + ".o")
             objects.append(obj)
             commands.append(
-                (f"{source} [{module}]", [hipcc] + FLAGS + recipe.flags_of(source) + define_flags
+                (f"{source} [{module}] for {'the host' if recipe.host_only else ARCH}", [hipcc] + base_flags + recipe.flags_of(source) + define_flags
                  + ["-I", recipe.directory, "-I", CSRC, "-c", os.path.join(recipe.directory, source), "-o", obj])
             )
         _run_with_heartbeat(commands, env)
         tmp_out = os.path.join(work, name)
-        _run_with_heartbeat([(f"link {module}", [hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", tmp_out] + objects)], env)
+        link = [hipcc, "-shared", "-fPIC", "-o", tmp_out] if recipe.host_only else [hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", tmp_out]
+        _run_with_heartbeat([(f"link {module}", link + objects)], env)
         final = os.path.join(out_dir, name)
         shutil.move(tmp_out, final)
         # older builds of the same module are of no use any more
@@ -268,7 +282,7 @@ def load_module(module: str, build_if_missing: bool = True) -> ctypes.CDLL:
 
 
 def all_prebuilt_modules() -> List[str]:
-    return ["core"] + [f"attn_hd{d}" for d in PREBUILT_HEAD_DIMS]
+    return ["core", "reference"] + [f"attn_hd{d}" for d in PREBUILT_HEAD_DIMS]
 
 
 def build_all(force: bool = True, jobs: int = 4) -> List[str]:

@@ -348,7 +348,13 @@ def step_tables(tok_slot: torch.Tensor, tok_pos: torch.Tensor, tokens: int, cos:
                 sequence_pages: bool = False) -> StepTables:
     """One kernel at the start of a step; see ``StepTables``.  ``cos`` / ``sin``:
     rotation tables [positions, half]; ``block_table``: int32 [slots, pages];
-    ``sequence_pages``: also each token's sequence's pages (a decode step)."""
+    ``sequence_pages``: also each token's sequence's pages (a decode step).
+    The positions live on the device, where nothing can refuse them: the
+    caller sees to it that every position is below ``cos.shape[0]`` and
+    below ``block_table.shape[1] * 64`` (the engine refuses a step beyond the
+    model's positions before it launches anything, and its tables reach that
+    far); the kernel's clamps of a position beyond either are a guard against
+    reading out of bounds, not a result."""
     _dev(tok_slot, "tok_slot"), _dev(tok_pos, "tok_pos")
     if tok_slot.dtype != torch.int32 or tok_pos.dtype != torch.int32 or min(tok_slot.numel(), tok_pos.numel()) < tokens:
         raise KernelError("step_tables: tok_slot / tok_pos must be int32 with one entry per token")
@@ -798,30 +804,31 @@ class KeyRuns:
 
 
 _DECODE_KERNELS = {"auto": 0, "columns": 1, "keys": 2}
-_decode_scratch = {}  # per device: every scratch made so far, the largest last
+_decode_scratch = {}  # per device: the scratch in use
 
 
 def decode_scratch(device, floats: int) -> torch.Tensor:
     """Scratch of the split decode attention, kept per device.  Calls on one
     device share it, so they must follow one another on one stream.  A call
     that needs more gets a larger tensor, made outside a graph capture only
-    (the run that warms a graph up sizes it); the smaller ones are kept until
-    the process ends, because a captured graph has the address it was captured
-    with baked in and goes on writing there on every replay.  (A graph also
-    holds the tensor it captured: ``engine/graph.py``.)"""
+    (the run that warms a graph up sizes it), and the smaller one is let go:
+    kernels already on the stream are ahead of whoever gets its memory next,
+    and a captured graph, which has the address it was captured with baked in
+    and goes on writing there on every replay, holds the tensor itself for as
+    long as it lives (``Part.held_buffers``, ``engine/graph.py``)."""
     key = (device.type, device.index)
-    held = _decode_scratch.setdefault(key, [])
-    if not held or held[-1].numel() < floats:
+    held = _decode_scratch.get(key)
+    if held is None or held.numel() < floats:
         if torch.cuda.is_current_stream_capturing():
             raise KernelError("attention: the decode scratch would have to grow inside a graph capture")
-        held.append(torch.empty(max(floats, 2 * held[-1].numel() if held else 1 << 16), dtype=torch.float32, device=device))
-    return held[-1]
+        held = _decode_scratch[key] = torch.empty(max(floats, 2 * held.numel() if held is not None else 1 << 16),
+                                                   dtype=torch.float32, device=device)
+    return held
 
 
 def decode_scratch_held(device):
     """The scratch a decode attention launched now would use (None: none made yet)."""
-    held = _decode_scratch.get((device.type, device.index))
-    return held[-1] if held else None
+    return _decode_scratch.get((device.type, device.index))
 
 
 def decode_max_waves(heads: int, kv_heads: int, head_dim: int) -> int:
