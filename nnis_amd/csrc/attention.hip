@@ -753,9 +753,16 @@ __global__ __launch_bounds__(64 * kBlockWaves) void attention_prefill_kernel(Mfm
     // shares in proportion to the pages, at least one wave each (a group of n waves needs n / 2 states of room, rounded
     // down, for its merge: the two groups' rooms lie behind one another and come to at most waves / 2 together).  With
     // even shares only, four waves went 2 + 2 whatever the pages: 30 pages beside 3 were 15 a wave where 3 + 1 give 10.
-    const int all_pages = pages_of[0] + pages_of[1];
-    int first_share = (2 * waves * pages_of[0] + all_pages) / (2 * all_pages);
-    first_share = first_share < 1 ? 1 : (first_share > waves - 1 ? waves - 1 : first_share);
+    // The shares that leave the busiest wave the fewest pages (in proportion to the pages, 21 beside 12 went 3 + 1:
+    // 12 pages on the light item's one wave where 2 + 2 give 11 and 6).
+    int first_share = 1, fewest = 0x7fffffff;
+    for (int share = 1; share < waves; ++share) {
+      const int most = max((pages_of[0] + share - 1) / share, (pages_of[1] + waves - share - 1) / (waves - share));
+      if (most < fewest) {
+        fewest = most;
+        first_share = share;
+      }
+    }
     if (wave < first_share) run_item(0, wave, first_share, merge, rounds);
     else run_item(1, wave - first_share, waves - first_share, merge + (size_t)(first_share / 2) * C * kStateFloats, rounds);
   }
