@@ -1341,7 +1341,9 @@ extern "C" int nnis_gemm_takes_pair(int m, int n, int k, size_t workspace_bytes)
 // nnis_gemm_residual_parts(m, n) are always enough.
 extern "C" int nnis_gemm_residual_parts(int m, int n) {
   (void)m;
-  return (n + 15) / 16;  // the kernel for few tokens: a part per strip of 16 columns; the tiled one uses fewer
+  // the kernel for few tokens: a part per strip of 16 columns; the tiled one a part per wave column of its tiles,
+  // which is fewer from 17 columns on and two for a single tile
+  return n > 16 ? (n + 15) / 16 : 2;
 }
 
 extern "C" int nnis_gemm_residual(const void* x, const void* w, float* resid, const void* gain, int gain_dtype, void* scaled,

@@ -860,6 +860,9 @@ AWKWARD = {
     # a width of 36 and a vocabulary of 61: smaller than any tile
     "width 36": dict(num_hidden_layers=1, hidden_size=36, num_attention_heads=3, num_key_value_heads=3, head_dim=16, intermediate_size=52,
                      vocab_size=61, tie_word_embeddings=True),
+    # a width of 16: one strip of the stream's projections, which the tiled product still gives two parts of a row's sum of squares
+    "width 16": dict(num_hidden_layers=2, hidden_size=16, num_attention_heads=2, num_key_value_heads=2, head_dim=16, intermediate_size=240,
+                     vocab_size=237, tie_word_embeddings=False),
     # heads of 192 channels: beyond what the decode kernel with keys on lanes takes
     "heads of 192": dict(num_hidden_layers=2, hidden_size=192, num_attention_heads=2, num_key_value_heads=1, head_dim=192, intermediate_size=264,
                          vocab_size=333, tie_word_embeddings=True),
