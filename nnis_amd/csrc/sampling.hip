@@ -344,7 +344,10 @@ __global__ __launch_bounds__(kSampleThreads) void sample_kernel(
   }
 
   const float p = top_p[at];
-  if (p > 0.0f && p <= 1.0f) {
+  // (A top_p of 1 keeps every candidate: the running sum reaches the whole weight at the last one that adds to it,
+  // and what lies behind that one has no weight to be drawn with.  It must not go through the search: sums of the
+  // same weights in another order may stay a rounding below the whole, and the search then finds no cut at all.)
+  if (p > 0.0f && p < 1.0f) {
     const double threshold = (double)p * total;
     const unsigned t = find_cut([&](double mass) { return mass >= threshold; });
     // t >= cut_key when limited, because the whole kept mass reaches the threshold

@@ -503,7 +503,8 @@ def test_command_line_with_text(model_dirs, tmp_path):
 
 
 @pytest.mark.parametrize("options", [dict(), dict(temperature=0.8), dict(top_k=40), dict(top_p=0.7),
-                                     dict(temperature=1.3, top_k=200, top_p=0.95), dict(top_k=1)])
+                                     dict(temperature=1.3, top_k=200, top_p=0.95), dict(top_k=1), dict(top_p=1.0),
+                                     dict(temperature=0.05, top_p=1.0)])
 @pytest.mark.parametrize("vocab", [1000, 5003, 20011, 49152, 70001])
 def test_device_sampling_matches_the_host_sampler(options, vocab):
     """Same logits, same seeds: the kernel picks what the reference's host
