@@ -875,12 +875,35 @@ AWKWARD = {
 def test_awkward_sizes(tmp_path, case, dtype):
     """Sizes that no kernel's tiles divide: three prompts of unequal length in one step and six tokens each one by
     one, every logit against the plain model."""
+    _prompts_and_tokens_agree(tmp_path, AWKWARD[case], case, dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_sizes_drawn_from_a_seed(tmp_path, dtype):
+    """The same at thirty configurations whose every size is drawn from a seed: one to three layers, heads of 16 to
+    256 channels in groups of one to eight, widths, inner sizes and vocabularies of any number (a width below a
+    strip of 16, a vocabulary of two), a head tied or of its own."""
+    import random
+
+    rng = random.Random(20)
+    for number in range(30):
+        head_dim = rng.choice([16, 16, 32, 32, 48, 64, 64, 80, 96, 112, 128, 192, 256])
+        kv_heads = rng.choice([1, 1, 2, 3, 4])
+        group = rng.choice([1, 1, 2, 3, 4, 5, 8]) if head_dim <= 128 else rng.choice([1, 2])
+        sizes = dict(num_hidden_layers=rng.randint(1, 3), hidden_size=rng.choice([rng.randint(9, 300), 8 * rng.randint(2, 60), 64 * rng.randint(1, 8)]),
+                     num_attention_heads=kv_heads * group, num_key_value_heads=kv_heads, head_dim=head_dim,
+                     intermediate_size=rng.choice([rng.randint(4, 500), 8 * rng.randint(1, 80)]),
+                     vocab_size=rng.choice([rng.randint(2, 3000), 64 * rng.randint(1, 40)]), tie_word_embeddings=rng.random() < 0.5)
+        _prompts_and_tokens_agree(tmp_path / str(number), sizes, f"drawn configuration {number} {sizes}", dtype)
+
+
+def _prompts_and_tokens_agree(tmp_path, sizes, case, dtype):
     import nnis_amd
     from configs import llama
     from nnis_amd.api import load_engine
     from nnis_amd.engine.batch import StepEntry
 
-    config = llama(rope_theta=10000.0, rms_norm_eps=1e-5, max_position_embeddings=256, torch_dtype="bfloat16", **AWKWARD[case])
+    config = llama(rope_theta=10000.0, rms_norm_eps=1e-5, max_position_embeddings=256, torch_dtype="bfloat16", **sizes)
     folder = str(tmp_path / "model")
     os.makedirs(folder)
     nnis_amd.write_random_model(folder, config, 3)
