@@ -361,3 +361,78 @@ def test_a_row_is_not_rewritten_before_its_copy_has_left():
     assert (event.recorded, event.waited) == (3, 2)
     cache.grow_by_one([b])  # inside its page
     assert (event.recorded, event.waited) == (3, 2)
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_operations_drawn_from_a_seed(seed):
+    """Four hundred operations in an order drawn from the seed -- sequences start, grow by prompts and by single
+    tokens (checked first, all or nothing), are cut back, reset, rolled back and ended -- against a model of the
+    lengths kept here.  After each one: every group holds exactly the pages its lengths need, no page twice, the
+    rows that the kernels read name them, and what is free and what is held add up."""
+    rng = random.Random(seed)
+    cache = _cache(max_tokens=10 * 64)
+    lengths = {}
+
+    def check():
+        assert {s: cache.length(s) for s in lengths} == lengths and set(cache.slots.held) == set(lengths)
+        assert cache.live_tokens() == sum(lengths.values())
+        for group in cache.kv_groups:
+            seen = []
+            for slot, n in lengths.items():
+                row = group.table.rows.get(slot, [])
+                assert len(row) == pages_for(n)
+                assert group.block_table_host[slot, :len(row)].tolist() == row
+                seen += row
+            assert len(seen) == len(set(seen)) and set(seen) == set(group.table.pool.held)
+            assert group.table.pool.free + len(seen) == 10
+
+    for _ in range(400):
+        action = rng.random()
+        if not lengths or (action < 0.12 and len(lengths) < cache.max_slots):
+            lengths[cache.acquire()] = 0
+        elif action < 0.2:
+            slot = rng.choice(sorted(lengths))
+            cache.release(slot)
+            del lengths[slot]
+        elif action < 0.3:
+            slot = rng.choice(sorted(lengths))
+            keep = rng.randint(0, lengths[slot])
+            cache.truncate(slot, keep)
+            lengths[slot] = keep
+        elif action < 0.35:
+            slot = rng.choice(sorted(lengths))
+            cache.reset(slot)
+            lengths[slot] = 0
+        elif action < 0.65:  # prompts: some sequences grow by any number of tokens, together or not at all
+            some = [s for s in sorted(lengths) if rng.random() < 0.6] or [rng.choice(sorted(lengths))]
+            growth = {s: rng.choice([1, 2, 63, 64, 65, rng.randint(1, 200)]) for s in some}
+            fits = (all(lengths[s] + n <= 300 for s, n in growth.items())
+                    and sum(pages_for(lengths[s] + n) - pages_for(lengths[s]) for s, n in growth.items()) <= cache.kv_groups[0].table.pool.free)
+            before = dict(lengths)
+            try:
+                cache.check_room(growth)
+                cache.grow(growth)
+                assert fits
+                for s, n in growth.items():
+                    lengths[s] += n
+                if rng.random() < 0.2:  # the step failed in flight: everything goes back
+                    cache.roll_back(before)
+                    lengths = before
+            except (CacheFull, InvalidInput):
+                assert not fits
+        else:  # one token each
+            some = [s for s in sorted(lengths) if rng.random() < 0.7] or [rng.choice(sorted(lengths))]
+            fits = (all(lengths[s] + 1 <= 300 for s in some)
+                    and sum(1 for s in some if lengths[s] % 64 == 0) <= cache.kv_groups[0].table.pool.free)
+            try:
+                checked = cache.check_one_more(some)
+                assert fits
+                assert cache.grow_by_one(some, checked if rng.random() < 0.5 else None) == [lengths[s] for s in some]
+                for s in some:
+                    lengths[s] += 1
+            except (CacheFull, InvalidInput):
+                assert not fits
+        check()
+    for slot in list(lengths):
+        cache.release(slot)
+    assert all(g.table.pool.free == 10 and not g.table.pool.held for g in cache.kv_groups) and not cache.slots.held
