@@ -25,7 +25,7 @@ For the SmolLM2 shapes there are further points at long contexts: decode at
 batch 8 and 64 over prompts of 7,800 to 8,000 tokens (``*_ctx8k``) and a prompt
 of 8,192 tokens in one step (``*_prefill_8192``).  A decode point is the
 median of three windows of K steps, one after the other on the same batch; a
-prefill figure is the median of three runs of a shape seen before.
+prefill figure is the median of seven runs of a shape seen before.
 ``--workload tinyllama-ragged`` runs that workload alone.
 
 Peaks used for the fractions are the published MI355X ones: HBM 8 TB/s; dense
@@ -196,7 +196,7 @@ def prefill_run(shape, rng, tokens=2048):
     engine.step([StepEntry(slot, warm, None)])  # another shape: kernels loaded, buffers made
     engine.end_sequence(slot)
     times = []
-    for _ in range(6):
+    for _ in range(10):
         slot = engine.start_sequence()
         torch.cuda.synchronize()
         start = time.perf_counter()
@@ -206,7 +206,7 @@ def prefill_run(shape, rng, tokens=2048):
         engine.end_sequence(slot)
     del engine
     torch.cuda.empty_cache()
-    seconds = sorted(times[3:])[1]  # the median of three runs of a shape that has come before (and is captured, where it is)
+    seconds = sorted(times[3:])[3]  # the median of seven runs of a shape that has come before (and is captured, where it is)
     flops = step_flops(shape.config, [tokens], 1)
     return {"value": round(tokens / seconds, 1), "tokens": tokens, "ms": round(1000.0 * seconds, 3),
             "frac": round(flops / seconds / FLOP_PEAK[shape.dtype], 5), "first_ms": round(1000.0 * times[0], 3)}
