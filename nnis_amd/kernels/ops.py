@@ -942,13 +942,25 @@ def prefill_plan_class(longest: int) -> int:
 PREFILL_CLASS_LENGTH = (1, 128, 512, 1024, 1280)  # a length of each class
 
 
+def _prefill_tile_arrays(new_tokens, first_positions, rows: int):
+    """``prefill_tile_items`` as two int64 arrays (a step of thousands of tokens has hundreds of tiles: arrays,
+    not a loop, while the GPU waits for the host)."""
+    import numpy as np
+
+    counts, pos0 = np.asarray(new_tokens, dtype=np.int64), np.asarray(first_positions, dtype=np.int64)
+    tiles = (counts + rows - 1) // rows  # of each sequence
+    seq = np.repeat(np.arange(counts.size, dtype=np.int64), tiles)
+    row0 = (np.arange(int(tiles.sum()), dtype=np.int64) - np.repeat(np.cumsum(tiles) - tiles, tiles)) * rows
+    last_key = pos0[seq] + np.minimum(row0 + rows, counts[seq])  # one beyond the last key that the tile's last row reads
+    order = np.lexsort((-row0, -seq, -last_key))  # most keys first; among equals the later sequence, the later row
+    return seq[order], row0[order]
+
+
 def prefill_tile_items(new_tokens, first_positions, rows: int):
     """Work items (sequence of the step, first row) of a prefill step for tiles of ``rows`` query rows: those
     with the most keys first."""
-    items = [(pos0 + min(row0 + rows, count), seq, row0)
-             for seq, (count, pos0) in enumerate(zip(new_tokens, first_positions)) for row0 in range(0, count, rows)]
-    items.sort(reverse=True)
-    return [seq for _, seq, _ in items], [row0 for _, _, row0 in items]
+    seq, row0 = _prefill_tile_arrays(new_tokens, first_positions, rows)
+    return seq.tolist(), row0.tolist()
 
 
 NO_ROWS = 1 << 24  # first row of a work item that has none: it lies beyond any sequence's tokens
@@ -961,7 +973,7 @@ def prefill_tile_list(new_tokens, first_positions, padded, rows: int):
     (rows of the step / rows of a tile + sequences), those beyond the step's own with no rows."""
     import numpy as np
 
-    seqs, row0s = prefill_tile_items(new_tokens, first_positions, rows)
+    seqs, row0s = _prefill_tile_arrays(new_tokens, first_positions, rows)
     count = len(seqs)
     if padded is not None:
         count = padded[1] // rows + padded[0]
