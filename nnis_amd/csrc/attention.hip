@@ -318,14 +318,15 @@ __device__ __forceinline__ void attend_block(AttnState<C>& st, const QFrag (&q)[
 // instructions, a few vector instructions, and so on.
 template <int C, bool AHEAD, int c>
 __device__ __forceinline__ void attend_unit_ahead(AttnState<C>& st, const QFrag (&q)[C], const BlockFrags& f, const BlockFrags& next,
-                                                  f32x4 (&s)[2], bf16x8& before, float scale_log2) {
+                                                  f32x4 (&s)[2], bf16x8& before, float scale_log2, float (&rise)[C]) {
   constexpr int kScores = 2 * (kFullD + (kTailD ? 1 : 0));
+  // rise[c]: the raw score (before the scale) above which column c's reference moves, (st.m[c] + kLazyRise) / scale:
+  // the test of every unit is then the scores' maximum against a register
   float block_max = -INFINITY;
 #pragma unroll
   for (int t = 0; t < 2; ++t)
 #pragma unroll
     for (int e = 0; e < 4; ++e) block_max = fmaxf(block_max, s[t][e]);
-  block_max *= scale_log2;
   {
     // the stretch that ends here: the unit before this one (the block before's last column, for column 0)
     constexpr int unit = c == 0 ? C - 1 : c - 1;
@@ -345,8 +346,8 @@ __device__ __forceinline__ void attend_unit_ahead(AttnState<C>& st, const QFrag 
       }
     }
   }
-  if (__any(block_max > st.m[c] + kLazyRise)) {  // (see attend_block)
-    float moved = fmaxf(st.m[c], block_max);
+  if (__any(block_max > rise[c])) {  // (see attend_block)
+    float moved = fmaxf(st.m[c], block_max * scale_log2);
     moved = fmaxf(moved, __shfl_xor(moved, 16, kWave));
     moved = fmaxf(moved, __shfl_xor(moved, 32, kWave));
     const float shrink = st.m[c] == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(st.m[c] - moved);
@@ -354,6 +355,7 @@ __device__ __forceinline__ void attend_unit_ahead(AttnState<C>& st, const QFrag 
 #pragma unroll
     for (int t = 0; t < kTilesD; ++t) st.o[c][t] = st.o[c][t] * shrink;
     st.m[c] = moved;
+    rise[c] = (moved + kLazyRise) / scale_log2;
   }
   f32x4 ahead[2];
   if constexpr (c + 1 < C) {
@@ -368,18 +370,18 @@ __device__ __forceinline__ void attend_unit_ahead(AttnState<C>& st, const QFrag 
     for (int t = 0; t < kTilesD; ++t)
       st.o[c - 1][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.values[t], before, st.o[c - 1][t], 0, 0, 0);
   }
-  const float base = st.m[c] == -INFINITY ? 0.0f : st.m[c];
+  // (No key of these blocks is masked: behind the test above the reference is a score's own size, never -inf.)
+  const float base = st.m[c];
   bf16x8 p;
-  float sum = 0.0f;
+  float w[8];
 #pragma unroll
   for (int t = 0; t < 2; ++t)
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      const float w = __builtin_amdgcn_exp2f(fmaf(s[t][e], scale_log2, -base));
-      sum += w;
-      p[4 * t + e] = (__bf16)w;
+      w[4 * t + e] = __builtin_amdgcn_exp2f(fmaf(s[t][e], scale_log2, -base));
+      p[4 * t + e] = (__bf16)w[4 * t + e];
     }
-  st.l[c] += sum;
+  st.l[c] += ((w[0] + w[1]) + (w[2] + w[3])) + ((w[4] + w[5]) + (w[6] + w[7]));
   if constexpr (c + 1 < C) {
     before = p;
   } else {
@@ -390,14 +392,14 @@ __device__ __forceinline__ void attend_unit_ahead(AttnState<C>& st, const QFrag 
     s[0] = ahead[0];
     s[1] = ahead[1];
   }
-  if constexpr (c + 1 < C) attend_unit_ahead<C, AHEAD, c + 1>(st, q, f, next, s, before, scale_log2);
+  if constexpr (c + 1 < C) attend_unit_ahead<C, AHEAD, c + 1>(st, q, f, next, s, before, scale_log2, rise);
 }
 
 template <int C, bool AHEAD>
 __device__ __forceinline__ void attend_block_ahead(AttnState<C>& st, const QFrag (&q)[C], const BlockFrags& f, const BlockFrags& next,
-                                                   f32x4 (&s)[2], float scale_log2) {
+                                                   f32x4 (&s)[2], float scale_log2, float (&rise)[C]) {
   bf16x8 before;  // the probabilities of the column before, whose outputs are still to be multiplied
-  attend_unit_ahead<C, AHEAD, 0>(st, q, f, next, s, before, scale_log2);
+  attend_unit_ahead<C, AHEAD, 0>(st, q, f, next, s, before, scale_log2, rise);
 }
 
 // The pages of a run of key blocks, 64 at a time in the lanes of the wave: a
@@ -605,6 +607,9 @@ __device__ __forceinline__ void attend_run(AttnState<C>& st, const QFrag (&q)[C]
 #pragma unroll
       for (int t = 0; t < 2; ++t) s[t] = score_tile(ring[0].keys[t], q[0]);
     }
+    float rise[C];
+#pragma unroll
+    for (int c = 0; c < C; ++c) rise[c] = (st.m[c] + kLazyRise) / a.scale_log2;  // (-inf before a column's first key)
     for (; b0 + 2 * RING <= blocks && b0 + RING <= inner_end; b0 += RING) {
 #pragma unroll
       for (int i = 0; i < RING; ++i) {
@@ -612,7 +617,7 @@ __device__ __forceinline__ void attend_run(AttnState<C>& st, const QFrag (&q)[C]
 #pragma unroll
           for (int t = 0; t < 2; ++t) s[t] = score_tile(ring[i].keys[t], q[0]);
         }
-        attend_block_ahead<C, kAhead>(st, q, ring[i], ring[(i + 1) % RING], s, a.scale_log2);
+        attend_block_ahead<C, kAhead>(st, q, ring[i], ring[(i + 1) % RING], s, a.scale_log2, rise);
         ask(ring[i], b0 + i + RING);
       }
     }
