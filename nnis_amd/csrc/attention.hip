@@ -536,6 +536,13 @@ template <int C, int RING>
 __device__ __forceinline__ void attend_run(AttnState<C>& st, const QFrag (&q)[C], const MfmaArgs& a, const int* pages,
                                            int kv_head, int first, int stride, int mine, int last_key,
                                            const int (&lo)[C], const int (&hi)[C], int lane) {
+  // (The run's bounds are the same in every lane -- they come from sums over the wave -- but the compiler has them
+  // in vector registers unless it is told: as scalars the loop's counters, the pages' numbers and the pages'
+  // addresses cost no vector instruction, of which the loop has none to spare.)
+  first = __builtin_amdgcn_readfirstlane(first);
+  stride = __builtin_amdgcn_readfirstlane(stride);
+  mine = __builtin_amdgcn_readfirstlane(mine);
+  last_key = __builtin_amdgcn_readfirstlane(last_key);
   if (mine <= 0) return;
   const int r = lane % 16, g = lane / 16;
   const bf16_t* k_base = k_page_ptr(a, 0, kv_head);
@@ -554,7 +561,7 @@ __device__ __forceinline__ void attend_run(AttnState<C>& st, const QFrag (&q)[C]
       run.first = first + n * stride;
       run.fill(lane);
     }
-    const int page = run.page(n & 63);
+    const int page = __builtin_amdgcn_readfirstlane(run.page(n & 63));
     load_block(into, k_base + page * k_page_stride, v_base + page * v_page_stride, b & 1, r, g);
   };
   auto work = [&](const BlockFrags& f, int b) {
@@ -583,6 +590,8 @@ __device__ __forceinline__ void attend_run(AttnState<C>& st, const QFrag (&q)[C]
     every_lo = max(every_lo, __shfl_xor(every_lo, offset, kWave));
     every_hi = min(every_hi, __shfl_xor(every_hi, offset, kWave));
   }
+  every_lo = __builtin_amdgcn_readfirstlane(every_lo);
+  every_hi = __builtin_amdgcn_readfirstlane(every_hi);
   const int whole_pages = (every_hi + 1) / kPageTokens;  // pages 0 .. whole_pages - 1 of the sequence end at or below every_hi
   const int inner_end = whole_pages > first ? 2 * min(mine, (whole_pages - first + stride - 1) / stride) : 0;  // in blocks of the run
   const int low_page = (every_lo + kPageTokens - 1) / kPageTokens;
