@@ -665,7 +665,7 @@ __global__ __launch_bounds__(64 * kBlockWaves) void attention_prefill_kernel(Mfm
                                                                             int per_tile) {
   extern __shared__ __attribute__((aligned(16))) float merge[];
   constexpr int C = QT * GH;
-  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave, r = lane % 16, g = lane / 16;
+  const int lane = threadIdx.x % kWave, wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), r = lane % 16, g = lane / 16;  // (the wave's number as a scalar)
   const int group = a.heads / a.kv_heads;
   const int chunks = (group + GH - 1) / GH;
   // both items' places in the step, asked for together: each is a chain of dependent loads
@@ -832,7 +832,7 @@ __device__ __forceinline__ void finish_decode(AttnState<C>& st, const bool (&liv
 template <int C>
 __global__ __launch_bounds__(64 * kBlockWaves) void attention_decode_kernel(MfmaArgs a, int waves) {
   extern __shared__ __attribute__((aligned(16))) float merge[];  // [waves / 2][C][kTilesD * 4 + 2][64]
-  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave, r = lane % 16, g = lane / 16;
+  const int lane = threadIdx.x % kWave, wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), r = lane % 16, g = lane / 16;  // (the wave's number as a scalar)
   const int token = a.heads_first ? blockIdx.y : blockIdx.x, kv_head = a.heads_first ? blockIdx.x : blockIdx.y, split = blockIdx.z;
   // With the step's tables a token's pages are a row of its own and nothing is asked of its slot: the first
   // pages' numbers are one round trip away, not two.  (A padding row then reads the page its row names, 0,
@@ -906,7 +906,7 @@ __global__ __launch_bounds__(64 * kKeysWaves) void attention_decode_keys_kernel(
   extern __shared__ __attribute__((aligned(16))) float merge[];  // [waves / 2][kTilesD * 4 + 2][64]
   constexpr int kStageRow = kPageTokens + 8;  // bfloat16 per head: a page's probabilities, rows apart in the banks
   __shared__ __attribute__((aligned(16))) bf16_t stage[kKeysWaves][4][kStageRow];
-  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave, r = lane % 16, g = lane / 16;
+  const int lane = threadIdx.x % kWave, wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), r = lane % 16, g = lane / 16;  // (the wave's number as a scalar)
   const int blk = lane / 4, j = lane % 4;  // the scores' layout: keys 4 blk .. 4 blk + 3 of a page, head j of the group
   const int token = a.heads_first ? blockIdx.y : blockIdx.x, kv_head = a.heads_first ? blockIdx.x : blockIdx.y, split = blockIdx.z;
   int slot = 0;
@@ -955,7 +955,7 @@ __global__ __launch_bounds__(64 * kKeysWaves) void attention_decode_keys_kernel(
         run.first = first + n * stride;
         run.fill(lane);
       }
-      const int page = run.page(n & 63);
+      const int page = __builtin_amdgcn_readfirstlane(run.page(n & 63));
       load_keys_page(into, k_base + page * k_page_stride, v_base + page * v_page_stride, lane);
     };
     bf16_t* mine_stage = &stage[wave][0][0];
